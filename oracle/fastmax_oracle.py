@@ -1,0 +1,343 @@
+"""CPU oracle for the Fastmax attention hot path.  TEST INFRASTRUCTURE ONLY.
+
+Nothing in the shipped package may import this module: it is the checker used by
+``tests/``, by ``__graft_entry__.smoke()`` and by the ``cpu_baseline`` leg of
+``bench.py``.  The product path is the HIP library and fails loudly without it.
+
+Two independent restatements of the reference's algorithm live here:
+
+* ``closed_form_*`` - the quadratic definition ``o = (M . f(QK^T/tau)) V / rowsum``
+  with ``f(s) = a0 + a1 s + a2 s^2``.  This is what the reference's own unit
+  tests build as ground truth (``test/test_einops_fastmax.py:25-75``) and what
+  ``fastattention_einops.compute_attn`` computes
+  (``attention_mechanisms/fastattention_einops.py:337-381``).  Gradients come
+  from torch autograd through that definition, which is how the reference pins
+  its hand-written backward (``gradcheck``, ``test/test_einops_fastmax.py:131-225``).
+* ``factorised_*`` - the linear-time moment algorithm, following the operation
+  sequence of the reference's einops implementation (einsum -> cumsum -> einsum,
+  ``fastattention_einops.py:186-322`` forward, ``:384-691`` backward).  It is
+  the timed CPU baseline (kind "port").
+
+Pinning (see tests/test_oracle.py): factorised == closed form in float64 to
+1e-9; factorised backward == autograd of the closed form; closed form ==
+pure-Python triple loops on tiny inputs; invariants that a dropped term, wrong
+sign or transposed operand would break (causality, o_0 = v_0, constant v,
+a1 = a2 = 0 running mean, key-permutation invariance, value linearity).
+Functions whose parity is unpinned: none of the numerical ones; the random
+feature dropout of ``score_function.py:84-86`` is out of scope (dropout_rate=0).
+
+Conventions.  ``tau`` is the divisor of the score: the einops front uses
+``normalize_term * sqrt(D)`` (``fastattention_einops.py:79-82``), the
+``score_function.fastmax`` front uses ``denum_term * sqrt(D)``
+(``score_function.py:57``) and the extension divides k by ``temperature``
+(``fastmax_cuda_forward.cu:288``).  Shapes are ``(B, H, N, D)`` unless said.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+
+__all__ = [
+    "tau_einops", "closed_form_forward", "closed_form_forward_backward",
+    "manual_backward_blocked", "factorised_forward", "factorised_backward",
+    "extension_forward", "extension_backward", "score_function_fastmax",
+    "normalize_feature_mean", "normalize_token_mean", "normalize_lim",
+    "rel_l2",
+]
+
+
+def rel_l2(a: torch.Tensor, b: torch.Tensor) -> float:
+    """||a-b||_2 / ||b||_2 in float64 (the parity metric of the whole project)."""
+    a = a.detach().double().cpu()
+    b = b.detach().double().cpu()
+    return float((a - b).norm() / b.norm().clamp_min(1e-300))
+
+
+def tau_einops(normalize_term: float, d: int, tensors_normalized: bool = False) -> float:
+    """Score divisor of the einops front (``fastattention_einops.py:78-82``)."""
+    return 1.0 if tensors_normalized else normalize_term * math.sqrt(d)
+
+
+def _coeffs(p: int, a0: float, a1: float, a2: float) -> Tuple[float, float, float]:
+    if p == 1:
+        return a0, a1, 0.0
+    if p == 2:
+        return a0, a1, a2
+    raise ValueError(f"p must be 1 or 2, got p={p}")
+
+
+# --------------------------------------------------------------------------
+# Quadratic closed form (ground truth)
+# --------------------------------------------------------------------------
+def closed_form_forward(q, k, v, *, mask: bool, tau: float, p: int = 2,
+                        a0: float = 1.0, a1: float = 1.0, a2: float = 0.5,
+                        return_attn: bool = False):
+    """``o_i = sum_j M_ij f(s_ij) v_j / g_i``, ``g_i = sum_j M_ij f(s_ij)``.
+
+    With ``nk >= nq`` and ``mask`` the queries are aligned to the tail of the
+    keys: query ``i`` sees keys ``0 .. nk-nq+i``
+    (``fastmax_cuda_forward.cu:160-172``).  Returns ``(o, g)`` (and the
+    row-normalised attention matrix if asked, ``fastattention_einops.py:337-381``).
+    """
+    c0, c1, c2 = _coeffs(p, a0, a1, a2)
+    s = torch.matmul(q, k.transpose(-1, -2)) / tau
+    f = c0 + c1 * s + c2 * s * s
+    if mask:
+        nq, nk = q.shape[-2], k.shape[-2]
+        keep = torch.ones(nq, nk, dtype=torch.bool, device=q.device).tril(diagonal=nk - nq)
+        f = f * keep.to(f.dtype)
+    g = f.sum(-1)
+    o = torch.matmul(f, v) / g.unsqueeze(-1)
+    if return_attn:
+        return o, g, f / g.unsqueeze(-1)
+    return o, g
+
+
+def closed_form_forward_backward(q, k, v, d_o, *, mask: bool, tau: float, p: int = 2,
+                                 a0: float = 1.0, a1: float = 1.0, a2: float = 0.5,
+                                 dtype=torch.float64):
+    """Forward plus torch-autograd gradients of the closed form, computed in
+    ``dtype`` (float64 by default), one (b, h) slice at a time so that the
+    ``N x N`` score matrix of a single head is the largest temporary."""
+    shape = q.shape
+    qf = q.reshape(-1, shape[-2], shape[-1]).to(dtype)
+    kf = k.reshape(-1, k.shape[-2], k.shape[-1]).to(dtype)
+    vf = v.reshape(-1, v.shape[-2], v.shape[-1]).to(dtype)
+    gf = d_o.reshape(-1, d_o.shape[-2], d_o.shape[-1]).to(dtype)
+    outs, gs, dqs, dks, dvs = [], [], [], [], []
+    for i in range(qf.shape[0]):
+        qi = qf[i].clone().requires_grad_(True)
+        ki = kf[i].clone().requires_grad_(True)
+        vi = vf[i].clone().requires_grad_(True)
+        o, g = closed_form_forward(qi, ki, vi, mask=mask, tau=tau, p=p, a0=a0, a1=a1, a2=a2)
+        dq, dk, dv = torch.autograd.grad(o, (qi, ki, vi), gf[i])
+        outs.append(o.detach()); gs.append(g.detach())
+        dqs.append(dq); dks.append(dk); dvs.append(dv)
+    o = torch.stack(outs).reshape(*shape[:-1], v.shape[-1])
+    g = torch.stack(gs).reshape(shape[:-1])
+    return (o, g, torch.stack(dqs).reshape(shape), torch.stack(dks).reshape(k.shape),
+            torch.stack(dvs).reshape(v.shape))
+
+
+def manual_backward_blocked(q, k, v, d_o, *, mask: bool, tau: float, p: int = 2,
+                            a0: float = 1.0, a1: float = 1.0, a2: float = 0.5,
+                            block: int = 1024, dtype=torch.float64):
+    """Row-blocked closed form with the analytic gradient
+
+        ghat_i = dO_i / g_i,  c_i = ghat_i . o_i,
+        dS_ij  = M_ij f'(s_ij) (ghat_i . v_j - c_i),   f'(s) = a1 + 2 a2 s,
+        dQ = dS K / tau,  dK = dS^T Q / tau,  dV = (M . f(S))^T ghat,
+
+    for sequences whose full score matrix does not fit.  Pinned against
+    ``closed_form_forward_backward`` in the tests.  Shapes ``(BH, N, D)`` or
+    ``(B, H, N, D)``; requires ``nq == nk`` when masked.
+    """
+    c0, c1, c2 = _coeffs(p, a0, a1, a2)
+    shape = q.shape
+    qf = q.reshape(-1, shape[-2], shape[-1]).to(dtype)
+    kf = k.reshape(-1, k.shape[-2], k.shape[-1]).to(dtype)
+    vf = v.reshape(-1, v.shape[-2], v.shape[-1]).to(dtype)
+    gf = d_o.reshape(-1, d_o.shape[-2], d_o.shape[-1]).to(dtype)
+    nq, nk = qf.shape[1], kf.shape[1]
+    o = torch.empty(qf.shape[0], nq, vf.shape[2], dtype=dtype)
+    g = torch.empty(qf.shape[0], nq, dtype=dtype)
+    dq = torch.zeros_like(qf); dk = torch.zeros_like(kf); dv = torch.zeros_like(vf)
+    for r0 in range(0, nq, block):
+        r1 = min(nq, r0 + block)
+        hi = nk if not mask else min(nk, nk - nq + r1)
+        qs = qf[:, r0:r1]
+        ks, vs = kf[:, :hi], vf[:, :hi]
+        s = torch.matmul(qs, ks.transpose(1, 2)) / tau
+        f = c0 + c1 * s + c2 * s * s
+        fp = c1 + 2.0 * c2 * s
+        if mask:
+            rows = torch.arange(r0, r1).unsqueeze(1) + (nk - nq)
+            keep = (torch.arange(hi).unsqueeze(0) <= rows).to(dtype)
+            f = f * keep
+            fp = fp * keep
+        gb = f.sum(-1)
+        ob = torch.matmul(f, vs) / gb.unsqueeze(-1)
+        gh = gf[:, r0:r1] / gb.unsqueeze(-1)
+        cb = (gh * ob).sum(-1, keepdim=True)
+        ds = fp * (torch.matmul(gh, vs.transpose(1, 2)) - cb)
+        dq[:, r0:r1] = torch.matmul(ds, ks) / tau
+        dk[:, :hi] += torch.matmul(ds.transpose(1, 2), qs) / tau
+        dv[:, :hi] += torch.matmul(f.transpose(1, 2), gh)
+        o[:, r0:r1] = ob
+        g[:, r0:r1] = gb
+    return (o.reshape(*shape[:-1], v.shape[-1]), g.reshape(shape[:-1]),
+            dq.reshape(shape), dk.reshape(k.shape), dv.reshape(v.shape))
+
+
+# --------------------------------------------------------------------------
+# Factorised (moment) algorithm - the reference's linear-time path
+# --------------------------------------------------------------------------
+def _rev_cumsum(x: torch.Tensor, dim: int) -> torch.Tensor:
+    """Suffix sums (the reference indexes with a reversed arange,
+    ``fastattention_einops.py:565-567``)."""
+    return torch.flip(torch.cumsum(torch.flip(x, (dim,)), dim), (dim,))
+
+
+def factorised_forward(q, k, v, *, mask: bool, tau: float, p: int = 2):
+    """Numerator F and denominator g from key/value moments, Taylor coefficients
+    (1, 1, 1/2).  Unmasked: global moments (``fastattention_einops.py:186-217,
+    253-284``).  Masked: per-token outer products, cumsum over the sequence,
+    contraction with q (``:219-250, 286-322``) - this materialises
+    ``(B, H, N, D, D, Dv)`` for p=2 exactly as the reference does.
+    Returns ``(o, g)``."""
+    if p not in (1, 2):
+        raise ValueError(f"p must be 1 or 2, got p={p}")
+    b, h, n, d = q.shape
+    if not mask:
+        nk = k.shape[2]
+        num = v.sum(2, keepdim=True).expand(b, h, n, v.shape[3])
+        kv = torch.einsum("bhnm,bhnj->bhmj", k, v)
+        num = num + torch.einsum("bhim,bhmj->bhij", q, kv) / tau
+        den = torch.full((b, h, n), float(nk), dtype=q.dtype, device=q.device)
+        den = den + torch.einsum("bhil,bhl->bhi", q, k.sum(2)) / tau
+        if p == 2:
+            kkv = torch.einsum("bhnm,bhnl,bhnj->bhmlj", k, k, v)
+            num = num + torch.einsum("bhim,bhil,bhmlj->bhij", q, q, kkv) / (2 * tau ** 2)
+            kk = torch.einsum("bhnl,bhnp->bhlp", k, k)
+            den = den + torch.einsum("bhil,bhip,bhlp->bhi", q, q, kk) / (2 * tau ** 2)
+    else:
+        num = torch.cumsum(v, 2)
+        kv = torch.cumsum(torch.einsum("bhnm,bhnj->bhnmj", k, v), 2)
+        num = num + torch.einsum("bhim,bhimj->bhij", q, kv) / tau
+        den = (torch.arange(n, device=q.device) + 1).to(q.dtype).expand(b, h, n)
+        den = den + torch.einsum("bhim,bhim->bhi", q, torch.cumsum(k, 2)) / tau
+        if p == 2:
+            kkv = torch.cumsum(torch.einsum("bhnm,bhnl,bhnj->bhnmlj", k, k, v), 2)
+            num = num + torch.einsum("bhim,bhil,bhimlj->bhij", q, q, kkv) / (2 * tau ** 2)
+            kk = torch.cumsum(torch.einsum("bhnm,bhnl->bhnml", k, k), 2)
+            den = den + torch.einsum("bhim,bhil,bhiml->bhi", q, q, kk) / (2 * tau ** 2)
+    return num / den.unsqueeze(-1), den
+
+
+def factorised_backward(q, k, v, o, g, d_o, *, mask: bool, tau: float, p: int = 2):
+    """Hand-factorised gradients (``fastattention_einops.py:384-691``).
+
+    With ``gh = dO / g`` and ``c = sum_j gh_j o_j``:
+      dQ uses prefix (or global) moments of k (x) v and k (x) k (``:384-485``),
+      dK and dV use suffix (or global) moments of q (x) gh and q (x) q (x) gh
+      (``:487-691``).  Returns ``(dq, dk, dv)``.
+    """
+    if p not in (1, 2):
+        raise ValueError(f"Expected p = 1 or 2, got p = {p}")
+    gh = d_o / g.unsqueeze(-1)
+    c = (gh * o).sum(-1)
+    if not mask:
+        kv = torch.einsum("bhlr,bhlj->bhrj", k, v)
+        dq = torch.einsum("bhpj,bhrj->bhpr", gh, kv) - c.unsqueeze(-1) * k.sum(2, keepdim=True)
+        qg = torch.einsum("bhir,bhij->bhrj", q, gh)
+        dk = torch.einsum("bhpj,bhrj->bhpr", v, qg) - torch.einsum("bhi,bhir->bhr", c, q).unsqueeze(2)
+        dv = gh.sum(2, keepdim=True) + torch.einsum("bhpm,bhmr->bhpr", k, qg) / tau
+        if p == 2:
+            kkv = torch.einsum("bhlm,bhlr,bhlj->bhmrj", k, k, v)
+            kk = torch.einsum("bhlm,bhlr->bhmr", k, k)
+            dq = dq + (torch.einsum("bhpm,bhpj,bhmrj->bhpr", q, gh, kkv)
+                       - c.unsqueeze(-1) * torch.einsum("bhpm,bhmr->bhpr", q, kk)) / tau
+            qqg = torch.einsum("bhim,bhir,bhij->bhmrj", q, q, gh)
+            qqc = torch.einsum("bhi,bhim,bhir->bhmr", c, q, q)
+            dk = dk + (torch.einsum("bhpm,bhpj,bhmrj->bhpr", k, v, qqg)
+                       - torch.einsum("bhpm,bhmr->bhpr", k, qqc)) / tau
+            dv = dv + torch.einsum("bhpm,bhpl,bhmlr->bhpr", k, k, qqg) / (2 * tau ** 2)
+        dv = dv.expand_as(v) if dv.shape != v.shape else dv
+        return dq / tau, dk / tau, dv.contiguous()
+    kv = torch.cumsum(torch.einsum("bhlj,bhlr->bhljr", v, k), 2)
+    dq = torch.einsum("bhpj,bhpjr->bhpr", gh, kv) - c.unsqueeze(-1) * torch.cumsum(k, 2)
+    qg = _rev_cumsum(torch.einsum("bhij,bhir->bhijr", gh, q), 2)
+    dk = torch.einsum("bhpj,bhpjr->bhpr", v, qg) - _rev_cumsum(c.unsqueeze(-1) * q, 2)
+    dv = _rev_cumsum(gh, 2) + torch.einsum("bhpm,bhprm->bhpr", k, qg) / tau
+    if p == 2:
+        kvk = torch.cumsum(torch.einsum("bhlm,bhlj,bhlr->bhlmjr", k, v, k), 2)
+        kk = torch.cumsum(torch.einsum("bhlr,bhlm->bhlrm", k, k), 2)
+        dq = dq + (torch.einsum("bhpm,bhpj,bhpmjr->bhpr", q, gh, kvk)
+                   - c.unsqueeze(-1) * torch.einsum("bhpm,bhprm->bhpr", q, kk)) / tau
+        gqq = _rev_cumsum(torch.einsum("bhij,bhim,bhir->bhijmr", gh, q, q), 2)
+        cqq = _rev_cumsum(torch.einsum("bhi,bhim,bhir->bhimr", c, q, q), 2)
+        dk = dk + (torch.einsum("bhpm,bhpj,bhpjmr->bhpr", k, v, gqq)
+                   - torch.einsum("bhpm,bhpmr->bhpr", k, cqq)) / tau
+        dv = dv + torch.einsum("bhpm,bhpl,bhprml->bhpr", k, k, gqq) / (2 * tau ** 2)
+    return dq / tau, dk / tau, dv
+
+
+# --------------------------------------------------------------------------
+# The two API fronts restated on top of the closed form
+# --------------------------------------------------------------------------
+def extension_forward(q, k, v, *, mask: bool, temperature: float, a0: float, a1: float,
+                      a2: float, p: int, dtype=torch.float64):
+    """Semantics of ``fastmax_cuda.forwardpass`` with ``normalize=False``
+    (``fastmax_cuda_forward.cu:366-456``): layout ``(n, bh, d)``, k divided by
+    the temperature, result ``(nq, bh, d+1)`` whose last column is g."""
+    qq = q.permute(1, 0, 2).to(dtype)
+    kk = k.permute(1, 0, 2).to(dtype)
+    vv = v.permute(1, 0, 2).to(dtype)
+    o, g = closed_form_forward(qq, kk, vv, mask=mask, tau=float(temperature), p=p,
+                               a0=a0, a1=a1, a2=a2)
+    return torch.cat([o, g.unsqueeze(-1)], dim=-1).permute(1, 0, 2).contiguous()
+
+
+def extension_backward(q, k_scaled, v, d_o, *, mask: bool, a0: float, a1: float, a2: float,
+                       p: int, dtype=torch.float64):
+    """Semantics of ``fastmax_cuda.backwardpass``
+    (``fastmax_cuda_backward.cu:518-613``): q and k are the tensors as left by
+    the forward (k already divided by the temperature), so the score is their
+    plain dot product and gradients are with respect to those tensors.
+    Layout ``(n, bh, d)``.  Returns ``(gradq, gradk, gradv)``."""
+    qq = q.permute(1, 0, 2); kk = k_scaled.permute(1, 0, 2)
+    vv = v.permute(1, 0, 2); gg = d_o.permute(1, 0, 2)
+    _, _, dq, dk, dv = closed_form_forward_backward(qq, kk, vv, gg, mask=mask, tau=1.0, p=p,
+                                                    a0=a0, a1=a1, a2=a2, dtype=dtype)
+    return tuple(t.permute(1, 0, 2).contiguous() for t in (dq, dk, dv))
+
+
+def normalize_feature_mean(q, k):
+    """``fastattention_einops.normalize`` (``fastattention_einops.py:324-334``):
+    subtract the mean over the feature axis, divide by the largest token norm
+    of each (b, h)."""
+    def one(x):
+        x = x - x.mean(-1, keepdim=True)
+        return x / torch.linalg.vector_norm(x, dim=-1).amax(-1)[..., None, None]
+    return one(q), one(k)
+
+
+def normalize_token_mean(q, k):
+    """``score_function.fastmax(normalize=1)`` (``score_function.py:40-55``):
+    subtract the mean over the token axis, divide by the largest token norm."""
+    def one(x):
+        x = x - x.mean(-2, keepdim=True)
+        return x / torch.linalg.vector_norm(x, dim=-1).amax(-1)[..., None, None]
+    return one(q), one(k)
+
+
+def normalize_lim(x, lim: float = 1.0):
+    """Intended semantics of the extension's ``normalize`` flag as written out in
+    ``transformer/model.py:97-102``: ``lim * x / max_n ||x_n||_2``, no centring."""
+    return lim * x / torch.linalg.vector_norm(x, dim=-1).amax(-1)[..., None, None]
+
+
+def score_function_fastmax(q, k, v, mask=None, denum_term=8, normalize=0, p=1,
+                           create_attn_matrix=False, dropout_rate=0):
+    """``attention_mechanisms/score_function.py:7-248`` restated on the closed
+    form (dropout_rate must be 0).  ``normalize == 1`` centres over tokens and
+    max-normalises, then uses tau = 1 (``:40-55``); otherwise
+    tau = denum_term * sqrt(D) (``:57``).  ``create_attn_matrix`` also returns
+    the row-normalised attention matrix (``:226-247``; that debug branch always
+    uses the quadratic kernel and tau = denum_term * sqrt(D))."""
+    if dropout_rate:
+        raise ValueError("the oracle covers dropout_rate=0 only")
+    if create_attn_matrix:
+        tau = denum_term * math.sqrt(q.shape[-1])
+        o, _, a = closed_form_forward(q, k, v, mask=bool(mask is not None and mask), tau=tau,
+                                      p=2, return_attn=True)
+        return o, a
+    if normalize == 1:
+        q, k = normalize_token_mean(q, k)
+        tau = 1.0
+    else:
+        tau = denum_term * math.sqrt(q.shape[-1])
+    o, _ = closed_form_forward(q, k, v, mask=bool(mask is not None and mask), tau=tau, p=p)
+    return o
