@@ -1,0 +1,116 @@
+/* C ABI of libfastmax_hip.so: the Fastmax attention hot path on MI355X (gfx950).
+ *
+ * Plain pointers and sizes only; no torch types.  Every entry point enqueues
+ * work on the given HIP stream and returns without synchronising.  Inputs are
+ * never written.  All functions are re-entrant; the library keeps no mutable
+ * global state besides per-kernel launch attributes.
+ *
+ * Tensors are addressed as (bh, n, d) through two element strides per tensor
+ * (the feature axis is contiguous), so the reference extension's (n, bh, d)
+ * layout and the model's (b, h, n, d) layout are both accepted without copies.
+ */
+#ifndef FASTMAX_HIP_H_
+#define FASTMAX_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  FASTMAX_OK = 0,
+  FASTMAX_ERR_NULL = 1,          /* a required pointer is null */
+  FASTMAX_ERR_SHAPE = 2,         /* sizes or strides are not valid */
+  FASTMAX_ERR_UNSUPPORTED = 3,   /* valid, but not implemented (head size, order, masked nk != nq) */
+  FASTMAX_ERR_WORKSPACE = 4,     /* workspace missing, too small or misaligned */
+  FASTMAX_ERR_LAUNCH = 5,        /* the HIP runtime refused a launch */
+  FASTMAX_ERR_DTYPE = 6          /* unknown element type */
+};
+
+enum { FASTMAX_F32 = 0, FASTMAX_BF16 = 1 };
+
+/* flags */
+enum {
+  FASTMAX_FLAG_FORCE_MOMENTS = 1,   /* unmasked: always use the moment (linear-time) path */
+  FASTMAX_FLAG_FORCE_DENSE = 2      /* never build moment states (quadratic-time path) */
+};
+
+typedef struct FastmaxStrides {
+  int64_t bh;   /* elements between consecutive batch*head slices */
+  int64_t n;    /* elements between consecutive tokens */
+} FastmaxStrides;
+
+/* Problem description shared by forward and backward.
+ * Score s_ij = (q_i . k_j) * inv_tau;  weight f(s) = a0 + a1 s + a2 s^2 (a2 ignored when p == 1);
+ * mask != 0: causal, query i sees keys 0..i (requires nq == nk). */
+typedef struct FastmaxDesc {
+  int32_t bh;        /* batch * heads */
+  int32_t nq, nk;    /* query and key/value tokens */
+  int32_t d;         /* head size, D == Dv; 32 or 64 */
+  int32_t dtype;     /* FASTMAX_F32 or FASTMAX_BF16: element type of q,k,v,o,dO,dq,dk,dv */
+  int32_t mask;
+  int32_t p;         /* 1 or 2 */
+  float a0, a1, a2;
+  float inv_tau;
+  int32_t chunk;     /* segment length of the causal moment scan; 0 = automatic */
+  int32_t flags;
+  FastmaxStrides sq, sk, sv, so, sg, sdo, sdq, sdk, sdv;   /* sg: strides of the fp32 denominator g (bh, n) */
+} FastmaxDesc;
+
+/* Replaces the tensor allocations inside forward_cuda / backward_cuda
+ * (reference fastmax_cuda_forward.cu:404-414, fastmax_cuda_backward.cu:563-571):
+ * the caller owns all memory and asks here how much scratch a call needs. */
+int fastmax_workspace_bytes(const FastmaxDesc* desc, size_t* forward_bytes, size_t* backward_bytes);
+
+/* Replaces forward_cuda (reference fastmax_cuda.cpp:17-24 -> fastmax_cuda_forward.cu:366-456):
+ * o (dtype) and the denominator g (fp32) for every query.  The reference returns both in one
+ * (nq, bh, d+1) tensor; that layout is expressed by pointing g at column d of that tensor
+ * with strides (d+1, bh*(d+1)).  workspace: >= forward_bytes, 256-byte aligned device memory. */
+int fastmax_forward(const FastmaxDesc* desc, const void* q, const void* k, const void* v,
+                    void* o, float* g, void* workspace, size_t workspace_bytes, void* hip_stream);
+
+/* Replaces backward_cuda (reference fastmax_cuda.cpp:26-32 -> fastmax_cuda_backward.cu:518-613):
+ * gradients of sum(o * dO) with respect to q, k and v, where s_ij = (q_i . k_j) * inv_tau.
+ * o and g are the forward results.  d_o is not modified (the reference divides it by g in place,
+ * fastmax_cuda_backward.cu:494-501). */
+int fastmax_backward(const FastmaxDesc* desc, const void* q, const void* k, const void* v,
+                     const void* o, const float* g, const void* d_o,
+                     void* dq, void* dk, void* dv,
+                     void* workspace, size_t workspace_bytes, void* hip_stream);
+
+/* Fused normalisation pass over one (bh, n, d) tensor.  Replaces apply_rpe_and_temp, calc_norms,
+ * find_max and apply_norm (reference fastmax_cuda_forward.cu:282-338) with the semantics the
+ * Python variants define:
+ *   y = scale * (x - centre) / max_n || x_n - centre ||_2     when max_norm != 0
+ *   y = scale * (x - centre)                                   otherwise
+ * centre: 0 none; 1 mean over the feature axis (fastattention_einops.py:327-334);
+ *         2 mean over the token axis (score_function.py:42-47).
+ * x and y may be the same buffer with the same strides.
+ * stats: device pointer to bh*(d+2) floats of scratch, or null when max_norm == 0 and centre != 2. */
+typedef struct FastmaxNormDesc {
+  int32_t bh, n, d;
+  int32_t dtype;
+  int32_t centre;
+  int32_t max_norm;
+  float scale;
+  FastmaxStrides sx, sy;
+} FastmaxNormDesc;
+int fastmax_normalize(const FastmaxNormDesc* desc, const void* x, void* y, float* stats,
+                      void* hip_stream);
+
+const char* fastmax_status_string(int status);
+
+/* Library version: major * 10000 + minor * 100 + patch. */
+int fastmax_version(void);
+
+/* Self-check of the matrix-core lane layout the kernels assume: runs one 32x32 MFMA tile per
+ * element type on known operands and writes, for each of the 64 lanes and 16 accumulator
+ * registers, the value found (out_f16 and out_f32: 1024 floats each, device memory). */
+int fastmax_probe_mfma(float* out_f16, float* out_f32, void* hip_stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FASTMAX_HIP_H_ */

@@ -1,0 +1,211 @@
+"""ctypes view of the C ABI declared in ``include/fastmax_hip.h``.
+
+This is plumbing: it turns torch tensors into (pointer, strides) pairs, asks the
+library how much scratch a call needs, allocates it with torch and passes torch's
+current HIP stream.  There is no fallback: if ``libfastmax_hip.so`` has not been
+built, importing the operator fails with an ImportError that says so.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import threading
+from typing import Optional, Tuple
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_NAME = "libfastmax_hip.so"
+
+F32, BF16 = 0, 1
+FLAG_FORCE_MOMENTS, FLAG_FORCE_DENSE = 1, 2
+STATUS_OK = 0
+
+
+class Strides(C.Structure):
+    _fields_ = [("bh", C.c_int64), ("n", C.c_int64)]
+
+
+class Desc(C.Structure):
+    _fields_ = [
+        ("bh", C.c_int32), ("nq", C.c_int32), ("nk", C.c_int32), ("d", C.c_int32),
+        ("dtype", C.c_int32), ("mask", C.c_int32), ("p", C.c_int32),
+        ("a0", C.c_float), ("a1", C.c_float), ("a2", C.c_float), ("inv_tau", C.c_float),
+        ("chunk", C.c_int32), ("flags", C.c_int32),
+        ("sq", Strides), ("sk", Strides), ("sv", Strides), ("so", Strides), ("sg", Strides),
+        ("sdo", Strides), ("sdq", Strides), ("sdk", Strides), ("sdv", Strides),
+    ]
+
+
+class NormDesc(C.Structure):
+    _fields_ = [
+        ("bh", C.c_int32), ("n", C.c_int32), ("d", C.c_int32), ("dtype", C.c_int32),
+        ("centre", C.c_int32), ("max_norm", C.c_int32), ("scale", C.c_float),
+        ("sx", Strides), ("sy", Strides),
+    ]
+
+
+EXPORTS = (
+    "fastmax_workspace_bytes", "fastmax_forward", "fastmax_backward", "fastmax_normalize",
+    "fastmax_status_string", "fastmax_version", "fastmax_probe_mfma",
+)
+
+
+class FastmaxError(RuntimeError):
+    pass
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return F32
+    if t.dtype == torch.bfloat16:
+        return BF16
+    raise FastmaxError(f"fastmax: dtype must be float32 or bfloat16, got {t.dtype}")
+
+
+def _strides(t: torch.Tensor) -> Strides:
+    if t.dim() != 3:
+        raise FastmaxError("fastmax: expected a (bh, n, d) view")
+    if t.shape[2] > 1 and t.stride(2) != 1:
+        raise FastmaxError("fastmax: the feature axis must be contiguous")
+    return Strides(t.stride(0), t.stride(1))
+
+
+class FastmaxLib:
+    """One loaded copy of the shared library."""
+
+    def __init__(self, path: Optional[str] = None):
+        path = path or os.path.join(_HERE, LIB_NAME)
+        if not os.path.exists(path):
+            raise ImportError(
+                f"{path} not found: build it with `python __graft_entry__.py` "
+                "(hipcc --offload-arch=gfx950); there is no CPU fallback")
+        self.path = path
+        self.lib = C.CDLL(path)
+        L = self.lib
+        L.fastmax_workspace_bytes.argtypes = [C.POINTER(Desc), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+        L.fastmax_workspace_bytes.restype = C.c_int
+        L.fastmax_forward.argtypes = [C.POINTER(Desc)] + [C.c_void_p] * 6 + [C.c_size_t, C.c_void_p]
+        L.fastmax_forward.restype = C.c_int
+        L.fastmax_backward.argtypes = [C.POINTER(Desc)] + [C.c_void_p] * 10 + [C.c_size_t, C.c_void_p]
+        L.fastmax_backward.restype = C.c_int
+        L.fastmax_normalize.argtypes = [C.POINTER(NormDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.fastmax_normalize.restype = C.c_int
+        L.fastmax_status_string.argtypes = [C.c_int]
+        L.fastmax_status_string.restype = C.c_char_p
+        L.fastmax_version.restype = C.c_int
+        L.fastmax_probe_mfma.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+        L.fastmax_probe_mfma.restype = C.c_int
+
+    # -- helpers ---------------------------------------------------------------
+    def status_string(self, st: int) -> str:
+        return self.lib.fastmax_status_string(st).decode()
+
+    def check(self, st: int, what: str) -> None:
+        if st != STATUS_OK:
+            raise FastmaxError(f"{what}: {self.status_string(st)} (status {st})")
+
+    @staticmethod
+    def _stream(t: torch.Tensor) -> int:
+        if t.is_cuda:
+            return torch.cuda.current_stream(t.device).cuda_stream
+        return 0
+
+    def make_desc(self, q, k, v, *, mask, inv_tau, a0, a1, a2, p, chunk=0, flags=0) -> Desc:
+        d = Desc()
+        d.bh, d.nq, d.d = q.shape
+        d.nk = k.shape[1]
+        if k.shape[0] != d.bh or v.shape[0] != d.bh or k.shape[2] != d.d or v.shape[2] != d.d or v.shape[1] != d.nk:
+            raise FastmaxError("fastmax: q, k, v must be (bh, nq, d), (bh, nk, d), (bh, nk, d)")
+        d.dtype = _dtype_code(q)
+        if k.dtype != q.dtype or v.dtype != q.dtype:
+            raise FastmaxError("fastmax: q, k, v must share one dtype")
+        d.mask, d.p = int(bool(mask)), int(p)
+        d.a0, d.a1, d.a2, d.inv_tau = float(a0), float(a1), float(a2), float(inv_tau)
+        d.chunk, d.flags = int(chunk), int(flags)
+        d.sq, d.sk, d.sv = _strides(q), _strides(k), _strides(v)
+        return d
+
+    def workspace_bytes(self, desc: Desc) -> Tuple[int, int]:
+        f, b = C.c_size_t(0), C.c_size_t(0)
+        self.check(self.lib.fastmax_workspace_bytes(C.byref(desc), C.byref(f), C.byref(b)), "fastmax_workspace_bytes")
+        return f.value, b.value
+
+    @staticmethod
+    def _workspace(nbytes: int, device) -> torch.Tensor:
+        # torch allocations are at least 256-byte aligned on the device; on the CPU
+        # (host simulator) over-allocate and slice to an aligned start
+        buf = torch.empty(nbytes + 256, dtype=torch.uint8, device=device)
+        off = (-buf.data_ptr()) % 256
+        return buf[off:off + nbytes]
+
+    # -- entry points ------------------------------------------------------------
+    def forward(self, q, k, v, *, mask, inv_tau, a0=1.0, a1=1.0, a2=0.5, p=2, chunk=0, flags=0,
+                out: Optional[torch.Tensor] = None, g: Optional[torch.Tensor] = None):
+        """q (bh, nq, d), k, v (bh, nk, d) views with contiguous features.
+        Returns (o, g): o like q, g (bh, nq) float32."""
+        desc = self.make_desc(q, k, v, mask=mask, inv_tau=inv_tau, a0=a0, a1=a1, a2=a2, p=p, chunk=chunk, flags=flags)
+        if out is None:
+            out = torch.empty((desc.bh, desc.nq, desc.d), dtype=q.dtype, device=q.device)
+        if g is None:
+            g = torch.empty((desc.bh, desc.nq), dtype=torch.float32, device=q.device)
+        desc.so = _strides(out)
+        desc.sg = Strides(g.stride(0), g.stride(1))
+        fwd, _ = self.workspace_bytes(desc)
+        ws = self._workspace(fwd, q.device)
+        st = self.lib.fastmax_forward(C.byref(desc), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                      g.data_ptr(), ws.data_ptr(), fwd, self._stream(q))
+        self.check(st, "fastmax_forward")
+        return out, g
+
+    def backward(self, q, k, v, o, g, d_o, *, mask, inv_tau, a0=1.0, a1=1.0, a2=0.5, p=2, chunk=0, flags=0):
+        """Gradients (dq, dk, dv) of sum(o * d_o); all tensors are (bh, n, d) views."""
+        desc = self.make_desc(q, k, v, mask=mask, inv_tau=inv_tau, a0=a0, a1=a1, a2=a2, p=p, chunk=chunk, flags=flags)
+        if o.dtype != q.dtype or d_o.dtype != q.dtype or g.dtype != torch.float32:
+            raise FastmaxError("fastmax: o and d_o must have q's dtype and g must be float32")
+        dq = torch.empty((desc.bh, desc.nq, desc.d), dtype=q.dtype, device=q.device)
+        dk = torch.empty((desc.bh, desc.nk, desc.d), dtype=q.dtype, device=q.device)
+        dv = torch.empty((desc.bh, desc.nk, desc.d), dtype=q.dtype, device=q.device)
+        desc.so, desc.sdo = _strides(o), _strides(d_o)
+        desc.sg = Strides(g.stride(0), g.stride(1))
+        desc.sdq, desc.sdk, desc.sdv = _strides(dq), _strides(dk), _strides(dv)
+        _, bwd = self.workspace_bytes(desc)
+        ws = self._workspace(bwd, q.device)
+        st = self.lib.fastmax_backward(C.byref(desc), q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                       g.data_ptr(), d_o.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                                       ws.data_ptr(), bwd, self._stream(q))
+        self.check(st, "fastmax_backward")
+        return dq, dk, dv
+
+    def normalize(self, x, *, centre=0, max_norm=True, scale=1.0, out: Optional[torch.Tensor] = None):
+        """x (bh, n, d) view; returns y = scale * (x - centre) / max_n ||.|| (see the header)."""
+        nd = NormDesc()
+        nd.bh, nd.n, nd.d = x.shape
+        nd.dtype = _dtype_code(x)
+        nd.centre, nd.max_norm, nd.scale = int(centre), int(bool(max_norm)), float(scale)
+        if out is None:
+            out = torch.empty(tuple(x.shape), dtype=x.dtype, device=x.device)
+        nd.sx, nd.sy = _strides(x), _strides(out)
+        stats = torch.empty(nd.bh * (nd.d + 2), dtype=torch.float32, device=x.device)
+        st = self.lib.fastmax_normalize(C.byref(nd), x.data_ptr(), out.data_ptr(), stats.data_ptr(), self._stream(x))
+        self.check(st, "fastmax_normalize")
+        return out
+
+    def probe_mfma(self, device):
+        a = torch.zeros(1024, dtype=torch.float32, device=device)
+        b = torch.zeros(1024, dtype=torch.float32, device=device)
+        self.check(self.lib.fastmax_probe_mfma(a.data_ptr(), b.data_ptr(), 0), "fastmax_probe_mfma")
+        return a.view(64, 16), b.view(64, 16)
+
+
+_lock = threading.Lock()
+_default: Optional[FastmaxLib] = None
+
+
+def get_lib() -> FastmaxLib:
+    """The process-wide library handle (loaded on first use)."""
+    global _default
+    with _lock:
+        if _default is None:
+            _default = FastmaxLib()
+        return _default

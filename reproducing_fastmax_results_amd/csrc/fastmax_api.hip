@@ -1,0 +1,285 @@
+// C ABI of libfastmax_hip.so: argument validation, workspace planning and the
+// launch sequences.  See include/fastmax_hip.h for the contract of each entry.
+#include "fastmax_hip.h"
+#include "fm_kernels.h"
+#include "fm_kernels_bwd.h"
+#include "fm_norm.h"
+
+namespace {
+
+#if defined(FM_HOSTSIM)
+inline int fm_after_launch() { return FASTMAX_OK; }
+inline void fm_allow_lds(const void*, size_t) {}
+#else
+inline int fm_after_launch() { return hipGetLastError() == hipSuccess ? FASTMAX_OK : FASTMAX_ERR_LAUNCH; }
+inline void fm_allow_lds(const void* fn, size_t bytes) {
+  // needed above the 64 KiB default; harmless below it
+  (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, int(bytes));
+}
+#endif
+
+inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+inline size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
+
+struct Plan {
+  bool half;            // compute type: _Float16 (bf16 interface) or float
+  int esz;              // sizeof compute element
+  int qw;               // tokens per workgroup of the token-side kernels
+  int L, nseg, nslots;
+  bool use_state, quad;
+  int npad_q, npad_k;
+  float c0, c1, c2;     // polynomial on the raw dot product
+  // workspace offsets (bytes)
+  size_t kt, vt, big, small, fwd_bytes;
+  size_t b_kt, b_vt, b_qt, b_qct, b_gh, b_ght, b_cv, b_bigq, b_smallq, b_bigk, b_smallk, b_bigv, b_smallv,
+      bwd_bytes;
+};
+
+bool strides_ok(const FastmaxStrides& s, int bh, int n, int d) {
+  if (s.n < d && n > 1) return false;
+  if (s.bh <= 0 && bh > 1) return false;
+  return s.n > 0 || n <= 1;
+}
+
+int validate(const FastmaxDesc* d) {
+  if (!d) return FASTMAX_ERR_NULL;
+  if (d->dtype != FASTMAX_F32 && d->dtype != FASTMAX_BF16) return FASTMAX_ERR_DTYPE;
+  if (d->bh <= 0 || d->nq <= 0 || d->nk <= 0 || d->d <= 0) return FASTMAX_ERR_SHAPE;
+  if (d->bh > 65535) return FASTMAX_ERR_SHAPE;
+  if (d->p != 1 && d->p != 2) return FASTMAX_ERR_UNSUPPORTED;
+  if (d->d != 32 && d->d != 64) return FASTMAX_ERR_UNSUPPORTED;
+  if (d->mask && d->nq != d->nk) return FASTMAX_ERR_UNSUPPORTED;
+  if (d->chunk < 0) return FASTMAX_ERR_SHAPE;
+  if (!(d->inv_tau == d->inv_tau)) return FASTMAX_ERR_SHAPE;
+  return FASTMAX_OK;
+}
+
+template <int DH> size_t big_bytes(int esz) { return size_t(StateDims<DH>::BIG) * esz; }
+
+int make_plan(const FastmaxDesc* d, Plan& p) {
+  int st = validate(d);
+  if (st != FASTMAX_OK) return st;
+  p.half = d->dtype == FASTMAX_BF16;
+  p.esz = p.half ? 2 : 4;
+  p.qw = p.half ? 256 : 128;
+  p.npad_q = int(round_up(d->nq, 256));
+  p.npad_k = int(round_up(d->nk, 256));
+  p.quad = d->p == 2 && d->a2 != 0.0f;
+  p.c0 = d->a0;
+  p.c1 = d->a1 * d->inv_tau;
+  p.c2 = p.quad ? d->a2 * d->inv_tau * d->inv_tau : 0.0f;
+  const bool force_dense = (d->flags & FASTMAX_FLAG_FORCE_DENSE) != 0;
+  if (d->mask) {
+    int L = d->chunk > 0 ? int(round_up(d->chunk, 256)) : (d->nq >= 2048 ? 1024 : p.npad_q);
+    if (force_dense || L > p.npad_q) L = p.npad_q;
+    p.L = L;
+    p.nseg = (d->nq + L - 1) / L;
+    p.use_state = p.nseg > 1;
+    p.nslots = p.use_state ? p.nseg : 0;
+  } else {
+    p.L = p.npad_k;
+    p.nseg = 1;
+    const bool force_m = (d->flags & FASTMAX_FLAG_FORCE_MOMENTS) != 0;
+    p.use_state = force_m || (!force_dense && int64_t(d->nk) > int64_t(d->d) * d->d + d->d);
+    p.nslots = p.use_state ? 1 : 0;
+  }
+  const size_t bigsz = d->d == 64 ? big_bytes<64>(p.esz) : big_bytes<32>(p.esz);
+  const size_t smallsz = size_t(d->d == 64 ? StateDims<64>::SMALL : StateDims<32>::SMALL) * 4;
+  const size_t tq = size_t(d->bh) * d->d * p.npad_q * p.esz;
+  const size_t tk = size_t(d->bh) * d->d * p.npad_k * p.esz;
+  size_t off = 0;
+  auto take = [&](size_t bytes) { size_t o = off; off = align256(off + bytes); return o; };
+  p.kt = take(p.use_state ? tk : 0);
+  p.vt = take(tk);
+  p.big = take(size_t(d->bh) * p.nslots * bigsz);
+  p.small = take(size_t(d->bh) * p.nslots * smallsz);
+  p.fwd_bytes = off ? off : 256;
+  off = 0;
+  p.b_kt = take(tk); p.b_vt = take(tk); p.b_qt = take(tq); p.b_qct = take(tq);
+  p.b_gh = take(tq); p.b_ght = take(tq);
+  p.b_cv = take(size_t(d->bh) * p.npad_q * 4);
+  p.b_bigq = take(size_t(d->bh) * p.nslots * bigsz); p.b_smallq = take(size_t(d->bh) * p.nslots * smallsz);
+  p.b_bigk = take(size_t(d->bh) * p.nslots * bigsz); p.b_smallk = take(size_t(d->bh) * p.nslots * smallsz);
+  p.b_bigv = take(size_t(d->bh) * p.nslots * bigsz); p.b_smallv = take(size_t(d->bh) * p.nslots * smallsz);
+  p.bwd_bytes = off ? off : 256;
+  return FASTMAX_OK;
+}
+
+template <typename T> bool vec_ok(const void* ptr, const FastmaxStrides& s) {
+  const int64_t a = 16 / int64_t(sizeof(T));          // elements per 16 bytes
+  return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && (s.n % a == 0) && (s.bh % a == 0);
+}
+template <typename T> TRef<const T> cref(const void* ptr, const FastmaxStrides& s) {
+  TRef<const T> r; r.p = static_cast<const T*>(ptr); r.s_bh = s.bh; r.s_n = s.n; r.vec = vec_ok<T>(ptr, s); return r;
+}
+template <typename T> TRef<T> mref(void* ptr, const FastmaxStrides& s) {
+  TRef<T> r; r.p = static_cast<T*>(ptr); r.s_bh = s.bh; r.s_n = s.n; r.vec = vec_ok<T>(ptr, s); return r;
+}
+
+template <typename TIO, typename E, int DH>
+int launch_transpose(const void* x, const FastmaxStrides& s, int bh, int n, int npad, E* xt, fm_stream_t stream) {
+  TRef<const TIO> r = cref<TIO>(x, s);
+  FM_KERNEL_LAUNCH((k_transpose<TIO, E, DH>), fm_dim3(npad / 64, bh), fm_dim3(FM_THREADS), 0, stream,
+                   r.p, r.s_bh, r.s_n, r.vec, n, npad, xt);
+  return fm_after_launch();
+}
+
+template <typename E, int DH>
+int launch_build(const BuildArgs<E>& a, int bh, fm_stream_t stream) {
+  constexpr int TT = 64;
+  constexpr int PT = TT + Mma<E>::PAD;
+  const size_t lds = size_t(4) * DH * PT * sizeof(E);
+  const int nsteps = a.mode == FM_WALK_TOTAL ? 1 : a.nseg - 1;
+  if (nsteps <= 0) return FASTMAX_OK;
+  // two values of a per wavefront when that still fills the GPU, else one
+  const bool na2 = int64_t(bh) * (DH / 8) >= 256;
+  if (na2) {
+    const int groups = a.quad ? DH / 8 : 0;
+    fm_allow_lds(reinterpret_cast<const void*>(&k_build<E, DH, 2, TT>), lds);
+    FM_KERNEL_LAUNCH((k_build<E, DH, 2, TT>), fm_dim3(groups + 1, bh), fm_dim3(FM_THREADS), lds, stream, a);
+  } else {
+    const int groups = a.quad ? DH / 4 : 0;
+    fm_allow_lds(reinterpret_cast<const void*>(&k_build<E, DH, 1, TT>), lds);
+    FM_KERNEL_LAUNCH((k_build<E, DH, 1, TT>), fm_dim3(groups + 1, bh), fm_dim3(FM_THREADS), lds, stream, a);
+  }
+  return fm_after_launch();
+}
+
+template <typename E, int DH, int QT> size_t tok_lds_bytes(int extra_floats) {
+  typedef TokCfg<E, DH, QT> C;
+  size_t region = size_t(2) * C::SLAB * sizeof(E);
+  const size_t dense = size_t(2) * (C::KT * C::PQ + DH * C::PV) * sizeof(E);
+  const size_t outst = size_t(C::QW) * (DH + 1) * 4;
+  if (dense > region) region = dense;
+  if (outst > region) region = outst;
+  return size_t(C::QW) * C::PQ * sizeof(E) + size_t(C::NZ) * DH * C::PS * sizeof(E) + size_t(2 * DH + extra_floats) * 4 + region;
+}
+
+template <typename TIO, typename E, int DH, int QT>
+int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* k, const void* v, void* o,
+                float* g, char* ws, fm_stream_t stream) {
+  E* kt = reinterpret_cast<E*>(ws + p.kt);
+  E* vt = reinterpret_cast<E*>(ws + p.vt);
+  E* big = reinterpret_cast<E*>(ws + p.big);
+  float* small = reinterpret_cast<float*>(ws + p.small);
+  int st = launch_transpose<TIO, E, DH>(v, d->sv, d->bh, d->nk, p.npad_k, vt, stream);
+  if (st) return st;
+  if (p.use_state) {
+    st = launch_transpose<TIO, E, DH>(k, d->sk, d->bh, d->nk, p.npad_k, kt, stream);
+    if (st) return st;
+    BuildArgs<E> b;
+    b.xt = kt; b.pt = vt; b.rt = kt; b.za = kt; b.zb = kt;
+    b.npad = p.npad_k; b.nseg = p.nseg; b.L = p.L; b.mode = d->mask ? FM_WALK_PREFIX : FM_WALK_TOTAL;
+    b.quad = p.quad; b.big = big; b.small = small; b.nslots = p.nslots;
+    b.coef2 = p.c2; b.coef1 = p.c1; b.coefz = p.c2; b.coefva = p.c1; b.coefvb = p.c0;
+    st = launch_build<E, DH>(b, d->bh, stream);
+    if (st) return st;
+  }
+  FwdArgs<TIO, E> a;
+  a.q = cref<TIO>(q, d->sq); a.k = cref<TIO>(k, d->sk); a.v = cref<TIO>(v, d->sv);
+  a.o = mref<TIO>(o, d->so);
+  a.g = g; a.g_s_bh = d->sg.bh; a.g_s_n = d->sg.n;
+  a.vt = vt; a.npad_k = p.npad_k;
+  a.big = big; a.small = small; a.nslots = p.nslots;
+  a.nq = d->nq; a.nk = d->nk; a.L = p.L; a.causal = d->mask != 0; a.use_state = p.use_state; a.quad = p.quad;
+  a.a0 = p.c0; a.c1 = p.c1; a.c2 = p.c2;
+  typedef TokCfg<E, DH, QT> C;
+  const size_t lds = tok_lds_bytes<E, DH, QT>(0);
+  fm_allow_lds(reinterpret_cast<const void*>(&k_fwd<TIO, E, DH, QT>), lds);
+  FM_KERNEL_LAUNCH((k_fwd<TIO, E, DH, QT>), fm_dim3((d->nq + C::QW - 1) / C::QW, d->bh), fm_dim3(FM_THREADS), lds,
+                   stream, a);
+  return fm_after_launch();
+}
+
+template <typename TIO, typename E, int DH, int QT>
+int run_backward(const FastmaxDesc* d, const Plan& p, const void* q, const void* k, const void* v, const void* o,
+                 const float* g, const void* d_o, void* dq, void* dk, void* dv, char* ws, fm_stream_t stream);
+
+}  // namespace
+
+#include "fastmax_api_bwd.inc"
+
+extern "C" {
+
+int fastmax_version(void) { return 100; }
+
+const char* fastmax_status_string(int status) {
+  switch (status) {
+    case FASTMAX_OK: return "ok";
+    case FASTMAX_ERR_NULL: return "null pointer";
+    case FASTMAX_ERR_SHAPE: return "invalid shape or strides";
+    case FASTMAX_ERR_UNSUPPORTED: return "unsupported configuration (d must be 32 or 64, p 1 or 2, masked needs nq == nk)";
+    case FASTMAX_ERR_WORKSPACE: return "workspace missing, too small or not 256-byte aligned";
+    case FASTMAX_ERR_LAUNCH: return "HIP launch failed";
+    case FASTMAX_ERR_DTYPE: return "unknown dtype";
+    default: return "unknown status";
+  }
+}
+
+int fastmax_workspace_bytes(const FastmaxDesc* desc, size_t* forward_bytes, size_t* backward_bytes) {
+  Plan p;
+  const int st = make_plan(desc, p);
+  if (st) return st;
+  if (forward_bytes) *forward_bytes = p.fwd_bytes;
+  if (backward_bytes) *backward_bytes = p.bwd_bytes;
+  return FASTMAX_OK;
+}
+
+int fastmax_forward(const FastmaxDesc* desc, const void* q, const void* k, const void* v, void* o, float* g,
+                    void* workspace, size_t workspace_bytes, void* hip_stream) {
+  Plan p;
+  int st = make_plan(desc, p);
+  if (st) return st;
+  if (!q || !k || !v || !o || !g) return FASTMAX_ERR_NULL;
+  if (!strides_ok(desc->sq, desc->bh, desc->nq, desc->d) || !strides_ok(desc->sk, desc->bh, desc->nk, desc->d) ||
+      !strides_ok(desc->sv, desc->bh, desc->nk, desc->d) || !strides_ok(desc->so, desc->bh, desc->nq, desc->d) ||
+      !strides_ok(desc->sg, desc->bh, desc->nq, 1))
+    return FASTMAX_ERR_SHAPE;
+  if (!workspace || workspace_bytes < p.fwd_bytes || reinterpret_cast<uintptr_t>(workspace) % 256)
+    return FASTMAX_ERR_WORKSPACE;
+  char* ws = static_cast<char*>(workspace);
+  fm_stream_t stream = static_cast<fm_stream_t>(hip_stream);
+  if (p.half) {
+    if (desc->d == 64) return run_forward<fm_bf16, fm_half, 64, 2>(desc, p, q, k, v, o, g, ws, stream);
+    return run_forward<fm_bf16, fm_half, 32, 2>(desc, p, q, k, v, o, g, ws, stream);
+  }
+  if (desc->d == 64) return run_forward<float, float, 64, 1>(desc, p, q, k, v, o, g, ws, stream);
+  return run_forward<float, float, 32, 1>(desc, p, q, k, v, o, g, ws, stream);
+}
+
+int fastmax_backward(const FastmaxDesc* desc, const void* q, const void* k, const void* v, const void* o,
+                     const float* g, const void* d_o, void* dq, void* dk, void* dv, void* workspace,
+                     size_t workspace_bytes, void* hip_stream) {
+  Plan p;
+  int st = make_plan(desc, p);
+  if (st) return st;
+  if (!q || !k || !v || !o || !g || !d_o || !dq || !dk || !dv) return FASTMAX_ERR_NULL;
+  if (!strides_ok(desc->sq, desc->bh, desc->nq, desc->d) || !strides_ok(desc->sk, desc->bh, desc->nk, desc->d) ||
+      !strides_ok(desc->sv, desc->bh, desc->nk, desc->d) || !strides_ok(desc->so, desc->bh, desc->nq, desc->d) ||
+      !strides_ok(desc->sg, desc->bh, desc->nq, 1) || !strides_ok(desc->sdo, desc->bh, desc->nq, desc->d) ||
+      !strides_ok(desc->sdq, desc->bh, desc->nq, desc->d) || !strides_ok(desc->sdk, desc->bh, desc->nk, desc->d) ||
+      !strides_ok(desc->sdv, desc->bh, desc->nk, desc->d))
+    return FASTMAX_ERR_SHAPE;
+  if (!workspace || workspace_bytes < p.bwd_bytes || reinterpret_cast<uintptr_t>(workspace) % 256)
+    return FASTMAX_ERR_WORKSPACE;
+  char* ws = static_cast<char*>(workspace);
+  fm_stream_t stream = static_cast<fm_stream_t>(hip_stream);
+  if (p.half) {
+    if (desc->d == 64) return run_backward<fm_bf16, fm_half, 64, 2>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, ws, stream);
+    return run_backward<fm_bf16, fm_half, 32, 2>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, ws, stream);
+  }
+  if (desc->d == 64) return run_backward<float, float, 64, 1>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, ws, stream);
+  return run_backward<float, float, 32, 1>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, ws, stream);
+}
+
+int fastmax_normalize(const FastmaxNormDesc* desc, const void* x, void* y, float* stats, void* hip_stream) {
+  return fm_normalize_dispatch(desc, x, y, stats, static_cast<fm_stream_t>(hip_stream));
+}
+
+int fastmax_probe_mfma(float* out_f16, float* out_f32, void* hip_stream) {
+  if (!out_f16 || !out_f32) return FASTMAX_ERR_NULL;
+  FM_KERNEL_LAUNCH(k_probe_mfma, fm_dim3(1), fm_dim3(64), 0, static_cast<fm_stream_t>(hip_stream), out_f16, out_f32);
+  return fm_after_launch();
+}
+
+}  // extern "C"

@@ -1,0 +1,704 @@
+// Fastmax kernels for gfx950 (also compiled by the host simulator for tests).
+//
+// Math (per batch*head), s_ij = q_i.k_j / tau, f(s) = a0 + a1 s + a2 s^2:
+//     F_i = sum_j M_ij f(s_ij) v_j,  g_i = sum_j M_ij f(s_ij),  o_i = F_i / g_i.
+// The sequence is cut into segments of L tokens.  Keys of earlier segments (all
+// keys when there is no mask) reach a query through moment states
+//     T[a][r][c] = coef * sum_t x_ta p_tr r_tc     (a < D: order 2,  a = D: order 1, x = 1)
+// and keys of the query's own segment through dense masked tiles f(Q K^T).
+// Reference behaviour being reproduced: fastmax_cuda_forward.cu:23-280 (running
+// sums per thread) and fastattention_einops.py:186-322 (cumsum of outer products).
+//
+// All contractions are computed "transposed": the accumulator column (lane) is
+// the token, the accumulator rows are features.  That keeps one token per lane,
+// so a per-token scalar (q_ia, 1/g_i, c_i) is a per-lane scalar.
+#pragma once
+#include "fm_mma.h"
+
+#if defined(FM_HOSTSIM)
+#define FM_SHARED static
+#else
+#define FM_SHARED __shared__
+#endif
+
+static constexpr int FM_THREADS = 256;   // four wavefronts per workgroup, everywhere
+
+// ------------------------------------------------------------------------------
+// tile movers (global -> registers -> LDS), 16-byte chunks, 256 threads
+// ------------------------------------------------------------------------------
+template <typename E, int ROWS, int TT>
+struct TileRegs {
+  static constexpr int VEC = Mma<E>::VEC;
+  static constexpr int CPR = TT / VEC;                 // chunks per row
+  static constexpr int TOTAL = ROWS * CPR;
+  static constexpr int N = (TOTAL + FM_THREADS - 1) / FM_THREADS;
+  fm_u32x4 r[N];
+  // src points at (row 0, first token of the tile); rows are row_stride apart
+  FM_DEVICE void load(const E* src, int64_t row_stride, int tid) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int c = tid + FM_THREADS * i;
+      if (TOTAL % FM_THREADS == 0 || c < TOTAL) {
+        const int row = c / CPR, col = (c % CPR) * VEC;
+        r[i] = *reinterpret_cast<const fm_u32x4*>(src + row * row_stride + col);
+      }
+    }
+  }
+  FM_DEVICE void store(E* lds, int pitch, int tid) const {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int c = tid + FM_THREADS * i;
+      if (TOTAL % FM_THREADS == 0 || c < TOTAL) {
+        const int row = c / CPR, col = (c % CPR) * VEC;
+        *reinterpret_cast<fm_u32x4*>(lds + row * pitch + col) = r[i];
+      }
+    }
+  }
+};
+
+// Rows of a caller tensor (interface type, strided, bounds-checked) -> LDS in the
+// compute type.  ROWS x DH elements, eight elements per chunk.
+template <typename TIO, typename E, int ROWS, int DH>
+struct RowRegs {
+  static constexpr int CPR = DH / 8;
+  static constexpr int TOTAL = ROWS * CPR;
+  static constexpr int N = (TOTAL + FM_THREADS - 1) / FM_THREADS;
+  float v[N][8];
+  // base points at (token 0, feature 0) of this batch*head; rows row0..row0+ROWS-1
+  FM_DEVICE void load(const TIO* base, int64_t s_n, bool vec, int row0, int nrows, int tid) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int c = tid + FM_THREADS * i;
+      if (TOTAL % FM_THREADS == 0 || c < TOTAL) {
+        const int row = row0 + c / CPR, col = (c % CPR) * 8;
+        if (row < nrows) {
+          IO<TIO>::ld8(base + int64_t(row) * s_n + col, vec, v[i]);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) v[i][j] = 0.f;
+        }
+      }
+    }
+  }
+  FM_DEVICE void store(E* lds, int pitch, int tid) const {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int c = tid + FM_THREADS * i;
+      if (TOTAL % FM_THREADS == 0 || c < TOTAL) {
+        const int row = c / CPR, col = (c % CPR) * 8;
+        CE<E>::st8(lds + row * pitch + col, v[i]);
+      }
+    }
+  }
+};
+
+// ------------------------------------------------------------------------------
+// k_transpose: x (bh, n, DH) strided, interface type  ->  xt [bh][DH][npad], compute
+// type, zero for tokens >= n.  grid (npad/64, bh).
+// ------------------------------------------------------------------------------
+template <typename TIO, typename E, int DH>
+FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS)
+k_transpose(const TIO* FM_RESTRICT x, int64_t s_bh, int64_t s_n, int vec, int n, int npad,
+            E* FM_RESTRICT xt) {
+  constexpr int PT = 64 + Mma<E>::PAD;
+  constexpr int VEC = Mma<E>::VEC;
+  FM_SHARED E tile[DH * PT];
+  const int tid = FM_TID_X, t0 = FM_BID_X * 64, bh = FM_BID_Y;
+  const TIO* xb = x + int64_t(bh) * s_bh;
+  for (int c = tid; c < 64 * (DH / 8); c += FM_THREADS) {
+    const int tok = c / (DH / 8), d0 = (c % (DH / 8)) * 8;
+    float v[8];
+    if (t0 + tok < n) {
+      IO<TIO>::ld8(xb + int64_t(t0 + tok) * s_n + d0, vec != 0, v);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) tile[(d0 + j) * PT + tok] = CE<E>::from(v[j]);
+  }
+  FM_SYNC();
+  E* ob = xt + int64_t(bh) * DH * npad + t0;
+  for (int c = tid; c < DH * (64 / VEC); c += FM_THREADS) {
+    const int d = c / (64 / VEC), tk = (c % (64 / VEC)) * VEC;
+    *reinterpret_cast<fm_u32x4*>(ob + int64_t(d) * npad + tk) =
+        *reinterpret_cast<const fm_u32x4*>(&tile[d * PT + tk]);
+  }
+}
+
+// ------------------------------------------------------------------------------
+// k_prep_bwd: per token  gh = dO / g,  c = gh . o ; writes
+//   gh  [bh][npad][DH]  (row-major, compute type)      ght [bh][DH][npad]
+//   qt  [bh][DH][npad]  (q transposed)                  qct [bh][DH][npad]  (c_i q_i)
+//   cv  [bh][npad]      (fp32)
+// Tokens >= n are written as zeros.  grid (npad/64, bh).
+// Reference: div_grad_output, fastmax_cuda_backward.cu:494-501, and the
+// "grad * o" row sums of fastattention_einops.py:405-407.
+// ------------------------------------------------------------------------------
+template <typename TIO> struct TRef { TIO* p; int64_t s_bh, s_n; int vec; };
+
+template <typename TIO, typename E, int DH>
+FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS)
+k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, const float* FM_RESTRICT g,
+           int64_t g_s_bh, int64_t g_s_n, int n, int npad, E* FM_RESTRICT gh, E* FM_RESTRICT ght,
+           E* FM_RESTRICT qt, E* FM_RESTRICT qct, float* FM_RESTRICT cv) {
+  constexpr int PT = 64 + Mma<E>::PAD;
+  constexpr int VEC = Mma<E>::VEC;
+  constexpr int EPT = DH / 4;                      // elements per thread (4 threads per token)
+  FM_SHARED E tg[DH * PT];
+  FM_SHARED E tq[DH * PT];
+  FM_SHARED E tc[DH * PT];
+  const int tid = FM_TID_X, t0 = FM_BID_X * 64, bh = FM_BID_Y;
+  const int tok = tid >> 2, part = tid & 3, d0 = part * EPT;
+  const int row = t0 + tok;
+  float vg[EPT], vq[EPT];
+  float csum = 0.f;
+  if (row < n) {
+    const float ginv = 1.0f / g[int64_t(bh) * g_s_bh + int64_t(row) * g_s_n];
+#pragma unroll
+    for (int j = 0; j < EPT; j += 8) {
+      float a[8], b[8], c[8];
+      IO<TIO>::ld8(d_o.p + int64_t(bh) * d_o.s_bh + int64_t(row) * d_o.s_n + d0 + j, d_o.vec != 0, a);
+      IO<TIO>::ld8(o.p + int64_t(bh) * o.s_bh + int64_t(row) * o.s_n + d0 + j, o.vec != 0, b);
+      IO<TIO>::ld8(q.p + int64_t(bh) * q.s_bh + int64_t(row) * q.s_n + d0 + j, q.vec != 0, c);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        vg[j + i] = a[i] * ginv;
+        csum += vg[j + i] * b[i];
+        vq[j + i] = c[i];
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) { vg[j] = 0.f; vq[j] = 0.f; }
+  }
+  csum += fm_shfl_xor(csum, 1);
+  csum += fm_shfl_xor(csum, 2);
+  if (part == 0) cv[int64_t(bh) * npad + row] = csum;
+  E* ghrow = gh + (int64_t(bh) * npad + row) * DH + d0;
+#pragma unroll
+  for (int j = 0; j < EPT; j += 8) CE<E>::st8(ghrow + j, &vg[j]);
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) {
+    tg[(d0 + j) * PT + tok] = CE<E>::from(vg[j]);
+    tq[(d0 + j) * PT + tok] = CE<E>::from(vq[j]);
+    tc[(d0 + j) * PT + tok] = CE<E>::from(vq[j] * csum);
+  }
+  FM_SYNC();
+  const int64_t ob = int64_t(bh) * DH * npad + t0;
+  for (int c = tid; c < DH * (64 / VEC); c += FM_THREADS) {
+    const int d = c / (64 / VEC), tk = (c % (64 / VEC)) * VEC;
+    const int64_t off = ob + int64_t(d) * npad + tk;
+    *reinterpret_cast<fm_u32x4*>(ght + off) = *reinterpret_cast<const fm_u32x4*>(&tg[d * PT + tk]);
+    *reinterpret_cast<fm_u32x4*>(qt + off) = *reinterpret_cast<const fm_u32x4*>(&tq[d * PT + tk]);
+    *reinterpret_cast<fm_u32x4*>(qct + off) = *reinterpret_cast<const fm_u32x4*>(&tc[d * PT + tk]);
+  }
+}
+
+// ------------------------------------------------------------------------------
+// Moment states.
+//   big   [slot][a = 0..DH][r][c]   compute type;  a < DH: coef2 * sum x_a p_r r_c,
+//                                                  a = DH: coef1 * sum p_r r_c
+//   small [slot]{ Z[DH][DH], va[DH], vb[DH] } fp32;  Z = coefz * sum za_r zb_c,
+//                                   va = coefva * sum za,  vb = coefvb * sum p
+// ------------------------------------------------------------------------------
+// `big` is padded to DH + 4 values of a so that a reader may fetch whole slabs of
+// up to four values of a starting at any a <= DH without leaving the state.
+template <int DH> struct StateDims {
+  static constexpr int64_t BIG = int64_t(DH + 4) * DH * DH;
+  static constexpr int64_t SMALL = int64_t(DH) * DH + 2 * DH;
+};
+
+enum { FM_WALK_PREFIX = 0, FM_WALK_SUFFIX = 1, FM_WALK_TOTAL = 2 };
+
+template <typename E> struct BuildArgs {
+  const E* xt; const E* pt; const E* rt; const E* za; const E* zb;   // [bh][DH][npad]
+  int npad, nseg, L, mode, quad;
+  E* big; float* small;                 // [bh][nslots] states
+  int nslots;
+  float coef2, coef1, coefz, coefva, coefvb;
+};
+
+FM_DEVICE void fm_walk_step(int mode, int nseg, int L, int npad, int w, int& tb, int& te, int& slot) {
+  if (mode == FM_WALK_PREFIX) { tb = w * L; te = tb + L; slot = w + 1; }
+  else if (mode == FM_WALK_SUFFIX) {
+    const int s = nseg - 1 - w;
+    tb = s * L; te = tb + L; if (te > npad) te = npad; slot = s - 1;
+  } else { tb = 0; te = npad; slot = 0; }
+}
+
+// k_build: one workgroup per (group of 4*NA values of a, batch*head) walks the
+// tokens once, keeping its slice of the order-2 state in accumulators and
+// writing a snapshot at every segment boundary, so the prefix (or suffix) scan
+// over segments is implicit.  The last workgroup in x builds the order-1 and
+// denominator states.  Replaces the running sums of fastmax_cuda_forward.cu:183-276
+// (one thread per feature, serial over tokens) and the cumsum of materialised
+// outer products of fastattention_einops.py:237-248.
+template <typename E, int DH, int NA, int TT>
+FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_build(BuildArgs<E> A) {
+  typedef Mma<E> M;
+  typedef typename M::frag frag;
+  constexpr int AW = 4 * NA;
+  constexpr int NT = DH / 32;               // 32-row tiles per feature axis
+  constexpr int PT = TT + M::PAD;
+  FM_DYN_SMEM(smem);
+  E* s0 = reinterpret_cast<E*>(smem);       // p tile   [DH][PT]
+  E* s1 = s0 + DH * PT;                      // r tile   [DH][PT]
+  E* s2 = s1 + DH * PT;                      // heavy: x rows [AW][PT]; small: za tile [DH][PT]
+  E* s3 = s2 + DH * PT;                      // small: zb tile [DH][PT]
+  const int tid = FM_TID_X, wave = tid >> 6, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int bh = FM_BID_Y;
+  const int ngroups = A.quad ? DH / AW : 0;
+  const bool small = (FM_BID_X == ngroups);
+  const int64_t tb_off = int64_t(bh) * DH * A.npad;
+  const int nsteps = (A.mode == FM_WALK_TOTAL) ? 1 : A.nseg - 1;
+  if (nsteps <= 0) return;
+  E* big = A.big + int64_t(bh) * A.nslots * StateDims<DH>::BIG;
+  float* sml = A.small + int64_t(bh) * A.nslots * StateDims<DH>::SMALL;
+
+  int w = 0, tb, te, slot;
+  fm_walk_step(A.mode, A.nseg, A.L, A.npad, 0, tb, te, slot);
+  int t = tb;
+
+  if (!small) {
+    const int a0 = FM_BID_X * AW;
+    TileRegs<E, DH, TT> rp, rr;
+    TileRegs<E, AW, TT> rx;
+    fm_f32x16 acc[NA][NT][NT];
+#pragma unroll
+    for (int i = 0; i < NA; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int k = 0; k < NT; ++k) acc[i][j][k] = fm_zero16();
+    rp.load(A.pt + tb_off + t, A.npad, tid);
+    rr.load(A.rt + tb_off + t, A.npad, tid);
+    rx.load(A.xt + tb_off + int64_t(a0) * A.npad + t, A.npad, tid);
+    bool have = true;
+    while (have) {
+      FM_SYNC();
+      rp.store(s0, PT, tid); rr.store(s1, PT, tid); rx.store(s2, PT, tid);
+      FM_SYNC();
+      int nt = t + TT, nw = w, ntb = tb, nte = te, nslot = slot;
+      const bool last = (nt >= te);
+      bool has_next = true;
+      if (last) {
+        nw = w + 1;
+        if (nw < nsteps) { fm_walk_step(A.mode, A.nseg, A.L, A.npad, nw, ntb, nte, nslot); nt = ntb; }
+        else has_next = false;
+      }
+      if (has_next) {
+        rp.load(A.pt + tb_off + nt, A.npad, tid);
+        rr.load(A.rt + tb_off + nt, A.npad, tid);
+        rx.load(A.xt + tb_off + int64_t(a0) * A.npad + nt, A.npad, tid);
+      }
+#pragma unroll 2
+      for (int ks = 0; ks < TT / M::KSTEP; ++ks) {
+        const int ko = ks * M::KSTEP + lh * M::KPL;
+        frag fb[NT], fp[NT];
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          fb[j] = M::load(s1 + (32 * j + lr) * PT + ko);
+          fp[j] = M::load(s0 + (32 * j + lr) * PT + ko);
+        }
+#pragma unroll
+        for (int i = 0; i < NA; ++i) {
+          const frag fx = M::load(s2 + (wave * NA + i) * PT + ko);
+#pragma unroll
+          for (int j = 0; j < NT; ++j) {
+            const frag fa = fp[j] * fx;
+#pragma unroll
+            for (int k = 0; k < NT; ++k) acc[i][j][k] = M::mma(fa, fb[k], acc[i][j][k]);
+          }
+        }
+      }
+      if (last) {
+        E* dst = big + int64_t(slot) * StateDims<DH>::BIG;
+#pragma unroll
+        for (int i = 0; i < NA; ++i) {
+          const int a = a0 + wave * NA + i;
+#pragma unroll
+          for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int k = 0; k < NT; ++k)
+#pragma unroll
+              for (int e = 0; e < 16; ++e) {
+                const int r = 32 * j + fm_acc_row(e, lh), c = 32 * k + lr;
+                dst[(int64_t(a) * DH + r) * DH + c] = CE<E>::from(A.coef2 * acc[i][j][k][e]);
+              }
+        }
+      }
+      t = nt; w = nw; tb = ntb; te = nte; slot = nslot; have = has_next;
+    }
+  } else {
+    // order-1 state (wave 0), denominator matrix Z (wave 1), vector sums (waves 2, 3)
+    const bool has_z = (A.za != nullptr);
+    TileRegs<E, DH, TT> rp, rr, ra, rb;
+    fm_f32x16 acc[NT][NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int k = 0; k < NT; ++k) acc[j][k] = fm_zero16();
+    float vsum = 0.f;
+    rp.load(A.pt + tb_off + t, A.npad, tid);
+    rr.load(A.rt + tb_off + t, A.npad, tid);
+    if (has_z) { ra.load(A.za + tb_off + t, A.npad, tid); rb.load(A.zb + tb_off + t, A.npad, tid); }
+    bool have = true;
+    while (have) {
+      FM_SYNC();
+      rp.store(s0, PT, tid); rr.store(s1, PT, tid);
+      if (has_z) { ra.store(s2, PT, tid); rb.store(s3, PT, tid); }
+      FM_SYNC();
+      int nt = t + TT, nw = w, ntb = tb, nte = te, nslot = slot;
+      const bool last = (nt >= te);
+      bool has_next = true;
+      if (last) {
+        nw = w + 1;
+        if (nw < nsteps) { fm_walk_step(A.mode, A.nseg, A.L, A.npad, nw, ntb, nte, nslot); nt = ntb; }
+        else has_next = false;
+      }
+      if (has_next) {
+        rp.load(A.pt + tb_off + nt, A.npad, tid);
+        rr.load(A.rt + tb_off + nt, A.npad, tid);
+        if (has_z) { ra.load(A.za + tb_off + nt, A.npad, tid); rb.load(A.zb + tb_off + nt, A.npad, tid); }
+      }
+      if (wave == 0 || (wave == 1 && has_z)) {
+        const E* sa = wave == 0 ? s0 : s2;
+        const E* sb = wave == 0 ? s1 : s3;
+        for (int ks = 0; ks < TT / M::KSTEP; ++ks) {
+          const int ko = ks * M::KSTEP + lh * M::KPL;
+          frag fa[NT], fb[NT];
+#pragma unroll
+          for (int j = 0; j < NT; ++j) {
+            fa[j] = M::load(sa + (32 * j + lr) * PT + ko);
+            fb[j] = M::load(sb + (32 * j + lr) * PT + ko);
+          }
+#pragma unroll
+          for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int k = 0; k < NT; ++k) acc[j][k] = M::mma(fa[j], fb[k], acc[j][k]);
+        }
+      } else if (wave >= 2 && lane < DH && (wave == 3 || has_z)) {
+        const E* sv = wave == 2 ? s2 : s0;          // wave 2: sum of za, wave 3: sum of p
+        float s = 0.f;
+        for (int j = 0; j < TT; ++j) s += float(sv[lane * PT + j]);
+        vsum += s;
+      }
+      if (last) {
+        float* ds = sml + int64_t(slot) * StateDims<DH>::SMALL;
+        if (wave == 0) {
+          E* dst = big + int64_t(slot) * StateDims<DH>::BIG + int64_t(DH) * DH * DH;
+#pragma unroll
+          for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int k = 0; k < NT; ++k)
+#pragma unroll
+              for (int e = 0; e < 16; ++e) {
+                const int r = 32 * j + fm_acc_row(e, lh), c = 32 * k + lr;
+                dst[r * DH + c] = CE<E>::from(A.coef1 * acc[j][k][e]);
+              }
+        } else if (wave == 1) {
+#pragma unroll
+          for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int k = 0; k < NT; ++k)
+#pragma unroll
+              for (int e = 0; e < 16; ++e) {
+                const int r = 32 * j + fm_acc_row(e, lh), c = 32 * k + lr;
+                ds[r * DH + c] = has_z ? A.coefz * acc[j][k][e] : 0.f;
+              }
+        } else if (lane < DH) {
+          if (wave == 2) ds[DH * DH + lane] = has_z ? A.coefva * vsum : 0.f;
+          else ds[DH * DH + DH + lane] = A.coefvb * vsum;
+        }
+      }
+      t = nt; w = nw; tb = ntb; te = nte; slot = nslot; have = has_next;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------
+// Shared pieces of the token-side kernels
+// ------------------------------------------------------------------------------
+// LDS sizes (in elements of E) used by k_fwd / k_dq / k_dkv; the host computes the
+// dynamic LDS bytes from the same struct.
+template <typename E, int DH, int QT>
+struct TokCfg {
+  typedef Mma<E> M;
+  static constexpr int NT = DH / 32;
+  static constexpr int NKS = DH / M::KSTEP;         // k-steps over a feature axis
+  static constexpr int QW = 4 * QT * 32;            // tokens per workgroup
+  static constexpr int PQ = DH + M::PAD;            // pitch of row-major token tiles
+  static constexpr int PS = DH + M::PAD;            // pitch of state rows
+  static constexpr int SA = sizeof(E) == 2 ? 4 : 2; // values of a per state slab
+  static constexpr int KT = 64;                     // tokens per stage of the dense loop
+  static constexpr int PV = KT + M::PAD;            // pitch of transposed token tiles
+  static constexpr int NZ = sizeof(E) == 2 ? 2 : 1; // hi/lo split of fp32 denominators
+  static constexpr int SLAB = SA * DH * PS;         // elements per slab buffer
+};
+
+// Moment readout, transposed:  acc[j][ct] (rows c, column = token of tile j) +=
+//   sum_{a, b} T[a][c][b] * x_a(token) * y_b(token)        a < DH
+//   sum_b      T[DH][c][b] * y_b(token)                    a = DH
+// xs: row-major token tile in LDS (pitch PQ) supplying x; yb[j][ks]: B fragments of y.
+// slab: two buffers of SA*DH*PS elements.  All 256 threads must call this.
+template <typename E, int DH, int QT, int NACC>
+FM_DEVICE void fm_readout(const E* FM_RESTRICT state, bool quad, const E* xs, const int* xrow,
+                          const typename Mma<E>::frag (*yb)[TokCfg<E, DH, QT>::NKS],
+                          E* slab, fm_f32x16 (*acc)[NACC], int tid) {
+  typedef TokCfg<E, DH, QT> C;
+  typedef Mma<E> M;
+  typedef typename M::frag frag;
+  const int lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int a_begin = quad ? 0 : DH;
+  TileRegs<E, C::SA * DH, DH> regs;
+  regs.load(state + int64_t(a_begin) * DH * DH, DH, tid);   // rows [a][c] are contiguous
+  int buf = 0;
+  for (int as = a_begin; as <= DH; as += C::SA) {
+    E* sb = slab + buf * C::SLAB;
+    regs.store(sb, C::PS, tid);
+    FM_SYNC();
+    if (as + C::SA <= DH) regs.load(state + int64_t(as + C::SA) * DH * DH, DH, tid);
+    const int na = (as + C::SA <= DH) ? C::SA : (DH + 1 - as);
+    for (int al = 0; al < na; ++al) {
+      const int a = as + al;
+      frag xr[QT];
+#pragma unroll
+      for (int j = 0; j < QT; ++j) xr[j] = (a < DH) ? M::splat(xs[xrow[j] * C::PQ + a]) : M::splat(E(1.0f));
+#pragma unroll
+      for (int ks = 0; ks < C::NKS; ++ks) {
+        const int ko = ks * M::KSTEP + lh * M::KPL;
+        frag fa[C::NT];
+#pragma unroll
+        for (int ct = 0; ct < C::NT; ++ct) fa[ct] = M::load(sb + (al * DH + 32 * ct + lr) * C::PS + ko);
+#pragma unroll
+        for (int j = 0; j < QT; ++j) {
+          const frag fb = yb[j][ks] * xr[j];
+#pragma unroll
+          for (int ct = 0; ct < C::NT; ++ct) acc[j][ct] = M::mma(fa[ct], fb, acc[j][ct]);
+        }
+      }
+    }
+    buf ^= 1;
+  }
+  FM_SYNC();
+}
+
+// ------------------------------------------------------------------------------
+// k_fwd: forward for one block of QW queries of one batch*head.
+//   [F_i, g_i] = (prefix or global moment readout) + (dense tiles over the keys
+//   kbeg .. kend of the query's own segment, causal on the diagonal);  o = F / g.
+// grid (ceil(nq / QW), bh).  Replaces calc_masked / calc_unmasked
+// (fastmax_cuda_forward.cu:23-280).
+// ------------------------------------------------------------------------------
+template <typename TIO, typename E> struct FwdArgs {
+  TRef<const TIO> q, k, v;
+  TRef<TIO> o;
+  float* g; int64_t g_s_bh, g_s_n;
+  const E* vt; int npad_k;             // V transposed [bh][DH][npad_k]
+  const E* big; const float* small; int nslots;
+  int nq, nk, L, causal, use_state, quad;
+  float a0, c1, c2;                    // f(x) = a0 + c1 x + c2 x^2 on the raw dot product x
+};
+
+template <typename TIO, typename E, int DH, int QT>
+FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_fwd(FwdArgs<TIO, E> A) {
+  typedef TokCfg<E, DH, QT> C;
+  typedef Mma<E> M;
+  typedef typename M::frag frag;
+  constexpr int NT = C::NT, NKS = C::NKS, QW = C::QW, PQ = C::PQ, PS = C::PS, KT = C::KT, PV = C::PV;
+  FM_DYN_SMEM(smem);
+  E* Qs = reinterpret_cast<E*>(smem);                 // [QW][PQ]
+  E* Zs = Qs + QW * PQ;                               // [NZ][DH][PS]
+  float* vecs = reinterpret_cast<float*>(Zs + C::NZ * DH * PS);   // va[DH], vb[DH]
+  E* R = reinterpret_cast<E*>(vecs + 2 * DH);         // slabs | dense-loop tiles | output staging
+  const int tid = FM_TID_X, wave = tid >> 6, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int bh = FM_BID_Y;
+  const int nqb = FM_GDIM_X;
+  const int qb = A.causal ? (nqb - 1 - FM_BID_X) : FM_BID_X;    // heavy blocks first
+  const int q0 = qb * QW;
+  const int seg = A.causal ? q0 / A.L : 0;
+  const bool use_state = A.use_state && (!A.causal || seg > 0);
+  const int slot = A.causal ? seg : 0;
+  const int kbeg = A.causal ? seg * A.L : 0;
+  int kend = A.causal ? (q0 + QW < A.nk ? q0 + QW : A.nk) : (A.use_state ? 0 : A.nk);
+  const float cnt = A.causal ? float(kbeg) : float(A.nk);       // keys covered by the state
+
+  // ---- stage Q (and the denominator states) ----
+  {
+    RowRegs<TIO, E, QW, DH> rq;
+    rq.load(A.q.p + int64_t(bh) * A.q.s_bh, A.q.s_n, A.q.vec != 0, q0, A.nq, tid);
+    rq.store(Qs, PQ, tid);
+  }
+  const float* sml = A.small + (int64_t(bh) * A.nslots + slot) * StateDims<DH>::SMALL;
+  if (use_state) {
+    for (int i = tid; i < DH * DH; i += FM_THREADS) {
+      const float z = sml[i];
+      const int r = i / DH, c = i % DH;
+      const E hi = CE<E>::from(z);
+      Zs[r * PS + c] = hi;
+      if (C::NZ == 2) Zs[DH * PS + r * PS + c] = CE<E>::from(z - float(hi));
+    }
+    if (tid < 2 * DH) vecs[tid] = sml[DH * DH + tid];
+  }
+  FM_SYNC();
+
+  int tw[QT], xrow[QT];
+#pragma unroll
+  for (int j = 0; j < QT; ++j) {
+    tw[j] = (j == 0) ? wave : (4 * QT - 1 - wave);   // pair a short and a long causal tile
+    xrow[j] = tw[j] * 32 + lr;
+  }
+  frag qf[QT][NKS];
+#pragma unroll
+  for (int j = 0; j < QT; ++j)
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) qf[j][ks] = M::load(Qs + xrow[j] * PQ + ks * M::KSTEP + lh * M::KPL);
+
+  fm_f32x16 acc[QT][NT];
+#pragma unroll
+  for (int j = 0; j < QT; ++j)
+#pragma unroll
+    for (int ct = 0; ct < NT; ++ct) acc[j][ct] = fm_zero16();
+  float gsum[QT];
+#pragma unroll
+  for (int j = 0; j < QT; ++j) gsum[j] = 0.f;
+
+  if (use_state) {
+    // denominator: g_i += sum_m q_im (va[m] + sum_l Z[m][l] q_il)
+#pragma unroll
+    for (int j = 0; j < QT; ++j) {
+#pragma unroll
+      for (int mt = 0; mt < NT; ++mt) {
+        fm_f32x16 y = fm_zero16();
+#pragma unroll
+        for (int z = 0; z < C::NZ; ++z)
+#pragma unroll
+          for (int ks = 0; ks < NKS; ++ks)
+            y = M::mma(M::load(Zs + z * DH * PS + (32 * mt + lr) * PS + ks * M::KSTEP + lh * M::KPL),
+                       qf[j][ks], y);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int m = 32 * mt + fm_acc_row(e, lh);
+          gsum[j] += (y[e] + vecs[m]) * float(Qs[xrow[j] * PQ + m]);
+        }
+      }
+    }
+    const E* state = A.big + (int64_t(bh) * A.nslots + slot) * StateDims<DH>::BIG;
+    fm_readout<E, DH, QT, NT>(state, A.quad != 0, Qs, xrow, qf, R, acc, tid);
+  }
+
+  // ---- dense tiles over the keys of this segment ----
+  if (kend > kbeg) {
+    E* Ks[2]; E* Vs[2];
+    Ks[0] = R; Vs[0] = R + KT * PQ; Ks[1] = Vs[0] + DH * PV; Vs[1] = Ks[1] + KT * PQ;
+    RowRegs<TIO, E, KT, DH> rk;
+    TileRegs<E, DH, KT> rv;
+    const TIO* kb = A.k.p + int64_t(bh) * A.k.s_bh;
+    const E* vtb = A.vt + int64_t(bh) * DH * A.npad_k;
+    rk.load(kb, A.k.s_n, A.k.vec != 0, kbeg, A.nk, tid);
+    rv.load(vtb + kbeg, A.npad_k, tid);
+    int buf = 0;
+    for (int kt0 = kbeg; kt0 < kend; kt0 += KT) {
+      rk.store(Ks[buf], PQ, tid);
+      rv.store(Vs[buf], PV, tid);
+      FM_SYNC();
+      if (kt0 + KT < kend) {
+        rk.load(kb, A.k.s_n, A.k.vec != 0, kt0 + KT, A.nk, tid);
+        rv.load(vtb + kt0 + KT, A.npad_k, tid);
+      }
+#pragma unroll
+      for (int st = 0; st < KT / 32; ++st) {
+        const int key0 = kt0 + 32 * st;
+        if (key0 >= kend) break;
+        frag kf[NKS];
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) kf[ks] = M::load(Ks[buf] + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL);
+#pragma unroll
+        for (int j = 0; j < QT; ++j) {
+          const int qlo = q0 + tw[j] * 32;             // first query of this tile
+          if (A.causal && key0 > qlo + 31) continue;   // tile entirely in the future
+          fm_f32x16 s = fm_zero16();
+#pragma unroll
+          for (int ks = 0; ks < NKS; ++ks) s = M::mma(kf[ks], qf[j][ks], s);
+          const bool edge = (A.causal && key0 + 31 > qlo) || (key0 + 31 >= A.nk);
+          const int qi = qlo + lr;
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const float x = s[e];
+            float pv = A.a0 + x * (A.c1 + A.c2 * x);
+            if (edge) {
+              const int t = key0 + fm_acc_row(e, lh);
+              if ((A.causal && t > qi) || t >= A.nk) pv = 0.f;
+            }
+            gsum[j] += pv;
+            s[e] = pv;
+          }
+#pragma unroll
+          for (int ss = 0; ss < M::ACC_KSTEPS; ++ss) {
+            const frag pb = M::from_acc(s, ss);
+#pragma unroll
+            for (int ct = 0; ct < NT; ++ct)
+              acc[j][ct] = M::mma(M::load_perm(Vs[buf] + (32 * ct + lr) * PV + 32 * st, ss, lh), pb, acc[j][ct]);
+          }
+        }
+      }
+      buf ^= 1;
+    }
+    FM_SYNC();
+  }
+
+  // ---- epilogue: o = (F + vb) / g, staged through LDS for coalesced stores ----
+  float* Os = reinterpret_cast<float*>(R);             // [QW][DH + 1]
+#pragma unroll
+  for (int j = 0; j < QT; ++j) {
+    float gt = gsum[j] + fm_shfl_xor(gsum[j], 32);
+    if (use_state) gt += A.a0 * cnt;
+    const float ginv = 1.0f / gt;
+#pragma unroll
+    for (int ct = 0; ct < NT; ++ct)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int c = 32 * ct + fm_acc_row(e, lh);
+        const float f = acc[j][ct][e] + (use_state ? vecs[DH + c] : 0.f);
+        Os[xrow[j] * (DH + 1) + c] = f * ginv;
+      }
+    const int qi = q0 + xrow[j];
+    if (lh == 0 && qi < A.nq) A.g[int64_t(bh) * A.g_s_bh + int64_t(qi) * A.g_s_n] = gt;
+  }
+  FM_SYNC();
+  TIO* ob = A.o.p + int64_t(bh) * A.o.s_bh;
+  for (int c = tid; c < QW * (DH / 8); c += FM_THREADS) {
+    const int row = c / (DH / 8), col = (c % (DH / 8)) * 8;
+    if (q0 + row < A.nq) {
+      float v[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = Os[row * (DH + 1) + col + i];
+      IO<TIO>::st8(ob + int64_t(q0 + row) * A.o.s_n + col, A.o.vec != 0, v);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------
+// k_probe_mfma: one wavefront; A[i][k] = i + 1 (k = 0) else 0 ... chosen so that
+// D[i][j] = (i + 1) * 100 + (j + 1) identifies which (row, col) every lane/register
+// holds.  A[i][k] = {i + 1 at k = 0, 1 at k = 1};  B[k][j] = {100 at k = 0, j + 1 at k = 1}.
+// ------------------------------------------------------------------------------
+FM_GLOBAL void k_probe_mfma(float* out_f16, float* out_f32) {
+  const int lane = FM_TID_X & 63, lr = lane & 31, lh = lane >> 5;
+  fm_half8 a, b;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) { a[i] = fm_half(0.f); b[i] = fm_half(0.f); }
+  if (lh == 0) { a[0] = fm_half(float(lr + 1)); a[1] = fm_half(1.f); b[0] = fm_half(100.f); b[1] = fm_half(float(lr + 1)); }
+  fm_f32x16 c = fm_zero16();
+  c = fm_mfma_f16(a, b, c);
+#pragma unroll
+  for (int e = 0; e < 16; ++e) out_f16[lane * 16 + e] = c[e];
+  // f32: k = 0 supplied by lanes 0..31, k = 1 by lanes 32..63
+  const float af = lh == 0 ? float(lr + 1) : 1.f;
+  const float bf = lh == 0 ? 100.f : float(lr + 1);
+  fm_f32x16 c2 = fm_zero16();
+  c2 = fm_mfma_f32(af, bf, c2);
+#pragma unroll
+  for (int e = 0; e < 16; ++e) out_f32[lane * 16 + e] = c2[e];
+}

@@ -1,0 +1,104 @@
+// Thin portability layer between the kernels and what runs them.
+//
+// The kernels are written once against the names below.  The normal build is
+// hipcc for gfx950.  A second, test-only build (-DFM_HOSTSIM, plain C++) maps
+// the same names onto a host-thread simulator so that indexing and lane layouts
+// can be checked without a GPU; the shipped library never defines FM_HOSTSIM.
+#pragma once
+#include <cstddef>
+#include <cstdint>
+
+typedef _Float16 fm_half;
+typedef _Float16 fm_half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 fm_half8 __attribute__((ext_vector_type(8)));
+typedef float fm_f32x4 __attribute__((ext_vector_type(4)));
+typedef float fm_f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t fm_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t fm_u32x2 __attribute__((ext_vector_type(2)));
+typedef uint16_t fm_bf16;  // raw storage of a bfloat16
+
+#if defined(FM_HOSTSIM)
+// ------------------------------------------------------------------ host simulator
+#include <cmath>
+#include "hostsim.h"
+#define FM_GLOBAL
+#define FM_DEVICE inline
+#define FM_LAUNCH_BOUNDS(n)
+#define FM_RESTRICT
+typedef void* fm_stream_t;
+typedef hostsim::Dim3 fm_dim3;
+#define FM_TID_X (int(hostsim::g_t.tid.x))
+#define FM_BID_X (int(hostsim::g_t.bid.x))
+#define FM_BID_Y (int(hostsim::g_t.bid.y))
+#define FM_BID_Z (int(hostsim::g_t.bid.z))
+#define FM_GDIM_X (int(hostsim::g_t.gdim.x))
+#define FM_SYNC() hostsim::syncthreads()
+#define FM_DYN_SMEM(name) unsigned char* name = hostsim::g_t.blk->dyn_smem
+#define FM_KERNEL_LAUNCH(kern, grid, block, smem, stream, ...) \
+  hostsim::launch((grid), (block), (smem), [=]() { kern(__VA_ARGS__); })
+
+FM_DEVICE fm_f32x16 fm_mfma_f16(fm_half8 a, fm_half8 b, fm_f32x16 c) {
+  fm_half av[8], bv[8]; float cv[16];
+  for (int i = 0; i < 8; ++i) { av[i] = a[i]; bv[i] = b[i]; }
+  for (int i = 0; i < 16; ++i) cv[i] = c[i];
+  hostsim::mfma_32x32<fm_half, 8>(av, bv, cv);
+  for (int i = 0; i < 16; ++i) c[i] = cv[i];
+  return c;
+}
+FM_DEVICE fm_f32x16 fm_mfma_f32(float a, float b, fm_f32x16 c) {
+  float cv[16];
+  for (int i = 0; i < 16; ++i) cv[i] = c[i];
+  hostsim::mfma_32x32<float, 1>(&a, &b, cv);
+  for (int i = 0; i < 16; ++i) c[i] = cv[i];
+  return c;
+}
+FM_DEVICE float fm_shfl_xor(float v, int m) { return hostsim::shfl(v, hostsim::g_t.lane ^ m); }
+FM_DEVICE float fm_fmaxf(float a, float b) { return a > b ? a : b; }
+FM_DEVICE float fm_rsqrtf(float a) { return 1.0f / std::sqrt(a); }
+FM_DEVICE float fm_sqrtf(float a) { return std::sqrt(a); }
+
+#else
+// ------------------------------------------------------------------ gfx950
+#include <hip/hip_runtime.h>
+#define FM_GLOBAL __global__
+#define FM_DEVICE __device__ __forceinline__
+#define FM_LAUNCH_BOUNDS(n) __launch_bounds__(n)
+#define FM_RESTRICT __restrict__
+typedef hipStream_t fm_stream_t;
+typedef dim3 fm_dim3;
+#define FM_TID_X (int(threadIdx.x))
+#define FM_BID_X (int(blockIdx.x))
+#define FM_BID_Y (int(blockIdx.y))
+#define FM_BID_Z (int(blockIdx.z))
+#define FM_GDIM_X (int(gridDim.x))
+#define FM_SYNC() __syncthreads()
+#define FM_DYN_SMEM(name) extern __shared__ __align__(16) unsigned char name[]
+#define FM_KERNEL_LAUNCH(kern, grid, block, smem, stream, ...) \
+  hipLaunchKernelGGL(kern, (grid), (block), (smem), (stream), __VA_ARGS__)
+
+FM_DEVICE fm_f32x16 fm_mfma_f16(fm_half8 a, fm_half8 b, fm_f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+FM_DEVICE fm_f32x16 fm_mfma_f32(float a, float b, fm_f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+FM_DEVICE float fm_shfl_xor(float v, int m) { return __shfl_xor(v, m, 64); }
+FM_DEVICE float fm_fmaxf(float a, float b) { return fmaxf(a, b); }
+FM_DEVICE float fm_rsqrtf(float a) { return rsqrtf(a); }
+FM_DEVICE float fm_sqrtf(float a) { return sqrtf(a); }
+#endif
+
+// ---- bf16 <-> f32 (round to nearest even), usable on both builds -------------
+FM_DEVICE float fm_bf16_to_f32(fm_bf16 v) {
+  uint32_t u = uint32_t(v) << 16;
+  float f;
+  __builtin_memcpy(&f, &u, 4);
+  return f;
+}
+FM_DEVICE fm_bf16 fm_f32_to_bf16(float f) {
+  uint32_t u;
+  __builtin_memcpy(&u, &f, 4);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return fm_bf16((u >> 16) | 0x40u);  // NaN stays NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return fm_bf16(u >> 16);
+}

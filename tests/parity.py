@@ -1,0 +1,53 @@
+"""Shared helpers of the parity tests: seeded inputs and comparison with the oracle."""
+import math
+
+import torch
+
+from oracle import fastmax_oracle as O
+
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}   # rel-L2 bars: fp32 1e-5, bf16 2e-2
+
+
+def make_inputs(bh, nq, nk, d, dtype, device, seed=0, scale=1.0):
+    gen = torch.Generator().manual_seed(seed)
+    q = (scale * torch.randn(bh, nq, d, generator=gen)).to(dtype)
+    k = (scale * torch.randn(bh, nk, d, generator=gen)).to(dtype)
+    v = (scale * torch.randn(bh, nk, d, generator=gen)).to(dtype)
+    go = torch.randn(bh, nq, d, generator=gen).to(dtype)
+    return tuple(t.to(device) for t in (q, k, v, go))
+
+
+def oracle_all(q, k, v, go, *, mask, tau, p, a=(1.0, 1.0, 0.5), block=1024):
+    """fp64 closed form on the (already rounded) inputs: o, g, dq, dk, dv."""
+    args = [t.detach().cpu().double() for t in (q, k, v, go)]
+    if mask or q.shape[1] * k.shape[1] > 1 << 22:
+        return O.manual_backward_blocked(*args, mask=mask, tau=tau, p=p, a0=a[0], a1=a[1], a2=a[2], block=block)
+    return O.closed_form_forward_backward(*args, mask=mask, tau=tau, p=p, a0=a[0], a1=a[1], a2=a[2])
+
+
+def check_forward(lib, bh, nq, d, dtype, device, *, mask, p, nk=None, chunk=0, flags=0, tau_mult=8.0,
+                  a=(1.0, 1.0, 0.5), seed=0, scale=1.0):
+    nk = nk or nq
+    q, k, v, go = make_inputs(bh, nq, nk, d, dtype, device, seed, scale)
+    tau = tau_mult * math.sqrt(d)
+    o, g = lib.forward(q, k, v, mask=mask, inv_tau=1.0 / tau, a0=a[0], a1=a[1], a2=a[2], p=p, chunk=chunk, flags=flags)
+    ref = oracle_all(q, k, v, go, mask=mask, tau=tau, p=p, a=a)
+    eo, eg = O.rel_l2(o, ref[0]), O.rel_l2(g, ref[1])
+    assert eo < TOL[dtype], f"o rel-L2 {eo:.3e}"
+    assert eg < TOL[dtype], f"g rel-L2 {eg:.3e}"
+    return eo, eg
+
+
+def check_forward_backward(lib, bh, nq, d, dtype, device, *, mask, p, nk=None, chunk=0, flags=0, tau_mult=8.0,
+                           a=(1.0, 1.0, 0.5), seed=0, scale=1.0):
+    nk = nk or nq
+    q, k, v, go = make_inputs(bh, nq, nk, d, dtype, device, seed, scale)
+    tau = tau_mult * math.sqrt(d)
+    kw = dict(mask=mask, inv_tau=1.0 / tau, a0=a[0], a1=a[1], a2=a[2], p=p, chunk=chunk, flags=flags)
+    o, g = lib.forward(q, k, v, **kw)
+    dq, dk, dv = lib.backward(q, k, v, o, g, go, **kw)
+    ref = oracle_all(q, k, v, go, mask=mask, tau=tau, p=p, a=a)
+    errs = {n: O.rel_l2(x, r) for n, x, r in zip(("o", "g", "dq", "dk", "dv"), (o, g, dq, dk, dv), ref)}
+    for n, e in errs.items():
+        assert e < TOL[dtype], f"{n} rel-L2 {e:.3e} (all: {errs})"
+    return errs

@@ -1,0 +1,73 @@
+"""GPU parity tests: the HIP path through the C ABI against the CPU oracle on the
+same seeded inputs.  Tolerances: rel-L2 1e-5 (fp32), 2e-2 (bf16, oracle fed the
+bf16-rounded inputs)."""
+import pytest
+import torch
+
+from tests.parity import check_forward, check_forward_backward
+from reproducing_fastmax_results_amd._capi import FLAG_FORCE_DENSE, FLAG_FORCE_MOMENTS
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from reproducing_fastmax_results_amd._capi import get_lib
+    return get_lib()
+
+
+DEV = "cuda:0"
+
+
+def test_mfma_lane_layout(lib):
+    """The kernels assume: lane l owns D[8*(e/4) + 4*(l/32) + e%4][l%32] of a 32x32 tile."""
+    a16, a32 = lib.probe_mfma(DEV)
+    torch.cuda.synchronize()
+    lane = torch.arange(64).view(64, 1)
+    e = torch.arange(16).view(1, 16)
+    row = 8 * (e // 4) + 4 * (lane // 32) + e % 4
+    col = lane % 32
+    want = ((row + 1) * 100 + (col + 1)).float()
+    assert torch.equal(a16.cpu(), want)
+    assert torch.equal(a32.cpu(), want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mask", [False, True])
+@pytest.mark.parametrize("p", [1, 2])
+@pytest.mark.parametrize("d", [32, 64])
+def test_forward_dense_small(lib, dtype, mask, p, d):
+    print(f"case dense dtype={dtype} mask={mask} p={p} d={d}", flush=True)
+    check_forward(lib, 3, 333, d, dtype, DEV, mask=mask, p=p, flags=FLAG_FORCE_DENSE, seed=1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mask", [False, True])
+@pytest.mark.parametrize("p", [1, 2])
+@pytest.mark.parametrize("d", [32, 64])
+def test_forward_moments_small(lib, dtype, mask, p, d):
+    print(f"case moments dtype={dtype} mask={mask} p={p} d={d}", flush=True)
+    check_forward(lib, 3, 1100, d, dtype, DEV, mask=mask, p=p, chunk=256, flags=FLAG_FORCE_MOMENTS, seed=2)
+
+
+def test_forward_config1(lib):
+    # Fastmax order-2 forward, unmasked, fp32: B=1, H=2, N=256, D=Dv=32
+    for flags in (FLAG_FORCE_DENSE, FLAG_FORCE_MOMENTS):
+        print(f"case config1 flags={flags}", flush=True)
+        check_forward(lib, 2, 256, 32, torch.float32, DEV, mask=False, p=2, flags=flags, seed=0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_forward_config2_heads(lib, dtype):
+    # causal order 2, N=4096, D=64: 4 of the 32 (b, h) slices against the fp64 closed form
+    print(f"case config2 fwd dtype={dtype}", flush=True)
+    check_forward(lib, 4, 4096, 64, dtype, DEV, mask=True, p=2, seed=1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_forward_ragged_and_cross(lib, dtype):
+    print(f"case ragged dtype={dtype}", flush=True)
+    check_forward(lib, 2, 1, 64, dtype, DEV, mask=True, p=2, seed=3)
+    check_forward(lib, 2, 50, 32, dtype, DEV, mask=False, p=2, seed=4)          # ViT shape: 49 patches + CLS
+    check_forward(lib, 2, 257, 64, dtype, DEV, mask=False, p=2, nk=513, seed=5)  # nq != nk, unmasked
+    check_forward(lib, 1, 700, 64, dtype, DEV, mask=False, p=2, nk=4500, seed=6)  # automatic moment path
