@@ -191,10 +191,6 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   return fm_after_launch();
 }
 
-template <typename TIO, typename E, int DH, int QT>
-int run_backward(const FastmaxDesc* d, const Plan& p, const void* q, const void* k, const void* v, const void* o,
-                 const float* g, const void* d_o, void* dq, void* dk, void* dv, char* ws, fm_stream_t stream);
-
 }  // namespace
 
 #include "fastmax_api_bwd.inc"

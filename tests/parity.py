@@ -17,6 +17,15 @@ def make_inputs(bh, nq, nk, d, dtype, device, seed=0, scale=1.0):
     return tuple(t.to(device) for t in (q, k, v, go))
 
 
+def rel_err(x, ref):
+    """rel-L2, except that a reference that is identically ~0 (dq, dk of a single causal
+    token: the two O(1) terms gh.v and c cancel exactly) is measured against an
+    absolute scale of 1e-2 per element, i.e. fp32 passes below 1e-7 per element."""
+    x = x.detach().double().cpu(); ref = ref.detach().double().cpu()
+    floor = 1e-2 * ref.numel() ** 0.5
+    return float((x - ref).norm() / max(float(ref.norm()), floor))
+
+
 def oracle_all(q, k, v, go, *, mask, tau, p, a=(1.0, 1.0, 0.5), block=1024):
     """fp64 closed form on the (already rounded) inputs: o, g, dq, dk, dv."""
     args = [t.detach().cpu().double() for t in (q, k, v, go)]
@@ -32,7 +41,7 @@ def check_forward(lib, bh, nq, d, dtype, device, *, mask, p, nk=None, chunk=0, f
     tau = tau_mult * math.sqrt(d)
     o, g = lib.forward(q, k, v, mask=mask, inv_tau=1.0 / tau, a0=a[0], a1=a[1], a2=a[2], p=p, chunk=chunk, flags=flags)
     ref = oracle_all(q, k, v, go, mask=mask, tau=tau, p=p, a=a)
-    eo, eg = O.rel_l2(o, ref[0]), O.rel_l2(g, ref[1])
+    eo, eg = rel_err(o, ref[0]), rel_err(g, ref[1])
     assert eo < TOL[dtype], f"o rel-L2 {eo:.3e}"
     assert eg < TOL[dtype], f"g rel-L2 {eg:.3e}"
     return eo, eg
@@ -47,7 +56,7 @@ def check_forward_backward(lib, bh, nq, d, dtype, device, *, mask, p, nk=None, c
     o, g = lib.forward(q, k, v, **kw)
     dq, dk, dv = lib.backward(q, k, v, o, g, go, **kw)
     ref = oracle_all(q, k, v, go, mask=mask, tau=tau, p=p, a=a)
-    errs = {n: O.rel_l2(x, r) for n, x, r in zip(("o", "g", "dq", "dk", "dv"), (o, g, dq, dk, dv), ref)}
+    errs = {n: rel_err(x, r) for n, x, r in zip(("o", "g", "dq", "dk", "dv"), (o, g, dq, dk, dv), ref)}
     for n, e in errs.items():
         assert e < TOL[dtype], f"{n} rel-L2 {e:.3e} (all: {errs})"
     return errs

@@ -71,3 +71,40 @@ def test_forward_ragged_and_cross(lib, dtype):
     check_forward(lib, 2, 50, 32, dtype, DEV, mask=False, p=2, seed=4)          # ViT shape: 49 patches + CLS
     check_forward(lib, 2, 257, 64, dtype, DEV, mask=False, p=2, nk=513, seed=5)  # nq != nk, unmasked
     check_forward(lib, 1, 700, 64, dtype, DEV, mask=False, p=2, nk=4500, seed=6)  # automatic moment path
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mask", [False, True])
+@pytest.mark.parametrize("p", [1, 2])
+@pytest.mark.parametrize("d", [32, 64])
+def test_backward_dense_small(lib, dtype, mask, p, d):
+    print(f"case bwd dense dtype={dtype} mask={mask} p={p} d={d}", flush=True)
+    check_forward_backward(lib, 3, 333, d, dtype, DEV, mask=mask, p=p, flags=FLAG_FORCE_DENSE, seed=7)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mask", [False, True])
+@pytest.mark.parametrize("p", [1, 2])
+@pytest.mark.parametrize("d", [32, 64])
+def test_backward_moments_small(lib, dtype, mask, p, d):
+    print(f"case bwd moments dtype={dtype} mask={mask} p={p} d={d}", flush=True)
+    check_forward_backward(lib, 3, 1100, d, dtype, DEV, mask=mask, p=p, chunk=256, flags=FLAG_FORCE_MOMENTS, seed=8)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_backward_config2_heads(lib, dtype):
+    # Fastmax order-2 causal forward and backward, N=4096, D=64 (4 of the 32 slices, fp64 closed form)
+    print(f"case config2 fwd+bwd dtype={dtype}", flush=True)
+    check_forward_backward(lib, 4, 4096, 64, dtype, DEV, mask=True, p=2, seed=9)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_backward_ragged_and_cross(lib, dtype):
+    print(f"case bwd ragged dtype={dtype}", flush=True)
+    check_forward_backward(lib, 2, 1, 64, dtype, DEV, mask=True, p=2, seed=10)
+    check_forward_backward(lib, 2, 50, 32, dtype, DEV, mask=False, p=2, seed=11)
+    check_forward_backward(lib, 2, 257, 64, dtype, DEV, mask=False, p=2, nk=513, seed=12)
+    check_forward_backward(lib, 1, 700, 64, dtype, DEV, mask=False, p=2, nk=4500, seed=13)
+    check_forward_backward(lib, 1, 2500, 64, dtype, DEV, mask=True, p=2, seed=14)       # ragged last segment
+    check_forward_backward(lib, 2, 777, 32, dtype, DEV, mask=True, p=2, a=(1.0, 1.166666, 0.145833), tau_mult=1.0,
+                           seed=15)                                                    # fitted (non-Taylor) coefficients
