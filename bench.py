@@ -1,0 +1,152 @@
+#!/usr/bin/env python3
+"""Benchmark of the Fastmax hot path on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+One step = one forward + one backward of causal order-2 Fastmax on one batch of
+synthetic input (BASELINE.json configs[1]: B=4, H=8, N=4096, D=Dv=64, bf16,
+q, k, v, dO ~ N(0,1), tau = 8*sqrt(D), Taylor coefficients), inputs resident in
+HBM, called through the C ABI (libfastmax_hip.so).  Prints ONE JSON line.
+
+Besides the contract fields the line carries
+  roofline:     the dominant kernel, measured live with HIP events on the launch
+                stream (fastmax_profile_begin/end), priced with the ALGORITHMIC
+                flop count 2*(D + D^2)*(Dv + 1) per (b, h, token) and unit of
+                work (state build, readout, dQ, dK, dV each count one unit);
+  cpu_baseline: the oracle's port of the reference's einops algorithm timed on
+                this box's host cores on a bounded sample (one (b, h) slice).
+Everything runs on one GPU; --gpus N > 1 is refused.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}      # MI355X dense matrix peaks (published)
+PEAK_HBM_GBS = 8000.0
+
+WORKLOAD = dict(name="configs[1]: causal order-2 fwd+bwd", B=4, H=8, N=4096, D=64, p=2, mask=True)
+
+# units of algorithmic work (each 2*M_p*(Dv+1) flop per (b, h, token)) per launch of each kernel
+UNITS = {"build": 1, "fwd": 1, "dq": 1, "dkv": 2}
+
+
+def alg_flops_unit(bh: int, n: int, d: int, p: int) -> float:
+    m = d + (d * d if p == 2 else 0)
+    return 2.0 * m * (d + 1) * bh * n
+
+
+def cpu_baseline(n: int, d: int, p: int, tokens_per_step: int, heads_total: int, max_n: int):
+    """Port of the reference's einops factorised path (oracle), fp32, one (b, h) slice."""
+    import torch
+    from oracle import fastmax_oracle as O
+    threads = torch.get_num_threads()          # follows OMP_NUM_THREADS (the box's CPU share)
+    n_run = min(n, max_n)
+    gen = torch.Generator().manual_seed(1)
+    q, k, v, go = (torch.randn(1, 1, n_run, d, generator=gen) for _ in range(4))
+    tau = 8.0 * math.sqrt(d)
+    t0 = time.perf_counter()
+    o, g = O.factorised_forward(q, k, v, mask=True, tau=tau, p=p)
+    dq, dk, dv = O.factorised_backward(q, k, v, o, g, go, mask=True, tau=tau, p=p)
+    dt = time.perf_counter() - t0
+    # linear-time algorithm: scale the slice to the full sequence and to all heads
+    t_step = dt * (n / n_run) * heads_total
+    sample = f"1 of {heads_total} (b,h) slices, N={n_run}" + ("" if n_run == n else f" (scaled linearly to N={n})") + \
+             f", fp32, fwd+bwd, scaled x{heads_total}; {dt:.1f} s measured"
+    return {"value": tokens_per_step / t_step, "unit": "tokens/s", "cores": threads, "kind": "port", "sample": sample}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "f32"])
+    ap.add_argument("--chunk", type=int, default=0, help="segment length of the causal moment scan (0 = library default)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-max-n", type=int, default=2048, help="longest slice the CPU baseline materialises")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (every (b,h) slice is independent; "
+              "see DESIGN.md for how the path would shard); run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import torch
+    from reproducing_fastmax_results_amd._capi import get_lib
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+    lib = get_lib()
+    dev = torch.device("cuda:0")
+    W = WORKLOAD
+    B, H, N, D, p = W["B"], W["H"], W["N"], W["D"], W["p"]
+    bh = B * H
+    tdtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    gen = torch.Generator(device="cpu").manual_seed(1)
+    q, k, v, go = (torch.randn(B, H, N, D, generator=gen).to(tdtype).to(dev).view(bh, N, D) for _ in range(4))
+    tau = 8.0 * math.sqrt(D)
+    kw = dict(mask=True, inv_tau=1.0 / tau, a0=1.0, a1=1.0, a2=0.5, p=p, chunk=args.chunk)
+
+    def step():
+        o, g = lib.forward(q, k, v, **kw)
+        return lib.backward(q, k, v, o, g, go, **kw)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = 1e3 * elapsed / args.steps
+    tokens = B * N
+    value = tokens * args.steps / elapsed
+
+    # per-kernel durations, HIP events on the launch stream
+    nprof = max(3, min(10, args.steps))
+    lib.profile_begin()
+    for _ in range(nprof):
+        step()
+    recs = lib.profile_end()
+    per_kernel = {}
+    for name, ms in recs:
+        tot, cnt = per_kernel.get(name, (0.0, 0))
+        per_kernel[name] = (tot + ms, cnt + 1)
+    dominant = max(per_kernel, key=lambda nme: per_kernel[nme][0])
+    avg_ms = per_kernel[dominant][0] / per_kernel[dominant][1]
+    unit = alg_flops_unit(bh, N, D, p)
+    achieved = UNITS.get(dominant, 0) * unit / (avg_ms * 1e-3) / 1e12
+    peak = PEAK_TFLOPS[args.dtype]
+    roofline = {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
+                "frac": achieved / peak, "traffic": None, "avg_ms": avg_ms,
+                "whole_step": {"achieved": 7 * unit / (ms_per_step * 1e-3) / 1e12,
+                               "frac": 7 * unit / (ms_per_step * 1e-3) / 1e12 / peak},
+                "kernels_ms_per_step": {nme: tot / nprof for nme, (tot, cnt) in sorted(per_kernel.items())}}
+
+    out = {
+        "metric": "Fastmax fwd+bwd tokens/s, causal order-2 N=4096 D=64",
+        "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic",
+        "config": {"workload": f"{W['name']} B={B} H={H} N={N} D=Dv={D} tau=8*sqrt(D) a=(1,1,0.5)",
+                   "chunk": args.chunk or "auto"},
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(N, D, p, tokens, bh, args.cpu_max_n)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

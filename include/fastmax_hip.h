@@ -105,6 +105,14 @@ const char* fastmax_status_string(int status);
 /* Library version: major * 10000 + minor * 100 + patch. */
 int fastmax_version(void);
 
+/* Per-kernel timing for benchmarks (no counterpart in the reference).  Between begin and end the
+ * library brackets every kernel it launches with HIP events on the launch stream; end waits for
+ * them and returns how many launches were recorded, filling up to `capacity` entries with the
+ * kernel id (0 transpose, 1 backward prep, 2 state build, 3 forward, 4 dQ, 5 dK/dV, 6 normalise)
+ * and its duration.  Process-global and not re-entrant: do not use from concurrent threads. */
+int fastmax_profile_begin(void);
+int fastmax_profile_end(int* kernel_ids, float* milliseconds, int capacity);
+
 /* Self-check of the matrix-core lane layout the kernels assume: runs one 32x32 MFMA tile per
  * element type on known operands and writes, for each of the 64 lanes and 16 accumulator
  * registers, the value found (out_f16 and out_f32: 1024 floats each, device memory). */

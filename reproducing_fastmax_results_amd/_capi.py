@@ -48,6 +48,7 @@ class NormDesc(C.Structure):
 EXPORTS = (
     "fastmax_workspace_bytes", "fastmax_forward", "fastmax_backward", "fastmax_normalize",
     "fastmax_status_string", "fastmax_version", "fastmax_probe_mfma",
+    "fastmax_profile_begin", "fastmax_profile_end",
 )
 
 
@@ -96,6 +97,9 @@ class FastmaxLib:
         L.fastmax_version.restype = C.c_int
         L.fastmax_probe_mfma.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
         L.fastmax_probe_mfma.restype = C.c_int
+        L.fastmax_profile_begin.restype = C.c_int
+        L.fastmax_profile_end.argtypes = [C.POINTER(C.c_int), C.POINTER(C.c_float), C.c_int]
+        L.fastmax_profile_end.restype = C.c_int
 
     # -- helpers ---------------------------------------------------------------
     def status_string(self, st: int) -> str:
@@ -190,6 +194,18 @@ class FastmaxLib:
         st = self.lib.fastmax_normalize(C.byref(nd), x.data_ptr(), out.data_ptr(), stats.data_ptr(), self._stream(x))
         self.check(st, "fastmax_normalize")
         return out
+
+    KERNEL_NAMES = ("transpose", "prep_bwd", "build", "fwd", "dq", "dkv", "normalize")
+
+    def profile_begin(self) -> None:
+        self.lib.fastmax_profile_begin()
+
+    def profile_end(self, capacity: int = 4096):
+        """[(kernel name, milliseconds)] for every launch since profile_begin()."""
+        ids = (C.c_int * capacity)()
+        ms = (C.c_float * capacity)()
+        n = min(self.lib.fastmax_profile_end(ids, ms, capacity), capacity)
+        return [(self.KERNEL_NAMES[ids[i]], float(ms[i])) for i in range(n)]
 
     def probe_mfma(self, device):
         a = torch.zeros(1024, dtype=torch.float32, device=device)

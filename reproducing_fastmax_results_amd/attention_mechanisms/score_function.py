@@ -1,0 +1,190 @@
+"""Operator fronts of the Fastmax path, on the HIP kernels.
+
+Mirrors, name for name, what a model written against the reference imports:
+
+* ``FASTMultiHeadAttention_Function`` / ``FASTMultiHeadAttention`` /
+  ``rpe_matrix_creator`` / ``fastmax_custom`` - the autograd wrapper around the
+  extension (reference ``transformer/model.py:14-74, 208-248``), same argument
+  list ``(q, k, v, drop_noise, rpe_matrix, mask, dropout, normalize,
+  temperature, a0, a1, a2, lim, p)``;
+* ``fastmax(q, k, v, mask, denum_term, normalize, p, create_attn_matrix,
+  dropout_rate)`` - the score function (reference
+  ``attention_mechanisms/score_function.py:7-17``);
+* ``fastmax_einops(q, k, v, mask, normalize_term, tensors_normalized, p, ...)`` -
+  the einops front (reference ``attention_mechanisms/fastattention_einops.py:7-27``).
+
+Differences from the reference wrapper, all deliberate:
+the (b,h,n,d) <-> (n,b*h,d) transposes and their copies are gone (the kernels take
+strides), nothing is mutated in place, and the gradient with respect to k carries
+the 1/temperature factor inside the kernel instead of a separate division.
+There is no fallback: without the built extension the import fails.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from .. import fastmax_cuda as _ext   # the torch binding built by __graft_entry__.build()
+
+__all__ = [
+    "FASTMultiHeadAttention_Function", "FASTMultiHeadAttention", "rpe_matrix_creator", "fastmax_custom",
+    "fastmax", "fastmax_einops", "FastmaxNormalize",
+]
+
+CENTRE_NONE, CENTRE_FEATURE, CENTRE_TOKEN = 0, 1, 2
+
+
+def _torch_normalize(x, centre: int, scale: float):
+    """Differentiable restatement of the normalisation kernel (used for its backward)."""
+    if centre == CENTRE_FEATURE:
+        x = x - x.mean(-1, keepdim=True)
+    elif centre == CENTRE_TOKEN:
+        x = x - x.mean(-2, keepdim=True)
+    m = torch.linalg.vector_norm(x.float(), dim=-1).amax(-1)
+    return (scale * x.float() / m[..., None, None]).to(x.dtype)
+
+
+class FastmaxNormalize(torch.autograd.Function):
+    """``y = scale * (x - centre) / max_n ||x_n - centre||_2`` per (b, h): forward on the
+    fused HIP pass, backward by differentiating the same formula (the reference's
+    extension drops this gradient; its Python variants carry it through autograd,
+    ``score_function.py:40-55``)."""
+
+    @staticmethod
+    def forward(ctx, x, centre: int = CENTRE_NONE, scale: float = 1.0):
+        ctx.save_for_backward(x)
+        ctx.centre, ctx.scale = centre, scale
+        return _ext.normalize(x, centre, True, scale)
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        (x,) = ctx.saved_tensors
+        with torch.enable_grad():
+            xr = x.detach().requires_grad_(True)
+            y = _torch_normalize(xr, ctx.centre, ctx.scale)
+            (gx,) = torch.autograd.grad(y, xr, grad_y)
+        return gx, None, None
+
+
+class FASTMultiHeadAttention_Function(torch.autograd.Function):
+    """Same call as reference ``transformer/model.py:16``.  q, k, v: ``(b, h, n, d)`` or
+    ``(b*h, n, d)``.  ``drop_noise``, ``rpe_matrix`` and ``dropout`` are accepted and unused,
+    as in the reference extension (``fastmax_cuda_forward.cu:289, 443``).  With
+    ``normalize`` the tensors are first mapped to ``lim * x / max_n ||x_n||`` (the
+    semantics spelled out in ``transformer/model.py:97-102``) and, like the reference,
+    the returned gradients are those with respect to the normalised q and k.
+    """
+
+    @staticmethod
+    def forward(ctx, q, k, v, drop_noise=None, rpe_matrix=None, mask=False, dropout=0.0, normalize=False,
+                temperature=1.0, a0=1.0, a1=1.0, a2=0.5, lim=1.0, p=2):
+        if q.dim() not in (3, 4):
+            raise ValueError("q, k, and v should be either 3 or 4 dimensional tensors. "
+                             "If 3D: (b*h,n,d), if 4D: (b,h,n,d).")
+        if normalize:
+            q = _ext.normalize(q, CENTRE_NONE, True, float(lim))
+            k = _ext.normalize(k, CENTRE_NONE, True, float(lim))
+        inv_tau = 1.0 / float(temperature)
+        o, g = _ext.forward_ex(q, k, v, bool(mask), inv_tau, float(a0), float(a1), float(a2), int(p), 0, 0)
+        ctx.save_for_backward(q, k, v, o, g)
+        ctx.cfg = (bool(mask), inv_tau, float(a0), float(a1), float(a2), int(p))
+        return o
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        q, k, v, o, g = ctx.saved_tensors
+        mask, inv_tau, a0, a1, a2, p = ctx.cfg
+        gq, gk, gv = _ext.backward_ex(q, k, v, o, g, grad_output, mask, inv_tau, a0, a1, a2, p, 0, 0)
+        return (gq, gk, gv) + (None,) * 11
+
+
+def fastmax_function(q, k, v, mask=0, dropout_rate=0.0, normalize=0, temperature=1, a0=1, a1=1, a2=0.5, lim=1, p=2):
+    """Functional form with the argument order of the reference's (disabled) pure-torch
+    twin ``fastmax_function`` (``transformer/model.py:77``); routed to the kernels."""
+    return FASTMultiHeadAttention_Function.apply(q, k, v, None, None, bool(mask), dropout_rate, bool(normalize),
+                                                 temperature, a0, a1, a2, lim, p)
+
+
+class FASTMultiHeadAttention(torch.nn.Module):
+    """Reference ``transformer/model.py:208-216``."""
+
+    def __init__(self, use_custom_gradient=True):
+        super().__init__()
+        self.use_custom_gradient = use_custom_gradient
+
+    def forward(self, q, k, v, drop_noise=None, rpe_matrix=None, mask=False, dropout=0.0, normalize=False,
+                temperature=1.0, a0=1.0, a1=1.0, a2=0.5, lim=1.0, p=2):
+        return FASTMultiHeadAttention_Function.apply(q, k, v, drop_noise, rpe_matrix, mask, dropout, normalize,
+                                                     temperature, a0, a1, a2, lim, p)
+
+
+def rpe_matrix_creator(n, d, device, dtype, structured=False, is_zero=True):
+    """``(2n-1, d)`` relative-position matrix (reference ``transformer/model.py:218-247``).
+    The kernels do not read it (neither does the reference extension); it exists so
+    that call sites written for the reference keep working."""
+    if structured:
+        position = torch.arange(0, n, device=device, dtype=dtype).unsqueeze(1)
+        div_term = torch.exp(torch.arange(0, d, 2, device=device, dtype=dtype) * -(math.log(10000.0) / d))
+        pos = torch.zeros(n, d, device=device, dtype=dtype)
+        neg = torch.zeros(n, d, device=device, dtype=dtype)
+        pos[:, 0::2] = torch.sin(position * div_term)
+        pos[:, 1::2] = torch.cos(position * div_term)
+        neg[:, 0::2] = torch.sin(-position * div_term)
+        neg[:, 1::2] = torch.cos(-position * div_term)
+        return torch.cat([torch.flip(pos, [0]), neg[1:]], dim=0)
+    if is_zero:
+        return torch.zeros(size=(2 * n - 1, d), device=device, dtype=dtype)
+    return torch.normal(0, 1, size=(2 * n - 1, d), device=device, dtype=dtype)
+
+
+fastmax_custom = FASTMultiHeadAttention()
+
+
+def _attn_matrix(q, k, mask, tau, p):
+    """Quadratic debug path (reference ``score_function.py:226-247``): explicit attention
+    matrix in torch; not a hot path."""
+    s = torch.matmul(q.float(), k.float().transpose(-1, -2)) / tau
+    f = 1 + s + (0.5 * s * s if p == 2 else 0)
+    if mask:
+        f = f * torch.ones_like(f).tril()
+    return f / f.sum(-1, keepdim=True)
+
+
+def fastmax(q, k, v, mask=None, denum_term=8, normalize=0, p=1, create_attn_matrix=False, dropout_rate=0):
+    """Same call as reference ``attention_mechanisms/score_function.py:7``.
+
+    ``normalize == 1``: q and k are centred over tokens and divided by their largest
+    token norm, and the score is their plain dot product; otherwise the score is
+    divided by ``denum_term * sqrt(d)``.  ``dropout_rate`` must be 0 (the reference's
+    random feature dropout has no seeded counterpart)."""
+    if dropout_rate:
+        raise NotImplementedError("fastmax: dropout_rate != 0 is not supported by the HIP path")
+    masked = False if mask is None else bool(mask)      # reference: `if mask is None or not mask` -> unmasked
+    d = q.shape[-1]
+    if create_attn_matrix:
+        a = _attn_matrix(q, k, masked, denum_term * math.sqrt(d), 2)
+        return torch.matmul(a, v.float()).to(q.dtype), a
+    if normalize == 1:
+        q = FastmaxNormalize.apply(q, CENTRE_TOKEN, 1.0)
+        k = FastmaxNormalize.apply(k, CENTRE_TOKEN, 1.0)
+        temperature = 1.0
+    else:
+        temperature = denum_term * math.sqrt(d)
+    return FASTMultiHeadAttention_Function.apply(q, k, v, None, None, masked, 0.0, False, temperature,
+                                                 1.0, 1.0, 0.5, 1.0, int(p))
+
+
+def fastmax_einops(q, k, v, mask=True, normalize_term=8, tensors_normalized=False, p=1, dropout_rate=0.0,
+                   create_attn=False):
+    """Same call as the reference's einops front (``fastattention_einops.py:7-27``): the
+    score is divided by ``normalize_term * sqrt(d)`` unless ``tensors_normalized``
+    (``:78-82``); ``mask`` follows the reference's identity test, anything but ``False``
+    means causal (``:85``)."""
+    d = q.shape[-1]
+    tau = 1.0 if tensors_normalized is True else normalize_term * math.sqrt(d)
+    masked = mask is not False
+    if create_attn:
+        a = _attn_matrix(q, k, masked, tau, int(p))
+        return torch.matmul(a, v.float()).to(q.dtype), a
+    return FASTMultiHeadAttention_Function.apply(q, k, v, None, None, masked, 0.0, False, tau, 1.0, 1.0, 0.5, 1.0, int(p))

@@ -4,6 +4,7 @@
 #include "fm_kernels.h"
 #include "fm_kernels_bwd.h"
 #include "fm_norm.h"
+#include <vector>
 
 namespace {
 
@@ -16,6 +17,27 @@ inline void fm_allow_lds(const void* fn, size_t bytes) {
   // needed above the 64 KiB default; harmless below it
   (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, int(bytes));
 }
+#endif
+
+// ---- optional per-kernel timing (used by the benchmark; not re-entrant) --------
+enum { FM_K_TRANSPOSE = 0, FM_K_PREP_BWD = 1, FM_K_BUILD = 2, FM_K_FWD = 3, FM_K_DQ = 4, FM_K_DKV = 5, FM_K_NORM = 6 };
+#if defined(FM_HOSTSIM)
+struct ProfScope { ProfScope(int, fm_stream_t) {} };
+#else
+struct ProfRec { int id; hipEvent_t a, b; };
+bool g_prof_on = false;
+std::vector<ProfRec> g_prof;
+struct ProfScope {
+  bool on; fm_stream_t s; size_t idx;
+  ProfScope(int id, fm_stream_t stream) : on(g_prof_on), s(stream), idx(0) {
+    if (!on) return;
+    ProfRec r; r.id = id;
+    hipEventCreate(&r.a); hipEventCreate(&r.b);
+    hipEventRecord(r.a, s);
+    g_prof.push_back(r); idx = g_prof.size() - 1;
+  }
+  ~ProfScope() { if (on) hipEventRecord(g_prof[idx].b, s); }
+};
 #endif
 
 inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
@@ -119,6 +141,7 @@ template <typename T> TRef<T> mref(void* ptr, const FastmaxStrides& s) {
 template <typename TIO, typename E, int DH>
 int launch_transpose(const void* x, const FastmaxStrides& s, int bh, int n, int npad, E* xt, fm_stream_t stream) {
   TRef<const TIO> r = cref<TIO>(x, s);
+  ProfScope prof(FM_K_TRANSPOSE, stream);
   FM_KERNEL_LAUNCH((k_transpose<TIO, E, DH>), fm_dim3(npad / 64, bh), fm_dim3(FM_THREADS), 0, stream,
                    r.p, r.s_bh, r.s_n, r.vec, n, npad, xt);
   return fm_after_launch();
@@ -131,6 +154,7 @@ int launch_build(const BuildArgs<E>& a, int bh, fm_stream_t stream) {
   const size_t lds = size_t(4) * DH * PT * sizeof(E);
   const int nsteps = a.mode == FM_WALK_TOTAL ? 1 : a.nseg - 1;
   if (nsteps <= 0) return FASTMAX_OK;
+  ProfScope prof(FM_K_BUILD, stream);
   // two values of a per wavefront when that still fills the GPU, else one
   const bool na2 = int64_t(bh) * (DH / 8) >= 256;
   if (na2) {
@@ -186,6 +210,7 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   typedef TokCfg<E, DH, QT> C;
   const size_t lds = tok_lds_bytes<E, DH, QT>(0);
   fm_allow_lds(reinterpret_cast<const void*>(&k_fwd<TIO, E, DH, QT>), lds);
+  ProfScope prof(FM_K_FWD, stream);
   FM_KERNEL_LAUNCH((k_fwd<TIO, E, DH, QT>), fm_dim3((d->nq + C::QW - 1) / C::QW, d->bh), fm_dim3(FM_THREADS), lds,
                    stream, a);
   return fm_after_launch();
@@ -270,6 +295,34 @@ int fastmax_backward(const FastmaxDesc* desc, const void* q, const void* k, cons
 
 int fastmax_normalize(const FastmaxNormDesc* desc, const void* x, void* y, float* stats, void* hip_stream) {
   return fm_normalize_dispatch(desc, x, y, stats, static_cast<fm_stream_t>(hip_stream));
+}
+
+int fastmax_profile_begin(void) {
+#if !defined(FM_HOSTSIM)
+  for (auto& r : g_prof) { hipEventDestroy(r.a); hipEventDestroy(r.b); }
+  g_prof.clear();
+  g_prof_on = true;
+#endif
+  return FASTMAX_OK;
+}
+
+int fastmax_profile_end(int* kernel_ids, float* milliseconds, int capacity) {
+  int n = 0;
+#if !defined(FM_HOSTSIM)
+  g_prof_on = false;
+  for (auto& r : g_prof) {
+    hipEventSynchronize(r.b);
+    float ms = 0.f;
+    hipEventElapsedTime(&ms, r.a, r.b);
+    if (n < capacity) { if (kernel_ids) kernel_ids[n] = r.id; if (milliseconds) milliseconds[n] = ms; }
+    ++n;
+    hipEventDestroy(r.a); hipEventDestroy(r.b);
+  }
+  g_prof.clear();
+#else
+  (void)kernel_ids; (void)milliseconds; (void)capacity;
+#endif
+  return n;
 }
 
 int fastmax_probe_mfma(float* out_f16, float* out_f32, void* hip_stream) {

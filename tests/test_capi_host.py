@@ -1,0 +1,99 @@
+"""CPU-side tests of the C ABI: the library loads, exports every symbol the header declares,
+and rejects bad arguments with the documented status codes (no kernel is launched)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from reproducing_fastmax_results_amd import _capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "reproducing_fastmax_results_amd", _capi.LIB_NAME)
+
+pytestmark = pytest.mark.skipif(not os.path.exists(LIB), reason="libfastmax_hip.so not built (run __graft_entry__.build())")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _capi.FastmaxLib(LIB)
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "fastmax_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fastmax_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_exports_match_header(lib):
+    names = declared_functions()
+    assert set(names) == set(_capi.EXPORTS)
+    for n in names:
+        assert getattr(lib.lib, n) is not None
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    with pytest.raises(ImportError, match="no CPU fallback"):
+        _capi.FastmaxLib(str(tmp_path / "libfastmax_hip.so"))
+
+
+def base_desc(**kw):
+    d = _capi.Desc()
+    d.bh, d.nq, d.nk, d.d = 4, 128, 128, 64
+    d.dtype, d.mask, d.p = _capi.BF16, 1, 2
+    d.a0, d.a1, d.a2, d.inv_tau = 1.0, 1.0, 0.5, 0.125
+    for name in ("sq", "sk", "sv", "so", "sdo", "sdq", "sdk", "sdv"):
+        setattr(d, name, _capi.Strides(128 * 64, 64))
+    d.sg = _capi.Strides(128, 1)
+    for k, v in kw.items():
+        setattr(d, k, v)
+    return d
+
+
+def ws(lib, d):
+    f, b = C.c_size_t(0), C.c_size_t(0)
+    st = lib.lib.fastmax_workspace_bytes(C.byref(d), C.byref(f), C.byref(b))
+    return st, f.value, b.value
+
+
+def test_workspace_sizes_and_status_codes(lib):
+    st, f, b = ws(lib, base_desc())
+    assert st == 0 and f >= 256 and b >= f
+    assert ws(lib, base_desc(d=48))[0] == 3          # unsupported head size
+    assert ws(lib, base_desc(p=3))[0] == 3           # unsupported order
+    assert ws(lib, base_desc(nk=256))[0] == 3        # masked needs nq == nk
+    assert ws(lib, base_desc(nk=256, mask=0))[0] == 0
+    assert ws(lib, base_desc(dtype=7))[0] == 6
+    assert ws(lib, base_desc(bh=0))[0] == 2
+    assert lib.lib.fastmax_workspace_bytes(None, None, None) == 1
+    # long sequences use the moment scan: scratch grows with the number of segments
+    small = ws(lib, base_desc(nq=1024, nk=1024))[1]
+    large = ws(lib, base_desc(nq=8192, nk=8192))[1]
+    assert large > 8 * small / 2
+    for code in range(0, 8):
+        assert isinstance(lib.status_string(code), str) and lib.status_string(code)
+
+
+def test_forward_backward_reject_bad_arguments_before_launching(lib):
+    d = base_desc()
+    one = C.c_void_p(256)     # never dereferenced: validation fails first
+    assert lib.lib.fastmax_forward(C.byref(d), None, one, one, one, one, one, 1 << 30, None) == 1
+    assert lib.lib.fastmax_forward(C.byref(d), one, one, one, one, one, None, 0, None) == 4      # no workspace
+    assert lib.lib.fastmax_forward(C.byref(d), one, one, one, one, one, C.c_void_p(264), 1 << 30, None) == 4  # misaligned
+    assert lib.lib.fastmax_forward(C.byref(d), one, one, one, one, one, one, 16, None) == 4     # too small
+    bad = base_desc()
+    bad.sq = _capi.Strides(128 * 64, 8)               # token stride smaller than the head size
+    assert lib.lib.fastmax_forward(C.byref(bad), one, one, one, one, one, one, 1 << 30, None) == 2
+    args = [one] * 9
+    assert lib.lib.fastmax_backward(C.byref(d), *args, None, 0, None) == 4
+    assert lib.lib.fastmax_backward(C.byref(d), None, *args[1:], one, 1 << 30, None) == 1
+    nd = _capi.NormDesc()
+    nd.bh, nd.n, nd.d, nd.dtype, nd.centre, nd.max_norm, nd.scale = 2, 10, 40, 0, 0, 1, 1.0
+    assert lib.lib.fastmax_normalize(C.byref(nd), one, one, one, None) == 3
+    nd.d, nd.centre = 64, 5
+    assert lib.lib.fastmax_normalize(C.byref(nd), one, one, one, None) == 3
+    nd.centre = 0
+    nd.sx = nd.sy = _capi.Strides(640, 64)
+    assert lib.lib.fastmax_normalize(C.byref(nd), one, one, None, None) == 4   # max_norm needs stats scratch
+    assert lib.lib.fastmax_probe_mfma(None, None, None) == 1
+    assert lib.lib.fastmax_version() >= 100

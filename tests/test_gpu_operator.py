@@ -1,0 +1,155 @@
+"""GPU tests of the torch binding (`fastmax_cuda`) and the operator fronts, against the oracle."""
+import math
+
+import pytest
+import torch
+
+from oracle import fastmax_oracle as O
+from tests.parity import TOL, rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ext():
+    from reproducing_fastmax_results_amd import fastmax_cuda
+    return fastmax_cuda
+
+
+@pytest.fixture(scope="module")
+def sf():
+    from reproducing_fastmax_results_amd.attention_mechanisms import score_function
+    return score_function
+
+
+def rnd(*shape, seed=0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed))
+
+
+@pytest.mark.parametrize("mask", [False, True])
+@pytest.mark.parametrize("p", [1, 2])
+def test_legacy_forwardpass_backwardpass(ext, mask, p):
+    """Reference call sequence of transformer/model.py:29-74 on (n, b*h, d) fp32 tensors."""
+    n, bh, d, t = 300, 6, 32, 3.7
+    q, k, v, go = (rnd(n, bh, d, seed=s) for s in (1, 2, 3, 4))
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    noise = torch.zeros_like(qd)
+    rpe = torch.zeros(2 * n - 1, d, device=DEV)
+    out = ext.forwardpass(qd, kd, vd, noise, rpe, mask, 0.1, False, t, 1.0, 1.0, 0.5, 1.0, p)
+    assert out.shape == (n, bh, d + 1) and out.dtype == torch.float32
+    # like the reference, k is left divided by the temperature (fastmax_cuda_forward.cu:288)
+    assert torch.allclose(kd.cpu(), k / t, rtol=1e-6, atol=1e-7)
+    assert torch.equal(qd.cpu(), q)
+    ref = O.extension_forward(q, k, v, mask=mask, temperature=t, a0=1.0, a1=1.0, a2=0.5, p=p)
+    assert rel_err(out, ref) < 1e-5
+    gq, gk, gv = ext.backwardpass(qd, kd, vd, out, go.to(DEV), mask, 1.0, 1.0, 0.5, p)
+    rq, rk, rv = O.extension_backward(q, k / t, v, go, mask=mask, a0=1.0, a1=1.0, a2=0.5, p=p)
+    for a, b in ((gq, rq), (gk, rk), (gv, rv)):
+        assert rel_err(a, b) < 1e-5
+
+
+def test_legacy_normalize_flag(ext):
+    n, bh, d = 130, 4, 64
+    q, k, v = (rnd(n, bh, d, seed=s) for s in (5, 6, 7))
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    out = ext.forwardpass(qd, kd, vd, torch.zeros_like(qd), torch.zeros(2 * n - 1, d, device=DEV), True, 0.0, True,
+                          2.0, 1.0, 1.0, 0.5, 1.5, 2)
+    qn = O.normalize_lim(q.permute(1, 0, 2).double(), 1.5).permute(1, 0, 2)
+    kn = O.normalize_lim(k.permute(1, 0, 2).double(), 1.5).permute(1, 0, 2)
+    assert rel_err(qd, qn) < 1e-5 and rel_err(kd, kn) < 1e-5
+    ref = O.extension_forward(qn, kn, v, mask=True, temperature=1.0, a0=1.0, a1=1.0, a2=0.5, p=2)
+    assert rel_err(out, ref) < 1e-5
+
+
+def test_legacy_errors(ext):
+    n, bh, d = 64, 2, 32
+    q = torch.randn(n, bh, d, device=DEV)
+    z = torch.zeros_like(q)
+    rpe = torch.zeros(2 * n - 1, d, device=DEV)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        ext.forwardpass(q.permute(1, 0, 2), q, q, z, rpe, True, 0.0, False, 1.0, 1.0, 1.0, 0.5, 1.0, 2)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        ext.forwardpass(q.cpu(), q, q, z, rpe, True, 0.0, False, 1.0, 1.0, 1.0, 0.5, 1.0, 2)
+    with pytest.raises(RuntimeError, match="unsupported"):
+        ext.forwardpass(q, q, q, z, rpe, True, 0.0, False, 1.0, 1.0, 1.0, 0.5, 1.0, 3)
+    q48 = torch.randn(n, bh, 48, device=DEV)
+    with pytest.raises(RuntimeError, match="unsupported"):
+        ext.forwardpass(q48, q48, q48, torch.zeros_like(q48), rpe, True, 0.0, False, 1.0, 1.0, 1.0, 0.5, 1.0, 2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("four_d", [False, True])
+def test_autograd_wrapper(sf, dtype, four_d):
+    b, h, n, d, t = 2, 3, 700, 64, 11.0
+    shape = (b, h, n, d) if four_d else (b * h, n, d)
+    q, k, v, go = (rnd(*shape, seed=s).to(dtype) for s in (8, 9, 10, 11))
+    qd, kd, vd = (x.to(DEV).requires_grad_(True) for x in (q, k, v))
+    noise = torch.zeros_like(qd)
+    rpe = sf.rpe_matrix_creator(n, d, DEV, torch.float32)
+    o = sf.FASTMultiHeadAttention_Function.apply(qd, kd, vd, noise, rpe, True, 0.1, False, t, 1.0, 1.0, 0.5, 1.0, 2)
+    assert o.shape == shape
+    o.backward(go.to(DEV))
+    ref = O.manual_backward_blocked(q.double(), k.double(), v.double(), go.double(), mask=True, tau=t, p=2)
+    assert rel_err(o, ref[0]) < TOL[dtype]
+    for got, want in ((qd.grad, ref[2]), (kd.grad, ref[3]), (vd.grad, ref[4])):
+        assert rel_err(got, want) < TOL[dtype]
+    # module form and the reference's model-side call (transformer/model.py:301-303)
+    o2 = sf.fastmax_custom(qd, kd, vd, noise, rpe, True, 0.1, False, t, 1.0, 1.0, 0.5, 1.0, 2)
+    assert torch.equal(o2, o)
+
+
+def test_transposed_projection_layout(sf):
+    """(b, n, h*d) projections viewed as (b, h, n, d) - the layout Attention.forward produces
+    (transformer/model.py:283-285) - are consumed through strides, without a copy."""
+    b, h, n, d = 2, 4, 260, 32
+    x = rnd(b, n, h * d, seed=12)
+    q = x.view(b, n, h, d).transpose(1, 2)
+    k = rnd(b, n, h * d, seed=13).view(b, n, h, d).transpose(1, 2)
+    v = rnd(b, n, h * d, seed=14).view(b, n, h, d).transpose(1, 2)
+    o = sf.fastmax_einops(q.to(DEV), k.to(DEV), v.to(DEV), mask=True, normalize_term=8, p=2)
+    ref, _ = O.closed_form_forward(q.double(), k.double(), v.double(), mask=True, tau=O.tau_einops(8, d), p=2)
+    assert rel_err(o, ref) < 1e-5
+
+
+@pytest.mark.parametrize("normalize", [0, 1])
+@pytest.mark.parametrize("mask", [None, True])
+@pytest.mark.parametrize("p", [1, 2])
+def test_score_function_front(sf, normalize, mask, p):
+    """fastmax(q,k,v,mask,denum_term,normalize,p) including gradients through the
+    token-mean / max-norm normalisation (score_function.py:40-57)."""
+    b, h, n, d = 1, 2, 150, 32
+    q, k, v, go = (rnd(b, h, n, d, seed=s) for s in (15, 16, 17, 18))
+    qd, kd, vd = (x.to(DEV).requires_grad_(True) for x in (q, k, v))
+    o = sf.fastmax(qd, kd, vd, mask=mask, denum_term=8, normalize=normalize, p=p)
+    o.backward(go.to(DEV))
+    qr, kr, vr = (x.double().requires_grad_(True) for x in (q, k, v))
+    oref = O.score_function_fastmax(qr, kr, vr, mask=mask, denum_term=8, normalize=normalize, p=p)
+    oref.backward(go.double())
+    assert rel_err(o, oref) < 1e-5
+    for got, want in ((qd.grad, qr.grad), (kd.grad, kr.grad), (vd.grad, vr.grad)):
+        assert rel_err(got, want) < 2e-5      # torch fp32 normalisation backward on top of the kernels
+
+
+def test_create_attn_matrix_debug_path(sf):
+    q, k, v = (rnd(1, 2, 40, 32, seed=s).to(DEV) for s in (19, 20, 21))
+    o, a = sf.fastmax(q, k, v, mask=True, p=2, create_attn_matrix=True)
+    assert torch.all(a.triu(1) == 0)                      # reference test_fastmax_iscausal
+    assert torch.allclose(a.sum(-1), torch.ones_like(a.sum(-1)), atol=1e-5)
+    o2 = sf.fastmax(q, k, v, mask=True, denum_term=8, p=2)
+    assert rel_err(o, o2) < 1e-5
+
+
+@pytest.mark.parametrize("centre", [0, 1, 2])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_normalize_kernel(ext, centre, dtype):
+    x = rnd(3, 2, 333, 64, seed=22).to(dtype)
+    y = ext.normalize(x.to(DEV), centre, True, 2.0)
+    xd = x.double()
+    if centre == 1:
+        ref = O.normalize_feature_mean(xd, xd)[0] * 2.0
+    elif centre == 2:
+        ref = O.normalize_token_mean(xd, xd)[0] * 2.0
+    else:
+        ref = O.normalize_lim(xd, 2.0)
+    assert rel_err(y, ref) < (1e-5 if dtype == torch.float32 else 1e-2)

@@ -1,0 +1,71 @@
+"""CPU run of the kernel sources through the host simulator (tests/hostsim/hostsim.h).
+
+The very same kernel templates the GPU runs are compiled as plain C++ with
+-DFM_HOSTSIM (work-items are OS threads, MFMA tiles are emulated with the lane
+layout the GPU probe test pins) and driven through the same C ABI.  This checks
+indexing, lane layouts, masks and ragged sizes without a GPU and, with
+FASTMAX_HOSTSIM_ASAN=1, under AddressSanitizer.  It is a test build only: the
+package never loads it.  Sizes are tiny because every work-item is a thread.
+"""
+import os
+import shutil
+import subprocess
+
+import pytest
+import torch
+
+from reproducing_fastmax_results_amd import _capi
+from tests.parity import check_forward, check_forward_backward
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CLANG = shutil.which("clang++", path="/opt/rocm/llvm/bin:" + os.environ.get("PATH", ""))
+
+pytestmark = pytest.mark.skipif(CLANG is None, reason="no clang++ for the host simulator build")
+
+
+@pytest.fixture(scope="module")
+def sim(tmp_path_factory):
+    out = str(tmp_path_factory.mktemp("hostsim") / "libfastmax_hostsim.so")
+    cmd = [CLANG, "-x", "c++", "-std=c++17", "-O2", "-DFM_HOSTSIM", "-Wno-psabi", "-fPIC", "-shared", "-pthread",
+           "-I", os.path.join(ROOT, "include"), "-I", os.path.join(ROOT, "tests", "hostsim"),
+           "-I", os.path.join(ROOT, "reproducing_fastmax_results_amd", "csrc"),
+           os.path.join(ROOT, "reproducing_fastmax_results_amd", "csrc", "fastmax_api.hip"), "-o", out]
+    subprocess.run(cmd, check=True, capture_output=True)
+    return _capi.FastmaxLib(out)
+
+
+def test_probe_matches_assumed_layout(sim):
+    a16, a32 = sim.probe_mfma("cpu")
+    lane = torch.arange(64).view(64, 1)
+    e = torch.arange(16).view(1, 16)
+    want = ((8 * (e // 4) + 4 * (lane // 32) + e % 4 + 1) * 100 + lane % 32 + 1).float()
+    assert torch.equal(a16, want) and torch.equal(a32, want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_dense_forward_backward(sim, dtype):
+    check_forward_backward(sim, 1, 70, 32, dtype, "cpu", mask=True, p=2, flags=_capi.FLAG_FORCE_DENSE, seed=1)
+    check_forward_backward(sim, 1, 33, 32, dtype, "cpu", mask=False, p=1, nk=45, seed=2)
+
+
+def test_moment_path_forward_backward_bf16(sim):
+    # two segments of 256: prefix state for the second, suffix state for the first
+    check_forward_backward(sim, 1, 300, 32, torch.bfloat16, "cpu", mask=True, p=2, chunk=256, seed=3)
+    check_forward_backward(sim, 1, 40, 32, torch.bfloat16, "cpu", mask=False, p=2, nk=260,
+                           flags=_capi.FLAG_FORCE_MOMENTS, seed=4)
+
+
+def test_moment_path_forward_fp32_d64(sim):
+    check_forward(sim, 1, 290, 64, torch.float32, "cpu", mask=True, p=2, chunk=256, seed=5)
+
+
+def test_normalize(sim):
+    from oracle import fastmax_oracle as O
+    x = torch.randn(2, 70, 32, generator=torch.Generator().manual_seed(6))
+    for centre, ref in ((0, O.normalize_lim(x.double(), 1.5)),
+                        (1, 1.5 * O.normalize_feature_mean(x.double(), x.double())[0]),
+                        (2, 1.5 * O.normalize_token_mean(x.double(), x.double())[0])):
+        y = sim.normalize(x, centre=centre, max_norm=True, scale=1.5)
+        assert O.rel_l2(y, ref) < 1e-6
+    y = sim.normalize(x, centre=0, max_norm=False, scale=0.25)
+    assert torch.allclose(y, 0.25 * x)
