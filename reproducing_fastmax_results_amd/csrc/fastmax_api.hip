@@ -4,6 +4,7 @@
 #include "fm_kernels.h"
 #include "fm_kernels_bwd.h"
 #include "fm_norm.h"
+#include <cmath>
 #include <vector>
 
 namespace {
@@ -50,11 +51,12 @@ struct Plan {
   int L, nseg, nslots;
   bool use_state, quad;
   int npad_q, npad_k;
-  float c0, c1, c2;     // polynomial on the raw dot product
+  float a0, a1, a2;     // polynomial on the score s = (q.k) / tau
+  float sc;             // sqrt(1/tau), folded into q and k when they are converted
+  float gscale;         // power of two folded into dO / g in the backward
   // workspace offsets (bytes)
   size_t kt, vt, big, small, fwd_bytes;
-  size_t b_kt, b_vt, b_qt, b_qct, b_gh, b_ght, b_cv, b_bigq, b_smallq, b_bigk, b_smallk, b_bigv, b_smallv,
-      bwd_bytes;
+  size_t b_kt, b_vt, b_qt, b_qct, b_gh, b_ght, b_cv, b_bigq, b_smallq, b_bigk, b_smallk, b_bigv, bwd_bytes;
 };
 
 bool strides_ok(const FastmaxStrides& s, int bh, int n, int d) {
@@ -72,7 +74,7 @@ int validate(const FastmaxDesc* d) {
   if (d->d != 32 && d->d != 64) return FASTMAX_ERR_UNSUPPORTED;
   if (d->mask && d->nq != d->nk) return FASTMAX_ERR_UNSUPPORTED;
   if (d->chunk < 0) return FASTMAX_ERR_SHAPE;
-  if (!(d->inv_tau == d->inv_tau)) return FASTMAX_ERR_SHAPE;
+  if (!(d->inv_tau > 0.0f) || !(d->inv_tau < 3.0e38f)) return FASTMAX_ERR_SHAPE;   // also rejects NaN
   return FASTMAX_OK;
 }
 
@@ -87,9 +89,15 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   p.npad_q = int(round_up(d->nq, 256));
   p.npad_k = int(round_up(d->nk, 256));
   p.quad = d->p == 2 && d->a2 != 0.0f;
-  p.c0 = d->a0;
-  p.c1 = d->a1 * d->inv_tau;
-  p.c2 = p.quad ? d->a2 * d->inv_tau * d->inv_tau : 0.0f;
+  p.a0 = d->a0;
+  p.a1 = d->a1;
+  p.a2 = p.quad ? d->a2 : 0.0f;
+  p.sc = std::sqrt(std::fabs(d->inv_tau));
+  {
+    int e = 0;
+    while ((int64_t(1) << e) < d->nq) ++e;
+    p.gscale = e > 6 ? float(int64_t(1) << (e - 6)) : 1.0f;
+  }
   const bool force_dense = (d->flags & FASTMAX_FLAG_FORCE_DENSE) != 0;
   if (d->mask) {
     int L = d->chunk > 0 ? int(round_up(d->chunk, 256)) : (d->nq >= 2048 ? 1024 : p.npad_q);
@@ -122,7 +130,7 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   p.b_cv = take(size_t(d->bh) * p.npad_q * 4);
   p.b_bigq = take(size_t(d->bh) * p.nslots * bigsz); p.b_smallq = take(size_t(d->bh) * p.nslots * smallsz);
   p.b_bigk = take(size_t(d->bh) * p.nslots * bigsz); p.b_smallk = take(size_t(d->bh) * p.nslots * smallsz);
-  p.b_bigv = take(size_t(d->bh) * p.nslots * bigsz); p.b_smallv = take(size_t(d->bh) * p.nslots * smallsz);
+  p.b_bigv = take(size_t(d->bh) * p.nslots * bigsz);
   p.bwd_bytes = off ? off : 256;
   return FASTMAX_OK;
 }
@@ -139,11 +147,12 @@ template <typename T> TRef<T> mref(void* ptr, const FastmaxStrides& s) {
 }
 
 template <typename TIO, typename E, int DH>
-int launch_transpose(const void* x, const FastmaxStrides& s, int bh, int n, int npad, E* xt, fm_stream_t stream) {
+int launch_transpose(const void* x, const FastmaxStrides& s, int bh, int n, int npad, E* xt, float scale,
+                     fm_stream_t stream) {
   TRef<const TIO> r = cref<TIO>(x, s);
   ProfScope prof(FM_K_TRANSPOSE, stream);
   FM_KERNEL_LAUNCH((k_transpose<TIO, E, DH>), fm_dim3(npad / 64, bh), fm_dim3(FM_THREADS), 0, stream,
-                   r.p, r.s_bh, r.s_n, r.vec, n, npad, xt);
+                   r.p, r.s_bh, r.s_n, r.vec, n, npad, xt, scale);
   return fm_after_launch();
 }
 
@@ -186,16 +195,17 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   E* vt = reinterpret_cast<E*>(ws + p.vt);
   E* big = reinterpret_cast<E*>(ws + p.big);
   float* small = reinterpret_cast<float*>(ws + p.small);
-  int st = launch_transpose<TIO, E, DH>(v, d->sv, d->bh, d->nk, p.npad_k, vt, stream);
+  int st = launch_transpose<TIO, E, DH>(v, d->sv, d->bh, d->nk, p.npad_k, vt, 1.0f, stream);
   if (st) return st;
   if (p.use_state) {
-    st = launch_transpose<TIO, E, DH>(k, d->sk, d->bh, d->nk, p.npad_k, kt, stream);
+    st = launch_transpose<TIO, E, DH>(k, d->sk, d->bh, d->nk, p.npad_k, kt, p.sc, stream);
     if (st) return st;
     BuildArgs<E> b;
     b.xt = kt; b.pt = vt; b.rt = kt; b.za = kt; b.zb = kt;
     b.npad = p.npad_k; b.nseg = p.nseg; b.L = p.L; b.mode = d->mask ? FM_WALK_PREFIX : FM_WALK_TOTAL;
     b.quad = p.quad; b.big = big; b.small = small; b.nslots = p.nslots;
-    b.coef2 = p.c2; b.coef1 = p.c1; b.coefz = p.c2; b.coefva = p.c1; b.coefvb = p.c0;
+    b.big2 = nullptr; b.vb_from_r = 0; b.coef2b = 0.0f; b.coef1b = 0.0f;
+    b.coef2 = p.a2; b.coef1 = p.a1; b.coefz = p.a2; b.coefva = p.a1; b.coefvb = p.a0;
     st = launch_build<E, DH>(b, d->bh, stream);
     if (st) return st;
   }
@@ -206,7 +216,7 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   a.vt = vt; a.npad_k = p.npad_k;
   a.big = big; a.small = small; a.nslots = p.nslots;
   a.nq = d->nq; a.nk = d->nk; a.L = p.L; a.causal = d->mask != 0; a.use_state = p.use_state; a.quad = p.quad;
-  a.a0 = p.c0; a.c1 = p.c1; a.c2 = p.c2;
+  a.a0 = p.a0; a.a1 = p.a1; a.a2 = p.a2; a.sc = p.sc;
   typedef TokCfg<E, DH, QT> C;
   const size_t lds = tok_lds_bytes<E, DH, QT>(0);
   fm_allow_lds(reinterpret_cast<const void*>(&k_fwd<TIO, E, DH, QT>), lds);

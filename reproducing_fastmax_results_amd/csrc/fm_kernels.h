@@ -80,13 +80,16 @@ struct RowRegs {
       }
     }
   }
-  FM_DEVICE void store(E* lds, int pitch, int tid) const {
+  FM_DEVICE void store(E* lds, int pitch, int tid, float scale) const {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
       const int c = tid + FM_THREADS * i;
       if (TOTAL % FM_THREADS == 0 || c < TOTAL) {
         const int row = c / CPR, col = (c % CPR) * 8;
-        CE<E>::st8(lds + row * pitch + col, v[i]);
+        float w[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) w[j] = v[i][j] * scale;
+        CE<E>::st8(lds + row * pitch + col, w);
       }
     }
   }
@@ -94,12 +97,12 @@ struct RowRegs {
 
 // ------------------------------------------------------------------------------
 // k_transpose: x (bh, n, DH) strided, interface type  ->  xt [bh][DH][npad], compute
-// type, zero for tokens >= n.  grid (npad/64, bh).
+// type, multiplied by `scale`, zero for tokens >= n.  grid (npad/64, bh).
 // ------------------------------------------------------------------------------
 template <typename TIO, typename E, int DH>
 FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS)
 k_transpose(const TIO* FM_RESTRICT x, int64_t s_bh, int64_t s_n, int vec, int n, int npad,
-            E* FM_RESTRICT xt) {
+            E* FM_RESTRICT xt, float scale) {
   constexpr int PT = 64 + Mma<E>::PAD;
   constexpr int VEC = Mma<E>::VEC;
   FM_SHARED E tile[DH * PT];
@@ -115,7 +118,7 @@ k_transpose(const TIO* FM_RESTRICT x, int64_t s_bh, int64_t s_n, int vec, int n,
       for (int j = 0; j < 8; ++j) v[j] = 0.f;
     }
 #pragma unroll
-    for (int j = 0; j < 8; ++j) tile[(d0 + j) * PT + tok] = CE<E>::from(v[j]);
+    for (int j = 0; j < 8; ++j) tile[(d0 + j) * PT + tok] = CE<E>::from(v[j] * scale);
   }
   FM_SYNC();
   E* ob = xt + int64_t(bh) * DH * npad + t0;
@@ -127,10 +130,13 @@ k_transpose(const TIO* FM_RESTRICT x, int64_t s_bh, int64_t s_n, int vec, int n,
 }
 
 // ------------------------------------------------------------------------------
-// k_prep_bwd: per token  gh = dO / g,  c = gh . o ; writes
+// k_prep_bwd: per token  gh = gscale * dO / g,  c = gh . o,  q' = qscale * q ; writes
 //   gh  [bh][npad][DH]  (row-major, compute type)      ght [bh][DH][npad]
-//   qt  [bh][DH][npad]  (q transposed)                  qct [bh][DH][npad]  (c_i q_i)
-//   cv  [bh][npad]      (fp32)
+//   qt  [bh][DH][npad]  (q' transposed)                 qct [bh][DH][npad]  (c_i q'_i)
+//   cv  [bh][npad]      (c, compute type)
+// gscale is a power of two that keeps gh inside the _Float16 range for long sequences
+// (g grows like the token index); every gradient is linear in (gh, c) and is divided
+// by gscale again when it is stored.
 // Tokens >= n are written as zeros.  grid (npad/64, bh).
 // Reference: div_grad_output, fastmax_cuda_backward.cu:494-501, and the
 // "grad * o" row sums of fastattention_einops.py:405-407.
@@ -141,7 +147,7 @@ template <typename TIO, typename E, int DH>
 FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS)
 k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, const float* FM_RESTRICT g,
            int64_t g_s_bh, int64_t g_s_n, int n, int npad, E* FM_RESTRICT gh, E* FM_RESTRICT ght,
-           E* FM_RESTRICT qt, E* FM_RESTRICT qct, float* FM_RESTRICT cv) {
+           E* FM_RESTRICT qt, E* FM_RESTRICT qct, E* FM_RESTRICT cv, float qscale, float gscale) {
   constexpr int PT = 64 + Mma<E>::PAD;
   constexpr int VEC = Mma<E>::VEC;
   constexpr int EPT = DH / 4;                      // elements per thread (4 threads per token)
@@ -154,7 +160,7 @@ k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, const floa
   float vg[EPT], vq[EPT];
   float csum = 0.f;
   if (row < n) {
-    const float ginv = 1.0f / g[int64_t(bh) * g_s_bh + int64_t(row) * g_s_n];
+    const float ginv = gscale / g[int64_t(bh) * g_s_bh + int64_t(row) * g_s_n];
 #pragma unroll
     for (int j = 0; j < EPT; j += 8) {
       float a[8], b[8], c[8];
@@ -165,7 +171,7 @@ k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, const floa
       for (int i = 0; i < 8; ++i) {
         vg[j + i] = a[i] * ginv;
         csum += vg[j + i] * b[i];
-        vq[j + i] = c[i];
+        vq[j + i] = c[i] * qscale;
       }
     }
   } else {
@@ -174,7 +180,7 @@ k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, const floa
   }
   csum += fm_shfl_xor(csum, 1);
   csum += fm_shfl_xor(csum, 2);
-  if (part == 0) cv[int64_t(bh) * npad + row] = csum;
+  if (part == 0) cv[int64_t(bh) * npad + row] = CE<E>::from(csum);
   E* ghrow = gh + (int64_t(bh) * npad + row) * DH + d0;
 #pragma unroll
   for (int j = 0; j < EPT; j += 8) CE<E>::st8(ghrow + j, &vg[j]);
@@ -200,7 +206,10 @@ k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, const floa
 //   big   [slot][a = 0..DH][r][c]   compute type;  a < DH: coef2 * sum x_a p_r r_c,
 //                                                  a = DH: coef1 * sum p_r r_c
 //   small [slot]{ Z[DH][DH], va[DH], vb[DH] } fp32;  Z = coefz * sum za_r zb_c,
-//                                   va = coefva * sum za,  vb = coefvb * sum p
+//                                   va = coefva * sum za,  vb = coefvb * sum p (or sum r)
+//   big2  [slot][a][c][r] = coefb * (same sums): the transposed tiles.  The state of
+//         (x, p, r) read with (r, p) exchanged is the state of (x, r, p), so one walk
+//         serves two consumers (dK wants [a][m][c], dV wants [a][c][m]).
 // ------------------------------------------------------------------------------
 // `big` is padded to DH + 4 values of a so that a reader may fetch whole slabs of
 // up to four values of a starting at any a <= DH without leaving the state.
@@ -215,8 +224,11 @@ template <typename E> struct BuildArgs {
   const E* xt; const E* pt; const E* rt; const E* za; const E* zb;   // [bh][DH][npad]
   int npad, nseg, L, mode, quad;
   E* big; float* small;                 // [bh][nslots] states
+  E* big2;                              // optional second copy with every [r][c] tile transposed
   int nslots;
+  int vb_from_r;                        // vb sums the r operand instead of p
   float coef2, coef1, coefz, coefva, coefvb;
+  float coef2b, coef1b;                 // coefficients of the transposed copy
 };
 
 FM_DEVICE void fm_walk_step(int mode, int nseg, int L, int npad, int w, int& tb, int& te, int& slot) {
@@ -235,7 +247,7 @@ FM_DEVICE void fm_walk_step(int mode, int nseg, int L, int npad, int w, int& tb,
 // (one thread per feature, serial over tokens) and the cumsum of materialised
 // outer products of fastattention_einops.py:237-248.
 template <typename E, int DH, int NA, int TT>
-FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_build(BuildArgs<E> A) {
+FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (sizeof(E) == 2 ? 2 : 1)) k_build(BuildArgs<E> A) {
   typedef Mma<E> M;
   typedef typename M::frag frag;
   constexpr int AW = 4 * NA;
@@ -254,6 +266,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_build(BuildArgs<E> A) {
   const int nsteps = (A.mode == FM_WALK_TOTAL) ? 1 : A.nseg - 1;
   if (nsteps <= 0) return;
   E* big = A.big + int64_t(bh) * A.nslots * StateDims<DH>::BIG;
+  E* big2 = A.big2 ? A.big2 + int64_t(bh) * A.nslots * StateDims<DH>::BIG : nullptr;
   float* sml = A.small + int64_t(bh) * A.nslots * StateDims<DH>::SMALL;
 
   int w = 0, tb, te, slot;
@@ -327,6 +340,22 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_build(BuildArgs<E> A) {
                 dst[(int64_t(a) * DH + r) * DH + c] = CE<E>::from(A.coef2 * acc[i][j][k][e]);
               }
         }
+        if (big2) {
+          E* dst2 = big2 + int64_t(slot) * StateDims<DH>::BIG;
+#pragma unroll
+          for (int i = 0; i < NA; ++i) {
+            const int a = a0 + wave * NA + i;
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+#pragma unroll
+              for (int k = 0; k < NT; ++k)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                  const int r = 32 * j + fm_acc_row(e, lh), c = 32 * k + lr;
+                  dst2[(int64_t(a) * DH + c) * DH + r] = CE<E>::from(A.coef2b * acc[i][j][k][e]);
+                }
+          }
+        }
       }
       t = nt; w = nw; tb = ntb; te = nte; slot = nslot; have = has_next;
     }
@@ -379,7 +408,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_build(BuildArgs<E> A) {
             for (int k = 0; k < NT; ++k) acc[j][k] = M::mma(fa[j], fb[k], acc[j][k]);
         }
       } else if (wave >= 2 && lane < DH && (wave == 3 || has_z)) {
-        const E* sv = wave == 2 ? s2 : s0;          // wave 2: sum of za, wave 3: sum of p
+        const E* sv = wave == 2 ? s2 : (A.vb_from_r ? s1 : s0);   // wave 2: sum of za, wave 3: sum of p (or r)
         float s = 0.f;
         for (int j = 0; j < TT; ++j) s += float(sv[lane * PT + j]);
         vsum += s;
@@ -396,6 +425,9 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_build(BuildArgs<E> A) {
               for (int e = 0; e < 16; ++e) {
                 const int r = 32 * j + fm_acc_row(e, lh), c = 32 * k + lr;
                 dst[r * DH + c] = CE<E>::from(A.coef1 * acc[j][k][e]);
+                if (big2)
+                  big2[int64_t(slot) * StateDims<DH>::BIG + int64_t(DH) * DH * DH + c * DH + r] =
+                      CE<E>::from(A.coef1b * acc[j][k][e]);
               }
         } else if (wave == 1) {
 #pragma unroll
@@ -442,6 +474,8 @@ struct TokCfg {
 //   sum_b      T[DH][c][b] * y_b(token)                    a = DH
 // xs: row-major token tile in LDS (pitch PQ) supplying x; yb[j][ks]: B fragments of y.
 // slab: two buffers of SA*DH*PS elements.  All 256 threads must call this.
+// The A fragments of step i+1 are fetched from LDS before the products of step i are
+// issued, so a single wavefront per SIMD keeps the matrix pipe fed.
 template <typename E, int DH, int QT, int NACC>
 FM_DEVICE void fm_readout(const E* FM_RESTRICT state, bool quad, const E* xs, const int* xrow,
                           const typename Mma<E>::frag (*yb)[TokCfg<E, DH, QT>::NKS],
@@ -454,12 +488,17 @@ FM_DEVICE void fm_readout(const E* FM_RESTRICT state, bool quad, const E* xs, co
   TileRegs<E, C::SA * DH, DH> regs;
   regs.load(state + int64_t(a_begin) * DH * DH, DH, tid);   // rows [a][c] are contiguous
   int buf = 0;
+  const int lane_off = lr * C::PS + lh * M::KPL;
   for (int as = a_begin; as <= DH; as += C::SA) {
     E* sb = slab + buf * C::SLAB;
     regs.store(sb, C::PS, tid);
     FM_SYNC();
     if (as + C::SA <= DH) regs.load(state + int64_t(as + C::SA) * DH * DH, DH, tid);
     const int na = (as + C::SA <= DH) ? C::SA : (DH + 1 - as);
+    const E* sl = sb + lane_off;
+    frag fa[C::NT];
+#pragma unroll
+    for (int ct = 0; ct < C::NT; ++ct) fa[ct] = M::load(sl + (32 * ct) * C::PS);
     for (int al = 0; al < na; ++al) {
       const int a = as + al;
       frag xr[QT];
@@ -467,16 +506,20 @@ FM_DEVICE void fm_readout(const E* FM_RESTRICT state, bool quad, const E* xs, co
       for (int j = 0; j < QT; ++j) xr[j] = (a < DH) ? M::splat(xs[xrow[j] * C::PQ + a]) : M::splat(E(1.0f));
 #pragma unroll
       for (int ks = 0; ks < C::NKS; ++ks) {
-        const int ko = ks * M::KSTEP + lh * M::KPL;
-        frag fa[C::NT];
+        // prefetch the fragments of the next (a, k-step); the last one of a slab re-reads a valid row
+        const int nks = (ks + 1 < C::NKS) ? ks + 1 : 0;
+        const int nal = (ks + 1 < C::NKS) ? al : (al + 1 < na ? al + 1 : al);
+        frag fn[C::NT];
 #pragma unroll
-        for (int ct = 0; ct < C::NT; ++ct) fa[ct] = M::load(sb + (al * DH + 32 * ct + lr) * C::PS + ko);
+        for (int ct = 0; ct < C::NT; ++ct) fn[ct] = M::load(sl + (nal * DH + 32 * ct) * C::PS + nks * M::KSTEP);
 #pragma unroll
         for (int j = 0; j < QT; ++j) {
           const frag fb = yb[j][ks] * xr[j];
 #pragma unroll
           for (int ct = 0; ct < C::NT; ++ct) acc[j][ct] = M::mma(fa[ct], fb, acc[j][ct]);
         }
+#pragma unroll
+        for (int ct = 0; ct < C::NT; ++ct) fa[ct] = fn[ct];
       }
     }
     buf ^= 1;
@@ -488,7 +531,8 @@ FM_DEVICE void fm_readout(const E* FM_RESTRICT state, bool quad, const E* xs, co
 // k_fwd: forward for one block of QW queries of one batch*head.
 //   [F_i, g_i] = (prefix or global moment readout) + (dense tiles over the keys
 //   kbeg .. kend of the query's own segment, causal on the diagonal);  o = F / g.
-// grid (ceil(nq / QW), bh).  Replaces calc_masked / calc_unmasked
+// q and k arrive multiplied by sqrt(1/tau) each, so the score is their plain dot
+// product.  grid (ceil(nq / QW), bh).  Replaces calc_masked / calc_unmasked
 // (fastmax_cuda_forward.cu:23-280).
 // ------------------------------------------------------------------------------
 template <typename TIO, typename E> struct FwdArgs {
@@ -498,21 +542,25 @@ template <typename TIO, typename E> struct FwdArgs {
   const E* vt; int npad_k;             // V transposed [bh][DH][npad_k]
   const E* big; const float* small; int nslots;
   int nq, nk, L, causal, use_state, quad;
-  float a0, c1, c2;                    // f(x) = a0 + c1 x + c2 x^2 on the raw dot product x
+  float a0, a1, a2;                    // f(s) = a0 + a1 s + a2 s^2
+  float sc;                            // sqrt(1/tau), applied to q and k on load
 };
 
 template <typename TIO, typename E, int DH, int QT>
 FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_fwd(FwdArgs<TIO, E> A) {
   typedef TokCfg<E, DH, QT> C;
   typedef Mma<E> M;
+  typedef TileMath<E> TM;
   typedef typename M::frag frag;
   constexpr int NT = C::NT, NKS = C::NKS, QW = C::QW, PQ = C::PQ, PS = C::PS, KT = C::KT, PV = C::PV;
+  constexpr int STAGE = KT * PQ + DH * PV;            // K rows, V transposed
   FM_DYN_SMEM(smem);
   E* Qs = reinterpret_cast<E*>(smem);                 // [QW][PQ]
   E* Zs = Qs + QW * PQ;                               // [NZ][DH][PS]
   float* vecs = reinterpret_cast<float*>(Zs + C::NZ * DH * PS);   // va[DH], vb[DH]
   E* R = reinterpret_cast<E*>(vecs + 2 * DH);         // slabs | dense-loop tiles | output staging
-  const int tid = FM_TID_X, wave = tid >> 6, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int tid = FM_TID_X, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int wave = FM_UNIFORM(tid >> 6);
   const int bh = FM_BID_Y;
   const int nqb = FM_GDIM_X;
   const int qb = A.causal ? (nqb - 1 - FM_BID_X) : FM_BID_X;    // heavy blocks first
@@ -521,14 +569,14 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_fwd(FwdArgs<TIO, E> A) {
   const bool use_state = A.use_state && (!A.causal || seg > 0);
   const int slot = A.causal ? seg : 0;
   const int kbeg = A.causal ? seg * A.L : 0;
-  int kend = A.causal ? (q0 + QW < A.nk ? q0 + QW : A.nk) : (A.use_state ? 0 : A.nk);
+  const int kend = A.causal ? (q0 + QW < A.nk ? q0 + QW : A.nk) : (A.use_state ? 0 : A.nk);
   const float cnt = A.causal ? float(kbeg) : float(A.nk);       // keys covered by the state
 
   // ---- stage Q (and the denominator states) ----
   {
     RowRegs<TIO, E, QW, DH> rq;
     rq.load(A.q.p + int64_t(bh) * A.q.s_bh, A.q.s_n, A.q.vec != 0, q0, A.nq, tid);
-    rq.store(Qs, PQ, tid);
+    rq.store(Qs, PQ, tid, A.sc);
   }
   const float* sml = A.small + (int64_t(bh) * A.nslots + slot) * StateDims<DH>::SMALL;
   if (use_state) {
@@ -590,8 +638,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_fwd(FwdArgs<TIO, E> A) {
 
   // ---- dense tiles over the keys of this segment ----
   if (kend > kbeg) {
-    E* Ks[2]; E* Vs[2];
-    Ks[0] = R; Vs[0] = R + KT * PQ; Ks[1] = Vs[0] + DH * PV; Vs[1] = Ks[1] + KT * PQ;
+    const typename TM::Coef coef = TM::coef(A.a0, A.a1, A.a2);
     RowRegs<TIO, E, KT, DH> rk;
     TileRegs<E, DH, KT> rv;
     const TIO* kb = A.k.p + int64_t(bh) * A.k.s_bh;
@@ -600,48 +647,59 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_fwd(FwdArgs<TIO, E> A) {
     rv.load(vtb + kbeg, A.npad_k, tid);
     int buf = 0;
     for (int kt0 = kbeg; kt0 < kend; kt0 += KT) {
-      rk.store(Ks[buf], PQ, tid);
-      rv.store(Vs[buf], PV, tid);
+      E* Ks = R + buf * STAGE;
+      E* Vs = Ks + KT * PQ;
+      rk.store(Ks, PQ, tid, A.sc);
+      rv.store(Vs, PV, tid);
       FM_SYNC();
       if (kt0 + KT < kend) {
         rk.load(kb, A.k.s_n, A.k.vec != 0, kt0 + KT, A.nk, tid);
         rv.load(vtb + kt0 + KT, A.npad_k, tid);
       }
+      // work items (sub-tile st, query tile j); the score tile of the next item is issued
+      // before the polynomial of the current one so that VALU and MFMA overlap
+      constexpr int NI = (KT / 32) * QT;
+      bool act[NI];
 #pragma unroll
-      for (int st = 0; st < KT / 32; ++st) {
-        const int key0 = kt0 + 32 * st;
-        if (key0 >= kend) break;
-        frag kf[NKS];
+      for (int it = 0; it < NI; ++it) {
+        const int key0 = kt0 + 32 * (it / QT), qlo = q0 + tw[it % QT] * 32;
+        act[it] = key0 < kend && !(A.causal && key0 > qlo + 31);
+      }
+      fm_f32x16 s_cur = fm_zero16();
+      if (act[0]) {
 #pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) kf[ks] = M::load(Ks[buf] + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL);
+        for (int ks = 0; ks < NKS; ++ks)
+          s_cur = M::mma(M::load(Ks + lr * PQ + ks * M::KSTEP + lh * M::KPL), qf[0][ks], s_cur);
+      }
 #pragma unroll
-        for (int j = 0; j < QT; ++j) {
-          const int qlo = q0 + tw[j] * 32;             // first query of this tile
-          if (A.causal && key0 > qlo + 31) continue;   // tile entirely in the future
-          fm_f32x16 s = fm_zero16();
+      for (int it = 0; it < NI; ++it) {
+        const int st = it / QT, j = it % QT;
+        fm_f32x16 s_nxt = fm_zero16();
+        if (it + 1 < NI && act[(it + 1 < NI) ? it + 1 : it]) {
+          const int st2 = (it + 1) / QT, j2 = (it + 1) % QT;
 #pragma unroll
-          for (int ks = 0; ks < NKS; ++ks) s = M::mma(kf[ks], qf[j][ks], s);
-          const bool edge = (A.causal && key0 + 31 > qlo) || (key0 + 31 >= A.nk);
-          const int qi = qlo + lr;
-#pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            const float x = s[e];
-            float pv = A.a0 + x * (A.c1 + A.c2 * x);
-            if (edge) {
-              const int t = key0 + fm_acc_row(e, lh);
-              if ((A.causal && t > qi) || t >= A.nk) pv = 0.f;
-            }
-            gsum[j] += pv;
-            s[e] = pv;
-          }
-#pragma unroll
-          for (int ss = 0; ss < M::ACC_KSTEPS; ++ss) {
-            const frag pb = M::from_acc(s, ss);
-#pragma unroll
-            for (int ct = 0; ct < NT; ++ct)
-              acc[j][ct] = M::mma(M::load_perm(Vs[buf] + (32 * ct + lr) * PV + 32 * st, ss, lh), pb, acc[j][ct]);
-          }
+          for (int ks = 0; ks < NKS; ++ks)
+            s_nxt = M::mma(M::load(Ks + (32 * st2 + lr) * PQ + ks * M::KSTEP + lh * M::KPL), qf[j2][ks], s_nxt);
         }
+        if (act[it]) {
+          const int key0 = kt0 + 32 * st, qlo = q0 + tw[j] * 32;
+          const bool edge = (A.causal && key0 + 31 > qlo) || (key0 + 31 >= A.nk);
+          int hi = A.nk - 1 - key0;
+          if (A.causal && qlo + lr - key0 < hi) hi = qlo + lr - key0;
+          frag pb[M::ACC_KSTEPS];
+          frag vf[NT][M::ACC_KSTEPS];
+#pragma unroll
+          for (int ct = 0; ct < NT; ++ct)
+#pragma unroll
+            for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
+              vf[ct][ss] = M::load_perm(Vs + (32 * ct + lr) * PV + 32 * st, ss, lh);
+          gsum[j] += TM::fwd(s_cur, coef, edge, 0, hi, lh, pb);
+#pragma unroll
+          for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
+#pragma unroll
+            for (int ct = 0; ct < NT; ++ct) acc[j][ct] = M::mma(vf[ct][ss], pb[ss], acc[j][ct]);
+        }
+        s_cur = s_nxt;
       }
       buf ^= 1;
     }

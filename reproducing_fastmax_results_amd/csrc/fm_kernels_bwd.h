@@ -15,14 +15,16 @@
 template <typename TIO, typename E> struct BwdArgs {
   TRef<const TIO> q, k, v;
   TRef<TIO> dq, dk, dv;
-  const E* gh; const E* ght; const E* qt; const E* kt; const float* cv;   // workspace copies
+  const E* gh; const E* ght; const E* qt; const E* kt; const E* cv;       // workspace copies
   int npad_q, npad_k;
   const E* bigq; const float* smallq;      // prefix (k, k, v)
   const E* bigk; const float* smallk;      // suffix (q, q, gh)
   const E* bigv; const float* smallv;      // suffix (q, gh, q)
   int nslots;
   int nq, nk, L, nseg, causal, use_state, quad;
-  float a0, c1, c2;
+  float a0, a1, a2;
+  float sc;                                // sqrt(1/tau): q and k are used as sc*q, sc*k
+  float gscale;                            // power of two folded into gh and c by k_prep_bwd
 };
 
 // Z (fp32, [DH][DH]) -> LDS in the compute type (hi/lo split for _Float16), va/vb -> vecs.
@@ -56,7 +58,7 @@ FM_DEVICE fm_f32x16 fm_zy(const E* Zs, const typename Mma<E>::frag* tf, int mt, 
 
 // Accumulators (rows = feature, column = token of tile j) -> caller tensor rows, through LDS.
 template <typename TIO, typename E, int DH, int QT>
-FM_DEVICE void fm_store_tokens(fm_f32x16 (*acc)[DH / 32], const int* xrow, const float* addvec, float* Os,
+FM_DEVICE void fm_store_tokens(fm_f32x16 (*acc)[DH / 32], const int* xrow, const float* addvec, float scale, float* Os,
                                TRef<TIO> out, int bh, int row0, int nrows, int tid) {
   typedef TokCfg<E, DH, QT> C;
   const int lane = tid & 63, lh = lane >> 5;
@@ -67,7 +69,7 @@ FM_DEVICE void fm_store_tokens(fm_f32x16 (*acc)[DH / 32], const int* xrow, const
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int c = 32 * ct + fm_acc_row(e, lh);
-        Os[xrow[j] * (DH + 1) + c] = acc[j][ct][e] + (addvec ? addvec[c] : 0.f);
+        Os[xrow[j] * (DH + 1) + c] = scale * (acc[j][ct][e] + (addvec ? addvec[c] : 0.f));
       }
   FM_SYNC();
   TIO* ob = out.p + int64_t(bh) * out.s_bh;
@@ -90,15 +92,18 @@ template <typename TIO, typename E, int DH, int QT>
 FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_dq(BwdArgs<TIO, E> A) {
   typedef TokCfg<E, DH, QT> C;
   typedef Mma<E> M;
+  typedef TileMath<E> TM;
   typedef typename M::frag frag;
   constexpr int NT = C::NT, NKS = C::NKS, QW = C::QW, PQ = C::PQ, KT = C::KT, PV = C::PV;
   constexpr int NBUF = sizeof(E) == 2 ? 2 : 1;
+  constexpr int STAGE = 2 * KT * PQ + DH * PV;        // K rows, V rows, K transposed
   FM_DYN_SMEM(smem);
   E* Qs = reinterpret_cast<E*>(smem);                 // [QW][PQ]  q rows
   E* Gs = Qs + QW * PQ;                               // [QW][PQ]  gh rows
   float* vecs = reinterpret_cast<float*>(Gs + QW * PQ);
   E* R = reinterpret_cast<E*>(vecs + 2 * DH);         // Z | slabs | dense tiles | output staging
-  const int tid = FM_TID_X, wave = tid >> 6, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int tid = FM_TID_X, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int wave = FM_UNIFORM(tid >> 6);
   const int bh = FM_BID_Y;
   const int nqb = FM_GDIM_X;
   const int qb = A.causal ? (nqb - 1 - FM_BID_X) : FM_BID_X;
@@ -112,7 +117,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_dq(BwdArgs<TIO, E> A) {
   {
     RowRegs<TIO, E, QW, DH> rq;
     rq.load(A.q.p + int64_t(bh) * A.q.s_bh, A.q.s_n, A.q.vec != 0, q0, A.nq, tid);
-    rq.store(Qs, PQ, tid);
+    rq.store(Qs, PQ, tid, A.sc);
     TileRegs<E, QW, DH> rg;                            // gh rows are dense [npad_q][DH]
     rg.load(A.gh + (int64_t(bh) * A.npad_q + q0) * DH, DH, tid);
     rg.store(Gs, PQ, tid);
@@ -127,7 +132,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_dq(BwdArgs<TIO, E> A) {
   for (int j = 0; j < QT; ++j) {
     tw[j] = (j == 0) ? wave : (4 * QT - 1 - wave);
     xrow[j] = tw[j] * 32 + lr;
-    ci[j] = A.cv[int64_t(bh) * A.npad_q + q0 + xrow[j]];
+    ci[j] = float(A.cv[int64_t(bh) * A.npad_q + q0 + xrow[j]]);
   }
   frag qf[QT][NKS], gf[QT][NKS];
 #pragma unroll
@@ -159,7 +164,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_dq(BwdArgs<TIO, E> A) {
   }
 
   if (kend > kbeg) {
-    constexpr int STAGE = 2 * KT * PQ + DH * PV;       // K rows, V rows, K transposed
+    const typename TM::Coef coef = TM::coef(A.a0, A.a1, A.a2);
     RowRegs<TIO, E, KT, DH> rk, rv;
     TileRegs<E, DH, KT> rkt;
     const TIO* kb = A.k.p + int64_t(bh) * A.k.s_bh;
@@ -168,62 +173,68 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_dq(BwdArgs<TIO, E> A) {
     rk.load(kb, A.k.s_n, A.k.vec != 0, kbeg, A.nk, tid);
     rv.load(vb, A.v.s_n, A.v.vec != 0, kbeg, A.nk, tid);
     rkt.load(ktb + kbeg, A.npad_k, tid);
-    const float c2x2 = 2.0f * A.c2;
     int buf = 0;
     for (int kt0 = kbeg; kt0 < kend; kt0 += KT) {
       E* Ks = R + buf * STAGE; E* Vs = Ks + KT * PQ; E* Kts = Vs + KT * PQ;
-      rk.store(Ks, PQ, tid); rv.store(Vs, PQ, tid); rkt.store(Kts, PV, tid);
+      rk.store(Ks, PQ, tid, A.sc); rv.store(Vs, PQ, tid, 1.0f); rkt.store(Kts, PV, tid);
       FM_SYNC();
       if (kt0 + KT < kend) {
         rk.load(kb, A.k.s_n, A.k.vec != 0, kt0 + KT, A.nk, tid);
         rv.load(vb, A.v.s_n, A.v.vec != 0, kt0 + KT, A.nk, tid);
         rkt.load(ktb + kt0 + KT, A.npad_k, tid);
       }
+      constexpr int NI = (KT / 32) * QT;
+      bool act[NI];
 #pragma unroll
-      for (int st = 0; st < KT / 32; ++st) {
-        const int key0 = kt0 + 32 * st;
-        if (key0 >= kend) break;
-        frag kf[NKS], vf[NKS];
+      for (int it = 0; it < NI; ++it) {
+        const int key0 = kt0 + 32 * (it / QT), qlo = q0 + tw[it % QT] * 32;
+        act[it] = key0 < kend && !(A.causal && key0 > qlo + 31);
+      }
+      fm_f32x16 s_cur = fm_zero16(), dp_cur = fm_zero16();
+      if (act[0]) {
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) {
-          kf[ks] = M::load(Ks + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL);
-          vf[ks] = M::load(Vs + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL);
+          s_cur = M::mma(M::load(Ks + lr * PQ + ks * M::KSTEP + lh * M::KPL), qf[0][ks], s_cur);
+          dp_cur = M::mma(M::load(Vs + lr * PQ + ks * M::KSTEP + lh * M::KPL), gf[0][ks], dp_cur);
         }
+      }
 #pragma unroll
-        for (int j = 0; j < QT; ++j) {
-          const int qlo = q0 + tw[j] * 32;
-          if (A.causal && key0 > qlo + 31) continue;
-          fm_f32x16 s = fm_zero16(), dp = fm_zero16();
+      for (int it = 0; it < NI; ++it) {
+        const int st = it / QT, j = it % QT;
+        fm_f32x16 s_nxt = fm_zero16(), dp_nxt = fm_zero16();
+        if (it + 1 < NI && act[(it + 1 < NI) ? it + 1 : it]) {
+          const int st2 = (it + 1) / QT, j2 = (it + 1) % QT;
 #pragma unroll
           for (int ks = 0; ks < NKS; ++ks) {
-            s = M::mma(kf[ks], qf[j][ks], s);
-            dp = M::mma(vf[ks], gf[j][ks], dp);
-          }
-          const bool edge = (A.causal && key0 + 31 > qlo) || (key0 + 31 >= A.nk);
-          const int qi = qlo + lr;
-#pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            float ds = (A.c1 + c2x2 * s[e]) * (dp[e] - ci[j]);
-            if (edge) {
-              const int t = key0 + fm_acc_row(e, lh);
-              if ((A.causal && t > qi) || t >= A.nk) ds = 0.f;
-            }
-            s[e] = ds;
-          }
-#pragma unroll
-          for (int ss = 0; ss < M::ACC_KSTEPS; ++ss) {
-            const frag db = M::from_acc(s, ss);
-#pragma unroll
-            for (int mt = 0; mt < NT; ++mt)
-              acc[j][mt] = M::mma(M::load_perm(Kts + (32 * mt + lr) * PV + 32 * st, ss, lh), db, acc[j][mt]);
+            s_nxt = M::mma(M::load(Ks + (32 * st2 + lr) * PQ + ks * M::KSTEP + lh * M::KPL), qf[j2][ks], s_nxt);
+            dp_nxt = M::mma(M::load(Vs + (32 * st2 + lr) * PQ + ks * M::KSTEP + lh * M::KPL), gf[j2][ks], dp_nxt);
           }
         }
+        if (act[it]) {
+          const int key0 = kt0 + 32 * st, qlo = q0 + tw[j] * 32;
+          const bool edge = (A.causal && key0 + 31 > qlo) || (key0 + 31 >= A.nk);
+          int hi = A.nk - 1 - key0;
+          if (A.causal && qlo + lr - key0 < hi) hi = qlo + lr - key0;
+          frag db[M::ACC_KSTEPS];
+          frag kf[NT][M::ACC_KSTEPS];
+#pragma unroll
+          for (int mt = 0; mt < NT; ++mt)
+#pragma unroll
+            for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
+              kf[mt][ss] = M::load_perm(Kts + (32 * mt + lr) * PV + 32 * st, ss, lh);
+          TM::dsc(s_cur, dp_cur, TM::splat_c(ci[j]), coef, edge, 0, hi, lh, db);
+#pragma unroll
+          for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
+#pragma unroll
+            for (int mt = 0; mt < NT; ++mt) acc[j][mt] = M::mma(kf[mt][ss], db[ss], acc[j][mt]);
+        }
+        s_cur = s_nxt; dp_cur = dp_nxt;
       }
       if (NBUF == 1) FM_SYNC(); else buf ^= 1;
     }
     if (NBUF == 2) FM_SYNC();
   }
-  fm_store_tokens<TIO, E, DH, QT>(acc, xrow, nullptr, reinterpret_cast<float*>(R), A.dq, bh, q0, A.nq, tid);
+  fm_store_tokens<TIO, E, DH, QT>(acc, xrow, nullptr, A.sc / A.gscale, reinterpret_cast<float*>(R), A.dq, bh, q0, A.nq, tid);
 }
 
 // ------------------------------------------------------------------------------
@@ -233,35 +244,36 @@ template <typename TIO, typename E, int DH, int QT>
 FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_dkv(BwdArgs<TIO, E> A) {
   typedef TokCfg<E, DH, QT> C;
   typedef Mma<E> M;
+  typedef TileMath<E> TM;
   typedef typename M::frag frag;
   constexpr int NT = C::NT, NKS = C::NKS, KW = C::QW, PQ = C::PQ, KT = C::KT, PV = C::PV;
   constexpr int NBUF = sizeof(E) == 2 ? 2 : 1;
+  constexpr int STAGE = 2 * KT * PQ + 2 * DH * PV;     // q rows, gh rows, q transposed, gh transposed
+  constexpr int STAGE_PAD = STAGE + 2 * KT;            // + c values (compute type, padded)
   FM_DYN_SMEM(smem);
   E* Ks = reinterpret_cast<E*>(smem);                 // [KW][PQ]  k rows
   E* Vs = Ks + KW * PQ;                               // [KW][PQ]  v rows
-  float* vecs = reinterpret_cast<float*>(Vs + KW * PQ);   // va (dK), vb (dK, unused), then vb of dV at [2*DH..)
-  float* vecv = vecs + 2 * DH;
-  E* R = reinterpret_cast<E*>(vecv + 2 * DH);
-  const int tid = FM_TID_X, wave = tid >> 6, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  float* vecs = reinterpret_cast<float*>(Vs + KW * PQ);   // va, vb of the (q, q, gh) state
+  E* R = reinterpret_cast<E*>(vecs + 2 * DH);
+  const int tid = FM_TID_X, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int wave = FM_UNIFORM(tid >> 6);
   const int bh = FM_BID_Y;
   const int k0 = FM_BID_X * KW;                        // early key blocks are the heavy ones
   const int seg = A.causal ? k0 / A.L : 0;
   const bool use_state = A.use_state && (!A.causal || seg < A.nseg - 1);
   const int slot = A.causal ? seg : 0;
   const int ibeg = A.causal ? k0 : 0;
-  int iend = A.causal ? ((seg + 1) * A.L < A.nq ? (seg + 1) * A.L : A.nq) : (A.use_state ? 0 : A.nq);
+  const int iend = A.causal ? ((seg + 1) * A.L < A.nq ? (seg + 1) * A.L : A.nq) : (A.use_state ? 0 : A.nq);
 
   {
     RowRegs<TIO, E, KW, DH> rk;
     rk.load(A.k.p + int64_t(bh) * A.k.s_bh, A.k.s_n, A.k.vec != 0, k0, A.nk, tid);
-    rk.store(Ks, PQ, tid);
+    rk.store(Ks, PQ, tid, A.sc);
     rk.load(A.v.p + int64_t(bh) * A.v.s_bh, A.v.s_n, A.v.vec != 0, k0, A.nk, tid);
-    rk.store(Vs, PQ, tid);
+    rk.store(Vs, PQ, tid, 1.0f);
   }
-  if (use_state) {
+  if (use_state)
     fm_stage_small<E, DH, QT>(A.smallk + (int64_t(bh) * A.nslots + slot) * StateDims<DH>::SMALL, R, vecs, tid);
-    if (tid < DH) vecv[tid] = A.smallv[(int64_t(bh) * A.nslots + slot) * StateDims<DH>::SMALL + DH * DH + DH + tid];
-  }
   FM_SYNC();
 
   int tw[QT], xrow[QT];
@@ -301,8 +313,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_dkv(BwdArgs<TIO, E> A) {
   }
 
   if (iend > ibeg) {
-    constexpr int STAGE = 2 * KT * PQ + 2 * DH * PV;   // q rows, gh rows, q transposed, gh transposed
-    constexpr int STAGE_PAD = STAGE + (KT * 4 + sizeof(E) - 1) / sizeof(E);   // + c values (fp32)
+    const typename TM::Coef coef = TM::coef(A.a0, A.a1, A.a2);
     RowRegs<TIO, E, KT, DH> rq;
     TileRegs<E, KT, DH> rg;
     TileRegs<E, DH, KT> rqt, rgt;
@@ -310,19 +321,18 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_dkv(BwdArgs<TIO, E> A) {
     const E* ghb = A.gh + int64_t(bh) * A.npad_q * DH;
     const E* qtb = A.qt + int64_t(bh) * DH * A.npad_q;
     const E* gtb = A.ght + int64_t(bh) * DH * A.npad_q;
-    const float* cvb = A.cv + int64_t(bh) * A.npad_q;
-    float creg = 0.f;
+    const E* cvb = A.cv + int64_t(bh) * A.npad_q;
+    E creg = E(0.f);
     rq.load(qb, A.q.s_n, A.q.vec != 0, ibeg, A.nq, tid);
     rg.load(ghb + int64_t(ibeg) * DH, DH, tid);
     rqt.load(qtb + ibeg, A.npad_q, tid);
     rgt.load(gtb + ibeg, A.npad_q, tid);
     if (tid < KT) creg = cvb[ibeg + tid];
-    const float c2x2 = 2.0f * A.c2;
     int buf = 0;
     for (int i0 = ibeg; i0 < iend; i0 += KT) {
       E* Qr = R + buf * STAGE_PAD; E* Gr = Qr + KT * PQ; E* Qts = Gr + KT * PQ; E* Gts = Qts + DH * PV;
-      float* cs = reinterpret_cast<float*>(Gts + DH * PV);
-      rq.store(Qr, PQ, tid); rg.store(Gr, PQ, tid); rqt.store(Qts, PV, tid); rgt.store(Gts, PV, tid);
+      E* cs = Gts + DH * PV;
+      rq.store(Qr, PQ, tid, A.sc); rg.store(Gr, PQ, tid); rqt.store(Qts, PV, tid); rgt.store(Gts, PV, tid);
       if (tid < KT) cs[tid] = creg;
       FM_SYNC();
       if (i0 + KT < iend) {
@@ -332,60 +342,67 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_dkv(BwdArgs<TIO, E> A) {
         rgt.load(gtb + i0 + KT, A.npad_q, tid);
         if (tid < KT) creg = cvb[i0 + KT + tid];
       }
+      constexpr int NI = (KT / 32) * QT;
+      bool act[NI];
 #pragma unroll
-      for (int st = 0; st < KT / 32; ++st) {
-        const int qi0 = i0 + 32 * st;
-        if (qi0 >= iend) break;
-        frag qf[NKS], gf[NKS];
+      for (int it = 0; it < NI; ++it) {
+        const int qi0 = i0 + 32 * (it / QT), klo = k0 + tw[it % QT] * 32;
+        act[it] = qi0 < iend && !(A.causal && qi0 + 31 < klo);   // skip queries that precede all keys
+      }
+      fm_f32x16 s_cur = fm_zero16(), dp_cur = fm_zero16();
+      if (act[0]) {
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) {
-          qf[ks] = M::load(Qr + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL);
-          gf[ks] = M::load(Gr + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL);
+          s_cur = M::mma(M::load(Qr + lr * PQ + ks * M::KSTEP + lh * M::KPL), kf[0][ks], s_cur);
+          dp_cur = M::mma(M::load(Gr + lr * PQ + ks * M::KSTEP + lh * M::KPL), vf[0][ks], dp_cur);
         }
-        float crow[16];
+      }
 #pragma unroll
-        for (int e = 0; e < 16; ++e) crow[e] = cs[32 * st + fm_acc_row(e, lh)];
-#pragma unroll
-        for (int j = 0; j < QT; ++j) {
-          const int klo = k0 + tw[j] * 32;             // first key of this tile
-          if (A.causal && qi0 + 31 < klo) continue;    // all these queries precede the keys
-          fm_f32x16 s = fm_zero16(), dp = fm_zero16();
+      for (int it = 0; it < NI; ++it) {
+        const int st = it / QT, j = it % QT;
+        fm_f32x16 s_nxt = fm_zero16(), dp_nxt = fm_zero16();
+        if (it + 1 < NI && act[(it + 1 < NI) ? it + 1 : it]) {
+          const int st2 = (it + 1) / QT, j2 = (it + 1) % QT;
 #pragma unroll
           for (int ks = 0; ks < NKS; ++ks) {
-            s = M::mma(qf[ks], kf[j][ks], s);
-            dp = M::mma(gf[ks], vf[j][ks], dp);
-          }
-          const bool edge = (A.causal && qi0 < klo + 31) || (qi0 + 31 >= A.nq);
-          const int kj = klo + lr;
-#pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            const float x = s[e];
-            float pv = A.a0 + x * (A.c1 + A.c2 * x);
-            float ds = (A.c1 + c2x2 * x) * (dp[e] - crow[e]);
-            if (edge) {
-              const int i = qi0 + fm_acc_row(e, lh);
-              if ((A.causal && i < kj) || i >= A.nq) { pv = 0.f; ds = 0.f; }
-            }
-            s[e] = pv;
-            dp[e] = ds;
-          }
-#pragma unroll
-          for (int ss = 0; ss < M::ACC_KSTEPS; ++ss) {
-            const frag pb = M::from_acc(s, ss);
-            const frag db = M::from_acc(dp, ss);
-#pragma unroll
-            for (int mt = 0; mt < NT; ++mt) {
-              av[j][mt] = M::mma(M::load_perm(Gts + (32 * mt + lr) * PV + 32 * st, ss, lh), pb, av[j][mt]);
-              ak[j][mt] = M::mma(M::load_perm(Qts + (32 * mt + lr) * PV + 32 * st, ss, lh), db, ak[j][mt]);
-            }
+            s_nxt = M::mma(M::load(Qr + (32 * st2 + lr) * PQ + ks * M::KSTEP + lh * M::KPL), kf[j2][ks], s_nxt);
+            dp_nxt = M::mma(M::load(Gr + (32 * st2 + lr) * PQ + ks * M::KSTEP + lh * M::KPL), vf[j2][ks], dp_nxt);
           }
         }
+        if (act[it]) {
+          const int qi0 = i0 + 32 * st, klo = k0 + tw[j] * 32;
+          const bool edge = (A.causal && qi0 < klo + 31) || (qi0 + 31 >= A.nq);
+          const int lo = A.causal ? klo + lr - qi0 : 0;
+          const int hi = A.nq - 1 - qi0;
+          frag pb[M::ACC_KSTEPS], db[M::ACC_KSTEPS], crow[M::ACC_KSTEPS];
+          frag gtf[NT][M::ACC_KSTEPS], qtf[NT][M::ACC_KSTEPS];
+#pragma unroll
+          for (int ss = 0; ss < M::ACC_KSTEPS; ++ss) {
+            crow[ss] = M::load_perm(cs + 32 * st, ss, lh);
+#pragma unroll
+            for (int mt = 0; mt < NT; ++mt) {
+              gtf[mt][ss] = M::load_perm(Gts + (32 * mt + lr) * PV + 32 * st, ss, lh);
+              qtf[mt][ss] = M::load_perm(Qts + (32 * mt + lr) * PV + 32 * st, ss, lh);
+            }
+          }
+          TM::both(s_cur, dp_cur, crow, coef, edge, lo, hi, lh, pb, db);
+#pragma unroll
+          for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
+#pragma unroll
+            for (int mt = 0; mt < NT; ++mt) {
+              av[j][mt] = M::mma(gtf[mt][ss], pb[ss], av[j][mt]);
+              ak[j][mt] = M::mma(qtf[mt][ss], db[ss], ak[j][mt]);
+            }
+        }
+        s_cur = s_nxt; dp_cur = dp_nxt;
       }
       if (NBUF == 1) FM_SYNC(); else buf ^= 1;
     }
     if (NBUF == 2) FM_SYNC();
   }
   // keys past nk are zero rows: their gradients are discarded by the bounds check
-  fm_store_tokens<TIO, E, DH, QT>(ak, xrow, nullptr, reinterpret_cast<float*>(R), A.dk, bh, k0, A.nk, tid);
-  fm_store_tokens<TIO, E, DH, QT>(av, xrow, use_state ? vecv : nullptr, reinterpret_cast<float*>(R), A.dv, bh, k0, A.nk, tid);
+  const float inv_gs = 1.0f / A.gscale;
+  fm_store_tokens<TIO, E, DH, QT>(ak, xrow, nullptr, A.sc * inv_gs, reinterpret_cast<float*>(R), A.dk, bh, k0, A.nk, tid);
+  fm_store_tokens<TIO, E, DH, QT>(av, xrow, use_state ? vecs + DH : nullptr, inv_gs, reinterpret_cast<float*>(R), A.dv, bh, k0, A.nk,
+                                  tid);
 }

@@ -148,3 +148,123 @@ template <> struct CE<float> {
     *reinterpret_cast<fm_f32x4*>(p + 4) = b;
   }
 };
+
+// ---- elementwise math on accumulator tiles --------------------------------------
+// A tile is the 16 accumulator entries a lane owns (rows fm_acc_row(e, lh), one column).
+// `edge` tiles apply the row window lo <= row <= hi (causal diagonal and sequence tail);
+// interior tiles skip the test.  Results come back as B fragments (ACC_KSTEPS of them),
+// ready for the next product.
+//   fwd : P  = a0 + s (a1 + a2 s)                      and the lane's partial row-sum of P
+//   dsc : dS = (a1 + 2 a2 s) (dp - c),  c one scalar per lane
+//   both: P and dS with c per accumulator row (given as fragments in accumulator order)
+// The _Float16 instantiation evaluates the polynomials on packed halves (v_pk_fma_f16)
+// and sums with v_dot2_f32_f16, which keeps the vector pipe off the critical path.
+template <typename E> struct TileMath;
+
+template <> struct TileMath<float> {
+  typedef float frag;
+  struct Coef { float a0, a1, a2, ta2; };
+  static FM_DEVICE Coef coef(float a0, float a1, float a2) { Coef c = {a0, a1, a2, 2.0f * a2}; return c; }
+  static FM_DEVICE float splat_c(float c) { return c; }
+  static FM_DEVICE float fwd(const fm_f32x16& s, const Coef& k, bool edge, int lo, int hi, int lh, frag* pb) {
+    float g = 0.f;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const float x = s[e];
+      float pv = k.a0 + x * (k.a1 + k.a2 * x);
+      if (edge) { const int r = fm_acc_row(e, lh); if (r < lo || r > hi) pv = 0.f; }
+      g += pv;
+      pb[e] = pv;
+    }
+    return g;
+  }
+  static FM_DEVICE void dsc(const fm_f32x16& s, const fm_f32x16& dp, float c, const Coef& k, bool edge, int lo, int hi,
+                            int lh, frag* db) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      float ds = (k.a1 + k.ta2 * s[e]) * (dp[e] - c);
+      if (edge) { const int r = fm_acc_row(e, lh); if (r < lo || r > hi) ds = 0.f; }
+      db[e] = ds;
+    }
+  }
+  static FM_DEVICE void both(const fm_f32x16& s, const fm_f32x16& dp, const frag* crow, const Coef& k, bool edge, int lo,
+                             int hi, int lh, frag* pb, frag* db) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const float x = s[e];
+      float pv = k.a0 + x * (k.a1 + k.a2 * x);
+      float ds = (k.a1 + k.ta2 * x) * (dp[e] - crow[e]);
+      if (edge) { const int r = fm_acc_row(e, lh); if (r < lo || r > hi) { pv = 0.f; ds = 0.f; } }
+      pb[e] = pv;
+      db[e] = ds;
+    }
+  }
+};
+
+template <> struct TileMath<fm_half> {
+  typedef fm_half8 frag;
+  struct Coef { fm_half8 a0, a1, a2, ta2; };
+  static FM_DEVICE Coef coef(float a0, float a1, float a2) {
+    Coef c;
+    c.a0 = Mma<fm_half>::splat(fm_half(a0)); c.a1 = Mma<fm_half>::splat(fm_half(a1));
+    c.a2 = Mma<fm_half>::splat(fm_half(a2)); c.ta2 = Mma<fm_half>::splat(fm_half(2.0f * a2));
+    return c;
+  }
+  static FM_DEVICE fm_half8 splat_c(float c) { return Mma<fm_half>::splat(CE<fm_half>::from(c)); }
+  static FM_DEVICE fm_half8 half_of(const fm_f32x16& s, int ss) {
+    fm_half8 h;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) h[i] = fm_half(s[8 * ss + i]);
+    return h;
+  }
+  static FM_DEVICE fm_half8 window(fm_half8 v, int ss, int lo, int hi, int lh) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int r = fm_acc_row(8 * ss + i, lh);
+      if (r < lo || r > hi) v[i] = fm_half(0.f);
+    }
+    return v;
+  }
+  static FM_DEVICE float sum8(fm_half8 p, float g) {
+    const fm_half2 one = {fm_half(1.f), fm_half(1.f)};
+    g = fm_dot2(__builtin_shufflevector(p, p, 0, 1), one, g);
+    g = fm_dot2(__builtin_shufflevector(p, p, 2, 3), one, g);
+    g = fm_dot2(__builtin_shufflevector(p, p, 4, 5), one, g);
+    g = fm_dot2(__builtin_shufflevector(p, p, 6, 7), one, g);
+    return g;
+  }
+  static FM_DEVICE float fwd(const fm_f32x16& s, const Coef& k, bool edge, int lo, int hi, int lh, frag* pb) {
+    float g = 0.f;
+#pragma unroll
+    for (int ss = 0; ss < 2; ++ss) {
+      const fm_half8 x = half_of(s, ss);
+      fm_half8 p = (x * k.a2 + k.a1) * x + k.a0;
+      if (edge) p = window(p, ss, lo, hi, lh);
+      g = sum8(p, g);
+      pb[ss] = p;
+    }
+    return g;
+  }
+  static FM_DEVICE void dsc(const fm_f32x16& s, const fm_f32x16& dp, fm_half8 c, const Coef& k, bool edge, int lo, int hi,
+                            int lh, frag* db) {
+#pragma unroll
+    for (int ss = 0; ss < 2; ++ss) {
+      const fm_half8 x = half_of(s, ss);
+      fm_half8 d = (x * k.ta2 + k.a1) * (half_of(dp, ss) - c);
+      if (edge) d = window(d, ss, lo, hi, lh);
+      db[ss] = d;
+    }
+  }
+  static FM_DEVICE void both(const fm_f32x16& s, const fm_f32x16& dp, const frag* crow, const Coef& k, bool edge, int lo,
+                             int hi, int lh, frag* pb, frag* db) {
+#pragma unroll
+    for (int ss = 0; ss < 2; ++ss) {
+      const fm_half8 x = half_of(s, ss);
+      fm_half8 p = (x * k.a2 + k.a1) * x + k.a0;
+      fm_half8 d = (x * k.ta2 + k.a1) * (half_of(dp, ss) - crow[ss]);
+      if (edge) { p = window(p, ss, lo, hi, lh); d = window(d, ss, lo, hi, lh); }
+      pb[ss] = p;
+      db[ss] = d;
+    }
+  }
+};

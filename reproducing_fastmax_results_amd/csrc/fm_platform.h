@@ -9,6 +9,7 @@
 #include <cstdint>
 
 typedef _Float16 fm_half;
+typedef _Float16 fm_half2 __attribute__((ext_vector_type(2)));
 typedef _Float16 fm_half4 __attribute__((ext_vector_type(4)));
 typedef _Float16 fm_half8 __attribute__((ext_vector_type(8)));
 typedef float fm_f32x4 __attribute__((ext_vector_type(4)));
@@ -24,7 +25,9 @@ typedef uint16_t fm_bf16;  // raw storage of a bfloat16
 #define FM_GLOBAL
 #define FM_DEVICE inline
 #define FM_LAUNCH_BOUNDS(n)
+#define FM_LAUNCH_BOUNDS2(n, m)
 #define FM_RESTRICT
+#define FM_UNIFORM(x) (x)
 typedef void* fm_stream_t;
 typedef hostsim::Dim3 fm_dim3;
 #define FM_TID_X (int(hostsim::g_t.tid.x))
@@ -53,6 +56,7 @@ FM_DEVICE fm_f32x16 fm_mfma_f32(float a, float b, fm_f32x16 c) {
   return c;
 }
 FM_DEVICE float fm_shfl_xor(float v, int m) { return hostsim::shfl(v, hostsim::g_t.lane ^ m); }
+FM_DEVICE float fm_dot2(fm_half2 a, fm_half2 b, float c) { return float(a[0]) * float(b[0]) + float(a[1]) * float(b[1]) + c; }
 FM_DEVICE float fm_fmaxf(float a, float b) { return a > b ? a : b; }
 FM_DEVICE float fm_rsqrtf(float a) { return 1.0f / std::sqrt(a); }
 FM_DEVICE float fm_sqrtf(float a) { return std::sqrt(a); }
@@ -63,7 +67,11 @@ FM_DEVICE float fm_sqrtf(float a) { return std::sqrt(a); }
 #define FM_GLOBAL __global__
 #define FM_DEVICE __device__ __forceinline__
 #define FM_LAUNCH_BOUNDS(n) __launch_bounds__(n)
+#define FM_LAUNCH_BOUNDS2(n, m) __launch_bounds__(n, m)
 #define FM_RESTRICT __restrict__
+// a value that is the same in every lane of the wavefront, moved to a scalar register so that
+// branches on it are scalar branches
+#define FM_UNIFORM(x) __builtin_amdgcn_readfirstlane(x)
 typedef hipStream_t fm_stream_t;
 typedef dim3 fm_dim3;
 #define FM_TID_X (int(threadIdx.x))
@@ -83,6 +91,7 @@ FM_DEVICE fm_f32x16 fm_mfma_f32(float a, float b, fm_f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }
 FM_DEVICE float fm_shfl_xor(float v, int m) { return __shfl_xor(v, m, 64); }
+FM_DEVICE float fm_dot2(fm_half2 a, fm_half2 b, float c) { return __builtin_amdgcn_fdot2(a, b, c, false); }
 FM_DEVICE float fm_fmaxf(float a, float b) { return fmaxf(a, b); }
 FM_DEVICE float fm_rsqrtf(float a) { return rsqrtf(a); }
 FM_DEVICE float fm_sqrtf(float a) { return sqrtf(a); }
