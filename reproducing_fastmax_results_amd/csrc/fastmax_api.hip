@@ -5,6 +5,7 @@
 #include "fm_kernels_bwd.h"
 #include "fm_norm.h"
 #include <cmath>
+#include <cstdlib>
 #include <vector>
 
 namespace {
@@ -55,8 +56,8 @@ struct Plan {
   float sc;             // sqrt(1/tau), folded into q and k when they are converted
   float gscale;         // power of two folded into dO / g in the backward
   // workspace offsets (bytes)
-  size_t kt, vt, big, small, fwd_bytes;
-  size_t b_kt, b_vt, b_qt, b_qct, b_gh, b_ght, b_cv, b_bigq, b_smallq, b_bigk, b_smallk, b_bigv, bwd_bytes;
+  size_t kt, vt, kr, big, small, fwd_bytes;
+  size_t b_kr, b_vr, b_qr, b_kt, b_vt, b_qt, b_qct, b_gh, b_ght, b_cv, b_bigq, b_smallq, b_bigk, b_smallk, b_bigv, bwd_bytes;
 };
 
 bool strides_ok(const FastmaxStrides& s, int bh, int n, int d) {
@@ -119,13 +120,15 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   const size_t tk = size_t(d->bh) * d->d * p.npad_k * p.esz;
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off = align256(off + bytes); return o; };
-  p.kt = take(p.use_state ? tk : 0);
+  p.kt = take(tk);
   p.vt = take(tk);
+  p.kr = take(tk);
   p.big = take(size_t(d->bh) * p.nslots * bigsz);
   p.small = take(size_t(d->bh) * p.nslots * smallsz);
   p.fwd_bytes = off ? off : 256;
   off = 0;
   p.b_kt = take(tk); p.b_vt = take(tk); p.b_qt = take(tq); p.b_qct = take(tq);
+  p.b_kr = take(tk); p.b_vr = take(tk); p.b_qr = take(tq);
   p.b_gh = take(tq); p.b_ght = take(tq);
   p.b_cv = take(size_t(d->bh) * p.npad_q * 4);
   p.b_bigq = take(size_t(d->bh) * p.nslots * bigsz); p.b_smallq = take(size_t(d->bh) * p.nslots * smallsz);
@@ -147,35 +150,52 @@ template <typename T> TRef<T> mref(void* ptr, const FastmaxStrides& s) {
 }
 
 template <typename TIO, typename E, int DH>
-int launch_transpose(const void* x, const FastmaxStrides& s, int bh, int n, int npad, E* xt, float scale,
+int launch_transpose(const void* x, const FastmaxStrides& s, int bh, int n, int npad, E* xt, E* xr, float scale,
                      fm_stream_t stream) {
   TRef<const TIO> r = cref<TIO>(x, s);
   ProfScope prof(FM_K_TRANSPOSE, stream);
   FM_KERNEL_LAUNCH((k_transpose<TIO, E, DH>), fm_dim3(npad / 64, bh), fm_dim3(FM_THREADS), 0, stream,
-                   r.p, r.s_bh, r.s_n, r.vec, n, npad, xt, scale);
+                   r.p, r.s_bh, r.s_n, r.vec, n, npad, xt, xr, scale);
+  return fm_after_launch();
+}
+
+template <typename E, int DH, int NA, int TT>
+int launch_build_cfg(const BuildArgs<E>& a, int bh, fm_stream_t stream) {
+  constexpr int PT = TT + Mma<E>::PAD;
+  constexpr int AW = 4 * NA;
+  size_t lds = size_t(3 * DH + AW) * PT * sizeof(E);                        // staged token tiles
+  const size_t red = size_t(2) * 4 * 64 * 16 * 4;                            // reduction scratch of the lower-order tiles
+  const size_t snap = size_t(AW) * DH * (DH + Mma<E>::PAD) * sizeof(E);      // snapshot staging
+  if (lds < red) lds = red;
+  if (lds < snap) lds = snap;
+  fm_allow_lds(reinterpret_cast<const void*>(&k_build<E, DH, NA, TT>), lds);
+  FM_KERNEL_LAUNCH((k_build<E, DH, NA, TT>), fm_dim3(DH / AW, bh), fm_dim3(FM_THREADS), lds, stream, a);
   return fm_after_launch();
 }
 
 template <typename E, int DH>
-int launch_build(const BuildArgs<E>& a, int bh, fm_stream_t stream) {
-  constexpr int TT = 64;
-  constexpr int PT = TT + Mma<E>::PAD;
-  const size_t lds = size_t(4) * DH * PT * sizeof(E);
-  const int nsteps = a.mode == FM_WALK_TOTAL ? 1 : a.nseg - 1;
+int launch_build(const BuildArgs<E>& a_in, int bh, fm_stream_t stream) {
+  const int nsteps = a_in.mode == FM_WALK_TOTAL ? 1 : a_in.nseg - 1;
   if (nsteps <= 0) return FASTMAX_OK;
   ProfScope prof(FM_K_BUILD, stream);
-  // two values of a per wavefront when that still fills the GPU, else one
-  const bool na2 = int64_t(bh) * (DH / 8) >= 256;
-  if (na2) {
-    const int groups = a.quad ? DH / 8 : 0;
-    fm_allow_lds(reinterpret_cast<const void*>(&k_build<E, DH, 2, TT>), lds);
-    FM_KERNEL_LAUNCH((k_build<E, DH, 2, TT>), fm_dim3(groups + 1, bh), fm_dim3(FM_THREADS), lds, stream, a);
-  } else {
-    const int groups = a.quad ? DH / 4 : 0;
-    fm_allow_lds(reinterpret_cast<const void*>(&k_build<E, DH, 1, TT>), lds);
-    FM_KERNEL_LAUNCH((k_build<E, DH, 1, TT>), fm_dim3(groups + 1, bh), fm_dim3(FM_THREADS), lds, stream, a);
+  BuildArgs<E> a = a_in;
+  a.dbg = 0;
+#if !defined(FM_HOSTSIM)
+  if (const char* v = getenv("FASTMAX_BUILD_DBG")) a.dbg = atoi(v);
+#endif
+  int variant = 0;
+#if !defined(FM_HOSTSIM)
+  if (const char* v = getenv("FASTMAX_BUILD_VARIANT")) variant = atoi(v);   // tuning aid
+#endif
+  if (sizeof(E) == 2) {
+    // two values of a per wavefront when that still fills the GPU, else one
+    const bool na2 = variant ? (variant & 1) : int64_t(bh) * (DH / 8) >= 256;
+    const bool tt128 = variant ? (variant & 2) : true;
+    if (na2) return tt128 ? launch_build_cfg<E, DH, 2, 128>(a, bh, stream) : launch_build_cfg<E, DH, 2, 64>(a, bh, stream);
+    return tt128 ? launch_build_cfg<E, DH, 1, 128>(a, bh, stream) : launch_build_cfg<E, DH, 1, 64>(a, bh, stream);
   }
-  return fm_after_launch();
+  if (int64_t(bh) * (DH / 8) >= 256) return launch_build_cfg<E, DH, 2, 64>(a, bh, stream);
+  return launch_build_cfg<E, DH, 1, 64>(a, bh, stream);
 }
 
 template <typename E, int DH, int QT> size_t tok_lds_bytes(int extra_floats) {
@@ -195,13 +215,14 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   E* vt = reinterpret_cast<E*>(ws + p.vt);
   E* big = reinterpret_cast<E*>(ws + p.big);
   float* small = reinterpret_cast<float*>(ws + p.small);
-  int st = launch_transpose<TIO, E, DH>(v, d->sv, d->bh, d->nk, p.npad_k, vt, 1.0f, stream);
+  E* kr = reinterpret_cast<E*>(ws + p.kr);
+  int st = launch_transpose<TIO, E, DH>(v, d->sv, d->bh, d->nk, p.npad_k, vt, static_cast<E*>(nullptr), 1.0f, stream);
+  if (st) return st;
+  st = launch_transpose<TIO, E, DH>(k, d->sk, d->bh, d->nk, p.npad_k, kt, kr, p.sc, stream);
   if (st) return st;
   if (p.use_state) {
-    st = launch_transpose<TIO, E, DH>(k, d->sk, d->bh, d->nk, p.npad_k, kt, p.sc, stream);
-    if (st) return st;
     BuildArgs<E> b;
-    b.xt = kt; b.pt = vt; b.rt = kt; b.za = kt; b.zb = kt;
+    b.xt = kt; b.pt = vt; b.rt = kt; b.zt = nullptr; b.za_sel = FM_SRC_R; b.zb_sel = FM_SRC_R;
     b.npad = p.npad_k; b.nseg = p.nseg; b.L = p.L; b.mode = d->mask ? FM_WALK_PREFIX : FM_WALK_TOTAL;
     b.quad = p.quad; b.big = big; b.small = small; b.nslots = p.nslots;
     b.big2 = nullptr; b.vb_from_r = 0; b.coef2b = 0.0f; b.coef1b = 0.0f;
@@ -213,7 +234,7 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   a.q = cref<TIO>(q, d->sq); a.k = cref<TIO>(k, d->sk); a.v = cref<TIO>(v, d->sv);
   a.o = mref<TIO>(o, d->so);
   a.g = g; a.g_s_bh = d->sg.bh; a.g_s_n = d->sg.n;
-  a.vt = vt; a.npad_k = p.npad_k;
+  a.vt = vt; a.kr = kr; a.npad_k = p.npad_k;
   a.big = big; a.small = small; a.nslots = p.nslots;
   a.nq = d->nq; a.nk = d->nk; a.L = p.L; a.causal = d->mask != 0; a.use_state = p.use_state; a.quad = p.quad;
   a.a0 = p.a0; a.a1 = p.a1; a.a2 = p.a2; a.sc = p.sc;

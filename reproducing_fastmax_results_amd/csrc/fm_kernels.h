@@ -23,6 +23,23 @@
 
 static constexpr int FM_THREADS = 256;   // four wavefronts per workgroup, everywhere
 
+// Workgroups are handed to the 8 XCDs round-robin in launch order, and each XCD has its own
+// L2.  All workgroups of one batch*head read the same tiles and states, so the launch index
+// is remapped to put them on one XCD: with `units` workgroups per batch*head and nbh a
+// multiple of 8, launch index id runs on XCD id % 8 and becomes unit (id / 8) % units of
+// batch*head id % 8 + 8 * ((id / 8) / units).  Otherwise the plain 2-D index is used.
+FM_DEVICE void fm_xcd_map(int units, int nbh, int& unit, int& bh) {
+  const int id = FM_BID_X + FM_GDIM_X * FM_BID_Y;
+  if ((nbh & 7) == 0) {
+    const int x = id & 7, j = id >> 3;
+    unit = j % units;
+    bh = x + 8 * (j / units);
+  } else {
+    unit = id % units;
+    bh = id / units;
+  }
+}
+
 // ------------------------------------------------------------------------------
 // tile movers (global -> registers -> LDS), 16-byte chunks, 256 threads
 // ------------------------------------------------------------------------------
@@ -96,13 +113,15 @@ struct RowRegs {
 };
 
 // ------------------------------------------------------------------------------
-// k_transpose: x (bh, n, DH) strided, interface type  ->  xt [bh][DH][npad], compute
-// type, multiplied by `scale`, zero for tokens >= n.  grid (npad/64, bh).
+// k_transpose: x (bh, n, DH) strided, interface type  ->  compute type, multiplied by
+// `scale`, zero for tokens >= n:  xt [bh][DH][npad] (transposed) and, when xr is not
+// null, xr [bh][npad][DH] (row-major).  The token-side kernels stage their tiles from
+// these copies with plain 16-byte moves.  grid (npad/64, bh).
 // ------------------------------------------------------------------------------
 template <typename TIO, typename E, int DH>
 FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS)
 k_transpose(const TIO* FM_RESTRICT x, int64_t s_bh, int64_t s_n, int vec, int n, int npad,
-            E* FM_RESTRICT xt, float scale) {
+            E* FM_RESTRICT xt, E* FM_RESTRICT xr, float scale) {
   constexpr int PT = 64 + Mma<E>::PAD;
   constexpr int VEC = Mma<E>::VEC;
   FM_SHARED E tile[DH * PT];
@@ -118,7 +137,10 @@ k_transpose(const TIO* FM_RESTRICT x, int64_t s_bh, int64_t s_n, int vec, int n,
       for (int j = 0; j < 8; ++j) v[j] = 0.f;
     }
 #pragma unroll
-    for (int j = 0; j < 8; ++j) tile[(d0 + j) * PT + tok] = CE<E>::from(v[j] * scale);
+    for (int j = 0; j < 8; ++j) v[j] *= scale;
+    if (xr) CE<E>::st8(xr + (int64_t(bh) * npad + t0 + tok) * DH + d0, v);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) tile[(d0 + j) * PT + tok] = CE<E>::from(v[j]);
   }
   FM_SYNC();
   E* ob = xt + int64_t(bh) * DH * npad + t0;
@@ -133,6 +155,7 @@ k_transpose(const TIO* FM_RESTRICT x, int64_t s_bh, int64_t s_n, int vec, int n,
 // k_prep_bwd: per token  gh = gscale * dO / g,  c = gh . o,  q' = qscale * q ; writes
 //   gh  [bh][npad][DH]  (row-major, compute type)      ght [bh][DH][npad]
 //   qt  [bh][DH][npad]  (q' transposed)                 qct [bh][DH][npad]  (c_i q'_i)
+//   qr  [bh][npad][DH]  (q' row-major)
 //   cv  [bh][npad]      (c, compute type)
 // gscale is a power of two that keeps gh inside the _Float16 range for long sequences
 // (g grows like the token index); every gradient is linear in (gh, c) and is divided
@@ -147,7 +170,7 @@ template <typename TIO, typename E, int DH>
 FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS)
 k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, const float* FM_RESTRICT g,
            int64_t g_s_bh, int64_t g_s_n, int n, int npad, E* FM_RESTRICT gh, E* FM_RESTRICT ght,
-           E* FM_RESTRICT qt, E* FM_RESTRICT qct, E* FM_RESTRICT cv, float qscale, float gscale) {
+           E* FM_RESTRICT qt, E* FM_RESTRICT qct, E* FM_RESTRICT qr, E* FM_RESTRICT cv, float qscale, float gscale) {
   constexpr int PT = 64 + Mma<E>::PAD;
   constexpr int VEC = Mma<E>::VEC;
   constexpr int EPT = DH / 4;                      // elements per thread (4 threads per token)
@@ -182,8 +205,9 @@ k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, const floa
   csum += fm_shfl_xor(csum, 2);
   if (part == 0) cv[int64_t(bh) * npad + row] = CE<E>::from(csum);
   E* ghrow = gh + (int64_t(bh) * npad + row) * DH + d0;
+  E* qrrow = qr + (int64_t(bh) * npad + row) * DH + d0;
 #pragma unroll
-  for (int j = 0; j < EPT; j += 8) CE<E>::st8(ghrow + j, &vg[j]);
+  for (int j = 0; j < EPT; j += 8) { CE<E>::st8(ghrow + j, &vg[j]); CE<E>::st8(qrrow + j, &vq[j]); }
 #pragma unroll
   for (int j = 0; j < EPT; ++j) {
     tg[(d0 + j) * PT + tok] = CE<E>::from(vg[j]);
@@ -220,15 +244,20 @@ template <int DH> struct StateDims {
 
 enum { FM_WALK_PREFIX = 0, FM_WALK_SUFFIX = 1, FM_WALK_TOTAL = 2 };
 
+enum { FM_SRC_P = 0, FM_SRC_R = 1, FM_SRC_Z = 2 };
+
 template <typename E> struct BuildArgs {
-  const E* xt; const E* pt; const E* rt; const E* za; const E* zb;   // [bh][DH][npad]
+  const E* xt; const E* pt; const E* rt;   // [bh][DH][npad] transposed operands
+  const E* zt;                             // optional third operand (rows of the Z product), or null
+  int za_sel, zb_sel;                      // Z = sum za_r zb_c with za, zb chosen among p, r, zt
   int npad, nseg, L, mode, quad;
-  E* big; float* small;                 // [bh][nslots] states
-  E* big2;                              // optional second copy with every [r][c] tile transposed
+  E* big; float* small;                    // [bh][nslots] states
+  E* big2;                                 // optional second copy with every [r][c] tile transposed
   int nslots;
-  int vb_from_r;                        // vb sums the r operand instead of p
+  int vb_from_r;                           // vb sums the r operand instead of p
   float coef2, coef1, coefz, coefva, coefvb;
-  float coef2b, coef1b;                 // coefficients of the transposed copy
+  float coef2b, coef1b;                    // coefficients of the transposed copy
+  int dbg;
 };
 
 FM_DEVICE void fm_walk_step(int mode, int nseg, int L, int npad, int w, int& tb, int& te, int& slot) {
@@ -239,213 +268,233 @@ FM_DEVICE void fm_walk_step(int mode, int nseg, int L, int npad, int w, int& tb,
   } else { tb = 0; te = npad; slot = 0; }
 }
 
-// k_build: one workgroup per (group of 4*NA values of a, batch*head) walks the
-// tokens once, keeping its slice of the order-2 state in accumulators and
-// writing a snapshot at every segment boundary, so the prefix (or suffix) scan
-// over segments is implicit.  The last workgroup in x builds the order-1 and
-// denominator states.  Replaces the running sums of fastmax_cuda_forward.cu:183-276
-// (one thread per feature, serial over tokens) and the cumsum of materialised
-// outer products of fastattention_einops.py:237-248.
+// k_build: one workgroup per (group of 4*NA values of a, batch*head) walks the tokens
+// once, keeping its slice of the order-2 state in accumulators and writing a snapshot at
+// every segment boundary, so the prefix (or suffix) scan over segments is implicit.
+// The order-1 state, the denominator matrix Z and the two vector sums are 2*NT*NT + 2*NT
+// further 32x32 tiles; they are dealt round-robin to the workgroups of a batch*head, and
+// inside a workgroup each wavefront adds its quarter of the k-steps, so every workgroup
+// does the same amount of work and the grid is exactly (DH / (4*NA)) x bh.
+// Replaces the running sums of fastmax_cuda_forward.cu:165-276 (one thread per feature,
+// serial over tokens) and the cumsum of materialised outer products of
+// fastattention_einops.py:237-248.
 template <typename E, int DH, int NA, int TT>
-FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (sizeof(E) == 2 ? 2 : 1)) k_build(BuildArgs<E> A) {
+FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 ? 2 : 1)) k_build(BuildArgs<E> A) {
   typedef Mma<E> M;
   typedef typename M::frag frag;
   constexpr int AW = 4 * NA;
-  constexpr int NT = DH / 32;               // 32-row tiles per feature axis
+  constexpr int G = DH / AW;                 // workgroups per batch*head
+  constexpr int NT = DH / 32;                // 32-row tiles per feature axis
   constexpr int PT = TT + M::PAD;
+  constexpr int NSMALL = 2 * NT * NT + 2 * NT;
+  constexpr int SPW = (NSMALL + G - 1) / G;  // small tiles per workgroup (at most)
+  constexpr int NSTEP = TT / M::KSTEP;
   FM_DYN_SMEM(smem);
-  E* s0 = reinterpret_cast<E*>(smem);       // p tile   [DH][PT]
+  E* s0 = reinterpret_cast<E*>(smem);        // p tile   [DH][PT]
   E* s1 = s0 + DH * PT;                      // r tile   [DH][PT]
-  E* s2 = s1 + DH * PT;                      // heavy: x rows [AW][PT]; small: za tile [DH][PT]
-  E* s3 = s2 + DH * PT;                      // small: zb tile [DH][PT]
-  const int tid = FM_TID_X, wave = tid >> 6, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
-  const int bh = FM_BID_Y;
-  const int ngroups = A.quad ? DH / AW : 0;
-  const bool small = (FM_BID_X == ngroups);
+  E* s2 = s1 + DH * PT;                      // x rows   [AW][PT]
+  E* s3 = s2 + AW * PT;                      // third operand tile [DH][PT] (when zt is given)
+  const int tid = FM_TID_X, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int wave = FM_UNIFORM(tid >> 6);
+  int grp, bh;
+  fm_xcd_map(G, FM_GDIM_Y, grp, bh);
   const int64_t tb_off = int64_t(bh) * DH * A.npad;
   const int nsteps = (A.mode == FM_WALK_TOTAL) ? 1 : A.nseg - 1;
   if (nsteps <= 0) return;
   E* big = A.big + int64_t(bh) * A.nslots * StateDims<DH>::BIG;
   E* big2 = A.big2 ? A.big2 + int64_t(bh) * A.nslots * StateDims<DH>::BIG : nullptr;
   float* sml = A.small + int64_t(bh) * A.nslots * StateDims<DH>::SMALL;
+  const bool has_z = A.zt != nullptr;
+  const bool quad = A.quad != 0;
+
+  // small tiles of this workgroup: offsets (elements from s0) of the operand rows in LDS for
+  // the A side and the B side (-1: a column of ones)
+  int sm_a[SPW], sm_b[SPW], sm_id[SPW];
+#pragma unroll
+  for (int s = 0; s < SPW; ++s) {
+    const int t = grp + s * G;
+    sm_id[s] = t < NSMALL ? t : -1;
+    const int o0 = 0, o1 = DH * PT, o3 = (2 * DH + AW) * PT;
+    const int oza = A.za_sel == FM_SRC_P ? o0 : (A.za_sel == FM_SRC_R ? o1 : o3);
+    const int ozb = A.zb_sel == FM_SRC_P ? o0 : (A.zb_sel == FM_SRC_R ? o1 : o3);
+    int pa = o0, pb = -1;
+    if (t < NT * NT) { pa = o0 + 32 * (t / NT) * PT; pb = o1 + 32 * (t % NT) * PT; }                    // order 1
+    else if (t < 2 * NT * NT) {
+      const int u = t - NT * NT;
+      pa = oza + 32 * (u / NT) * PT; pb = ozb + 32 * (u % NT) * PT;                                      // Z
+    } else if (t < 2 * NT * NT + NT) pa = oza + 32 * (t - 2 * NT * NT) * PT;                             // va
+    else if (t < NSMALL) pa = (A.vb_from_r ? o1 : o0) + 32 * (t - 2 * NT * NT - NT) * PT;                // vb
+    sm_a[s] = pa + lr * PT + lh * M::KPL;
+    sm_b[s] = pb >= 0 ? pb + lr * PT + lh * M::KPL : -1;
+  }
 
   int w = 0, tb, te, slot;
   fm_walk_step(A.mode, A.nseg, A.L, A.npad, 0, tb, te, slot);
   int t = tb;
-
-  if (!small) {
-    const int a0 = FM_BID_X * AW;
-    TileRegs<E, DH, TT> rp, rr;
-    TileRegs<E, AW, TT> rx;
-    fm_f32x16 acc[NA][NT][NT];
+  const int a0 = grp * AW;
+  TileRegs<E, DH, TT> rp, rr, rz;
+  TileRegs<E, AW, TT> rx;
+  fm_f32x16 acc[NA][NT][NT];
+  fm_f32x16 sacc[SPW];
 #pragma unroll
-    for (int i = 0; i < NA; ++i)
+  for (int i = 0; i < NA; ++i)
 #pragma unroll
-      for (int j = 0; j < NT; ++j)
+    for (int j = 0; j < NT; ++j)
 #pragma unroll
-        for (int k = 0; k < NT; ++k) acc[i][j][k] = fm_zero16();
-    rp.load(A.pt + tb_off + t, A.npad, tid);
-    rr.load(A.rt + tb_off + t, A.npad, tid);
-    rx.load(A.xt + tb_off + int64_t(a0) * A.npad + t, A.npad, tid);
-    bool have = true;
-    while (have) {
-      FM_SYNC();
-      rp.store(s0, PT, tid); rr.store(s1, PT, tid); rx.store(s2, PT, tid);
-      FM_SYNC();
-      int nt = t + TT, nw = w, ntb = tb, nte = te, nslot = slot;
-      const bool last = (nt >= te);
-      bool has_next = true;
-      if (last) {
-        nw = w + 1;
-        if (nw < nsteps) { fm_walk_step(A.mode, A.nseg, A.L, A.npad, nw, ntb, nte, nslot); nt = ntb; }
-        else has_next = false;
-      }
-      if (has_next) {
-        rp.load(A.pt + tb_off + nt, A.npad, tid);
-        rr.load(A.rt + tb_off + nt, A.npad, tid);
-        rx.load(A.xt + tb_off + int64_t(a0) * A.npad + nt, A.npad, tid);
-      }
+      for (int k = 0; k < NT; ++k) acc[i][j][k] = fm_zero16();
+#pragma unroll
+  for (int s = 0; s < SPW; ++s) sacc[s] = fm_zero16();
+  rp.load(A.pt + tb_off + t, A.npad, tid);
+  rr.load(A.rt + tb_off + t, A.npad, tid);
+  if (quad) rx.load(A.xt + tb_off + int64_t(a0) * A.npad + t, A.npad, tid);
+  if (has_z) rz.load(A.zt + tb_off + t, A.npad, tid);
+  bool have = true;
+  while (have) {
+    if (!(A.dbg & 2) || t == tb) {
+    FM_SYNC();
+    rp.store(s0, PT, tid); rr.store(s1, PT, tid);
+    if (quad) rx.store(s2, PT, tid);
+    if (has_z) rz.store(s3, PT, tid);
+    FM_SYNC();
+    }
+    int nt = t + TT, nw = w, ntb = tb, nte = te, nslot = slot;
+    const bool last = (nt >= te);
+    bool has_next = true;
+    if (last) {
+      nw = w + 1;
+      if (nw < nsteps) { fm_walk_step(A.mode, A.nseg, A.L, A.npad, nw, ntb, nte, nslot); nt = ntb; }
+      else has_next = false;
+    }
+    if (has_next && !(A.dbg & 1)) {
+      rp.load(A.pt + tb_off + nt, A.npad, tid);
+      rr.load(A.rt + tb_off + nt, A.npad, tid);
+      if (quad) rx.load(A.xt + tb_off + int64_t(a0) * A.npad + nt, A.npad, tid);
+      if (has_z) rz.load(A.zt + tb_off + nt, A.npad, tid);
+    }
+    if (quad && !(A.dbg & 4)) {
+      // fragments of k-step ks+1 are fetched while the products of k-step ks are issued
+      const E* pb_ = s0 + lr * PT + lh * M::KPL;
+      const E* rb_ = s1 + lr * PT + lh * M::KPL;
+      const E* xb_ = s2 + (wave * NA) * PT + lh * M::KPL;
+      frag fb[NT], fp[NT], fx[NA];
+#pragma unroll
+      for (int j = 0; j < NT; ++j) { fb[j] = M::load(rb_ + 32 * j * PT); fp[j] = M::load(pb_ + 32 * j * PT); }
+#pragma unroll
+      for (int i = 0; i < NA; ++i) fx[i] = M::load(xb_ + i * PT);
 #pragma unroll 2
-      for (int ks = 0; ks < TT / M::KSTEP; ++ks) {
-        const int ko = ks * M::KSTEP + lh * M::KPL;
-        frag fb[NT], fp[NT];
+      for (int ks = 0; ks < NSTEP; ++ks) {
+        const int kn = (ks + 1 < NSTEP ? ks + 1 : ks) * M::KSTEP;
+        frag nb[NT], np[NT], nx[NA];
 #pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          fb[j] = M::load(s1 + (32 * j + lr) * PT + ko);
-          fp[j] = M::load(s0 + (32 * j + lr) * PT + ko);
-        }
+        for (int j = 0; j < NT; ++j) { nb[j] = M::load(rb_ + 32 * j * PT + kn); np[j] = M::load(pb_ + 32 * j * PT + kn); }
+#pragma unroll
+        for (int i = 0; i < NA; ++i) nx[i] = M::load(xb_ + i * PT + kn);
 #pragma unroll
         for (int i = 0; i < NA; ++i) {
-          const frag fx = M::load(s2 + (wave * NA + i) * PT + ko);
 #pragma unroll
           for (int j = 0; j < NT; ++j) {
-            const frag fa = fp[j] * fx;
+            const frag fa = fp[j] * fx[i];
 #pragma unroll
             for (int k = 0; k < NT; ++k) acc[i][j][k] = M::mma(fa, fb[k], acc[i][j][k]);
           }
         }
-      }
-      if (last) {
-        E* dst = big + int64_t(slot) * StateDims<DH>::BIG;
 #pragma unroll
-        for (int i = 0; i < NA; ++i) {
-          const int a = a0 + wave * NA + i;
+        for (int j = 0; j < NT; ++j) { fb[j] = nb[j]; fp[j] = np[j]; }
+#pragma unroll
+        for (int i = 0; i < NA; ++i) fx[i] = nx[i];
+      }
+    }
+    // the lower-order tiles: this wavefront takes the k-steps ks = wave (mod 4)
+#pragma unroll
+    for (int s = 0; s < SPW; ++s) {
+      if (sm_id[s] >= 0 && !(A.dbg & 8)) {
+        for (int ks = wave; ks < NSTEP; ks += 4) {
+          const frag fa = M::load(s0 + sm_a[s] + ks * M::KSTEP);
+          const frag fo = sm_b[s] >= 0 ? M::load(s0 + sm_b[s] + ks * M::KSTEP) : M::splat(E(1.0f));
+          sacc[s] = M::mma(fa, fo, sacc[s]);
+        }
+      }
+    }
+    if (last) {
+      if (quad) {
+        // snapshot through LDS (the token tiles are spent): accumulators -> staged tiles ->
+        // coalesced 16-byte stores; a second pass writes the transposed tiles
+        constexpr int SP = DH + M::PAD;
+        constexpr int VEC = M::VEC;
+        E* stg = reinterpret_cast<E*>(smem);                 // [AW][DH][SP]
+        FM_SYNC();
+#pragma unroll
+        for (int i = 0; i < NA; ++i)
 #pragma unroll
           for (int j = 0; j < NT; ++j)
 #pragma unroll
             for (int k = 0; k < NT; ++k)
 #pragma unroll
-              for (int e = 0; e < 16; ++e) {
-                const int r = 32 * j + fm_acc_row(e, lh), c = 32 * k + lr;
-                dst[(int64_t(a) * DH + r) * DH + c] = CE<E>::from(A.coef2 * acc[i][j][k][e]);
-              }
+              for (int e = 0; e < 16; ++e)
+                stg[((wave * NA + i) * DH + 32 * j + fm_acc_row(e, lh)) * SP + 32 * k + lr] =
+                    CE<E>::from(A.coef2 * acc[i][j][k][e]);
+        FM_SYNC();
+        E* dst = big + int64_t(slot) * StateDims<DH>::BIG + int64_t(a0) * DH * DH;
+        for (int c = tid; c < AW * DH * (DH / VEC); c += FM_THREADS) {
+          const int row = c / (DH / VEC), col = (c % (DH / VEC)) * VEC;
+          *reinterpret_cast<fm_u32x4*>(dst + row * DH + col) = *reinterpret_cast<const fm_u32x4*>(stg + row * SP + col);
         }
         if (big2) {
-          E* dst2 = big2 + int64_t(slot) * StateDims<DH>::BIG;
+          FM_SYNC();
 #pragma unroll
-          for (int i = 0; i < NA; ++i) {
-            const int a = a0 + wave * NA + i;
+          for (int i = 0; i < NA; ++i)
 #pragma unroll
             for (int j = 0; j < NT; ++j)
 #pragma unroll
               for (int k = 0; k < NT; ++k)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                  const int r = 32 * j + fm_acc_row(e, lh), c = 32 * k + lr;
-                  dst2[(int64_t(a) * DH + c) * DH + r] = CE<E>::from(A.coef2b * acc[i][j][k][e]);
-                }
+                for (int e = 0; e < 16; ++e)
+                  stg[((wave * NA + i) * DH + 32 * k + lr) * SP + 32 * j + fm_acc_row(e, lh)] =
+                      CE<E>::from(A.coef2b * acc[i][j][k][e]);
+          FM_SYNC();
+          E* dst2 = big2 + int64_t(slot) * StateDims<DH>::BIG + int64_t(a0) * DH * DH;
+          for (int c = tid; c < AW * DH * (DH / VEC); c += FM_THREADS) {
+            const int row = c / (DH / VEC), col = (c % (DH / VEC)) * VEC;
+            *reinterpret_cast<fm_u32x4*>(dst2 + row * DH + col) = *reinterpret_cast<const fm_u32x4*>(stg + row * SP + col);
           }
         }
       }
-      t = nt; w = nw; tb = ntb; te = nte; slot = nslot; have = has_next;
-    }
-  } else {
-    // order-1 state (wave 0), denominator matrix Z (wave 1), vector sums (waves 2, 3)
-    const bool has_z = (A.za != nullptr);
-    TileRegs<E, DH, TT> rp, rr, ra, rb;
-    fm_f32x16 acc[NT][NT];
-#pragma unroll
-    for (int j = 0; j < NT; ++j)
-#pragma unroll
-      for (int k = 0; k < NT; ++k) acc[j][k] = fm_zero16();
-    float vsum = 0.f;
-    rp.load(A.pt + tb_off + t, A.npad, tid);
-    rr.load(A.rt + tb_off + t, A.npad, tid);
-    if (has_z) { ra.load(A.za + tb_off + t, A.npad, tid); rb.load(A.zb + tb_off + t, A.npad, tid); }
-    bool have = true;
-    while (have) {
+      // reduce the four wavefronts' partial lower-order tiles through LDS (the token tiles are spent)
       FM_SYNC();
-      rp.store(s0, PT, tid); rr.store(s1, PT, tid);
-      if (has_z) { ra.store(s2, PT, tid); rb.store(s3, PT, tid); }
+      float* red = reinterpret_cast<float*>(smem);           // [SPW][4 waves][64 lanes][16]
+#pragma unroll
+      for (int s = 0; s < SPW; ++s)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) red[((s * 4 + wave) * 16 + e) * 64 + lane] = sacc[s][e];
       FM_SYNC();
-      int nt = t + TT, nw = w, ntb = tb, nte = te, nslot = slot;
-      const bool last = (nt >= te);
-      bool has_next = true;
-      if (last) {
-        nw = w + 1;
-        if (nw < nsteps) { fm_walk_step(A.mode, A.nseg, A.L, A.npad, nw, ntb, nte, nslot); nt = ntb; }
-        else has_next = false;
-      }
-      if (has_next) {
-        rp.load(A.pt + tb_off + nt, A.npad, tid);
-        rr.load(A.rt + tb_off + nt, A.npad, tid);
-        if (has_z) { ra.load(A.za + tb_off + nt, A.npad, tid); rb.load(A.zb + tb_off + nt, A.npad, tid); }
-      }
-      if (wave == 0 || (wave == 1 && has_z)) {
-        const E* sa = wave == 0 ? s0 : s2;
-        const E* sb = wave == 0 ? s1 : s3;
-        for (int ks = 0; ks < TT / M::KSTEP; ++ks) {
-          const int ko = ks * M::KSTEP + lh * M::KPL;
-          frag fa[NT], fb[NT];
-#pragma unroll
-          for (int j = 0; j < NT; ++j) {
-            fa[j] = M::load(sa + (32 * j + lr) * PT + ko);
-            fb[j] = M::load(sb + (32 * j + lr) * PT + ko);
-          }
-#pragma unroll
-          for (int j = 0; j < NT; ++j)
-#pragma unroll
-            for (int k = 0; k < NT; ++k) acc[j][k] = M::mma(fa[j], fb[k], acc[j][k]);
-        }
-      } else if (wave >= 2 && lane < DH && (wave == 3 || has_z)) {
-        const E* sv = wave == 2 ? s2 : (A.vb_from_r ? s1 : s0);   // wave 2: sum of za, wave 3: sum of p (or r)
-        float s = 0.f;
-        for (int j = 0; j < TT; ++j) s += float(sv[lane * PT + j]);
-        vsum += s;
-      }
-      if (last) {
+      if (wave == 0) {
         float* ds = sml + int64_t(slot) * StateDims<DH>::SMALL;
-        if (wave == 0) {
-          E* dst = big + int64_t(slot) * StateDims<DH>::BIG + int64_t(DH) * DH * DH;
 #pragma unroll
-          for (int j = 0; j < NT; ++j)
+        for (int s = 0; s < SPW; ++s) {
+          const int tl = sm_id[s];
+          if (tl < 0) continue;
 #pragma unroll
-            for (int k = 0; k < NT; ++k)
-#pragma unroll
-              for (int e = 0; e < 16; ++e) {
-                const int r = 32 * j + fm_acc_row(e, lh), c = 32 * k + lr;
-                dst[r * DH + c] = CE<E>::from(A.coef1 * acc[j][k][e]);
-                if (big2)
-                  big2[int64_t(slot) * StateDims<DH>::BIG + int64_t(DH) * DH * DH + c * DH + r] =
-                      CE<E>::from(A.coef1b * acc[j][k][e]);
-              }
-        } else if (wave == 1) {
-#pragma unroll
-          for (int j = 0; j < NT; ++j)
-#pragma unroll
-            for (int k = 0; k < NT; ++k)
-#pragma unroll
-              for (int e = 0; e < 16; ++e) {
-                const int r = 32 * j + fm_acc_row(e, lh), c = 32 * k + lr;
-                ds[r * DH + c] = has_z ? A.coefz * acc[j][k][e] : 0.f;
-              }
-        } else if (lane < DH) {
-          if (wave == 2) ds[DH * DH + lane] = has_z ? A.coefva * vsum : 0.f;
-          else ds[DH * DH + DH + lane] = A.coefvb * vsum;
+          for (int e = 0; e < 16; ++e) {
+            const float v = red[((s * 4 + 0) * 16 + e) * 64 + lane] + red[((s * 4 + 1) * 16 + e) * 64 + lane] +
+                            red[((s * 4 + 2) * 16 + e) * 64 + lane] + red[((s * 4 + 3) * 16 + e) * 64 + lane];
+            const int rr_ = fm_acc_row(e, lh);
+            if (tl < NT * NT) {
+              const int r = 32 * (tl / NT) + rr_, c = 32 * (tl % NT) + lr;
+              big[int64_t(slot) * StateDims<DH>::BIG + int64_t(DH) * DH * DH + r * DH + c] = CE<E>::from(A.coef1 * v);
+              if (big2)
+                big2[int64_t(slot) * StateDims<DH>::BIG + int64_t(DH) * DH * DH + c * DH + r] = CE<E>::from(A.coef1b * v);
+            } else if (tl < 2 * NT * NT) {
+              const int u = tl - NT * NT;
+              ds[(32 * (u / NT) + rr_) * DH + 32 * (u % NT) + lr] = A.coefz * v;
+            } else if (lr == 0) {
+              if (tl < 2 * NT * NT + NT) ds[DH * DH + 32 * (tl - 2 * NT * NT) + rr_] = A.coefva * v;
+              else ds[DH * DH + DH + 32 * (tl - 2 * NT * NT - NT) + rr_] = A.coefvb * v;
+            }
+          }
         }
       }
-      t = nt; w = nw; tb = ntb; te = nte; slot = nslot; have = has_next;
     }
+    t = nt; w = nw; tb = ntb; te = nte; slot = nslot; have = has_next;
   }
 }
 
@@ -539,7 +588,7 @@ template <typename TIO, typename E> struct FwdArgs {
   TRef<const TIO> q, k, v;
   TRef<TIO> o;
   float* g; int64_t g_s_bh, g_s_n;
-  const E* vt; int npad_k;             // V transposed [bh][DH][npad_k]
+  const E* vt; const E* kr; int npad_k; // V transposed [bh][DH][npad_k], K row-major [bh][npad_k][DH] (scaled)
   const E* big; const float* small; int nslots;
   int nq, nk, L, causal, use_state, quad;
   float a0, a1, a2;                    // f(s) = a0 + a1 s + a2 s^2
@@ -561,9 +610,10 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_fwd(FwdArgs<TIO, E> A) {
   E* R = reinterpret_cast<E*>(vecs + 2 * DH);         // slabs | dense-loop tiles | output staging
   const int tid = FM_TID_X, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   const int wave = FM_UNIFORM(tid >> 6);
-  const int bh = FM_BID_Y;
   const int nqb = FM_GDIM_X;
-  const int qb = A.causal ? (nqb - 1 - FM_BID_X) : FM_BID_X;    // heavy blocks first
+  int unit, bh;
+  fm_xcd_map(nqb, FM_GDIM_Y, unit, bh);
+  const int qb = A.causal ? (nqb - 1 - unit) : unit;            // heavy blocks first
   const int q0 = qb * QW;
   const int seg = A.causal ? q0 / A.L : 0;
   const bool use_state = A.use_state && (!A.causal || seg > 0);
@@ -639,21 +689,21 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_fwd(FwdArgs<TIO, E> A) {
   // ---- dense tiles over the keys of this segment ----
   if (kend > kbeg) {
     const typename TM::Coef coef = TM::coef(A.a0, A.a1, A.a2);
-    RowRegs<TIO, E, KT, DH> rk;
+    TileRegs<E, KT, DH> rk;
     TileRegs<E, DH, KT> rv;
-    const TIO* kb = A.k.p + int64_t(bh) * A.k.s_bh;
+    const E* kb = A.kr + int64_t(bh) * A.npad_k * DH;
     const E* vtb = A.vt + int64_t(bh) * DH * A.npad_k;
-    rk.load(kb, A.k.s_n, A.k.vec != 0, kbeg, A.nk, tid);
+    rk.load(kb + int64_t(kbeg) * DH, DH, tid);
     rv.load(vtb + kbeg, A.npad_k, tid);
     int buf = 0;
     for (int kt0 = kbeg; kt0 < kend; kt0 += KT) {
       E* Ks = R + buf * STAGE;
       E* Vs = Ks + KT * PQ;
-      rk.store(Ks, PQ, tid, A.sc);
+      rk.store(Ks, PQ, tid);
       rv.store(Vs, PV, tid);
       FM_SYNC();
       if (kt0 + KT < kend) {
-        rk.load(kb, A.k.s_n, A.k.vec != 0, kt0 + KT, A.nk, tid);
+        rk.load(kb + int64_t(kt0 + KT) * DH, DH, tid);
         rv.load(vtb + kt0 + KT, A.npad_k, tid);
       }
       // work items (sub-tile st, query tile j); the score tile of the next item is issued
@@ -665,8 +715,9 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_fwd(FwdArgs<TIO, E> A) {
         const int key0 = kt0 + 32 * (it / QT), qlo = q0 + tw[it % QT] * 32;
         act[it] = key0 < kend && !(A.causal && key0 > qlo + 31);
       }
-      fm_f32x16 s_cur = fm_zero16();
+      fm_f32x16 s_cur;
       if (act[0]) {
+        s_cur = fm_zero16();
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks)
           s_cur = M::mma(M::load(Ks + lr * PQ + ks * M::KSTEP + lh * M::KPL), qf[0][ks], s_cur);
@@ -674,8 +725,9 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_fwd(FwdArgs<TIO, E> A) {
 #pragma unroll
       for (int it = 0; it < NI; ++it) {
         const int st = it / QT, j = it % QT;
-        fm_f32x16 s_nxt = fm_zero16();
+        fm_f32x16 s_nxt;
         if (it + 1 < NI && act[(it + 1 < NI) ? it + 1 : it]) {
+          s_nxt = fm_zero16();
           const int st2 = (it + 1) / QT, j2 = (it + 1) % QT;
 #pragma unroll
           for (int ks = 0; ks < NKS; ++ks)

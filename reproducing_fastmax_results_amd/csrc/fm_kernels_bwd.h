@@ -15,7 +15,7 @@
 template <typename TIO, typename E> struct BwdArgs {
   TRef<const TIO> q, k, v;
   TRef<TIO> dq, dk, dv;
-  const E* gh; const E* ght; const E* qt; const E* kt; const E* cv;       // workspace copies
+  const E* gh; const E* ght; const E* qt; const E* qr; const E* kt; const E* kr; const E* vr; const E* cv;   // workspace copies
   int npad_q, npad_k;
   const E* bigq; const float* smallq;      // prefix (k, k, v)
   const E* bigk; const float* smallk;      // suffix (q, q, gh)
@@ -104,9 +104,10 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_dq(BwdArgs<TIO, E> A) {
   E* R = reinterpret_cast<E*>(vecs + 2 * DH);         // Z | slabs | dense tiles | output staging
   const int tid = FM_TID_X, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   const int wave = FM_UNIFORM(tid >> 6);
-  const int bh = FM_BID_Y;
   const int nqb = FM_GDIM_X;
-  const int qb = A.causal ? (nqb - 1 - FM_BID_X) : FM_BID_X;
+  int unit, bh;
+  fm_xcd_map(nqb, FM_GDIM_Y, unit, bh);
+  const int qb = A.causal ? (nqb - 1 - unit) : unit;
   const int q0 = qb * QW;
   const int seg = A.causal ? q0 / A.L : 0;
   const bool use_state = A.use_state && (!A.causal || seg > 0);
@@ -165,22 +166,22 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_dq(BwdArgs<TIO, E> A) {
 
   if (kend > kbeg) {
     const typename TM::Coef coef = TM::coef(A.a0, A.a1, A.a2);
-    RowRegs<TIO, E, KT, DH> rk, rv;
+    TileRegs<E, KT, DH> rk, rv;
     TileRegs<E, DH, KT> rkt;
-    const TIO* kb = A.k.p + int64_t(bh) * A.k.s_bh;
-    const TIO* vb = A.v.p + int64_t(bh) * A.v.s_bh;
+    const E* kb = A.kr + int64_t(bh) * A.npad_k * DH;
+    const E* vb = A.vr + int64_t(bh) * A.npad_k * DH;
     const E* ktb = A.kt + int64_t(bh) * DH * A.npad_k;
-    rk.load(kb, A.k.s_n, A.k.vec != 0, kbeg, A.nk, tid);
-    rv.load(vb, A.v.s_n, A.v.vec != 0, kbeg, A.nk, tid);
+    rk.load(kb + int64_t(kbeg) * DH, DH, tid);
+    rv.load(vb + int64_t(kbeg) * DH, DH, tid);
     rkt.load(ktb + kbeg, A.npad_k, tid);
     int buf = 0;
     for (int kt0 = kbeg; kt0 < kend; kt0 += KT) {
       E* Ks = R + buf * STAGE; E* Vs = Ks + KT * PQ; E* Kts = Vs + KT * PQ;
-      rk.store(Ks, PQ, tid, A.sc); rv.store(Vs, PQ, tid, 1.0f); rkt.store(Kts, PV, tid);
+      rk.store(Ks, PQ, tid); rv.store(Vs, PQ, tid); rkt.store(Kts, PV, tid);
       FM_SYNC();
       if (kt0 + KT < kend) {
-        rk.load(kb, A.k.s_n, A.k.vec != 0, kt0 + KT, A.nk, tid);
-        rv.load(vb, A.v.s_n, A.v.vec != 0, kt0 + KT, A.nk, tid);
+        rk.load(kb + int64_t(kt0 + KT) * DH, DH, tid);
+        rv.load(vb + int64_t(kt0 + KT) * DH, DH, tid);
         rkt.load(ktb + kt0 + KT, A.npad_k, tid);
       }
       constexpr int NI = (KT / 32) * QT;
@@ -190,8 +191,9 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_dq(BwdArgs<TIO, E> A) {
         const int key0 = kt0 + 32 * (it / QT), qlo = q0 + tw[it % QT] * 32;
         act[it] = key0 < kend && !(A.causal && key0 > qlo + 31);
       }
-      fm_f32x16 s_cur = fm_zero16(), dp_cur = fm_zero16();
+      fm_f32x16 s_cur, dp_cur;
       if (act[0]) {
+        s_cur = fm_zero16(); dp_cur = fm_zero16();
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) {
           s_cur = M::mma(M::load(Ks + lr * PQ + ks * M::KSTEP + lh * M::KPL), qf[0][ks], s_cur);
@@ -201,8 +203,9 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_dq(BwdArgs<TIO, E> A) {
 #pragma unroll
       for (int it = 0; it < NI; ++it) {
         const int st = it / QT, j = it % QT;
-        fm_f32x16 s_nxt = fm_zero16(), dp_nxt = fm_zero16();
+        fm_f32x16 s_nxt, dp_nxt;
         if (it + 1 < NI && act[(it + 1 < NI) ? it + 1 : it]) {
+          s_nxt = fm_zero16(); dp_nxt = fm_zero16();
           const int st2 = (it + 1) / QT, j2 = (it + 1) % QT;
 #pragma unroll
           for (int ks = 0; ks < NKS; ++ks) {
@@ -257,8 +260,9 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_dkv(BwdArgs<TIO, E> A) {
   E* R = reinterpret_cast<E*>(vecs + 2 * DH);
   const int tid = FM_TID_X, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   const int wave = FM_UNIFORM(tid >> 6);
-  const int bh = FM_BID_Y;
-  const int k0 = FM_BID_X * KW;                        // early key blocks are the heavy ones
+  int unit, bh;
+  fm_xcd_map(FM_GDIM_X, FM_GDIM_Y, unit, bh);
+  const int k0 = unit * KW;                            // early key blocks are the heavy ones
   const int seg = A.causal ? k0 / A.L : 0;
   const bool use_state = A.use_state && (!A.causal || seg < A.nseg - 1);
   const int slot = A.causal ? seg : 0;
@@ -314,16 +318,15 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_dkv(BwdArgs<TIO, E> A) {
 
   if (iend > ibeg) {
     const typename TM::Coef coef = TM::coef(A.a0, A.a1, A.a2);
-    RowRegs<TIO, E, KT, DH> rq;
-    TileRegs<E, KT, DH> rg;
+    TileRegs<E, KT, DH> rq, rg;
     TileRegs<E, DH, KT> rqt, rgt;
-    const TIO* qb = A.q.p + int64_t(bh) * A.q.s_bh;
+    const E* qb = A.qr + int64_t(bh) * A.npad_q * DH;
     const E* ghb = A.gh + int64_t(bh) * A.npad_q * DH;
     const E* qtb = A.qt + int64_t(bh) * DH * A.npad_q;
     const E* gtb = A.ght + int64_t(bh) * DH * A.npad_q;
     const E* cvb = A.cv + int64_t(bh) * A.npad_q;
     E creg = E(0.f);
-    rq.load(qb, A.q.s_n, A.q.vec != 0, ibeg, A.nq, tid);
+    rq.load(qb + int64_t(ibeg) * DH, DH, tid);
     rg.load(ghb + int64_t(ibeg) * DH, DH, tid);
     rqt.load(qtb + ibeg, A.npad_q, tid);
     rgt.load(gtb + ibeg, A.npad_q, tid);
@@ -332,11 +335,11 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_dkv(BwdArgs<TIO, E> A) {
     for (int i0 = ibeg; i0 < iend; i0 += KT) {
       E* Qr = R + buf * STAGE_PAD; E* Gr = Qr + KT * PQ; E* Qts = Gr + KT * PQ; E* Gts = Qts + DH * PV;
       E* cs = Gts + DH * PV;
-      rq.store(Qr, PQ, tid, A.sc); rg.store(Gr, PQ, tid); rqt.store(Qts, PV, tid); rgt.store(Gts, PV, tid);
+      rq.store(Qr, PQ, tid); rg.store(Gr, PQ, tid); rqt.store(Qts, PV, tid); rgt.store(Gts, PV, tid);
       if (tid < KT) cs[tid] = creg;
       FM_SYNC();
       if (i0 + KT < iend) {
-        rq.load(qb, A.q.s_n, A.q.vec != 0, i0 + KT, A.nq, tid);
+        rq.load(qb + int64_t(i0 + KT) * DH, DH, tid);
         rg.load(ghb + int64_t(i0 + KT) * DH, DH, tid);
         rqt.load(qtb + i0 + KT, A.npad_q, tid);
         rgt.load(gtb + i0 + KT, A.npad_q, tid);
@@ -349,8 +352,9 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_dkv(BwdArgs<TIO, E> A) {
         const int qi0 = i0 + 32 * (it / QT), klo = k0 + tw[it % QT] * 32;
         act[it] = qi0 < iend && !(A.causal && qi0 + 31 < klo);   // skip queries that precede all keys
       }
-      fm_f32x16 s_cur = fm_zero16(), dp_cur = fm_zero16();
+      fm_f32x16 s_cur, dp_cur;
       if (act[0]) {
+        s_cur = fm_zero16(); dp_cur = fm_zero16();
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) {
           s_cur = M::mma(M::load(Qr + lr * PQ + ks * M::KSTEP + lh * M::KPL), kf[0][ks], s_cur);
@@ -360,8 +364,9 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_dkv(BwdArgs<TIO, E> A) {
 #pragma unroll
       for (int it = 0; it < NI; ++it) {
         const int st = it / QT, j = it % QT;
-        fm_f32x16 s_nxt = fm_zero16(), dp_nxt = fm_zero16();
+        fm_f32x16 s_nxt, dp_nxt;
         if (it + 1 < NI && act[(it + 1 < NI) ? it + 1 : it]) {
+          s_nxt = fm_zero16(); dp_nxt = fm_zero16();
           const int st2 = (it + 1) / QT, j2 = (it + 1) % QT;
 #pragma unroll
           for (int ks = 0; ks < NKS; ++ks) {

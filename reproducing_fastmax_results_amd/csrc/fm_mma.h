@@ -136,7 +136,11 @@ template <> struct CE<fm_half> {
   static FM_DEVICE void st8(fm_half* p, const float in[8]) {
     fm_half8 h;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) h[i] = from(in[i]);
+    for (int i = 0; i < 8; ++i) h[i] = fm_half(in[i]);
+    // saturate after the conversion, on packed halves (an overflowing float converts to inf)
+    const fm_half8 lim = {fm_half(65504.f), fm_half(65504.f), fm_half(65504.f), fm_half(65504.f),
+                          fm_half(65504.f), fm_half(65504.f), fm_half(65504.f), fm_half(65504.f)};
+    h = __builtin_elementwise_min(__builtin_elementwise_max(h, -lim), lim);
     *reinterpret_cast<fm_half8*>(p) = h;
   }
 };

@@ -108,3 +108,13 @@ def test_backward_ragged_and_cross(lib, dtype):
     check_forward_backward(lib, 1, 2500, 64, dtype, DEV, mask=True, p=2, seed=14)       # ragged last segment
     check_forward_backward(lib, 2, 777, 32, dtype, DEV, mask=True, p=2, a=(1.0, 1.166666, 0.145833), tau_mult=1.0,
                            seed=15)                                                    # fitted (non-Taylor) coefficients
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("d,bh", [(64, 32), (32, 64)])
+def test_many_heads_uses_two_states_per_wavefront(lib, dtype, d, bh):
+    # with bh*d/8 >= 256 the state build keeps two values of `a` per wavefront (the shape
+    # of the benchmark, B*H = 32 at D = 64); same parity bar
+    print(f"case many heads dtype={dtype} d={d} bh={bh}", flush=True)
+    check_forward_backward(lib, bh, 1100, d, dtype, DEV, mask=True, p=2, chunk=256, seed=16)
+    check_forward_backward(lib, bh, 600, d, dtype, DEV, mask=False, p=2, flags=FLAG_FORCE_MOMENTS, seed=17)
