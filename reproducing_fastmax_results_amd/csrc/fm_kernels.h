@@ -140,7 +140,7 @@ k_transpose(const TIO* FM_RESTRICT x, int64_t s_bh, int64_t s_n, int vec, int n,
     for (int j = 0; j < 8; ++j) v[j] *= scale;
     if (xr) CE<E>::st8(xr + (int64_t(bh) * npad + t0 + tok) * DH + d0, v);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) tile[(d0 + j) * PT + tok] = CE<E>::from(v[j]);
+    for (int j = 0; j < 8; ++j) tile[(d0 + j) * PT + Mma<E>::tperm(tok)] = CE<E>::from(v[j]);
   }
   FM_SYNC();
   E* ob = xt + int64_t(bh) * DH * npad + t0;
@@ -203,16 +203,16 @@ k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, const floa
   }
   csum += fm_shfl_xor(csum, 1);
   csum += fm_shfl_xor(csum, 2);
-  if (part == 0) cv[int64_t(bh) * npad + row] = CE<E>::from(csum);
+  if (part == 0) cv[int64_t(bh) * npad + t0 + Mma<E>::tperm(tok)] = CE<E>::from(csum);
   E* ghrow = gh + (int64_t(bh) * npad + row) * DH + d0;
   E* qrrow = qr + (int64_t(bh) * npad + row) * DH + d0;
 #pragma unroll
   for (int j = 0; j < EPT; j += 8) { CE<E>::st8(ghrow + j, &vg[j]); CE<E>::st8(qrrow + j, &vq[j]); }
 #pragma unroll
   for (int j = 0; j < EPT; ++j) {
-    tg[(d0 + j) * PT + tok] = CE<E>::from(vg[j]);
-    tq[(d0 + j) * PT + tok] = CE<E>::from(vq[j]);
-    tc[(d0 + j) * PT + tok] = CE<E>::from(vq[j] * csum);
+    tg[(d0 + j) * PT + Mma<E>::tperm(tok)] = CE<E>::from(vg[j]);
+    tq[(d0 + j) * PT + Mma<E>::tperm(tok)] = CE<E>::from(vq[j]);
+    tc[(d0 + j) * PT + Mma<E>::tperm(tok)] = CE<E>::from(vq[j] * csum);
   }
   FM_SYNC();
   const int64_t ob = int64_t(bh) * DH * npad + t0;

@@ -133,7 +133,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_dq(BwdArgs<TIO, E> A) {
   for (int j = 0; j < QT; ++j) {
     tw[j] = (j == 0) ? wave : (4 * QT - 1 - wave);
     xrow[j] = tw[j] * 32 + lr;
-    ci[j] = float(A.cv[int64_t(bh) * A.npad_q + q0 + xrow[j]]);
+    ci[j] = float(A.cv[int64_t(bh) * A.npad_q + q0 + M::tperm(xrow[j])]);   // c is stored in tile order
   }
   frag qf[QT][NKS], gf[QT][NKS];
 #pragma unroll

@@ -25,11 +25,14 @@ template <> struct Mma<fm_half> {
   static FM_DEVICE fm_f32x16 mma(frag a, frag b, fm_f32x16 c) { return fm_mfma_f16(a, b, c); }
   static FM_DEVICE frag load(const fm_half* p) { return *reinterpret_cast<const fm_half8*>(p); }
   static FM_DEVICE frag splat(fm_half x) { frag r = {x, x, x, x, x, x, x, x}; return r; }
+  // Transposed token tiles are stored with the 16 tokens of every group in the order
+  // 0-3, 8-11, 4-7, 12-15 (`tperm`), so that the eight accumulator rows a lane needs for
+  // accumulator k-step s (16s + 4lh + {0..3}, 16s + 8 + 4lh + {0..3}) are one 16-byte read.
+  // A contraction over tokens does not care about their order as long as both operands
+  // share it, so the same tiles serve the plain `load`.
+  static FM_DEVICE int tperm(int t) { return (t & ~15) | (t & 3) | ((t & 8) >> 1) | ((t & 4) << 1); }
   static FM_DEVICE frag load_perm(const fm_half* row, int s, int lh) {
-    const fm_half4 lo = *reinterpret_cast<const fm_half4*>(row + 16 * s + 4 * lh);
-    const fm_half4 hi = *reinterpret_cast<const fm_half4*>(row + 16 * s + 8 + 4 * lh);
-    frag r = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    return r;
+    return *reinterpret_cast<const fm_half8*>(row + 16 * s + 8 * lh);
   }
   static FM_DEVICE frag from_acc(const fm_f32x16& c, int s) {
     frag r;
@@ -49,6 +52,7 @@ template <> struct Mma<float> {
   static FM_DEVICE fm_f32x16 mma(frag a, frag b, fm_f32x16 c) { return fm_mfma_f32(a, b, c); }
   static FM_DEVICE frag load(const float* p) { return *p; }
   static FM_DEVICE frag splat(float x) { return x; }
+  static FM_DEVICE int tperm(int t) { return t; }
   static FM_DEVICE frag load_perm(const float* row, int s, int lh) { return row[8 * (s / 4) + 4 * lh + (s % 4)]; }
   static FM_DEVICE frag from_acc(const fm_f32x16& c, int s) { return c[s]; }
 };
