@@ -257,7 +257,6 @@ template <typename E> struct BuildArgs {
   int vb_from_r;                           // vb sums the r operand instead of p
   float coef2, coef1, coefz, coefva, coefvb;
   float coef2b, coef1b;                    // coefficients of the transposed copy
-  int dbg;
 };
 
 FM_DEVICE void fm_walk_step(int mode, int nseg, int L, int npad, int w, int& tb, int& te, int& slot) {
@@ -350,13 +349,11 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 ? 2 : 1)
   if (has_z) rz.load(A.zt + tb_off + t, A.npad, tid);
   bool have = true;
   while (have) {
-    if (!(A.dbg & 2) || t == tb) {
     FM_SYNC();
     rp.store(s0, PT, tid); rr.store(s1, PT, tid);
     if (quad) rx.store(s2, PT, tid);
     if (has_z) rz.store(s3, PT, tid);
     FM_SYNC();
-    }
     int nt = t + TT, nw = w, ntb = tb, nte = te, nslot = slot;
     const bool last = (nt >= te);
     bool has_next = true;
@@ -365,13 +362,13 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 ? 2 : 1)
       if (nw < nsteps) { fm_walk_step(A.mode, A.nseg, A.L, A.npad, nw, ntb, nte, nslot); nt = ntb; }
       else has_next = false;
     }
-    if (has_next && !(A.dbg & 1)) {
+    if (has_next) {
       rp.load(A.pt + tb_off + nt, A.npad, tid);
       rr.load(A.rt + tb_off + nt, A.npad, tid);
       if (quad) rx.load(A.xt + tb_off + int64_t(a0) * A.npad + nt, A.npad, tid);
       if (has_z) rz.load(A.zt + tb_off + nt, A.npad, tid);
     }
-    if (quad && !(A.dbg & 4)) {
+    if (quad) {
       // fragments of k-step ks+1 are fetched while the products of k-step ks are issued
       const E* pb_ = s0 + lr * PT + lh * M::KPL;
       const E* rb_ = s1 + lr * PT + lh * M::KPL;
@@ -407,7 +404,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 ? 2 : 1)
     // the lower-order tiles: this wavefront takes the k-steps ks = wave (mod 4)
 #pragma unroll
     for (int s = 0; s < SPW; ++s) {
-      if (sm_id[s] >= 0 && !(A.dbg & 8)) {
+      if (sm_id[s] >= 0) {
         for (int ks = wave; ks < NSTEP; ks += 4) {
           const frag fa = M::load(s0 + sm_a[s] + ks * M::KSTEP);
           const frag fo = sm_b[s] >= 0 ? M::load(s0 + sm_b[s] + ks * M::KSTEP) : M::splat(E(1.0f));

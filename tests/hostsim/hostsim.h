@@ -63,7 +63,7 @@ void launch(Dim3 grid, Dim3 block, size_t dyn_smem_bytes, F&& body) {
   if (nthreads % 64 != 0) { std::fprintf(stderr, "hostsim: block size must be a multiple of 64\n"); std::abort(); }
   BlockCtx blk;
   blk.waves = std::vector<WaveCtx>(nthreads / 64);
-  std::vector<unsigned char> smem(dyn_smem_bytes + 64);
+  
   for (unsigned bz = 0; bz < grid.z; ++bz)
     for (unsigned by = 0; by < grid.y; ++by)
       for (unsigned bx = 0; bx < grid.x; ++bx) {

@@ -112,9 +112,9 @@ def test_backward_ragged_and_cross(lib, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("d,bh", [(64, 32), (32, 64)])
-def test_many_heads_uses_two_states_per_wavefront(lib, dtype, d, bh):
-    # with bh*d/8 >= 256 the state build keeps two values of `a` per wavefront (the shape
-    # of the benchmark, B*H = 32 at D = 64); same parity bar
+def test_many_heads(lib, dtype, d, bh):
+    # the head count of the benchmark (B*H = 32 at D = 64): exercises the XCD-aware
+    # workgroup mapping (B*H a multiple of 8) and grids larger than the GPU
     print(f"case many heads dtype={dtype} d={d} bh={bh}", flush=True)
     check_forward_backward(lib, bh, 1100, d, dtype, DEV, mask=True, p=2, chunk=256, seed=16)
     check_forward_backward(lib, bh, 600, d, dtype, DEV, mask=False, p=2, flags=FLAG_FORCE_MOMENTS, seed=17)
