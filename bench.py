@@ -44,23 +44,28 @@ def alg_flops_unit(bh: int, n: int, d: int, p: int) -> float:
     return 2.0 * m * (d + 1) * bh * n
 
 
-def cpu_baseline(n: int, d: int, p: int, tokens_per_step: int, heads_total: int, max_n: int):
-    """Port of the reference's einops factorised path (oracle), fp32, one (b, h) slice."""
+def cpu_baseline(n: int, d: int, p: int, tokens_per_step: int, heads_total: int, max_n: int, slices: int = 4):
+    """Port of the reference's einops factorised path (oracle), fp32, a few (b, h) slices one after another."""
     import torch
     from oracle import fastmax_oracle as O
     threads = torch.get_num_threads()          # follows OMP_NUM_THREADS (the box's CPU share)
     n_run = min(n, max_n)
     gen = torch.Generator().manual_seed(1)
-    q, k, v, go = (torch.randn(1, 1, n_run, d, generator=gen) for _ in range(4))
+    slices = max(1, min(slices, heads_total))
     tau = 8.0 * math.sqrt(d)
-    t0 = time.perf_counter()
-    o, g = O.factorised_forward(q, k, v, mask=True, tau=tau, p=p)
-    dq, dk, dv = O.factorised_backward(q, k, v, o, g, go, mask=True, tau=tau, p=p)
-    dt = time.perf_counter() - t0
-    # linear-time algorithm: scale the slice to the full sequence and to all heads
-    t_step = dt * (n / n_run) * heads_total
-    sample = f"1 of {heads_total} (b,h) slices, N={n_run}" + ("" if n_run == n else f" (scaled linearly to N={n})") + \
-             f", fp32, fwd+bwd, scaled x{heads_total}; {dt:.1f} s measured"
+    dt = 0.0
+    for _ in range(slices):
+        q, k, v, go = (torch.randn(1, 1, n_run, d, generator=gen) for _ in range(4))
+        t0 = time.perf_counter()
+        o, g = O.factorised_forward(q, k, v, mask=True, tau=tau, p=p)
+        dq, dk, dv = O.factorised_backward(q, k, v, o, g, go, mask=True, tau=tau, p=p)
+        dt += time.perf_counter() - t0
+        del o, g, dq, dk, dv
+    # linear-time algorithm: scale the slices to the full sequence and to all heads
+    t_step = dt * (n / n_run) * heads_total / slices
+    sample = f"{slices} of {heads_total} (b,h) slices, N={n_run}" + \
+             ("" if n_run == n else f" (scaled linearly to N={n})") + \
+             f", fp32, fwd+bwd, scaled x{heads_total / slices:g}; {dt:.1f} s measured"
     return {"value": tokens_per_step / t_step, "unit": "tokens/s", "cores": threads, "kind": "port", "sample": sample}
 
 
@@ -71,6 +76,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f32"])
     ap.add_argument("--chunk", type=int, default=0, help="segment length of the causal moment scan (0 = library default)")
+    ap.add_argument("--independent-backward", action="store_true",
+                    help="backward rebuilds the key-side copies and states instead of taking them from the forward")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-max-n", type=int, default=2048, help="longest slice the CPU baseline materialises")
     args = ap.parse_args()
@@ -97,8 +104,13 @@ def main() -> int:
     kw = dict(mask=True, inv_tau=1.0 / tau, a0=1.0, a1=1.0, a2=0.5, p=p, chunk=args.chunk)
 
     def step():
-        o, g = lib.forward(q, k, v, **kw)
-        return lib.backward(q, k, v, o, g, go, **kw)
+        # the training step of the autograd wrapper: the forward keeps its workspace
+        # (key-side copies, prefix states) and the backward of the same step reads it
+        if args.independent_backward:
+            o, g = lib.forward(q, k, v, **kw)
+            return lib.backward(q, k, v, o, g, go, **kw)
+        o, g, saved = lib.forward(q, k, v, save=True, **kw)
+        return lib.backward(q, k, v, o, g, go, saved=saved, **kw)
 
     for _ in range(args.warmup):
         step()

@@ -34,7 +34,10 @@ enum { FASTMAX_F32 = 0, FASTMAX_BF16 = 1 };
 /* flags */
 enum {
   FASTMAX_FLAG_FORCE_MOMENTS = 1,   /* unmasked: always use the moment (linear-time) path */
-  FASTMAX_FLAG_FORCE_DENSE = 2      /* never build moment states (quadratic-time path) */
+  FASTMAX_FLAG_FORCE_DENSE = 2,     /* never build moment states (quadratic-time path) */
+  FASTMAX_FLAG_SAVE_FOR_BACKWARD = 4 /* forward: also leave in its workspace what the backward of the same
+                                        problem can reuse (converted k, v and the key-side moment states);
+                                        forward_bytes grows accordingly */
 };
 
 typedef struct FastmaxStrides {
@@ -79,6 +82,16 @@ int fastmax_backward(const FastmaxDesc* desc, const void* q, const void* k, cons
                      const void* o, const float* g, const void* d_o,
                      void* dq, void* dk, void* dv,
                      void* workspace, size_t workspace_bytes, void* hip_stream);
+
+/* Same as fastmax_backward, reusing the workspace a forward call with FASTMAX_FLAG_SAVE_FOR_BACKWARD
+ * left behind for the same desc, q, k, v (no counterpart in the reference, which recomputes
+ * everything: fastmax_cuda_backward.cu:101-188 rebuilds the running key sums).  The key-side
+ * conversions and the prefix-state build are skipped.  forward_workspace is only read. */
+int fastmax_backward_saved(const FastmaxDesc* desc, const void* q, const void* k, const void* v,
+                           const void* o, const float* g, const void* d_o,
+                           void* dq, void* dk, void* dv,
+                           const void* forward_workspace, size_t forward_workspace_bytes,
+                           void* workspace, size_t workspace_bytes, void* hip_stream);
 
 /* Fused normalisation pass over one (bh, n, d) tensor.  Replaces apply_rpe_and_temp, calc_norms,
  * find_max and apply_norm (reference fastmax_cuda_forward.cu:282-338) with the semantics the

@@ -18,7 +18,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_NAME = "libfastmax_hip.so"
 
 F32, BF16 = 0, 1
-FLAG_FORCE_MOMENTS, FLAG_FORCE_DENSE = 1, 2
+FLAG_FORCE_MOMENTS, FLAG_FORCE_DENSE, FLAG_SAVE_FOR_BACKWARD = 1, 2, 4
 STATUS_OK = 0
 
 
@@ -46,7 +46,7 @@ class NormDesc(C.Structure):
 
 
 EXPORTS = (
-    "fastmax_workspace_bytes", "fastmax_forward", "fastmax_backward", "fastmax_normalize",
+    "fastmax_workspace_bytes", "fastmax_forward", "fastmax_backward", "fastmax_backward_saved", "fastmax_normalize",
     "fastmax_status_string", "fastmax_version", "fastmax_probe_mfma",
     "fastmax_profile_begin", "fastmax_profile_end",
 )
@@ -90,6 +90,8 @@ class FastmaxLib:
         L.fastmax_forward.restype = C.c_int
         L.fastmax_backward.argtypes = [C.POINTER(Desc)] + [C.c_void_p] * 10 + [C.c_size_t, C.c_void_p]
         L.fastmax_backward.restype = C.c_int
+        L.fastmax_backward_saved.argtypes = [C.POINTER(Desc)] + [C.c_void_p] * 10 + [C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p]
+        L.fastmax_backward_saved.restype = C.c_int
         L.fastmax_normalize.argtypes = [C.POINTER(NormDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         L.fastmax_normalize.restype = C.c_int
         L.fastmax_status_string.argtypes = [C.c_int]
@@ -145,9 +147,12 @@ class FastmaxLib:
 
     # -- entry points ------------------------------------------------------------
     def forward(self, q, k, v, *, mask, inv_tau, a0=1.0, a1=1.0, a2=0.5, p=2, chunk=0, flags=0,
-                out: Optional[torch.Tensor] = None, g: Optional[torch.Tensor] = None):
+                out: Optional[torch.Tensor] = None, g: Optional[torch.Tensor] = None, save: bool = False):
         """q (bh, nq, d), k, v (bh, nk, d) views with contiguous features.
-        Returns (o, g): o like q, g (bh, nq) float32."""
+        Returns (o, g): o like q, g (bh, nq) float32; with ``save`` also the workspace
+        tensor that ``backward(..., saved=...)`` can reuse."""
+        if save:
+            flags |= FLAG_SAVE_FOR_BACKWARD
         desc = self.make_desc(q, k, v, mask=mask, inv_tau=inv_tau, a0=a0, a1=a1, a2=a2, p=p, chunk=chunk, flags=flags)
         if out is None:
             out = torch.empty((desc.bh, desc.nq, desc.d), dtype=q.dtype, device=q.device)
@@ -160,10 +165,16 @@ class FastmaxLib:
         st = self.lib.fastmax_forward(C.byref(desc), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                                       g.data_ptr(), ws.data_ptr(), fwd, self._stream(q))
         self.check(st, "fastmax_forward")
+        if save:
+            return out, g, ws
         return out, g
 
-    def backward(self, q, k, v, o, g, d_o, *, mask, inv_tau, a0=1.0, a1=1.0, a2=0.5, p=2, chunk=0, flags=0):
-        """Gradients (dq, dk, dv) of sum(o * d_o); all tensors are (bh, n, d) views."""
+    def backward(self, q, k, v, o, g, d_o, *, mask, inv_tau, a0=1.0, a1=1.0, a2=0.5, p=2, chunk=0, flags=0,
+                 saved: Optional[torch.Tensor] = None):
+        """Gradients (dq, dk, dv) of sum(o * d_o); all tensors are (bh, n, d) views.
+        ``saved``: the workspace returned by ``forward(..., save=True)`` for the same problem."""
+        if saved is not None:
+            flags |= FLAG_SAVE_FOR_BACKWARD
         desc = self.make_desc(q, k, v, mask=mask, inv_tau=inv_tau, a0=a0, a1=a1, a2=a2, p=p, chunk=chunk, flags=flags)
         if o.dtype != q.dtype or d_o.dtype != q.dtype or g.dtype != torch.float32:
             raise FastmaxError("fastmax: o and d_o must have q's dtype and g must be float32")
@@ -175,9 +186,15 @@ class FastmaxLib:
         desc.sdq, desc.sdk, desc.sdv = _strides(dq), _strides(dk), _strides(dv)
         _, bwd = self.workspace_bytes(desc)
         ws = self._workspace(bwd, q.device)
-        st = self.lib.fastmax_backward(C.byref(desc), q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
-                                       g.data_ptr(), d_o.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
-                                       ws.data_ptr(), bwd, self._stream(q))
+        if saved is not None:
+            st = self.lib.fastmax_backward_saved(C.byref(desc), q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                                 g.data_ptr(), d_o.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                                                 dv.data_ptr(), saved.data_ptr(), saved.numel(), ws.data_ptr(), bwd,
+                                                 self._stream(q))
+        else:
+            st = self.lib.fastmax_backward(C.byref(desc), q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                           g.data_ptr(), d_o.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                                           ws.data_ptr(), bwd, self._stream(q))
         self.check(st, "fastmax_backward")
         return dq, dk, dv
 

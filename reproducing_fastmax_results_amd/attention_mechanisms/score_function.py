@@ -86,16 +86,21 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
             q = _ext.normalize(q, CENTRE_NONE, True, float(lim))
             k = _ext.normalize(k, CENTRE_NONE, True, float(lim))
         inv_tau = 1.0 / float(temperature)
-        o, g = _ext.forward_ex(q, k, v, bool(mask), inv_tau, float(a0), float(a1), float(a2), int(p), 0, 0)
-        ctx.save_for_backward(q, k, v, o, g)
+        needs_grad = any(ctx.needs_input_grad[:3])
+        if needs_grad:
+            # keep the key-side copies and prefix states the forward built: the backward reuses them
+            o, g, saved = _ext.forward_save(q, k, v, bool(mask), inv_tau, float(a0), float(a1), float(a2), int(p), 0, 0)
+            ctx.save_for_backward(q, k, v, o, g, saved)
+        else:
+            o, g = _ext.forward_ex(q, k, v, bool(mask), inv_tau, float(a0), float(a1), float(a2), int(p), 0, 0)
         ctx.cfg = (bool(mask), inv_tau, float(a0), float(a1), float(a2), int(p))
         return o
 
     @staticmethod
     def backward(ctx, grad_output):
-        q, k, v, o, g = ctx.saved_tensors
+        q, k, v, o, g, saved = ctx.saved_tensors
         mask, inv_tau, a0, a1, a2, p = ctx.cfg
-        gq, gk, gv = _ext.backward_ex(q, k, v, o, g, grad_output, mask, inv_tau, a0, a1, a2, p, 0, 0)
+        gq, gk, gv = _ext.backward_saved(q, k, v, o, g, grad_output, saved, mask, inv_tau, a0, a1, a2, p, 0, 0)
         return (gq, gk, gv) + (None,) * 11
 
 

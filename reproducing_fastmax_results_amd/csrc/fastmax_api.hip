@@ -55,7 +55,8 @@ struct Plan {
   float sc;             // sqrt(1/tau), folded into q and k when they are converted
   float gscale;         // power of two folded into dO / g in the backward
   // workspace offsets (bytes)
-  size_t kt, vt, kr, big, small, fwd_bytes;
+  size_t kt, vt, kr, vr, big, big2, small, fwd_bytes;
+  bool save;
   size_t b_kr, b_vr, b_qr, b_kt, b_vt, b_qt, b_qct, b_gh, b_ght, b_cv, b_bigq, b_smallq, b_bigk, b_smallk, b_bigv, bwd_bytes;
 };
 
@@ -124,6 +125,9 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   p.kr = take(tk);
   p.big = take(size_t(d->bh) * p.nslots * bigsz);
   p.small = take(size_t(d->bh) * p.nslots * smallsz);
+  p.save = (d->flags & FASTMAX_FLAG_SAVE_FOR_BACKWARD) != 0;
+  p.vr = take(p.save ? tk : 0);
+  p.big2 = take(p.save ? size_t(d->bh) * p.nslots * bigsz : 0);
   p.fwd_bytes = off ? off : 256;
   off = 0;
   p.b_kt = take(tk); p.b_vt = take(tk); p.b_qt = take(tq); p.b_qct = take(tq);
@@ -202,7 +206,8 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   E* big = reinterpret_cast<E*>(ws + p.big);
   float* small = reinterpret_cast<float*>(ws + p.small);
   E* kr = reinterpret_cast<E*>(ws + p.kr);
-  int st = launch_transpose<TIO, E, DH>(v, d->sv, d->bh, d->nk, p.npad_k, vt, static_cast<E*>(nullptr), 1.0f, stream);
+  E* vr = p.save ? reinterpret_cast<E*>(ws + p.vr) : nullptr;
+  int st = launch_transpose<TIO, E, DH>(v, d->sv, d->bh, d->nk, p.npad_k, vt, vr, 1.0f, stream);
   if (st) return st;
   st = launch_transpose<TIO, E, DH>(k, d->sk, d->bh, d->nk, p.npad_k, kt, kr, p.sc, stream);
   if (st) return st;
@@ -211,7 +216,9 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
     b.xt = kt; b.pt = vt; b.rt = kt; b.zt = nullptr; b.za_sel = FM_SRC_R; b.zb_sel = FM_SRC_R;
     b.npad = p.npad_k; b.nseg = p.nseg; b.L = p.L; b.mode = d->mask ? FM_WALK_PREFIX : FM_WALK_TOTAL;
     b.quad = p.quad; b.big = big; b.small = small; b.nslots = p.nslots;
-    b.big2 = nullptr; b.vb_from_r = 0; b.coef2b = 0.0f; b.coef1b = 0.0f;
+    // saved for the backward: the transposed tiles are the (k, k, v) state that dQ reads
+    b.big2 = p.save ? reinterpret_cast<E*>(ws + p.big2) : nullptr;
+    b.vb_from_r = 0; b.coef2b = 2.0f * p.a2; b.coef1b = p.a1;
     b.coef2 = p.a2; b.coef1 = p.a1; b.coefz = p.a2; b.coefva = p.a1; b.coefvb = p.a0;
     st = launch_build<E, DH>(b, d->bh, stream);
     if (st) return st;
@@ -285,9 +292,9 @@ int fastmax_forward(const FastmaxDesc* desc, const void* q, const void* k, const
   return run_forward<float, float, 32, 1>(desc, p, q, k, v, o, g, ws, stream);
 }
 
-int fastmax_backward(const FastmaxDesc* desc, const void* q, const void* k, const void* v, const void* o,
-                     const float* g, const void* d_o, void* dq, void* dk, void* dv, void* workspace,
-                     size_t workspace_bytes, void* hip_stream) {
+static int backward_impl(const FastmaxDesc* desc, const void* q, const void* k, const void* v, const void* o,
+                         const float* g, const void* d_o, void* dq, void* dk, void* dv, const void* fwd_ws,
+                         size_t fwd_ws_bytes, void* workspace, size_t workspace_bytes, void* hip_stream) {
   Plan p;
   int st = make_plan(desc, p);
   if (st) return st;
@@ -300,14 +307,34 @@ int fastmax_backward(const FastmaxDesc* desc, const void* q, const void* k, cons
     return FASTMAX_ERR_SHAPE;
   if (!workspace || workspace_bytes < p.bwd_bytes || reinterpret_cast<uintptr_t>(workspace) % 256)
     return FASTMAX_ERR_WORKSPACE;
+  if (fwd_ws) {
+    if (!p.save) return FASTMAX_ERR_SHAPE;          // desc must carry the flag the forward was run with
+    if (fwd_ws_bytes < p.fwd_bytes || reinterpret_cast<uintptr_t>(fwd_ws) % 256) return FASTMAX_ERR_WORKSPACE;
+  }
   char* ws = static_cast<char*>(workspace);
+  const char* fws = static_cast<const char*>(fwd_ws);
   fm_stream_t stream = static_cast<fm_stream_t>(hip_stream);
   if (p.half) {
-    if (desc->d == 64) return run_backward<fm_bf16, fm_half, 64, 2>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, ws, stream);
-    return run_backward<fm_bf16, fm_half, 32, 2>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, ws, stream);
+    if (desc->d == 64) return run_backward<fm_bf16, fm_half, 64, 2>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);
+    return run_backward<fm_bf16, fm_half, 32, 2>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);
   }
-  if (desc->d == 64) return run_backward<float, float, 64, 1>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, ws, stream);
-  return run_backward<float, float, 32, 1>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, ws, stream);
+  if (desc->d == 64) return run_backward<float, float, 64, 1>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);
+  return run_backward<float, float, 32, 1>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);
+}
+
+int fastmax_backward(const FastmaxDesc* desc, const void* q, const void* k, const void* v, const void* o,
+                     const float* g, const void* d_o, void* dq, void* dk, void* dv, void* workspace,
+                     size_t workspace_bytes, void* hip_stream) {
+  return backward_impl(desc, q, k, v, o, g, d_o, dq, dk, dv, nullptr, 0, workspace, workspace_bytes, hip_stream);
+}
+
+int fastmax_backward_saved(const FastmaxDesc* desc, const void* q, const void* k, const void* v, const void* o,
+                           const float* g, const void* d_o, void* dq, void* dk, void* dv,
+                           const void* forward_workspace, size_t forward_workspace_bytes, void* workspace,
+                           size_t workspace_bytes, void* hip_stream) {
+  if (!forward_workspace) return FASTMAX_ERR_NULL;
+  return backward_impl(desc, q, k, v, o, g, d_o, dq, dk, dv, forward_workspace, forward_workspace_bytes, workspace,
+                       workspace_bytes, hip_stream);
 }
 
 int fastmax_normalize(const FastmaxNormDesc* desc, const void* x, void* y, float* stats, void* hip_stream) {

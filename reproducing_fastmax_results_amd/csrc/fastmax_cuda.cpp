@@ -186,9 +186,8 @@ FastmaxDesc ex_desc(const torch::Tensor& q, const torch::Tensor& k, const torch:
   return d;
 }
 
-std::tuple<torch::Tensor, torch::Tensor> forward_ex(torch::Tensor q_, torch::Tensor k_, torch::Tensor v_, bool mask,
-                                                    double inv_tau, double a0, double a1, double a2, int64_t p,
-                                                    int64_t chunk, int64_t flags) {
+std::vector<torch::Tensor> forward_any(torch::Tensor q_, torch::Tensor k_, torch::Tensor v_, bool mask, double inv_tau,
+                                       double a0, double a1, double a2, int64_t p, int64_t chunk, int64_t flags) {
   torch::Tensor q = as_bhnd(q_, "q"), k = as_bhnd(k_, "k"), v = as_bhnd(v_, "v");
   FastmaxDesc d = ex_desc(q, k, v, mask, inv_tau, a0, a1, a2, p, chunk, flags);
   torch::Tensor o = torch::empty({d.bh, d.nq, d.d}, q.options());
@@ -200,13 +199,31 @@ std::tuple<torch::Tensor, torch::Tensor> forward_ex(torch::Tensor q_, torch::Ten
   torch::Tensor ws = workspace(fwd, q);
   check_status(fastmax_forward(&d, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), g.data_ptr<float>(),
                                ws.data_ptr(), fwd, stream_of(q)), "fastmax_forward");
-  if (q_.dim() == 4) return {o.view({q_.size(0), q_.size(1), d.nq, d.d}), g.view({q_.size(0), q_.size(1), d.nq})};
-  return {o, g};
+  if (q_.dim() == 4) return {o.view({q_.size(0), q_.size(1), d.nq, d.d}), g.view({q_.size(0), q_.size(1), d.nq}), ws};
+  return {o, g, ws};
 }
 
-std::vector<torch::Tensor> backward_ex(torch::Tensor q_, torch::Tensor k_, torch::Tensor v_, torch::Tensor o_,
-                                       torch::Tensor g_, torch::Tensor go_, bool mask, double inv_tau, double a0,
-                                       double a1, double a2, int64_t p, int64_t chunk, int64_t flags) {
+std::tuple<torch::Tensor, torch::Tensor> forward_ex(torch::Tensor q, torch::Tensor k, torch::Tensor v, bool mask,
+                                                    double inv_tau, double a0, double a1, double a2, int64_t p,
+                                                    int64_t chunk, int64_t flags) {
+  std::vector<torch::Tensor> r = forward_any(q, k, v, mask, inv_tau, a0, a1, a2, p, chunk,
+                                             flags & ~int64_t(FASTMAX_FLAG_SAVE_FOR_BACKWARD));
+  return {r[0], r[1]};
+}
+
+// Forward that keeps its workspace (key-side copies and prefix states) for backward_saved.
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> forward_save(torch::Tensor q, torch::Tensor k, torch::Tensor v,
+                                                                   bool mask, double inv_tau, double a0, double a1,
+                                                                   double a2, int64_t p, int64_t chunk, int64_t flags) {
+  std::vector<torch::Tensor> r = forward_any(q, k, v, mask, inv_tau, a0, a1, a2, p, chunk,
+                                             flags | FASTMAX_FLAG_SAVE_FOR_BACKWARD);
+  return {r[0], r[1], r[2]};
+}
+
+std::vector<torch::Tensor> backward_any(torch::Tensor q_, torch::Tensor k_, torch::Tensor v_, torch::Tensor o_,
+                                        torch::Tensor g_, torch::Tensor go_, const torch::Tensor* saved, bool mask,
+                                        double inv_tau, double a0, double a1, double a2, int64_t p, int64_t chunk,
+                                        int64_t flags) {
   torch::Tensor q = as_bhnd(q_, "q"), k = as_bhnd(k_, "k"), v = as_bhnd(v_, "v");
   torch::Tensor o = as_bhnd(o_, "o"), go = as_bhnd(go_, "grad_output");
   FastmaxDesc d = ex_desc(q, k, v, mask, inv_tau, a0, a1, a2, p, chunk, flags);
@@ -222,14 +239,39 @@ std::vector<torch::Tensor> backward_ex(torch::Tensor q_, torch::Tensor k_, torch
   size_t fwd = 0, bwd = 0;
   check_status(fastmax_workspace_bytes(&d, &fwd, &bwd), "fastmax_workspace_bytes");
   torch::Tensor ws = workspace(bwd, q);
-  check_status(fastmax_backward(&d, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), g.data_ptr<float>(),
-                                go.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), bwd,
-                                stream_of(q)), "fastmax_backward");
+  if (saved) {
+    TORCH_CHECK(saved->is_cuda() && saved->scalar_type() == torch::kUInt8 && saved->is_contiguous(),
+                "saved workspace must be the uint8 tensor returned by forward_save");
+    check_status(fastmax_backward_saved(&d, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), g.data_ptr<float>(),
+                                        go.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), saved->data_ptr(),
+                                        size_t(saved->numel()), ws.data_ptr(), bwd, stream_of(q)),
+                 "fastmax_backward_saved");
+  } else {
+    check_status(fastmax_backward(&d, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), g.data_ptr<float>(),
+                                  go.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), bwd,
+                                  stream_of(q)), "fastmax_backward");
+  }
   if (q_.dim() == 4) {
     const int64_t b = q_.size(0), h = q_.size(1);
     return {dq.view({b, h, d.nq, d.d}), dk.view({b, h, d.nk, d.d}), dv.view({b, h, d.nk, d.d})};
   }
   return {dq, dk, dv};
+}
+
+std::vector<torch::Tensor> backward_ex(torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor o,
+                                       torch::Tensor g, torch::Tensor go, bool mask, double inv_tau, double a0,
+                                       double a1, double a2, int64_t p, int64_t chunk, int64_t flags) {
+  return backward_any(q, k, v, o, g, go, nullptr, mask, inv_tau, a0, a1, a2, p, chunk,
+                      flags & ~int64_t(FASTMAX_FLAG_SAVE_FOR_BACKWARD));
+}
+
+// Backward on the workspace forward_save returned for the same q, k, v and parameters.
+std::vector<torch::Tensor> backward_saved(torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor o,
+                                          torch::Tensor g, torch::Tensor go, torch::Tensor saved, bool mask,
+                                          double inv_tau, double a0, double a1, double a2, int64_t p, int64_t chunk,
+                                          int64_t flags) {
+  return backward_any(q, k, v, o, g, go, &saved, mask, inv_tau, a0, a1, a2, p, chunk,
+                      flags | FASTMAX_FLAG_SAVE_FOR_BACKWARD);
 }
 
 // y = scale * (x - centre) / max_n ||x_n - centre||  (see fastmax_normalize in the C header)
@@ -255,6 +297,8 @@ PYBIND11_MODULE(fastmax_cuda, m) {
   m.def("backwardpass", &backwardpass, "backwardpass");
   m.def("forward_ex", &forward_ex, "strided forward: returns (o, g)");
   m.def("backward_ex", &backward_ex, "strided backward: returns [dq, dk, dv]");
+  m.def("forward_save", &forward_save, "strided forward keeping its workspace: returns (o, g, saved)");
+  m.def("backward_saved", &backward_saved, "strided backward on a saved forward workspace: returns [dq, dk, dv]");
   m.def("normalize", &normalize, "fused normalisation pass");
   m.def("version", []() { return fastmax_version(); });
 }

@@ -25,14 +25,15 @@ template <typename TIO, typename E> struct BwdArgs {
   float a0, a1, a2;
   float sc;                                // sqrt(1/tau): q and k are used as sc*q, sc*k
   float gscale;                            // power of two folded into gh and c by k_prep_bwd
+  float zscale_q;                          // factor on the Z of the (k, k, v) state (2 when the forward's state is reused)
 };
 
 // Z (fp32, [DH][DH]) -> LDS in the compute type (hi/lo split for _Float16), va/vb -> vecs.
 template <typename E, int DH, int QT>
-FM_DEVICE void fm_stage_small(const float* sml, E* Zs, float* vecs, int tid) {
+FM_DEVICE void fm_stage_small(const float* sml, E* Zs, float* vecs, int tid, float zscale = 1.0f) {
   typedef TokCfg<E, DH, QT> C;
   for (int i = tid; i < DH * DH; i += FM_THREADS) {
-    const float z = sml[i];
+    const float z = sml[i] * zscale;
     const int r = i / DH, c = i % DH;
     const E hi = CE<E>::from(z);
     Zs[r * C::PS + c] = hi;
@@ -124,7 +125,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_dq(BwdArgs<TIO, E> A) {
     rg.store(Gs, PQ, tid);
   }
   if (use_state)
-    fm_stage_small<E, DH, QT>(A.smallq + (int64_t(bh) * A.nslots + slot) * StateDims<DH>::SMALL, R, vecs, tid);
+    fm_stage_small<E, DH, QT>(A.smallq + (int64_t(bh) * A.nslots + slot) * StateDims<DH>::SMALL, R, vecs, tid, A.zscale_q);
   FM_SYNC();
 
   int tw[QT], xrow[QT];

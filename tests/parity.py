@@ -48,13 +48,19 @@ def check_forward(lib, bh, nq, d, dtype, device, *, mask, p, nk=None, chunk=0, f
 
 
 def check_forward_backward(lib, bh, nq, d, dtype, device, *, mask, p, nk=None, chunk=0, flags=0, tau_mult=8.0,
-                           a=(1.0, 1.0, 0.5), seed=0, scale=1.0):
+                           a=(1.0, 1.0, 0.5), seed=0, scale=1.0, saved=False):
+    """saved: run the backward on the workspace the forward leaves behind
+    (FASTMAX_FLAG_SAVE_FOR_BACKWARD / fastmax_backward_saved)."""
     nk = nk or nq
     q, k, v, go = make_inputs(bh, nq, nk, d, dtype, device, seed, scale)
     tau = tau_mult * math.sqrt(d)
     kw = dict(mask=mask, inv_tau=1.0 / tau, a0=a[0], a1=a[1], a2=a[2], p=p, chunk=chunk, flags=flags)
-    o, g = lib.forward(q, k, v, **kw)
-    dq, dk, dv = lib.backward(q, k, v, o, g, go, **kw)
+    if saved:
+        o, g, ws = lib.forward(q, k, v, save=True, **kw)
+        dq, dk, dv = lib.backward(q, k, v, o, g, go, saved=ws, **kw)
+    else:
+        o, g = lib.forward(q, k, v, **kw)
+        dq, dk, dv = lib.backward(q, k, v, o, g, go, **kw)
     ref = oracle_all(q, k, v, go, mask=mask, tau=tau, p=p, a=a)
     errs = {n: rel_err(x, r) for n, x, r in zip(("o", "g", "dq", "dk", "dv"), (o, g, dq, dk, dv), ref)}
     for n, e in errs.items():

@@ -118,3 +118,15 @@ def test_many_heads(lib, dtype, d, bh):
     print(f"case many heads dtype={dtype} d={d} bh={bh}", flush=True)
     check_forward_backward(lib, bh, 1100, d, dtype, DEV, mask=True, p=2, chunk=256, seed=16)
     check_forward_backward(lib, bh, 600, d, dtype, DEV, mask=False, p=2, flags=FLAG_FORCE_MOMENTS, seed=17)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mask", [False, True])
+@pytest.mark.parametrize("p", [1, 2])
+def test_backward_on_saved_forward_workspace(lib, dtype, mask, p):
+    # fastmax_backward_saved: key-side copies and the prefix state come from the forward
+    print(f"case saved dtype={dtype} mask={mask} p={p}", flush=True)
+    check_forward_backward(lib, 8, 1100, 64, dtype, DEV, mask=mask, p=p, chunk=256, flags=FLAG_FORCE_MOMENTS,
+                           seed=18, saved=True)
+    check_forward_backward(lib, 3, 333, 32, dtype, DEV, mask=mask, p=p, flags=FLAG_FORCE_DENSE, seed=19, saved=True)
+    check_forward_backward(lib, 2, 2500, 64, dtype, DEV, mask=mask, p=p, seed=20, saved=True)

@@ -51,6 +51,7 @@ def test_dense_forward_backward(sim, dtype):
 def test_moment_path_forward_backward_bf16(sim):
     # two segments of 256: prefix state for the second, suffix state for the first
     check_forward_backward(sim, 1, 300, 32, torch.bfloat16, "cpu", mask=True, p=2, chunk=256, seed=3)
+    check_forward_backward(sim, 1, 300, 32, torch.bfloat16, "cpu", mask=True, p=2, chunk=256, seed=3, saved=True)
     check_forward_backward(sim, 1, 40, 32, torch.bfloat16, "cpu", mask=False, p=2, nk=260,
                            flags=_capi.FLAG_FORCE_MOMENTS, seed=4)
 
