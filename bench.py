@@ -36,7 +36,7 @@ PEAK_HBM_GBS = 8000.0
 WORKLOAD = dict(name="configs[1]: causal order-2 fwd+bwd", B=4, H=8, N=4096, D=64, p=2, mask=True)
 
 # units of algorithmic work (each 2*M_p*(Dv+1) flop per (b, h, token)) per launch of each kernel
-UNITS = {"build": 1, "fwd": 1, "dq": 1, "dkv": 2}
+UNITS = {"build": 1, "fwd": 1, "dq": 1, "dk": 1, "dv": 1}
 
 
 def alg_flops_unit(bh: int, n: int, d: int, p: int) -> float:

@@ -212,7 +212,7 @@ class FastmaxLib:
         self.check(st, "fastmax_normalize")
         return out
 
-    KERNEL_NAMES = ("transpose", "prep_bwd", "build", "fwd", "dq", "dkv", "normalize")
+    KERNEL_NAMES = ("transpose", "prep_bwd", "build", "fwd", "dq", "dk", "normalize", "dv")
 
     def profile_begin(self) -> None:
         self.lib.fastmax_profile_begin()

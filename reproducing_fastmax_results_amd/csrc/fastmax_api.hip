@@ -2,7 +2,7 @@
 // launch sequences.  See include/fastmax_hip.h for the contract of each entry.
 #include "fastmax_hip.h"
 #include "fm_kernels.h"
-#include "fm_kernels_bwd.h"
+#include "fm_tok.h"
 #include "fm_norm.h"
 #include <cmath>
 #include <vector>
@@ -21,7 +21,7 @@ inline void fm_allow_lds(const void* fn, size_t bytes) {
 #endif
 
 // ---- optional per-kernel timing (used by the benchmark; not re-entrant) --------
-enum { FM_K_TRANSPOSE = 0, FM_K_PREP_BWD = 1, FM_K_BUILD = 2, FM_K_FWD = 3, FM_K_DQ = 4, FM_K_DKV = 5, FM_K_NORM = 6 };
+enum { FM_K_TRANSPOSE = 0, FM_K_PREP_BWD = 1, FM_K_BUILD = 2, FM_K_FWD = 3, FM_K_DQ = 4, FM_K_DK = 5, FM_K_NORM = 6, FM_K_DV = 7 };
 #if defined(FM_HOSTSIM)
 struct ProfScope { ProfScope(int, fm_stream_t) {} };
 #else
@@ -188,14 +188,51 @@ int launch_build(const BuildArgs<E>& a, int bh, fm_stream_t stream) {
   return launch_build_cfg<E, DH, 1, 64>(a, bh, stream);
 }
 
-template <typename E, int DH, int QT> size_t tok_lds_bytes(int extra_floats) {
+// Dynamic LDS of k_pv and k_ds (one size for both): va, vb | own rows | region, where the
+// dense stages of k_ds and the output staging lie over the own rows and the region.
+template <typename E, int DH, int QT> size_t tok_lds_bytes() {
   typedef TokCfg<E, DH, QT> C;
   size_t region = size_t(2) * C::SLAB * sizeof(E);
-  const size_t dense = size_t(2) * (C::KT * C::PQ + DH * C::PV) * sizeof(E);
-  const size_t outst = size_t(C::QW) * (DH + 1) * 4;
+  const size_t dense = size_t(2) * C::PV_STAGE * sizeof(E);
+  const size_t zs = size_t(C::NZ) * DH * C::PS * sizeof(E);
   if (dense > region) region = dense;
-  if (outst > region) region = outst;
-  return size_t(C::QW) * C::PQ * sizeof(E) + size_t(C::NZ) * DH * C::PS * sizeof(E) + size_t(2 * DH + extra_floats) * 4 + region;
+  if (zs > region) region = zs;
+  size_t body = size_t(C::QW) * C::PQ * sizeof(E) + region;
+  const size_t outst = size_t(C::QW) * (DH + 1) * 4;
+  const size_t ds = size_t(C::DS_NBUF) * C::DS_STAGE * sizeof(E);
+  if (outst > body) body = outst;
+  if (ds > body) body = ds;
+  return size_t(2 * DH) * 4 + body;
+}
+
+template <typename TIO, typename E> void tok_common(TokArgs<TIO, E>& a, const FastmaxDesc* d, const Plan& p) {
+  a.own_io = TRef<const TIO>{nullptr, 0, 0, 0};
+  a.own_r = nullptr; a.own2_r = nullptr; a.cv = nullptr; a.xr = nullptr; a.yr = nullptr; a.zt = nullptr;
+  a.g = nullptr; a.g_s_bh = 0; a.g_s_n = 0;
+  a.nslots = p.nslots; a.L = p.L; a.nseg = p.nseg; a.causal = d->mask != 0; a.use_state = p.use_state;
+  a.quad = p.quad; a.a0 = p.a0; a.a1 = p.a1; a.a2 = p.a2; a.sc = p.sc; a.out_scale = 1.0f; a.zscale = 1.0f;
+}
+
+template <typename TIO, typename E, int DH, int QT, int OWN>
+int launch_pv(const TokArgs<TIO, E>& a, int bh, int kernel_id, fm_stream_t stream) {
+  typedef TokCfg<E, DH, QT> C;
+  const size_t lds = tok_lds_bytes<E, DH, QT>();
+  fm_allow_lds(reinterpret_cast<const void*>(&k_pv<TIO, E, DH, QT, OWN>), lds);
+  ProfScope prof(kernel_id, stream);
+  FM_KERNEL_LAUNCH((k_pv<TIO, E, DH, QT, OWN>), fm_dim3((a.n_own + C::QW - 1) / C::QW, bh), fm_dim3(FM_THREADS), lds,
+                   stream, a);
+  return fm_after_launch();
+}
+
+template <typename TIO, typename E, int DH, int QT, int OWN>
+int launch_ds(const TokArgs<TIO, E>& a, int bh, int kernel_id, fm_stream_t stream) {
+  typedef TokCfg<E, DH, QT> C;
+  const size_t lds = tok_lds_bytes<E, DH, QT>();
+  fm_allow_lds(reinterpret_cast<const void*>(&k_ds<TIO, E, DH, QT, OWN>), lds);
+  ProfScope prof(kernel_id, stream);
+  FM_KERNEL_LAUNCH((k_ds<TIO, E, DH, QT, OWN>), fm_dim3((a.n_own + C::QW - 1) / C::QW, bh), fm_dim3(FM_THREADS), lds,
+                   stream, a);
+  return fm_after_launch();
 }
 
 template <typename TIO, typename E, int DH, int QT>
@@ -223,21 +260,15 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
     st = launch_build<E, DH>(b, d->bh, stream);
     if (st) return st;
   }
-  FwdArgs<TIO, E> a;
-  a.q = cref<TIO>(q, d->sq); a.k = cref<TIO>(k, d->sk); a.v = cref<TIO>(v, d->sv);
-  a.o = mref<TIO>(o, d->so);
+  TokArgs<TIO, E> a;
+  tok_common(a, d, p);
+  a.own_io = cref<TIO>(q, d->sq);
+  a.xr = kr; a.zt = vt; a.npad_own = p.npad_q; a.npad_str = p.npad_k;
+  a.big = big; a.small = small;
+  a.out = mref<TIO>(o, d->so);
   a.g = g; a.g_s_bh = d->sg.bh; a.g_s_n = d->sg.n;
-  a.vt = vt; a.kr = kr; a.npad_k = p.npad_k;
-  a.big = big; a.small = small; a.nslots = p.nslots;
-  a.nq = d->nq; a.nk = d->nk; a.L = p.L; a.causal = d->mask != 0; a.use_state = p.use_state; a.quad = p.quad;
-  a.a0 = p.a0; a.a1 = p.a1; a.a2 = p.a2; a.sc = p.sc;
-  typedef TokCfg<E, DH, QT> C;
-  const size_t lds = tok_lds_bytes<E, DH, QT>(0);
-  fm_allow_lds(reinterpret_cast<const void*>(&k_fwd<TIO, E, DH, QT>), lds);
-  ProfScope prof(FM_K_FWD, stream);
-  FM_KERNEL_LAUNCH((k_fwd<TIO, E, DH, QT>), fm_dim3((d->nq + C::QW - 1) / C::QW, d->bh), fm_dim3(FM_THREADS), lds,
-                   stream, a);
-  return fm_after_launch();
+  a.n_own = d->nq; a.n_str = d->nk;
+  return launch_pv<TIO, E, DH, QT, FM_OWN_Q>(a, d->bh, FM_K_FWD, stream);
 }
 
 }  // namespace

@@ -51,13 +51,16 @@ struct TileRegs {
   static constexpr int N = (TOTAL + FM_THREADS - 1) / FM_THREADS;
   fm_u32x4 r[N];
   // src points at (row 0, first token of the tile); rows are row_stride apart
-  FM_DEVICE void load(const E* src, int64_t row_stride, int tid) {
+  // (src is the same in every lane; the per-lane part is an unsigned 32-bit element offset, so
+  // the address is a scalar base plus a vector offset and no 64-bit pointer is kept per lane)
+  FM_DEVICE void load(const E* src, int row_stride, int tid) {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
       const int c = tid + FM_THREADS * i;
       if (TOTAL % FM_THREADS == 0 || c < TOTAL) {
-        const int row = c / CPR, col = (c % CPR) * VEC;
-        r[i] = *reinterpret_cast<const fm_u32x4*>(src + row * row_stride + col);
+        const uint32_t row = uint32_t(c / CPR), col = uint32_t((c % CPR) * VEC);
+        const uint32_t off = row * uint32_t(row_stride) + col;
+        r[i] = *reinterpret_cast<const fm_u32x4*>(src + off);
       }
     }
   }
@@ -508,11 +511,15 @@ struct TokCfg {
   static constexpr int QW = 4 * QT * 32;            // tokens per workgroup
   static constexpr int PQ = DH + M::PAD;            // pitch of row-major token tiles
   static constexpr int PS = DH + M::PAD;            // pitch of state rows
-  static constexpr int SA = sizeof(E) == 2 ? 4 : 2; // values of a per state slab
+  static constexpr int OCC = sizeof(E) == 2 ? 2 : 1;   // workgroups per CU the kernels are sized for
+  static constexpr int SA = 2;                      // values of a per state slab
   static constexpr int KT = 64;                     // tokens per stage of the dense loop
   static constexpr int PV = KT + M::PAD;            // pitch of transposed token tiles
   static constexpr int NZ = sizeof(E) == 2 ? 2 : 1; // hi/lo split of fp32 denominators
   static constexpr int SLAB = SA * DH * PS;         // elements per slab buffer
+  static constexpr int PV_STAGE = KT * PQ + DH * PV;            // k_pv: stream rows, stream transposed
+  static constexpr int DS_STAGE = 2 * KT * PQ + DH * PV + KT;   // k_ds: two row tiles, transposed tile, c values
+  static constexpr int DS_NBUF = sizeof(E) == 2 ? 2 : 1;
 };
 
 // Moment readout, transposed:  acc[j][ct] (rows c, column = token of tile j) +=
@@ -571,219 +578,6 @@ FM_DEVICE void fm_readout(const E* FM_RESTRICT state, bool quad, const E* xs, co
     buf ^= 1;
   }
   FM_SYNC();
-}
-
-// ------------------------------------------------------------------------------
-// k_fwd: forward for one block of QW queries of one batch*head.
-//   [F_i, g_i] = (prefix or global moment readout) + (dense tiles over the keys
-//   kbeg .. kend of the query's own segment, causal on the diagonal);  o = F / g.
-// q and k arrive multiplied by sqrt(1/tau) each, so the score is their plain dot
-// product.  grid (ceil(nq / QW), bh).  Replaces calc_masked / calc_unmasked
-// (fastmax_cuda_forward.cu:23-280).
-// ------------------------------------------------------------------------------
-template <typename TIO, typename E> struct FwdArgs {
-  TRef<const TIO> q, k, v;
-  TRef<TIO> o;
-  float* g; int64_t g_s_bh, g_s_n;
-  const E* vt; const E* kr; int npad_k; // V transposed [bh][DH][npad_k], K row-major [bh][npad_k][DH] (scaled)
-  const E* big; const float* small; int nslots;
-  int nq, nk, L, causal, use_state, quad;
-  float a0, a1, a2;                    // f(s) = a0 + a1 s + a2 s^2
-  float sc;                            // sqrt(1/tau), applied to q and k on load
-};
-
-template <typename TIO, typename E, int DH, int QT>
-FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_fwd(FwdArgs<TIO, E> A) {
-  typedef TokCfg<E, DH, QT> C;
-  typedef Mma<E> M;
-  typedef TileMath<E> TM;
-  typedef typename M::frag frag;
-  constexpr int NT = C::NT, NKS = C::NKS, QW = C::QW, PQ = C::PQ, PS = C::PS, KT = C::KT, PV = C::PV;
-  constexpr int STAGE = KT * PQ + DH * PV;            // K rows, V transposed
-  FM_DYN_SMEM(smem);
-  E* Qs = reinterpret_cast<E*>(smem);                 // [QW][PQ]
-  E* Zs = Qs + QW * PQ;                               // [NZ][DH][PS]
-  float* vecs = reinterpret_cast<float*>(Zs + C::NZ * DH * PS);   // va[DH], vb[DH]
-  E* R = reinterpret_cast<E*>(vecs + 2 * DH);         // slabs | dense-loop tiles | output staging
-  const int tid = FM_TID_X, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
-  const int wave = FM_UNIFORM(tid >> 6);
-  const int nqb = FM_GDIM_X;
-  int unit, bh;
-  fm_xcd_map(nqb, FM_GDIM_Y, unit, bh);
-  const int qb = A.causal ? (nqb - 1 - unit) : unit;            // heavy blocks first
-  const int q0 = qb * QW;
-  const int seg = A.causal ? q0 / A.L : 0;
-  const bool use_state = A.use_state && (!A.causal || seg > 0);
-  const int slot = A.causal ? seg : 0;
-  const int kbeg = A.causal ? seg * A.L : 0;
-  const int kend = A.causal ? (q0 + QW < A.nk ? q0 + QW : A.nk) : (A.use_state ? 0 : A.nk);
-  const float cnt = A.causal ? float(kbeg) : float(A.nk);       // keys covered by the state
-
-  // ---- stage Q (and the denominator states) ----
-  {
-    RowRegs<TIO, E, QW, DH> rq;
-    rq.load(A.q.p + int64_t(bh) * A.q.s_bh, A.q.s_n, A.q.vec != 0, q0, A.nq, tid);
-    rq.store(Qs, PQ, tid, A.sc);
-  }
-  const float* sml = A.small + (int64_t(bh) * A.nslots + slot) * StateDims<DH>::SMALL;
-  if (use_state) {
-    for (int i = tid; i < DH * DH; i += FM_THREADS) {
-      const float z = sml[i];
-      const int r = i / DH, c = i % DH;
-      const E hi = CE<E>::from(z);
-      Zs[r * PS + c] = hi;
-      if (C::NZ == 2) Zs[DH * PS + r * PS + c] = CE<E>::from(z - float(hi));
-    }
-    if (tid < 2 * DH) vecs[tid] = sml[DH * DH + tid];
-  }
-  FM_SYNC();
-
-  int tw[QT], xrow[QT];
-#pragma unroll
-  for (int j = 0; j < QT; ++j) {
-    tw[j] = (j == 0) ? wave : (4 * QT - 1 - wave);   // pair a short and a long causal tile
-    xrow[j] = tw[j] * 32 + lr;
-  }
-  frag qf[QT][NKS];
-#pragma unroll
-  for (int j = 0; j < QT; ++j)
-#pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) qf[j][ks] = M::load(Qs + xrow[j] * PQ + ks * M::KSTEP + lh * M::KPL);
-
-  fm_f32x16 acc[QT][NT];
-#pragma unroll
-  for (int j = 0; j < QT; ++j)
-#pragma unroll
-    for (int ct = 0; ct < NT; ++ct) acc[j][ct] = fm_zero16();
-  float gsum[QT];
-#pragma unroll
-  for (int j = 0; j < QT; ++j) gsum[j] = 0.f;
-
-  if (use_state) {
-    // denominator: g_i += sum_m q_im (va[m] + sum_l Z[m][l] q_il)
-#pragma unroll
-    for (int j = 0; j < QT; ++j) {
-#pragma unroll
-      for (int mt = 0; mt < NT; ++mt) {
-        fm_f32x16 y = fm_zero16();
-#pragma unroll
-        for (int z = 0; z < C::NZ; ++z)
-#pragma unroll
-          for (int ks = 0; ks < NKS; ++ks)
-            y = M::mma(M::load(Zs + z * DH * PS + (32 * mt + lr) * PS + ks * M::KSTEP + lh * M::KPL),
-                       qf[j][ks], y);
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int m = 32 * mt + fm_acc_row(e, lh);
-          gsum[j] += (y[e] + vecs[m]) * float(Qs[xrow[j] * PQ + m]);
-        }
-      }
-    }
-    const E* state = A.big + (int64_t(bh) * A.nslots + slot) * StateDims<DH>::BIG;
-    fm_readout<E, DH, QT, NT>(state, A.quad != 0, Qs, xrow, qf, R, acc, tid);
-  }
-
-  // ---- dense tiles over the keys of this segment ----
-  if (kend > kbeg) {
-    const typename TM::Coef coef = TM::coef(A.a0, A.a1, A.a2);
-    TileRegs<E, KT, DH> rk;
-    TileRegs<E, DH, KT> rv;
-    const E* kb = A.kr + int64_t(bh) * A.npad_k * DH;
-    const E* vtb = A.vt + int64_t(bh) * DH * A.npad_k;
-    rk.load(kb + int64_t(kbeg) * DH, DH, tid);
-    rv.load(vtb + kbeg, A.npad_k, tid);
-    int buf = 0;
-    for (int kt0 = kbeg; kt0 < kend; kt0 += KT) {
-      E* Ks = R + buf * STAGE;
-      E* Vs = Ks + KT * PQ;
-      rk.store(Ks, PQ, tid);
-      rv.store(Vs, PV, tid);
-      FM_SYNC();
-      if (kt0 + KT < kend) {
-        rk.load(kb + int64_t(kt0 + KT) * DH, DH, tid);
-        rv.load(vtb + kt0 + KT, A.npad_k, tid);
-      }
-      // work items (sub-tile st, query tile j); the score tile of the next item is issued
-      // before the polynomial of the current one so that VALU and MFMA overlap
-      constexpr int NI = (KT / 32) * QT;
-      bool act[NI];
-#pragma unroll
-      for (int it = 0; it < NI; ++it) {
-        const int key0 = kt0 + 32 * (it / QT), qlo = q0 + tw[it % QT] * 32;
-        act[it] = key0 < kend && !(A.causal && key0 > qlo + 31);
-      }
-      fm_f32x16 s_cur;
-      if (act[0]) {
-        s_cur = fm_zero16();
-#pragma unroll
-        for (int ks = 0; ks < NKS; ++ks)
-          s_cur = M::mma(M::load(Ks + lr * PQ + ks * M::KSTEP + lh * M::KPL), qf[0][ks], s_cur);
-      }
-#pragma unroll
-      for (int it = 0; it < NI; ++it) {
-        const int st = it / QT, j = it % QT;
-        fm_f32x16 s_nxt;
-        if (it + 1 < NI && act[(it + 1 < NI) ? it + 1 : it]) {
-          s_nxt = fm_zero16();
-          const int st2 = (it + 1) / QT, j2 = (it + 1) % QT;
-#pragma unroll
-          for (int ks = 0; ks < NKS; ++ks)
-            s_nxt = M::mma(M::load(Ks + (32 * st2 + lr) * PQ + ks * M::KSTEP + lh * M::KPL), qf[j2][ks], s_nxt);
-        }
-        if (act[it]) {
-          const int key0 = kt0 + 32 * st, qlo = q0 + tw[j] * 32;
-          const bool edge = (A.causal && key0 + 31 > qlo) || (key0 + 31 >= A.nk);
-          int hi = A.nk - 1 - key0;
-          if (A.causal && qlo + lr - key0 < hi) hi = qlo + lr - key0;
-          frag pb[M::ACC_KSTEPS];
-          frag vf[NT][M::ACC_KSTEPS];
-#pragma unroll
-          for (int ct = 0; ct < NT; ++ct)
-#pragma unroll
-            for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
-              vf[ct][ss] = M::load_perm(Vs + (32 * ct + lr) * PV + 32 * st, ss, lh);
-          gsum[j] += TM::fwd(s_cur, coef, edge, 0, hi, lh, pb);
-#pragma unroll
-          for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
-#pragma unroll
-            for (int ct = 0; ct < NT; ++ct) acc[j][ct] = M::mma(vf[ct][ss], pb[ss], acc[j][ct]);
-        }
-        s_cur = s_nxt;
-      }
-      buf ^= 1;
-    }
-    FM_SYNC();
-  }
-
-  // ---- epilogue: o = (F + vb) / g, staged through LDS for coalesced stores ----
-  float* Os = reinterpret_cast<float*>(R);             // [QW][DH + 1]
-#pragma unroll
-  for (int j = 0; j < QT; ++j) {
-    float gt = gsum[j] + fm_shfl_xor(gsum[j], 32);
-    if (use_state) gt += A.a0 * cnt;
-    const float ginv = 1.0f / gt;
-#pragma unroll
-    for (int ct = 0; ct < NT; ++ct)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int c = 32 * ct + fm_acc_row(e, lh);
-        const float f = acc[j][ct][e] + (use_state ? vecs[DH + c] : 0.f);
-        Os[xrow[j] * (DH + 1) + c] = f * ginv;
-      }
-    const int qi = q0 + xrow[j];
-    if (lh == 0 && qi < A.nq) A.g[int64_t(bh) * A.g_s_bh + int64_t(qi) * A.g_s_n] = gt;
-  }
-  FM_SYNC();
-  TIO* ob = A.o.p + int64_t(bh) * A.o.s_bh;
-  for (int c = tid; c < QW * (DH / 8); c += FM_THREADS) {
-    const int row = c / (DH / 8), col = (c % (DH / 8)) * 8;
-    if (q0 + row < A.nq) {
-      float v[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) v[i] = Os[row * (DH + 1) + col + i];
-      IO<TIO>::st8(ob + int64_t(q0 + row) * A.o.s_n + col, A.o.vec != 0, v);
-    }
-  }
 }
 
 // ------------------------------------------------------------------------------

@@ -164,7 +164,7 @@ template <> struct CE<float> {
 // ready for the next product.
 //   fwd : P  = a0 + s (a1 + a2 s)                      and the lane's partial row-sum of P
 //   dsc : dS = (a1 + 2 a2 s) (dp - c),  c one scalar per lane
-//   both: P and dS with c per accumulator row (given as fragments in accumulator order)
+//   dsr : the same with c per accumulator row (given as fragments in accumulator order)
 // The _Float16 instantiation evaluates the polynomials on packed halves (v_pk_fma_f16)
 // and sums with v_dot2_f32_f16, which keeps the vector pipe off the critical path.
 template <typename E> struct TileMath;
@@ -173,6 +173,7 @@ template <> struct TileMath<float> {
   typedef float frag;
   struct Coef { float a0, a1, a2, ta2; };
   static FM_DEVICE Coef coef(float a0, float a1, float a2) { Coef c = {a0, a1, a2, 2.0f * a2}; return c; }
+  typedef float CSplat;
   static FM_DEVICE float splat_c(float c) { return c; }
   static FM_DEVICE float fwd(const fm_f32x16& s, const Coef& k, bool edge, int lo, int hi, int lh, frag* pb) {
     float g = 0.f;
@@ -195,15 +196,12 @@ template <> struct TileMath<float> {
       db[e] = ds;
     }
   }
-  static FM_DEVICE void both(const fm_f32x16& s, const fm_f32x16& dp, const frag* crow, const Coef& k, bool edge, int lo,
-                             int hi, int lh, frag* pb, frag* db) {
+  static FM_DEVICE void dsr(const fm_f32x16& s, const fm_f32x16& dp, const frag* crow, const Coef& k, bool edge, int lo,
+                            int hi, int lh, frag* db) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      const float x = s[e];
-      float pv = k.a0 + x * (k.a1 + k.a2 * x);
-      float ds = (k.a1 + k.ta2 * x) * (dp[e] - crow[e]);
-      if (edge) { const int r = fm_acc_row(e, lh); if (r < lo || r > hi) { pv = 0.f; ds = 0.f; } }
-      pb[e] = pv;
+      float ds = (k.a1 + k.ta2 * s[e]) * (dp[e] - crow[e]);
+      if (edge) { const int r = fm_acc_row(e, lh); if (r < lo || r > hi) ds = 0.f; }
       db[e] = ds;
     }
   }
@@ -211,68 +209,73 @@ template <> struct TileMath<float> {
 
 template <> struct TileMath<fm_half> {
   typedef fm_half8 frag;
-  struct Coef { fm_half8 a0, a1, a2, ta2; };
+  // every constant is one packed pair (one register); all arithmetic is written on pairs so
+  // that it maps to v_cvt_pk_f16_f32 / v_pk_fma_f16 / v_pk_mul_f16 / v_pk_add_f16
+  struct Coef { fm_half2 a0, a1, a2, ta2; };
+  static FM_DEVICE fm_half2 pair(float x) { const fm_half h = CE<fm_half>::from(x); fm_half2 r = {h, h}; return r; }
   static FM_DEVICE Coef coef(float a0, float a1, float a2) {
     Coef c;
-    c.a0 = Mma<fm_half>::splat(fm_half(a0)); c.a1 = Mma<fm_half>::splat(fm_half(a1));
-    c.a2 = Mma<fm_half>::splat(fm_half(a2)); c.ta2 = Mma<fm_half>::splat(fm_half(2.0f * a2));
+    c.a0 = pair(a0); c.a1 = pair(a1); c.a2 = pair(a2); c.ta2 = pair(2.0f * a2);
     return c;
   }
-  static FM_DEVICE fm_half8 splat_c(float c) { return Mma<fm_half>::splat(CE<fm_half>::from(c)); }
-  static FM_DEVICE fm_half8 half_of(const fm_f32x16& s, int ss) {
-    fm_half8 h;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) h[i] = fm_half(s[8 * ss + i]);
-    return h;
+  typedef fm_half2 CSplat;
+  static FM_DEVICE fm_half2 splat_c(float c) { return pair(c); }
+  static FM_DEVICE fm_half2 cvt2(float a, float b) {
+    fm_f32x2 v = {a, b};
+    return __builtin_convertvector(v, fm_half2);
   }
-  static FM_DEVICE fm_half8 window(fm_half8 v, int ss, int lo, int hi, int lh) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int r = fm_acc_row(8 * ss + i, lh);
-      if (r < lo || r > hi) v[i] = fm_half(0.f);
-    }
+  static FM_DEVICE fm_half2 get2(const fm_half8& v, int i) {
+    fm_half2 r = {v[2 * i], v[2 * i + 1]};
+    return r;
+  }
+  static FM_DEVICE void put2(fm_half8& v, int i, fm_half2 x) { v[2 * i] = x[0]; v[2 * i + 1] = x[1]; }
+  // zero the entries whose accumulator row is outside [lo, hi]
+  static FM_DEVICE fm_half2 window2(fm_half2 v, int e, int lo, int hi, int lh) {
+    const int r0 = fm_acc_row(e, lh), r1 = fm_acc_row(e + 1, lh);
+    if (r0 < lo || r0 > hi) v[0] = fm_half(0.f);
+    if (r1 < lo || r1 > hi) v[1] = fm_half(0.f);
     return v;
   }
-  static FM_DEVICE float sum8(fm_half8 p, float g) {
-    const fm_half2 one = {fm_half(1.f), fm_half(1.f)};
-    g = fm_dot2(__builtin_shufflevector(p, p, 0, 1), one, g);
-    g = fm_dot2(__builtin_shufflevector(p, p, 2, 3), one, g);
-    g = fm_dot2(__builtin_shufflevector(p, p, 4, 5), one, g);
-    g = fm_dot2(__builtin_shufflevector(p, p, 6, 7), one, g);
-    return g;
-  }
   static FM_DEVICE float fwd(const fm_f32x16& s, const Coef& k, bool edge, int lo, int hi, int lh, frag* pb) {
+    const fm_half2 one = {fm_half(1.f), fm_half(1.f)};
     float g = 0.f;
 #pragma unroll
-    for (int ss = 0; ss < 2; ++ss) {
-      const fm_half8 x = half_of(s, ss);
-      fm_half8 p = (x * k.a2 + k.a1) * x + k.a0;
-      if (edge) p = window(p, ss, lo, hi, lh);
-      g = sum8(p, g);
-      pb[ss] = p;
-    }
+    for (int ss = 0; ss < 2; ++ss)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int e = 8 * ss + 2 * i;
+        const fm_half2 x = cvt2(s[e], s[e + 1]);
+        fm_half2 p = (x * k.a2 + k.a1) * x + k.a0;
+        if (edge) p = window2(p, e, lo, hi, lh);
+        g = fm_dot2(p, one, g);
+        put2(pb[ss], i, p);
+      }
     return g;
   }
-  static FM_DEVICE void dsc(const fm_f32x16& s, const fm_f32x16& dp, fm_half8 c, const Coef& k, bool edge, int lo, int hi,
+  static FM_DEVICE void dsc(const fm_f32x16& s, const fm_f32x16& dp, fm_half2 c, const Coef& k, bool edge, int lo, int hi,
                             int lh, frag* db) {
 #pragma unroll
-    for (int ss = 0; ss < 2; ++ss) {
-      const fm_half8 x = half_of(s, ss);
-      fm_half8 d = (x * k.ta2 + k.a1) * (half_of(dp, ss) - c);
-      if (edge) d = window(d, ss, lo, hi, lh);
-      db[ss] = d;
-    }
-  }
-  static FM_DEVICE void both(const fm_f32x16& s, const fm_f32x16& dp, const frag* crow, const Coef& k, bool edge, int lo,
-                             int hi, int lh, frag* pb, frag* db) {
+    for (int ss = 0; ss < 2; ++ss)
 #pragma unroll
-    for (int ss = 0; ss < 2; ++ss) {
-      const fm_half8 x = half_of(s, ss);
-      fm_half8 p = (x * k.a2 + k.a1) * x + k.a0;
-      fm_half8 d = (x * k.ta2 + k.a1) * (half_of(dp, ss) - crow[ss]);
-      if (edge) { p = window(p, ss, lo, hi, lh); d = window(d, ss, lo, hi, lh); }
-      pb[ss] = p;
-      db[ss] = d;
-    }
+      for (int i = 0; i < 4; ++i) {
+        const int e = 8 * ss + 2 * i;
+        const fm_half2 x = cvt2(s[e], s[e + 1]);
+        fm_half2 d = (x * k.ta2 + k.a1) * (cvt2(dp[e], dp[e + 1]) - c);
+        if (edge) d = window2(d, e, lo, hi, lh);
+        put2(db[ss], i, d);
+      }
+  }
+  static FM_DEVICE void dsr(const fm_f32x16& s, const fm_f32x16& dp, const frag* crow, const Coef& k, bool edge, int lo,
+                            int hi, int lh, frag* db) {
+#pragma unroll
+    for (int ss = 0; ss < 2; ++ss)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int e = 8 * ss + 2 * i;
+        const fm_half2 x = cvt2(s[e], s[e + 1]);
+        fm_half2 d = (x * k.ta2 + k.a1) * (cvt2(dp[e], dp[e + 1]) - get2(crow[ss], i));
+        if (edge) d = window2(d, e, lo, hi, lh);
+        put2(db[ss], i, d);
+      }
   }
 };

@@ -12,6 +12,7 @@ typedef _Float16 fm_half;
 typedef _Float16 fm_half2 __attribute__((ext_vector_type(2)));
 typedef _Float16 fm_half4 __attribute__((ext_vector_type(4)));
 typedef _Float16 fm_half8 __attribute__((ext_vector_type(8)));
+typedef float fm_f32x2 __attribute__((ext_vector_type(2)));
 typedef float fm_f32x4 __attribute__((ext_vector_type(4)));
 typedef float fm_f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t fm_u32x4 __attribute__((ext_vector_type(4)));
@@ -28,6 +29,8 @@ typedef uint16_t fm_bf16;  // raw storage of a bfloat16
 #define FM_LAUNCH_BOUNDS2(n, m)
 #define FM_RESTRICT
 #define FM_UNIFORM(x) (x)
+#define FM_OPAQUE_ZERO() 0
+#define FM_SCHED_FENCE()
 typedef void* fm_stream_t;
 typedef hostsim::Dim3 fm_dim3;
 #define FM_TID_X (int(hostsim::g_t.tid.x))
@@ -73,6 +76,12 @@ FM_DEVICE float fm_sqrtf(float a) { return std::sqrt(a); }
 // a value that is the same in every lane of the wavefront, moved to a scalar register so that
 // branches on it are scalar branches
 #define FM_UNIFORM(x) __builtin_amdgcn_readfirstlane(x)
+// A zero the optimiser cannot see through: added to an LDS offset it keeps two reads of the
+// same tile apart, so the second is a fresh read instead of 16 more live registers.
+static __device__ __forceinline__ int fm_opaque_zero() { int z = 0; asm volatile("" : "+v"(z)); return z; }
+#define FM_OPAQUE_ZERO() fm_opaque_zero()
+// Nothing is scheduled across this point (keeps the live ranges of one phase out of the next).
+#define FM_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
 typedef hipStream_t fm_stream_t;
 typedef dim3 fm_dim3;
 #define FM_TID_X (int(threadIdx.x))

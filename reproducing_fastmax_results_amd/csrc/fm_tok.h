@@ -1,0 +1,587 @@
+// Token-side kernels: the forward and the three gradients as two kernel shapes.
+//
+// A workgroup owns QW tokens of one batch*head ("own" tokens: one 32-token tile per
+// accumulator column group, QT tiles per wavefront) and streams the tokens of the
+// other side past them in stages of KT.  With x_ij = q_i.k_j (q, k pre-multiplied
+// by sqrt(1/tau)), f(x) = a0 + a1 x + a2 x^2 and, per query, gh_i = dO_i / g_i,
+// c_i = gh_i.o_i:
+//
+//   k_pv  own = queries:  F_i  = sum_j M_ij f(x_ij) v_j,  g_i = sum_j M_ij f(x_ij)      (forward)
+//         own = keys:     dV_j = sum_i M_ij f(x_ij) gh_i
+//   k_ds  own = queries:  dQ_i = sum_j dS_ij k_j          dS_ij = M_ij f'(x_ij) (gh_i.v_j - c_i)
+//         own = keys:     dK_j = sum_i dS_ij q_i
+//
+// Stream tokens outside the own token's segment arrive through a moment state
+// (fm_readout), those inside it through dense 32x32 tiles.  A stage whose tiles are
+// all unmasked takes the fast path: every fragment read from LDS feeds the products
+// of all QT own tiles of the wavefront.  Stages on the causal diagonal or at the end
+// of the sequence take the general path with per-tile activity and row windows.
+//
+// Replaces calc_masked / calc_unmasked (fastmax_cuda_forward.cu:23-280) and
+// calc_gradq/k/v_* (fastmax_cuda_backward.cu:26-491), which walk the tokens serially
+// with one thread per feature; the formulas are those of
+// fastattention_einops.py:186-322 (forward) and :384-691 (backward).
+#pragma once
+#include "fm_kernels.h"
+
+enum { FM_OWN_Q = 0, FM_OWN_K = 1 };
+
+template <typename TIO, typename E> struct TokArgs {
+  TRef<const TIO> own_io;   // k_pv, own = queries: q in the caller's tensor (multiplied by sc on load)
+  const E* own_r;           // otherwise: own tokens, row-major compute-type copy [bh][npad_own][DH]
+  const E* own2_r;          // k_ds: second own operand rows (gh for own = queries, v for own = keys)
+  const E* cv;              // k_ds: c per query [bh][npad_q] in tile order
+  const E* xr;              // stream rows that form the scores      [bh][npad_str][DH]
+  const E* yr;              // k_ds: stream rows that form gh.v      [bh][npad_str][DH]
+  const E* zt;              // stream tokens, transposed             [bh][DH][npad_str]
+  int npad_own, npad_str;
+  const E* big; const float* small; int nslots;
+  TRef<TIO> out;
+  float* g; int64_t g_s_bh, g_s_n;      // k_pv, own = queries: denominators
+  int n_own, n_str, L, nseg, causal, use_state, quad;
+  float a0, a1, a2;                     // f(x) = a0 + a1 x + a2 x^2
+  float sc;                             // sqrt(1/tau)
+  float out_scale;                      // factor on the stored gradient
+  float zscale;                         // factor on the Z of the state (k_ds)
+};
+
+// Z (fp32, [DH][DH]) -> LDS in the compute type (hi/lo split for _Float16), va/vb -> vecs.
+template <typename E, int DH, int QT>
+FM_DEVICE void fm_stage_small(const float* sml, E* Zs, float* vecs, int tid, float zscale) {
+  typedef TokCfg<E, DH, QT> C;
+  for (int i = tid; i < DH * DH; i += FM_THREADS) {
+    const float z = sml[i] * zscale;
+    const int r = i / DH, c = i % DH;
+    const E hi = CE<E>::from(z);
+    Zs[r * C::PS + c] = hi;
+    if (C::NZ == 2) Zs[DH * C::PS + r * C::PS + c] = CE<E>::from(z - float(hi));
+  }
+  if (tid < 2 * DH) vecs[tid] = sml[DH * DH + tid];
+}
+
+// y[mt] (rows m, column = token) = sum_l Z[m][l] * tok_l, from the staged Z and the
+// token's B fragments.
+template <typename E, int DH, int QT>
+FM_DEVICE fm_f32x16 fm_zy(const E* Zs, const typename Mma<E>::frag* tf, int mt, int lr, int lh) {
+  typedef TokCfg<E, DH, QT> C;
+  typedef Mma<E> M;
+  fm_f32x16 y = fm_zero16();
+#pragma unroll
+  for (int z = 0; z < C::NZ; ++z)
+#pragma unroll
+    for (int ks = 0; ks < C::NKS; ++ks)
+      y = M::mma(M::load(Zs + z * DH * C::PS + (32 * mt + lr) * C::PS + ks * M::KSTEP + lh * M::KPL), tf[ks], y);
+  return y;
+}
+
+// Accumulators (rows = feature, column = token of tile j) -> caller tensor rows, through LDS.
+template <typename TIO, typename E, int DH, int QT>
+FM_DEVICE void fm_store_tokens(fm_f32x16 (*acc)[DH / 32], const int* xrow, const float* addvec, float scale, float* Os,
+                               TRef<TIO> out, int bh, int row0, int nrows, int tid) {
+  typedef TokCfg<E, DH, QT> C;
+  const int lane = tid & 63, lh = lane >> 5;
+#pragma unroll
+  for (int j = 0; j < QT; ++j)
+#pragma unroll
+    for (int ct = 0; ct < C::NT; ++ct)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int c = 32 * ct + fm_acc_row(e, lh);
+        Os[xrow[j] * (DH + 1) + c] = scale * (acc[j][ct][e] + (addvec ? addvec[c] : 0.f));
+      }
+  FM_SYNC();
+  TIO* ob = out.p + int64_t(bh) * out.s_bh;
+  for (int c = tid; c < C::QW * (DH / 8); c += FM_THREADS) {
+    const int row = c / (DH / 8), col = (c % (DH / 8)) * 8;
+    if (row0 + row < nrows) {
+      float v[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = Os[row * (DH + 1) + col + i];
+      IO<TIO>::st8(ob + int64_t(row0 + row) * out.s_n + col, out.vec != 0, v);
+    }
+  }
+  FM_SYNC();
+}
+
+// Placement of the blocks of own tokens.  A causal block's work is its dense part (1 .. L/QW
+// units of QW x QW tiles, growing with the position inside its segment for queries, shrinking
+// for keys) plus the state readout (the same for every block that has a state), so blocks
+// differ by up to an order of magnitude, and at B*H = 32, N = 4096 a launch has exactly as
+// many workgroups as the chip has slots (two per CU): there is no second wave of workgroups
+// to even things out.  Workgroups go round-robin to the 8 XCDs and, inside an XCD, to its
+// 32 CUs in launch order, so the XCD-local launch index j is turned into a weight rank
+// boustrophedon-wise over rounds of 32: the CU that got the heaviest block of one round gets
+// the lightest of the next.  All blocks of one batch*head stay on one XCD (one L2).
+FM_DEVICE int fm_snake_rank(int j, int total) {
+  const int r = j >> 5, pos = j & 31, base = r << 5;
+  if ((r & 1) == 0) return j;
+  const int cnt = total - base < 32 ? total - base : 32;
+  return base + cnt - 1 - pos;
+}
+
+// rank (0 = heaviest) -> block index, for a causal launch with bps blocks per segment
+template <int OWN> FM_DEVICE int fm_block_of_rank(int rank, int nblk, int bps) {
+  const int nseg = (nblk + bps - 1) / bps;
+  int n = 0;
+  if (OWN == FM_OWN_Q) {
+    // with a state (segments >= 1): late positions first; then segment 0
+    for (int w = bps - 1; w >= 0; --w)
+      for (int sg = nseg - 1; sg >= 1; --sg) {
+        const int b = sg * bps + w;
+        if (b < nblk) { if (n == rank) return b; ++n; }
+      }
+    for (int w = bps - 1; w >= 0; --w)
+      if (w < nblk) { if (n == rank) return w; ++n; }
+  } else {
+    // with a state (all but the last segment): early positions first; then the last segment
+    for (int w = 0; w < bps; ++w)
+      for (int sg = 0; sg < nseg - 1; ++sg) {
+        const int b = sg * bps + w;
+        if (b < nblk) { if (n == rank) return b; ++n; }
+      }
+    for (int w = 0; w < bps; ++w) {
+      const int b = (nseg - 1) * bps + w;
+      if (b < nblk) { if (n == rank) return b; ++n; }
+    }
+  }
+  return rank;   // not reached
+}
+
+// Which part of the stream a block of own tokens starting at t0 sees densely, and which state slot.
+template <int OWN, int QW, typename A_>
+struct TokGeom {
+  int unit, bh, t0, seg, slot, sbeg, send;
+  bool use_state;
+  FM_DEVICE void init(const A_& A) {
+    const int nblk = FM_GDIM_X, nbh = FM_GDIM_Y;
+    const int id = FM_BID_X + nblk * FM_BID_Y;
+    if ((nbh & 7) == 0) {
+      const int nb = nbh >> 3;                       // batch*heads per XCD
+      const int rank = fm_snake_rank(id >> 3, nblk * nb);
+      unit = rank / nb;
+      bh = (id & 7) + 8 * (rank % nb);
+    } else {
+      unit = id % nblk;
+      bh = id / nblk;
+    }
+    const int blk = A.causal ? fm_block_of_rank<OWN>(unit, nblk, A.L / QW) : unit;
+    t0 = blk * QW;
+    seg = A.causal ? t0 / A.L : 0;
+    slot = A.causal ? seg : 0;
+    if (OWN == FM_OWN_Q) {
+      use_state = A.use_state && (!A.causal || seg > 0);
+      sbeg = A.causal ? seg * A.L : 0;
+      send = A.causal ? (t0 + QW < A.n_str ? t0 + QW : A.n_str) : (A.use_state ? 0 : A.n_str);
+    } else {
+      use_state = A.use_state && (!A.causal || seg < A.nseg - 1);
+      sbeg = A.causal ? t0 : 0;
+      send = A.causal ? ((seg + 1) * A.L < A.n_str ? (seg + 1) * A.L : A.n_str) : (A.use_state ? 0 : A.n_str);
+    }
+  }
+  // every 32x32 tile of the stage starting at s0 is fully inside the mask and the sequence
+  FM_DEVICE bool fast_stage(bool causal, int s0, int KT, int n_str) const {
+    if (s0 + KT > n_str) return false;
+    if (!causal) return true;
+    return OWN == FM_OWN_Q ? (s0 + KT <= t0) : (s0 >= t0 + QW);
+  }
+};
+
+// one 32-token stream tile starting at s0 against the own tile starting at lo
+template <int OWN> FM_DEVICE bool fm_tile_active(bool causal, int s0, int lo, int send) {
+  if (s0 >= send) return false;
+  if (!causal) return true;
+  return OWN == FM_OWN_Q ? (s0 <= lo + 31) : (s0 + 31 >= lo);
+}
+template <int OWN> FM_DEVICE bool fm_tile_edge(bool causal, int s0, int lo, int n_str) {
+  if (s0 + 31 >= n_str) return true;
+  if (!causal) return false;
+  return OWN == FM_OWN_Q ? (s0 + 31 > lo) : (s0 < lo + 31);
+}
+// rows (stream tokens of the tile) that the lane's own token lo + lr may see
+template <int OWN> FM_DEVICE void fm_tile_window(bool causal, int s0, int lo, int lr, int n_str, int& wlo, int& whi) {
+  wlo = 0;
+  whi = n_str - 1 - s0;
+  if (causal) {
+    const int dgl = lo + lr - s0;
+    if (OWN == FM_OWN_Q) { if (dgl < whi) whi = dgl; } else wlo = dgl;
+  }
+}
+
+// ------------------------------------------------------------------------------
+// k_pv: forward (own = queries) and dV (own = keys).  grid (ceil(n_own / QW), bh).
+// LDS: va, vb | own rows [QW][PQ] | region (Z, then state slabs, then two dense stages);
+// the output staging lies over the own rows and the region once they are spent.
+// ------------------------------------------------------------------------------
+template <typename TIO, typename E, int DH, int QT, int OWN>
+FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (sizeof(E) == 2 ? 2 : 1)) k_pv(TokArgs<TIO, E> A) {
+  typedef TokCfg<E, DH, QT> C;
+  typedef Mma<E> M;
+  typedef TileMath<E> TM;
+  typedef typename M::frag frag;
+  constexpr int NT = C::NT, NKS = C::NKS, QW = C::QW, PQ = C::PQ, PS = C::PS, KT = C::KT, PV = C::PV;
+  constexpr int STAGE = C::PV_STAGE;
+  FM_DYN_SMEM(smem);
+  float* vecs = reinterpret_cast<float*>(smem);       // va[DH], vb[DH]
+  E* Own = reinterpret_cast<E*>(vecs + 2 * DH);       // [QW][PQ]
+  E* R = Own + QW * PQ;
+  const int tid = FM_TID_X, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int wave = FM_UNIFORM(tid >> 6);
+  TokGeom<OWN, QW, TokArgs<TIO, E> > G;
+  G.init(A);
+  const int bh = G.bh, t0 = G.t0;
+  const bool causal = A.causal != 0;
+
+  // ---- stage the own rows (and the small states) ----
+  if (OWN == FM_OWN_Q) {
+    RowRegs<TIO, E, QW, DH> rq;
+    rq.load(A.own_io.p + int64_t(bh) * A.own_io.s_bh, A.own_io.s_n, A.own_io.vec != 0, t0, A.n_own, tid);
+    rq.store(Own, PQ, tid, A.sc);
+  } else {
+    TileRegs<E, QW, DH> ro;
+    ro.load(A.own_r + (int64_t(bh) * A.npad_own + t0) * DH, DH, tid);
+    ro.store(Own, PQ, tid);
+  }
+  const float* sml = A.small + (int64_t(bh) * A.nslots + G.slot) * StateDims<DH>::SMALL;
+  if (G.use_state) {
+    if (OWN == FM_OWN_Q) fm_stage_small<E, DH, QT>(sml, R, vecs, tid, 1.0f);
+    else if (tid < 2 * DH) vecs[tid] = sml[DH * DH + tid];
+  }
+  FM_SYNC();
+
+  int tw[QT], xrow[QT];
+#pragma unroll
+  for (int j = 0; j < QT; ++j) {
+    tw[j] = (j == 0) ? wave : (4 * QT - 1 - wave);   // pair a short and a long causal tile
+    xrow[j] = tw[j] * 32 + lr;
+  }
+  frag of[QT][NKS];
+#pragma unroll
+  for (int j = 0; j < QT; ++j)
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) of[j][ks] = M::load(Own + xrow[j] * PQ + ks * M::KSTEP + lh * M::KPL);
+
+  fm_f32x16 acc[QT][NT];
+#pragma unroll
+  for (int j = 0; j < QT; ++j)
+#pragma unroll
+    for (int ct = 0; ct < NT; ++ct) acc[j][ct] = fm_zero16();
+  float gsum[QT];
+#pragma unroll
+  for (int j = 0; j < QT; ++j) gsum[j] = 0.f;
+
+  if (G.use_state) {
+    if (OWN == FM_OWN_Q) {
+      // denominator: g_i += sum_m q_im (va[m] + sum_l Z[m][l] q_il)
+#pragma unroll
+      for (int j = 0; j < QT; ++j)
+#pragma unroll
+        for (int mt = 0; mt < NT; ++mt) {
+          const fm_f32x16 y = fm_zy<E, DH, QT>(R, of[j], mt, lr, lh);
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int m = 32 * mt + fm_acc_row(e, lh);
+            gsum[j] += (y[e] + vecs[m]) * float(Own[xrow[j] * PQ + m]);
+          }
+        }
+      FM_SYNC();                                       // Z is overwritten by the slabs
+    }
+    const E* state = A.big + (int64_t(bh) * A.nslots + G.slot) * StateDims<DH>::BIG;
+    fm_readout<E, DH, QT, NT>(state, A.quad != 0, Own, xrow, of, R, acc, tid);
+  }
+
+  // ---- dense tiles over the stream tokens of this segment ----
+  if (G.send > G.sbeg) {
+    const typename TM::Coef coef = TM::coef(A.a0, A.a1, A.a2);
+    TileRegs<E, KT, DH> rx;
+    TileRegs<E, DH, KT> rz;
+    const E* xb = A.xr + int64_t(bh) * A.npad_str * DH;
+    const E* zb = A.zt + int64_t(bh) * DH * A.npad_str;
+    rx.load(xb + int64_t(G.sbeg) * DH, DH, tid);
+    rz.load(zb + G.sbeg, A.npad_str, tid);
+    int buf = 0;
+    for (int s0 = G.sbeg; s0 < G.send; s0 += KT) {
+      E* Xs = R + buf * STAGE;
+      E* Zt = Xs + KT * PQ;
+      rx.store(Xs, PQ, tid);
+      rz.store(Zt, PV, tid);
+      FM_SYNC();
+      if (s0 + KT < G.send) {
+        rx.load(xb + int64_t(s0 + KT) * DH, DH, tid);
+        rz.load(zb + s0 + KT, A.npad_str, tid);
+      }
+      if (G.fast_stage(causal, s0, KT, A.n_str)) {
+#pragma unroll
+        for (int st = 0; st < KT / 32; ++st) {
+          fm_f32x16 s[QT];
+#pragma unroll
+          for (int j = 0; j < QT; ++j) s[j] = fm_zero16();
+#pragma unroll
+          for (int ks = 0; ks < NKS; ++ks) {
+            const frag xf = M::load(Xs + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL);
+#pragma unroll
+            for (int j = 0; j < QT; ++j) s[j] = M::mma(xf, of[j][ks], s[j]);
+          }
+          frag zf[NT][M::ACC_KSTEPS];
+#pragma unroll
+          for (int ct = 0; ct < NT; ++ct)
+#pragma unroll
+            for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
+              zf[ct][ss] = M::load_perm(Zt + (32 * ct + lr) * PV + 32 * st, ss, lh);
+#pragma unroll
+          for (int j = 0; j < QT; ++j) {
+            frag pb[M::ACC_KSTEPS];
+            const float gs = TM::fwd(s[j], coef, false, 0, 0, lh, pb);
+            if (OWN == FM_OWN_Q) gsum[j] += gs;
+#pragma unroll
+            for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
+#pragma unroll
+              for (int ct = 0; ct < NT; ++ct) acc[j][ct] = M::mma(zf[ct][ss], pb[ss], acc[j][ct]);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int st = 0; st < KT / 32; ++st)
+#pragma unroll
+          for (int j = 0; j < QT; ++j) {
+            const int ss0 = s0 + 32 * st, lo = t0 + tw[j] * 32;
+            if (!fm_tile_active<OWN>(causal, ss0, lo, G.send)) continue;
+            const bool edge = fm_tile_edge<OWN>(causal, ss0, lo, A.n_str);
+            int wlo, whi;
+            fm_tile_window<OWN>(causal, ss0, lo, lr, A.n_str, wlo, whi);
+            fm_f32x16 s = fm_zero16();
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks)
+              s = M::mma(M::load(Xs + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL), of[j][ks], s);
+            frag pb[M::ACC_KSTEPS];
+            const float gs = TM::fwd(s, coef, edge, wlo, whi, lh, pb);
+            if (OWN == FM_OWN_Q) gsum[j] += gs;
+#pragma unroll
+            for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
+#pragma unroll
+              for (int ct = 0; ct < NT; ++ct)
+                acc[j][ct] = M::mma(M::load_perm(Zt + (32 * ct + lr) * PV + 32 * st, ss, lh), pb[ss], acc[j][ct]);
+          }
+      }
+      buf ^= 1;
+    }
+    FM_SYNC();
+  }
+
+  // ---- epilogue, staged through LDS for coalesced stores ----
+  float* Os = reinterpret_cast<float*>(Own);           // [QW][DH + 1]
+  if (OWN == FM_OWN_Q) {
+    // o = (F + vb) / g
+    const float cnt = causal ? float(G.sbeg) : float(A.n_str);   // keys covered by the state
+#pragma unroll
+    for (int j = 0; j < QT; ++j) {
+      float gt = gsum[j] + fm_shfl_xor(gsum[j], 32);
+      if (G.use_state) gt += A.a0 * cnt;
+      const float ginv = 1.0f / gt;
+#pragma unroll
+      for (int ct = 0; ct < NT; ++ct)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int c = 32 * ct + fm_acc_row(e, lh);
+          const float f = acc[j][ct][e] + (G.use_state ? vecs[DH + c] : 0.f);
+          Os[xrow[j] * (DH + 1) + c] = f * ginv;
+        }
+      const int qi = t0 + xrow[j];
+      if (lh == 0 && qi < A.n_own) A.g[int64_t(bh) * A.g_s_bh + int64_t(qi) * A.g_s_n] = gt;
+    }
+    FM_SYNC();
+    TIO* ob = A.out.p + int64_t(bh) * A.out.s_bh;
+    for (int c = tid; c < QW * (DH / 8); c += FM_THREADS) {
+      const int row = c / (DH / 8), col = (c % (DH / 8)) * 8;
+      if (t0 + row < A.n_own) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = Os[row * (DH + 1) + col + i];
+        IO<TIO>::st8(ob + int64_t(t0 + row) * A.out.s_n + col, A.out.vec != 0, v);
+      }
+    }
+  } else {
+    // dV = (sums + vb) * out_scale; keys past n_own are discarded by the bounds check
+    fm_store_tokens<TIO, E, DH, QT>(acc, xrow, G.use_state ? vecs + DH : nullptr, A.out_scale, Os, A.out, bh, t0,
+                                    A.n_own, tid);
+  }
+}
+
+// ------------------------------------------------------------------------------
+// k_ds: dQ (own = queries) and dK (own = keys).  grid (ceil(n_own / QW), bh).
+// LDS: va, vb | own rows [QW][PQ] | region (Z, then state slabs); the dense stages
+// (stream rows for the scores, stream rows for gh.v, stream transposed, c values)
+// and the output staging lie over the own rows and the region once they are spent.
+// ------------------------------------------------------------------------------
+template <typename TIO, typename E, int DH, int QT, int OWN>
+FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (sizeof(E) == 2 ? 2 : 1)) k_ds(TokArgs<TIO, E> A) {
+  typedef TokCfg<E, DH, QT> C;
+  typedef Mma<E> M;
+  typedef TileMath<E> TM;
+  typedef typename M::frag frag;
+  constexpr int NT = C::NT, NKS = C::NKS, QW = C::QW, PQ = C::PQ, KT = C::KT, PV = C::PV;
+  constexpr int NBUF = C::DS_NBUF;
+  constexpr int STAGE = C::DS_STAGE;
+  FM_DYN_SMEM(smem);
+  float* vecs = reinterpret_cast<float*>(smem);
+  E* Own = reinterpret_cast<E*>(vecs + 2 * DH);       // [QW][PQ]
+  E* R = Own + QW * PQ;
+  const int tid = FM_TID_X, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int wave = FM_UNIFORM(tid >> 6);
+  TokGeom<OWN, QW, TokArgs<TIO, E> > G;
+  G.init(A);
+  const int bh = G.bh, t0 = G.t0;
+  const bool causal = A.causal != 0;
+
+  {
+    TileRegs<E, QW, DH> ro;
+    ro.load(A.own_r + (int64_t(bh) * A.npad_own + t0) * DH, DH, tid);
+    ro.store(Own, PQ, tid);
+  }
+  if (G.use_state)
+    fm_stage_small<E, DH, QT>(A.small + (int64_t(bh) * A.nslots + G.slot) * StateDims<DH>::SMALL, R, vecs, tid, A.zscale);
+  FM_SYNC();
+
+  int tw[QT], xrow[QT];
+  float ci[QT];
+  typename TM::CSplat cs_own[QT];                      // own = queries: c of the lane's query
+#pragma unroll
+  for (int j = 0; j < QT; ++j) {
+    tw[j] = (j == 0) ? wave : (4 * QT - 1 - wave);
+    xrow[j] = tw[j] * 32 + lr;
+    ci[j] = (OWN == FM_OWN_Q) ? float(A.cv[int64_t(bh) * A.npad_own + t0 + M::tperm(xrow[j])]) : 1.0f;
+    cs_own[j] = TM::splat_c(ci[j]);
+  }
+  frag of[QT][NKS], of2[QT][NKS];
+#pragma unroll
+  for (int j = 0; j < QT; ++j) {
+    const E* o2 = A.own2_r + (int64_t(bh) * A.npad_own + t0 + xrow[j]) * DH + lh * M::KPL;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      of[j][ks] = M::load(Own + xrow[j] * PQ + ks * M::KSTEP + lh * M::KPL);
+      of2[j][ks] = M::load(o2 + ks * M::KSTEP);
+    }
+  }
+  fm_f32x16 acc[QT][NT];
+#pragma unroll
+  for (int j = 0; j < QT; ++j)
+#pragma unroll
+    for (int mt = 0; mt < NT; ++mt) acc[j][mt] = fm_zero16();
+
+  if (G.use_state) {
+    // - c * (va[m] + sum_l Z[m][l] own_l)   (c = c_i for own = queries; folded into Z and va for own = keys)
+#pragma unroll
+    for (int j = 0; j < QT; ++j)
+#pragma unroll
+      for (int mt = 0; mt < NT; ++mt) {
+        const fm_f32x16 y = fm_zy<E, DH, QT>(R, of[j], mt, lr, lh);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[j][mt][e] = -ci[j] * (y[e] + vecs[32 * mt + fm_acc_row(e, lh)]);
+      }
+    FM_SYNC();                                         // Z is overwritten by the slabs
+    const E* state = A.big + (int64_t(bh) * A.nslots + G.slot) * StateDims<DH>::BIG;
+    fm_readout<E, DH, QT, NT>(state, A.quad != 0, Own, xrow, of2, R, acc, tid);
+  } else {
+    FM_SYNC();                                         // own rows are overwritten by the dense stages
+  }
+
+  if (G.send > G.sbeg) {
+    const typename TM::Coef coef = TM::coef(A.a0, A.a1, A.a2);
+    const E* xb = A.xr + int64_t(bh) * A.npad_str * DH;
+    const E* yb = A.yr + int64_t(bh) * A.npad_str * DH;
+    const E* zb = A.zt + int64_t(bh) * DH * A.npad_str;
+    const E* cvb = A.cv + int64_t(bh) * A.npad_str;    // own = keys: c of the streamed queries
+    int buf = 0;
+    for (int s0 = G.sbeg; s0 < G.send; s0 += KT) {
+      // no register prefetch across the products: the second workgroup of the CU covers the
+      // load latency, and the registers go to the fragments of both own tiles instead
+      E* Xs = Own + buf * STAGE; E* Ys = Xs + KT * PQ; E* Zt = Ys + KT * PQ; E* cs = Zt + DH * PV;
+      {
+        TileRegs<E, KT, DH> rx, ry;
+        TileRegs<E, DH, KT> rz;
+        E creg = E(0.f);
+        rx.load(xb + int64_t(s0) * DH, DH, tid);
+        ry.load(yb + int64_t(s0) * DH, DH, tid);
+        rz.load(zb + s0, A.npad_str, tid);
+        if (OWN == FM_OWN_K && tid < KT) creg = cvb[s0 + tid];
+        rx.store(Xs, PQ, tid); ry.store(Ys, PQ, tid); rz.store(Zt, PV, tid);
+        if (OWN == FM_OWN_K && tid < KT) cs[tid] = creg;
+      }
+      FM_SYNC();
+      FM_SCHED_FENCE();
+      if (G.fast_stage(causal, s0, KT, A.n_str)) {
+#pragma unroll
+        for (int st = 0; st < KT / 32; ++st) {
+          // the score fragments and the transposed fragments serve both own tiles; gh.v is formed
+          // per own tile (its fragments are read again) to keep the live accumulators within
+          // the register budget of two workgroups per CU
+          fm_f32x16 s[QT];
+#pragma unroll
+          for (int j = 0; j < QT; ++j) s[j] = fm_zero16();
+#pragma unroll
+          for (int ks = 0; ks < NKS; ++ks) {
+            const frag xf = M::load(Xs + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL);
+#pragma unroll
+            for (int j = 0; j < QT; ++j) s[j] = M::mma(xf, of[j][ks], s[j]);
+          }
+          frag zf[NT][M::ACC_KSTEPS], crow[M::ACC_KSTEPS];
+#pragma unroll
+          for (int ss = 0; ss < M::ACC_KSTEPS; ++ss) {
+            if (OWN == FM_OWN_K) crow[ss] = M::load_perm(cs + 32 * st, ss, lh);
+#pragma unroll
+            for (int mt = 0; mt < NT; ++mt) zf[mt][ss] = M::load_perm(Zt + (32 * mt + lr) * PV + 32 * st, ss, lh);
+          }
+#pragma unroll
+          for (int j = 0; j < QT; ++j) {
+            FM_SCHED_FENCE();
+            fm_f32x16 dp = fm_zero16();
+            const E* yrow = Ys + (32 * st + lr) * PQ + lh * M::KPL + FM_OPAQUE_ZERO();
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) dp = M::mma(M::load(yrow + ks * M::KSTEP), of2[j][ks], dp);
+            frag db[M::ACC_KSTEPS];
+            if (OWN == FM_OWN_Q) TM::dsc(s[j], dp, cs_own[j], coef, false, 0, 0, lh, db);
+            else TM::dsr(s[j], dp, crow, coef, false, 0, 0, lh, db);
+#pragma unroll
+            for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
+#pragma unroll
+              for (int mt = 0; mt < NT; ++mt) acc[j][mt] = M::mma(zf[mt][ss], db[ss], acc[j][mt]);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int st = 0; st < KT / 32; ++st)
+#pragma unroll
+          for (int j = 0; j < QT; ++j) {
+            const int ss0 = s0 + 32 * st, lo = t0 + tw[j] * 32;
+            if (!fm_tile_active<OWN>(causal, ss0, lo, G.send)) continue;
+            const bool edge = fm_tile_edge<OWN>(causal, ss0, lo, A.n_str);
+            int wlo, whi;
+            fm_tile_window<OWN>(causal, ss0, lo, lr, A.n_str, wlo, whi);
+            fm_f32x16 s = fm_zero16(), dp = fm_zero16();
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) {
+              s = M::mma(M::load(Xs + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL), of[j][ks], s);
+              dp = M::mma(M::load(Ys + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL), of2[j][ks], dp);
+            }
+            frag db[M::ACC_KSTEPS];
+            if (OWN == FM_OWN_Q) {
+              TM::dsc(s, dp, cs_own[j], coef, edge, wlo, whi, lh, db);
+            } else {
+              frag crow[M::ACC_KSTEPS];
+#pragma unroll
+              for (int ss = 0; ss < M::ACC_KSTEPS; ++ss) crow[ss] = M::load_perm(cs + 32 * st, ss, lh);
+              TM::dsr(s, dp, crow, coef, edge, wlo, whi, lh, db);
+            }
+#pragma unroll
+            for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
+#pragma unroll
+              for (int mt = 0; mt < NT; ++mt)
+                acc[j][mt] = M::mma(M::load_perm(Zt + (32 * mt + lr) * PV + 32 * st, ss, lh), db[ss], acc[j][mt]);
+          }
+      }
+      if (NBUF == 1) FM_SYNC(); else buf ^= 1;
+    }
+    if (NBUF == 2) FM_SYNC();
+  }
+  fm_store_tokens<TIO, E, DH, QT>(acc, xrow, nullptr, A.out_scale, reinterpret_cast<float*>(Own), A.out, bh, t0,
+                                  A.n_own, tid);
+}
