@@ -86,7 +86,7 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   if (st != FASTMAX_OK) return st;
   p.half = d->dtype == FASTMAX_BF16;
   p.esz = p.half ? 2 : 4;
-  p.qw = p.half ? 256 : 128;
+  p.qw = 128;
   p.npad_q = int(round_up(d->nq, 256));
   p.npad_k = int(round_up(d->nk, 256));
   p.quad = d->p == 2 && d->a2 != 0.0f;
@@ -101,7 +101,10 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   }
   const bool force_dense = (d->flags & FASTMAX_FLAG_FORCE_DENSE) != 0;
   if (d->mask) {
-    int L = d->chunk > 0 ? int(round_up(d->chunk, 256)) : (d->nq >= 2048 ? 1024 : p.npad_q);
+    // Segment length.  Dense tiles cost grows with L, the moment states cost the same per token
+    // whatever L is (readout) plus the walk that builds them.  Measured on MI355X (D = 64, bf16):
+    // one segment (no states at all) wins up to about 6000 tokens, 1024-token segments beyond.
+    int L = d->chunk > 0 ? int(round_up(d->chunk, 256)) : (d->nq > 6144 ? 1024 : p.npad_q);
     if (force_dense || L > p.npad_q) L = p.npad_q;
     p.L = L;
     p.nseg = (d->nq + L - 1) / L;
@@ -316,8 +319,8 @@ int fastmax_forward(const FastmaxDesc* desc, const void* q, const void* k, const
   char* ws = static_cast<char*>(workspace);
   fm_stream_t stream = static_cast<fm_stream_t>(hip_stream);
   if (p.half) {
-    if (desc->d == 64) return run_forward<fm_bf16, fm_half, 64, 2>(desc, p, q, k, v, o, g, ws, stream);
-    return run_forward<fm_bf16, fm_half, 32, 2>(desc, p, q, k, v, o, g, ws, stream);
+    if (desc->d == 64) return run_forward<fm_bf16, fm_half, 64, 1>(desc, p, q, k, v, o, g, ws, stream);
+    return run_forward<fm_bf16, fm_half, 32, 1>(desc, p, q, k, v, o, g, ws, stream);
   }
   if (desc->d == 64) return run_forward<float, float, 64, 1>(desc, p, q, k, v, o, g, ws, stream);
   return run_forward<float, float, 32, 1>(desc, p, q, k, v, o, g, ws, stream);
@@ -346,8 +349,8 @@ static int backward_impl(const FastmaxDesc* desc, const void* q, const void* k, 
   const char* fws = static_cast<const char*>(fwd_ws);
   fm_stream_t stream = static_cast<fm_stream_t>(hip_stream);
   if (p.half) {
-    if (desc->d == 64) return run_backward<fm_bf16, fm_half, 64, 2>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);
-    return run_backward<fm_bf16, fm_half, 32, 2>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);
+    if (desc->d == 64) return run_backward<fm_bf16, fm_half, 64, 1>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);
+    return run_backward<fm_bf16, fm_half, 32, 1>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);
   }
   if (desc->d == 64) return run_backward<float, float, 64, 1>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);
   return run_backward<float, float, 32, 1>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);

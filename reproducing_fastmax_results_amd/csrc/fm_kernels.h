@@ -357,6 +357,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 ? 2 : 1)
     if (quad) rx.store(s2, PT, tid);
     if (has_z) rz.store(s3, PT, tid);
     FM_SYNC();
+
     int nt = t + TT, nw = w, ntb = tb, nte = te, nslot = slot;
     const bool last = (nt >= te);
     bool has_next = true;
@@ -511,9 +512,14 @@ struct TokCfg {
   static constexpr int QW = 4 * QT * 32;            // tokens per workgroup
   static constexpr int PQ = DH + M::PAD;            // pitch of row-major token tiles
   static constexpr int PS = DH + M::PAD;            // pitch of state rows
-  static constexpr int OCC = sizeof(E) == 2 ? 2 : 1;   // workgroups per CU the kernels are sized for
-  static constexpr int SA = 2;                      // values of a per state slab
-  static constexpr int KT = 64;                     // tokens per stage of the dense loop
+  // _Float16: one tile per wavefront, small slabs and stages, so that four (k_pv) or three
+  // (k_ds) workgroups share a CU: 12 to 16 wavefronts hide each other's LDS and MFMA latency.
+  // On MI355X at B*H = 32, N = 4096, D = 64 this measured faster than two tiles per wavefront
+  // at two workgroups per CU, dense tiles 0.47 vs 0.56 ms for the four kernels together.
+  static constexpr int OCC_PV = sizeof(E) == 2 ? 4 : 1;   // workgroups per CU the kernels are sized for
+  static constexpr int OCC_DS = sizeof(E) == 2 ? 3 : 1;
+  static constexpr int SA = sizeof(E) == 2 ? 1 : 2;       // values of a per state slab
+  static constexpr int KT = sizeof(E) == 2 ? 32 : 64;    // tokens per stage of the dense loop
   static constexpr int PV = KT + M::PAD;            // pitch of transposed token tiles
   static constexpr int NZ = sizeof(E) == 2 ? 2 : 1; // hi/lo split of fp32 denominators
   static constexpr int SLAB = SA * DH * PS;         // elements per slab buffer

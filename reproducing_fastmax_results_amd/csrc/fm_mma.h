@@ -131,20 +131,16 @@ template <> struct IO<fm_bf16> {
 // out-of-range input degrades instead of producing infinities.
 template <typename E> struct CE;
 template <> struct CE<fm_half> {
-  static FM_DEVICE fm_half from(float x) {
-    const float lim = 65504.f;
-    x = x > lim ? lim : (x < -lim ? -lim : x);
-    return fm_half(x);
-  }
+  static FM_DEVICE fm_half from(float x) { return fm_half(fm_clampf(x, 65504.f)); }
   // eight consecutive elements to LDS / workspace (16-byte aligned)
   static FM_DEVICE void st8(fm_half* p, const float in[8]) {
     fm_half8 h;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) h[i] = fm_half(in[i]);
-    // saturate after the conversion, on packed halves (an overflowing float converts to inf)
-    const fm_half8 lim = {fm_half(65504.f), fm_half(65504.f), fm_half(65504.f), fm_half(65504.f),
-                          fm_half(65504.f), fm_half(65504.f), fm_half(65504.f), fm_half(65504.f)};
-    h = __builtin_elementwise_min(__builtin_elementwise_max(h, -lim), lim);
+    for (int i = 0; i < 8; i += 2) {
+      fm_f32x2 v = {fm_clampf(in[i], 65504.f), fm_clampf(in[i + 1], 65504.f)};
+      const fm_half2 c = __builtin_convertvector(v, fm_half2);
+      h[i] = c[0]; h[i + 1] = c[1];
+    }
     *reinterpret_cast<fm_half8*>(p) = h;
   }
 };

@@ -62,6 +62,7 @@ FM_DEVICE fm_f32x16 fm_mfma_f32(float a, float b, fm_f32x16 c) {
 FM_DEVICE float fm_shfl_xor(float v, int m) { return hostsim::shfl(v, hostsim::g_t.lane ^ m); }
 FM_DEVICE float fm_dot2(fm_half2 a, fm_half2 b, float c) { return float(a[0]) * float(b[0]) + float(a[1]) * float(b[1]) + c; }
 FM_DEVICE float fm_fmaxf(float a, float b) { return a > b ? a : b; }
+FM_DEVICE float fm_clampf(float x, float lim) { return x > lim ? lim : (x < -lim ? -lim : x); }
 FM_DEVICE float fm_rsqrtf(float a) { return 1.0f / std::sqrt(a); }
 FM_DEVICE float fm_sqrtf(float a) { return std::sqrt(a); }
 
@@ -104,6 +105,8 @@ FM_DEVICE fm_f32x16 fm_mfma_f32(float a, float b, fm_f32x16 c) {
 FM_DEVICE float fm_shfl_xor(float v, int m) { return __shfl_xor(v, m, 64); }
 FM_DEVICE float fm_dot2(fm_half2 a, fm_half2 b, float c) { return __builtin_amdgcn_fdot2(a, b, c, false); }
 FM_DEVICE float fm_fmaxf(float a, float b) { return fmaxf(a, b); }
+// clamp to [-lim, lim] in one instruction (v_med3_f32)
+FM_DEVICE float fm_clampf(float x, float lim) { return __builtin_amdgcn_fmed3f(x, -lim, lim); }
 FM_DEVICE float fm_rsqrtf(float a) { return rsqrtf(a); }
 FM_DEVICE float fm_sqrtf(float a) { return sqrtf(a); }
 #endif

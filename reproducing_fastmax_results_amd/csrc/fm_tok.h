@@ -213,7 +213,7 @@ template <int OWN> FM_DEVICE void fm_tile_window(bool causal, int s0, int lo, in
 // the output staging lies over the own rows and the region once they are spent.
 // ------------------------------------------------------------------------------
 template <typename TIO, typename E, int DH, int QT, int OWN>
-FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (sizeof(E) == 2 ? 2 : 1)) k_pv(TokArgs<TIO, E> A) {
+FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(TokArgs<TIO, E> A) {
   typedef TokCfg<E, DH, QT> C;
   typedef Mma<E> M;
   typedef TileMath<E> TM;
@@ -413,7 +413,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (sizeof(E) == 2 ? 2 : 1)) k_pv(TokA
 // and the output staging lie over the own rows and the region once they are spent.
 // ------------------------------------------------------------------------------
 template <typename TIO, typename E, int DH, int QT, int OWN>
-FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (sizeof(E) == 2 ? 2 : 1)) k_ds(TokArgs<TIO, E> A) {
+FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_DS)) k_ds(TokArgs<TIO, E> A) {
   typedef TokCfg<E, DH, QT> C;
   typedef Mma<E> M;
   typedef TileMath<E> TM;

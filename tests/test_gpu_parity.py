@@ -58,10 +58,12 @@ def test_forward_config1(lib):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_forward_config2_heads(lib, dtype):
-    # causal order 2, N=4096, D=64: 4 of the 32 (b, h) slices against the fp64 closed form
-    print(f"case config2 fwd dtype={dtype}", flush=True)
-    check_forward(lib, 4, 4096, 64, dtype, DEV, mask=True, p=2, seed=1)
+@pytest.mark.parametrize("chunk", [0, 1024, 2048])
+def test_forward_config2_heads(lib, dtype, chunk):
+    # causal order 2, N=4096, D=64: 4 of the 32 (b, h) slices against the fp64 closed form;
+    # chunk 0 is the library's own choice (one segment at this length), the others go through the states
+    print(f"case config2 fwd dtype={dtype} chunk={chunk}", flush=True)
+    check_forward(lib, 4, 4096, 64, dtype, DEV, mask=True, p=2, seed=1, chunk=chunk)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -92,10 +94,19 @@ def test_backward_moments_small(lib, dtype, mask, p, d):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_backward_config2_heads(lib, dtype):
+@pytest.mark.parametrize("chunk", [0, 1024, 2048])
+def test_backward_config2_heads(lib, dtype, chunk):
     # Fastmax order-2 causal forward and backward, N=4096, D=64 (4 of the 32 slices, fp64 closed form)
-    print(f"case config2 fwd+bwd dtype={dtype}", flush=True)
-    check_forward_backward(lib, 4, 4096, 64, dtype, DEV, mask=True, p=2, seed=9)
+    print(f"case config2 fwd+bwd dtype={dtype} chunk={chunk}", flush=True)
+    check_forward_backward(lib, 4, 4096, 64, dtype, DEV, mask=True, p=2, seed=9, chunk=chunk)
+    check_forward_backward(lib, 4, 4096, 64, dtype, DEV, mask=True, p=2, seed=9, chunk=chunk, saved=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_long_sequence_default_segments(lib, dtype):
+    # beyond 6144 tokens the library cuts the sequence into 1024-token segments on its own
+    print(f"case long dtype={dtype}", flush=True)
+    check_forward_backward(lib, 1, 7000, 64, dtype, DEV, mask=True, p=2, seed=21, saved=True)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -105,7 +116,7 @@ def test_backward_ragged_and_cross(lib, dtype):
     check_forward_backward(lib, 2, 50, 32, dtype, DEV, mask=False, p=2, seed=11)
     check_forward_backward(lib, 2, 257, 64, dtype, DEV, mask=False, p=2, nk=513, seed=12)
     check_forward_backward(lib, 1, 700, 64, dtype, DEV, mask=False, p=2, nk=4500, seed=13)
-    check_forward_backward(lib, 1, 2500, 64, dtype, DEV, mask=True, p=2, seed=14)       # ragged last segment
+    check_forward_backward(lib, 1, 2500, 64, dtype, DEV, mask=True, p=2, seed=14, chunk=1024)   # ragged last segment
     check_forward_backward(lib, 2, 777, 32, dtype, DEV, mask=True, p=2, a=(1.0, 1.166666, 0.145833), tau_mult=1.0,
                            seed=15)                                                    # fitted (non-Taylor) coefficients
 
@@ -129,4 +140,4 @@ def test_backward_on_saved_forward_workspace(lib, dtype, mask, p):
     check_forward_backward(lib, 8, 1100, 64, dtype, DEV, mask=mask, p=p, chunk=256, flags=FLAG_FORCE_MOMENTS,
                            seed=18, saved=True)
     check_forward_backward(lib, 3, 333, 32, dtype, DEV, mask=mask, p=p, flags=FLAG_FORCE_DENSE, seed=19, saved=True)
-    check_forward_backward(lib, 2, 2500, 64, dtype, DEV, mask=mask, p=p, seed=20, saved=True)
+    check_forward_backward(lib, 2, 2500, 64, dtype, DEV, mask=mask, p=p, seed=20, saved=True, chunk=1024)
