@@ -33,10 +33,21 @@ if ROOT not in sys.path:
 PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}      # MI355X dense matrix peaks (published)
 PEAK_HBM_GBS = 8000.0
 
+# HBM bytes per launch of the dominant kernel at the workload below, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of this file scaled by a copy of known size; keyed by (dtype, --chunk, kernel).
+TRAFFIC_BYTES = {("bf16", 0, "dk"): 224271 * 1024}
+
 WORKLOAD = dict(name="configs[1]: causal order-2 fwd+bwd", B=4, H=8, N=4096, D=64, p=2, mask=True)
 
-# units of algorithmic work (each 2*M_p*(Dv+1) flop per (b, h, token)) per launch of each kernel
-UNITS = {"build": 1, "fwd": 1, "dq": 1, "dk": 1, "dv": 1}
+# Units of algorithmic work (each 2*M_p*(Dv+1) flop per (b, h, token)) carried by one launch of
+# each kernel; 7 units per forward+backward in both cases (fwd 4, bwd 10 of the 14*M_p*(Dv+1)).
+# With moment states: two state walks (forward, backward) of one unit each, the readouts one
+# each, and dQ also carries the unit of the prefix rebuild it is spared by reading the forward's.
+# Without (a sequence short enough for one segment) each kernel carries its walk as well.
+UNITS_STATE = {"build": 1, "fwd": 1, "dq": 2, "dk": 1, "dv": 1}
+UNITS_DENSE = {"fwd": 2, "dq": 2, "dk": 2, "dv": 1}
+# 32x32x16 MFMA instructions per 32x32 score tile in the dense loops of each kernel
+MFMA_PER_TILE = {"fwd": 8, "dv": 8, "dq": 12, "dk": 12}
 
 
 def alg_flops_unit(bh: int, n: int, d: int, p: int) -> float:
@@ -79,6 +90,8 @@ def main() -> int:
     ap.add_argument("--independent-backward", action="store_true",
                     help="backward rebuilds the key-side copies and states instead of taking them from the forward")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB device copy, the yardstick for the HBM traffic counters")
     ap.add_argument("--cpu-max-n", type=int, default=2048, help="longest slice the CPU baseline materialises")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -134,16 +147,28 @@ def main() -> int:
     for name, ms in recs:
         tot, cnt = per_kernel.get(name, (0.0, 0))
         per_kernel[name] = (tot + ms, cnt + 1)
-    dominant = max(per_kernel, key=lambda nme: per_kernel[nme][0])
+    units = UNITS_STATE if "build" in per_kernel else UNITS_DENSE
+    heavy = {nme: v for nme, v in per_kernel.items() if nme in units}
+    dominant = max(heavy, key=lambda nme: heavy[nme][0] / heavy[nme][1])
     avg_ms = per_kernel[dominant][0] / per_kernel[dominant][1]
     unit = alg_flops_unit(bh, N, D, p)
-    achieved = UNITS.get(dominant, 0) * unit / (avg_ms * 1e-3) / 1e12
+    achieved = units[dominant] * unit / (avg_ms * 1e-3) / 1e12
     peak = PEAK_TFLOPS[args.dtype]
     roofline = {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
                 "frac": achieved / peak, "traffic": None, "avg_ms": avg_ms,
                 "whole_step": {"achieved": 7 * unit / (ms_per_step * 1e-3) / 1e12,
                                "frac": 7 * unit / (ms_per_step * 1e-3) / 1e12 / peak},
                 "kernels_ms_per_step": {nme: tot / nprof for nme, (tot, cnt) in sorted(per_kernel.items())}}
+    if "build" not in per_kernel and args.dtype == "bf16":
+        # what the matrix cores actually execute when one segment covers the sequence: causal 32x32 tiles only
+        nt = (N + 31) // 32
+        tiles = bh * nt * (nt + 1) // 2
+        executed = sum(MFMA_PER_TILE.values()) * tiles * 2.0 * 32 * 32 * 16
+        roofline["executed_mfma"] = {"flop_per_step": executed,
+                                     "achieved": executed / (ms_per_step * 1e-3) / 1e12,
+                                     "frac": executed / (ms_per_step * 1e-3) / 1e12 / peak}
+    if TRAFFIC_BYTES.get((args.dtype, args.chunk, dominant)) is not None:
+        roofline["traffic"] = TRAFFIC_BYTES[(args.dtype, args.chunk, dominant)]
 
     out = {
         "metric": "Fastmax fwd+bwd tokens/s, causal order-2 N=4096 D=64",
@@ -154,6 +179,11 @@ def main() -> int:
                    "chunk": args.chunk or "auto"},
         "roofline": roofline,
     }
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(N, D, p, tokens, bh, args.cpu_max_n)
     print(json.dumps(out))

@@ -196,14 +196,14 @@ int launch_build(const BuildArgs<E>& a, int bh, fm_stream_t stream) {
 template <typename E, int DH, int QT> size_t tok_lds_bytes() {
   typedef TokCfg<E, DH, QT> C;
   size_t region = size_t(2) * C::SLAB * sizeof(E);
-  const size_t dense = size_t(2) * C::PV_STAGE * sizeof(E);
   const size_t zs = size_t(C::NZ) * DH * C::PS * sizeof(E);
-  if (dense > region) region = dense;
   if (zs > region) region = zs;
   size_t body = size_t(C::QW) * C::PQ * sizeof(E) + region;
   const size_t outst = size_t(C::QW) * (DH + 1) * 4;
+  const size_t pv = size_t(2) * C::PV_STAGE * sizeof(E);
   const size_t ds = size_t(C::DS_NBUF) * C::DS_STAGE * sizeof(E);
   if (outst > body) body = outst;
+  if (pv > body) body = pv;
   if (ds > body) body = ds;
   return size_t(2 * DH) * 4 + body;
 }

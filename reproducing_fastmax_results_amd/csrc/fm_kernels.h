@@ -502,8 +502,21 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 ? 2 : 1)
 // ------------------------------------------------------------------------------
 // Shared pieces of the token-side kernels
 // ------------------------------------------------------------------------------
-// LDS sizes (in elements of E) used by k_fwd / k_dq / k_dkv; the host computes the
-// dynamic LDS bytes from the same struct.
+// LDS sizes (in elements of E) used by k_pv / k_ds; the host computes the dynamic LDS
+// bytes from the same struct.
+// Tuning knobs of the _Float16 token kernels (the values are the ones measured best on MI355X).
+#ifndef FM_TUNE_OCC_PV
+#define FM_TUNE_OCC_PV 4
+#endif
+#ifndef FM_TUNE_OCC_DS
+#define FM_TUNE_OCC_DS 3
+#endif
+#ifndef FM_TUNE_KT_PV
+#define FM_TUNE_KT_PV 32
+#endif
+#ifndef FM_TUNE_KT_DS
+#define FM_TUNE_KT_DS 32
+#endif
 template <typename E, int DH, int QT>
 struct TokCfg {
   typedef Mma<E> M;
@@ -516,15 +529,18 @@ struct TokCfg {
   // (k_ds) workgroups share a CU: 12 to 16 wavefronts hide each other's LDS and MFMA latency.
   // On MI355X at B*H = 32, N = 4096, D = 64 this measured faster than two tiles per wavefront
   // at two workgroups per CU, dense tiles 0.47 vs 0.56 ms for the four kernels together.
-  static constexpr int OCC_PV = sizeof(E) == 2 ? 4 : 1;   // workgroups per CU the kernels are sized for
-  static constexpr int OCC_DS = sizeof(E) == 2 ? 3 : 1;
+  static constexpr int OCC_PV = sizeof(E) == 2 ? FM_TUNE_OCC_PV : 1;   // workgroups per CU the kernels are sized for
+  static constexpr int OCC_DS = sizeof(E) == 2 ? FM_TUNE_OCC_DS : 1;
   static constexpr int SA = sizeof(E) == 2 ? 1 : 2;       // values of a per state slab
-  static constexpr int KT = sizeof(E) == 2 ? 32 : 64;    // tokens per stage of the dense loop
-  static constexpr int PV = KT + M::PAD;            // pitch of transposed token tiles
+  // (64-token stages for _Float16 measured slower on MI355X: the larger tile movers cost registers)
+  static constexpr int KT_PV = sizeof(E) == 2 ? FM_TUNE_KT_PV : 64;   // stream tokens per stage of the dense loop, k_pv
+  static constexpr int KT_DS = sizeof(E) == 2 ? FM_TUNE_KT_DS : 64;   //                                           k_ds
+  static constexpr int PV_PV = KT_PV + M::PAD;      // pitch of the transposed token tiles
+  static constexpr int PV_DS = KT_DS + M::PAD;
   static constexpr int NZ = sizeof(E) == 2 ? 2 : 1; // hi/lo split of fp32 denominators
   static constexpr int SLAB = SA * DH * PS;         // elements per slab buffer
-  static constexpr int PV_STAGE = KT * PQ + DH * PV;            // k_pv: stream rows, stream transposed
-  static constexpr int DS_STAGE = 2 * KT * PQ + DH * PV + KT;   // k_ds: two row tiles, transposed tile, c values
+  static constexpr int PV_STAGE = KT_PV * PQ + DH * PV_PV;                // k_pv: stream rows, stream transposed
+  static constexpr int DS_STAGE = 2 * KT_DS * PQ + DH * PV_DS + KT_DS;    // k_ds: two row tiles, transposed tile, c values
   static constexpr int DS_NBUF = sizeof(E) == 2 ? 2 : 1;
 };
 

@@ -225,27 +225,32 @@ template <> struct TileMath<fm_half> {
     return r;
   }
   static FM_DEVICE void put2(fm_half8& v, int i, fm_half2 x) { v[2 * i] = x[0]; v[2 * i + 1] = x[1]; }
-  // zero the entries whose accumulator row is outside [lo, hi]
-  static FM_DEVICE fm_half2 window2(fm_half2 v, int e, int lo, int hi, int lh) {
-    const int r0 = fm_acc_row(e, lh), r1 = fm_acc_row(e + 1, lh);
-    if (r0 < lo || r0 > hi) v[0] = fm_half(0.f);
-    if (r1 < lo || r1 > hi) v[1] = fm_half(0.f);
-    return v;
+  // zero the entries of both fragments whose accumulator row is outside [lo, hi]
+  static FM_DEVICE void window_frags(frag* f, int lo, int hi, int lh) {
+#pragma unroll
+    for (int ss = 0; ss < 2; ++ss)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int r = fm_acc_row(8 * ss + i, lh);
+        if (r < lo || r > hi) f[ss][i] = fm_half(0.f);
+      }
   }
   static FM_DEVICE float fwd(const fm_f32x16& s, const Coef& k, bool edge, int lo, int hi, int lh, frag* pb) {
     const fm_half2 one = {fm_half(1.f), fm_half(1.f)};
-    float g = 0.f;
 #pragma unroll
     for (int ss = 0; ss < 2; ++ss)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int e = 8 * ss + 2 * i;
         const fm_half2 x = cvt2(s[e], s[e + 1]);
-        fm_half2 p = (x * k.a2 + k.a1) * x + k.a0;
-        if (edge) p = window2(p, e, lo, hi, lh);
-        g = fm_dot2(p, one, g);
-        put2(pb[ss], i, p);
+        put2(pb[ss], i, (x * k.a2 + k.a1) * x + k.a0);
       }
+    if (edge) { FM_KEEP_BRANCH(); window_frags(pb, lo, hi, lh); }
+    float g = 0.f;
+#pragma unroll
+    for (int ss = 0; ss < 2; ++ss)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) g = fm_dot2(get2(pb[ss], i), one, g);
     return g;
   }
   static FM_DEVICE void dsc(const fm_f32x16& s, const fm_f32x16& dp, fm_half2 c, const Coef& k, bool edge, int lo, int hi,
@@ -256,10 +261,9 @@ template <> struct TileMath<fm_half> {
       for (int i = 0; i < 4; ++i) {
         const int e = 8 * ss + 2 * i;
         const fm_half2 x = cvt2(s[e], s[e + 1]);
-        fm_half2 d = (x * k.ta2 + k.a1) * (cvt2(dp[e], dp[e + 1]) - c);
-        if (edge) d = window2(d, e, lo, hi, lh);
-        put2(db[ss], i, d);
+        put2(db[ss], i, (x * k.ta2 + k.a1) * (cvt2(dp[e], dp[e + 1]) - c));
       }
+    if (edge) { FM_KEEP_BRANCH(); window_frags(db, lo, hi, lh); }
   }
   static FM_DEVICE void dsr(const fm_f32x16& s, const fm_f32x16& dp, const frag* crow, const Coef& k, bool edge, int lo,
                             int hi, int lh, frag* db) {
@@ -269,9 +273,8 @@ template <> struct TileMath<fm_half> {
       for (int i = 0; i < 4; ++i) {
         const int e = 8 * ss + 2 * i;
         const fm_half2 x = cvt2(s[e], s[e + 1]);
-        fm_half2 d = (x * k.ta2 + k.a1) * (cvt2(dp[e], dp[e + 1]) - get2(crow[ss], i));
-        if (edge) d = window2(d, e, lo, hi, lh);
-        put2(db[ss], i, d);
+        put2(db[ss], i, (x * k.ta2 + k.a1) * (cvt2(dp[e], dp[e + 1]) - get2(crow[ss], i)));
       }
+    if (edge) { FM_KEEP_BRANCH(); window_frags(db, lo, hi, lh); }
   }
 };

@@ -31,6 +31,7 @@ typedef uint16_t fm_bf16;  // raw storage of a bfloat16
 #define FM_UNIFORM(x) (x)
 #define FM_OPAQUE_ZERO() 0
 #define FM_SCHED_FENCE()
+#define FM_KEEP_BRANCH()
 typedef void* fm_stream_t;
 typedef hostsim::Dim3 fm_dim3;
 #define FM_TID_X (int(hostsim::g_t.tid.x))
@@ -83,6 +84,9 @@ static __device__ __forceinline__ int fm_opaque_zero() { int z = 0; asm volatile
 #define FM_OPAQUE_ZERO() fm_opaque_zero()
 // Nothing is scheduled across this point (keeps the live ranges of one phase out of the next).
 #define FM_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+// Inside a rarely taken wavefront-uniform branch: keeps it a branch (the optimiser would
+// otherwise run its body on every pass and select the result).
+#define FM_KEEP_BRANCH() asm volatile("")
 typedef hipStream_t fm_stream_t;
 typedef dim3 fm_dim3;
 #define FM_TID_X (int(threadIdx.x))

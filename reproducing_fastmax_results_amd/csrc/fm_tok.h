@@ -12,10 +12,8 @@
 //         own = keys:     dK_j = sum_i dS_ij q_i
 //
 // Stream tokens outside the own token's segment arrive through a moment state
-// (fm_readout), those inside it through dense 32x32 tiles.  A stage whose tiles are
-// all unmasked takes the fast path: every fragment read from LDS feeds the products
-// of all QT own tiles of the wavefront.  Stages on the causal diagonal or at the end
-// of the sequence take the general path with per-tile activity and row windows.
+// (fm_readout), those inside it through dense 32x32 tiles; tiles on the causal diagonal
+// or at the end of the sequence zero the entries outside their row window.
 //
 // Replaces calc_masked / calc_unmasked (fastmax_cuda_forward.cu:23-280) and
 // calc_gradq/k/v_* (fastmax_cuda_backward.cu:26-491), which walk the tokens serially
@@ -178,20 +176,9 @@ struct TokGeom {
       send = A.causal ? ((seg + 1) * A.L < A.n_str ? (seg + 1) * A.L : A.n_str) : (A.use_state ? 0 : A.n_str);
     }
   }
-  // every 32x32 tile of the stage starting at s0 is fully inside the mask and the sequence
-  FM_DEVICE bool fast_stage(bool causal, int s0, int KT, int n_str) const {
-    if (s0 + KT > n_str) return false;
-    if (!causal) return true;
-    return OWN == FM_OWN_Q ? (s0 + KT <= t0) : (s0 >= t0 + QW);
-  }
 };
 
 // one 32-token stream tile starting at s0 against the own tile starting at lo
-template <int OWN> FM_DEVICE bool fm_tile_active(bool causal, int s0, int lo, int send) {
-  if (s0 >= send) return false;
-  if (!causal) return true;
-  return OWN == FM_OWN_Q ? (s0 <= lo + 31) : (s0 + 31 >= lo);
-}
 template <int OWN> FM_DEVICE bool fm_tile_edge(bool causal, int s0, int lo, int n_str) {
   if (s0 + 31 >= n_str) return true;
   if (!causal) return false;
@@ -209,8 +196,8 @@ template <int OWN> FM_DEVICE void fm_tile_window(bool causal, int s0, int lo, in
 
 // ------------------------------------------------------------------------------
 // k_pv: forward (own = queries) and dV (own = keys).  grid (ceil(n_own / QW), bh).
-// LDS: va, vb | own rows [QW][PQ] | region (Z, then state slabs, then two dense stages);
-// the output staging lies over the own rows and the region once they are spent.
+// LDS: va, vb | own rows [QW][PQ] | region (Z, then state slabs); the two dense stages and the
+// output staging lie over the own rows and the region once they are spent.
 // ------------------------------------------------------------------------------
 template <typename TIO, typename E, int DH, int QT, int OWN>
 FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(TokArgs<TIO, E> A) {
@@ -218,7 +205,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
   typedef Mma<E> M;
   typedef TileMath<E> TM;
   typedef typename M::frag frag;
-  constexpr int NT = C::NT, NKS = C::NKS, QW = C::QW, PQ = C::PQ, PS = C::PS, KT = C::KT, PV = C::PV;
+  constexpr int NT = C::NT, NKS = C::NKS, QW = C::QW, PQ = C::PQ, KT = C::KT_PV, PV = C::PV_PV;
   constexpr int STAGE = C::PV_STAGE;
   FM_DYN_SMEM(smem);
   float* vecs = reinterpret_cast<float*>(smem);       // va[DH], vb[DH]
@@ -287,6 +274,8 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
     }
     const E* state = A.big + (int64_t(bh) * A.nslots + G.slot) * StateDims<DH>::BIG;
     fm_readout<E, DH, QT, NT>(state, A.quad != 0, Own, xrow, of, R, acc, tid);
+  } else {
+    FM_SYNC();                                         // own rows are overwritten by the dense stages
   }
 
   // ---- dense tiles over the stream tokens of this segment ----
@@ -300,7 +289,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
     rz.load(zb + G.sbeg, A.npad_str, tid);
     int buf = 0;
     for (int s0 = G.sbeg; s0 < G.send; s0 += KT) {
-      E* Xs = R + buf * STAGE;
+      E* Xs = Own + buf * STAGE;                        // the own rows and the slabs are spent
       E* Zt = Xs + KT * PQ;
       rx.store(Xs, PQ, tid);
       rz.store(Zt, PV, tid);
@@ -309,58 +298,40 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
         rx.load(xb + int64_t(s0 + KT) * DH, DH, tid);
         rz.load(zb + s0 + KT, A.npad_str, tid);
       }
-      if (G.fast_stage(causal, s0, KT, A.n_str)) {
+      // One code path for every tile: the products always run, and a tile that touches the mask
+      // or the end of the sequence (a wavefront-uniform test) zeroes the entries outside its row
+      // window before they are used; a tile wholly outside the mask has an empty window.
 #pragma unroll
-        for (int st = 0; st < KT / 32; ++st) {
-          fm_f32x16 s[QT];
+      for (int st = 0; st < KT / 32; ++st) {
+        fm_f32x16 s[QT];
 #pragma unroll
-          for (int j = 0; j < QT; ++j) s[j] = fm_zero16();
+        for (int j = 0; j < QT; ++j) s[j] = fm_zero16();
 #pragma unroll
-          for (int ks = 0; ks < NKS; ++ks) {
-            const frag xf = M::load(Xs + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL);
+        for (int ks = 0; ks < NKS; ++ks) {
+          const frag xf = M::load(Xs + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL);
 #pragma unroll
-            for (int j = 0; j < QT; ++j) s[j] = M::mma(xf, of[j][ks], s[j]);
-          }
-          frag zf[NT][M::ACC_KSTEPS];
-#pragma unroll
-          for (int ct = 0; ct < NT; ++ct)
-#pragma unroll
-            for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
-              zf[ct][ss] = M::load_perm(Zt + (32 * ct + lr) * PV + 32 * st, ss, lh);
-#pragma unroll
-          for (int j = 0; j < QT; ++j) {
-            frag pb[M::ACC_KSTEPS];
-            const float gs = TM::fwd(s[j], coef, false, 0, 0, lh, pb);
-            if (OWN == FM_OWN_Q) gsum[j] += gs;
-#pragma unroll
-            for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
-#pragma unroll
-              for (int ct = 0; ct < NT; ++ct) acc[j][ct] = M::mma(zf[ct][ss], pb[ss], acc[j][ct]);
-          }
+          for (int j = 0; j < QT; ++j) s[j] = M::mma(xf, of[j][ks], s[j]);
         }
-      } else {
+        frag zf[NT][M::ACC_KSTEPS];
 #pragma unroll
-        for (int st = 0; st < KT / 32; ++st)
+        for (int ct = 0; ct < NT; ++ct)
 #pragma unroll
-          for (int j = 0; j < QT; ++j) {
-            const int ss0 = s0 + 32 * st, lo = t0 + tw[j] * 32;
-            if (!fm_tile_active<OWN>(causal, ss0, lo, G.send)) continue;
-            const bool edge = fm_tile_edge<OWN>(causal, ss0, lo, A.n_str);
-            int wlo, whi;
-            fm_tile_window<OWN>(causal, ss0, lo, lr, A.n_str, wlo, whi);
-            fm_f32x16 s = fm_zero16();
+          for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
+            zf[ct][ss] = M::load_perm(Zt + (32 * ct + lr) * PV + 32 * st, ss, lh);
 #pragma unroll
-            for (int ks = 0; ks < NKS; ++ks)
-              s = M::mma(M::load(Xs + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL), of[j][ks], s);
-            frag pb[M::ACC_KSTEPS];
-            const float gs = TM::fwd(s, coef, edge, wlo, whi, lh, pb);
-            if (OWN == FM_OWN_Q) gsum[j] += gs;
+        for (int j = 0; j < QT; ++j) {
+          const int ss0 = s0 + 32 * st, lo = t0 + tw[j] * 32;
+          const bool edge = fm_tile_edge<OWN>(causal, ss0, lo, A.n_str);
+          int wlo, whi;
+          fm_tile_window<OWN>(causal, ss0, lo, lr, A.n_str, wlo, whi);
+          frag pb[M::ACC_KSTEPS];
+          const float gs = TM::fwd(s[j], coef, edge, wlo, whi, lh, pb);
+          if (OWN == FM_OWN_Q) gsum[j] += gs;
 #pragma unroll
-            for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
+          for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
 #pragma unroll
-              for (int ct = 0; ct < NT; ++ct)
-                acc[j][ct] = M::mma(M::load_perm(Zt + (32 * ct + lr) * PV + 32 * st, ss, lh), pb[ss], acc[j][ct]);
-          }
+            for (int ct = 0; ct < NT; ++ct) acc[j][ct] = M::mma(zf[ct][ss], pb[ss], acc[j][ct]);
+        }
       }
       buf ^= 1;
     }
@@ -418,7 +389,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_DS)) k_ds(T
   typedef Mma<E> M;
   typedef TileMath<E> TM;
   typedef typename M::frag frag;
-  constexpr int NT = C::NT, NKS = C::NKS, QW = C::QW, PQ = C::PQ, KT = C::KT, PV = C::PV;
+  constexpr int NT = C::NT, NKS = C::NKS, QW = C::QW, PQ = C::PQ, KT = C::KT_DS, PV = C::PV_DS;
   constexpr int NBUF = C::DS_NBUF;
   constexpr int STAGE = C::DS_STAGE;
   FM_DYN_SMEM(smem);
@@ -507,76 +478,44 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_DS)) k_ds(T
         if (OWN == FM_OWN_K && tid < KT) cs[tid] = creg;
       }
       FM_SYNC();
-      FM_SCHED_FENCE();
-      if (G.fast_stage(causal, s0, KT, A.n_str)) {
+      // One code path for every tile (see k_pv).  The score fragments and the transposed fragments
+      // serve all own tiles of the wavefront; gh.v is formed per own tile.
 #pragma unroll
-        for (int st = 0; st < KT / 32; ++st) {
-          // the score fragments and the transposed fragments serve both own tiles; gh.v is formed
-          // per own tile (its fragments are read again) to keep the live accumulators within
-          // the register budget of two workgroups per CU
-          fm_f32x16 s[QT];
+      for (int st = 0; st < KT / 32; ++st) {
+        fm_f32x16 s[QT];
 #pragma unroll
-          for (int j = 0; j < QT; ++j) s[j] = fm_zero16();
+        for (int j = 0; j < QT; ++j) s[j] = fm_zero16();
 #pragma unroll
-          for (int ks = 0; ks < NKS; ++ks) {
-            const frag xf = M::load(Xs + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL);
+        for (int ks = 0; ks < NKS; ++ks) {
+          const frag xf = M::load(Xs + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL);
 #pragma unroll
-            for (int j = 0; j < QT; ++j) s[j] = M::mma(xf, of[j][ks], s[j]);
-          }
-          frag zf[NT][M::ACC_KSTEPS], crow[M::ACC_KSTEPS];
-#pragma unroll
-          for (int ss = 0; ss < M::ACC_KSTEPS; ++ss) {
-            if (OWN == FM_OWN_K) crow[ss] = M::load_perm(cs + 32 * st, ss, lh);
-#pragma unroll
-            for (int mt = 0; mt < NT; ++mt) zf[mt][ss] = M::load_perm(Zt + (32 * mt + lr) * PV + 32 * st, ss, lh);
-          }
-#pragma unroll
-          for (int j = 0; j < QT; ++j) {
-            FM_SCHED_FENCE();
-            fm_f32x16 dp = fm_zero16();
-            const E* yrow = Ys + (32 * st + lr) * PQ + lh * M::KPL + FM_OPAQUE_ZERO();
-#pragma unroll
-            for (int ks = 0; ks < NKS; ++ks) dp = M::mma(M::load(yrow + ks * M::KSTEP), of2[j][ks], dp);
-            frag db[M::ACC_KSTEPS];
-            if (OWN == FM_OWN_Q) TM::dsc(s[j], dp, cs_own[j], coef, false, 0, 0, lh, db);
-            else TM::dsr(s[j], dp, crow, coef, false, 0, 0, lh, db);
-#pragma unroll
-            for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
-#pragma unroll
-              for (int mt = 0; mt < NT; ++mt) acc[j][mt] = M::mma(zf[mt][ss], db[ss], acc[j][mt]);
-          }
+          for (int j = 0; j < QT; ++j) s[j] = M::mma(xf, of[j][ks], s[j]);
         }
-      } else {
+        frag zf[NT][M::ACC_KSTEPS], crow[M::ACC_KSTEPS];
 #pragma unroll
-        for (int st = 0; st < KT / 32; ++st)
+        for (int ss = 0; ss < M::ACC_KSTEPS; ++ss) {
+          if (OWN == FM_OWN_K) crow[ss] = M::load_perm(cs + 32 * st, ss, lh);
 #pragma unroll
-          for (int j = 0; j < QT; ++j) {
-            const int ss0 = s0 + 32 * st, lo = t0 + tw[j] * 32;
-            if (!fm_tile_active<OWN>(causal, ss0, lo, G.send)) continue;
-            const bool edge = fm_tile_edge<OWN>(causal, ss0, lo, A.n_str);
-            int wlo, whi;
-            fm_tile_window<OWN>(causal, ss0, lo, lr, A.n_str, wlo, whi);
-            fm_f32x16 s = fm_zero16(), dp = fm_zero16();
+          for (int mt = 0; mt < NT; ++mt) zf[mt][ss] = M::load_perm(Zt + (32 * mt + lr) * PV + 32 * st, ss, lh);
+        }
 #pragma unroll
-            for (int ks = 0; ks < NKS; ++ks) {
-              s = M::mma(M::load(Xs + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL), of[j][ks], s);
-              dp = M::mma(M::load(Ys + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL), of2[j][ks], dp);
-            }
-            frag db[M::ACC_KSTEPS];
-            if (OWN == FM_OWN_Q) {
-              TM::dsc(s, dp, cs_own[j], coef, edge, wlo, whi, lh, db);
-            } else {
-              frag crow[M::ACC_KSTEPS];
+        for (int j = 0; j < QT; ++j) {
+          const int ss0 = s0 + 32 * st, lo = t0 + tw[j] * 32;
+          const bool edge = fm_tile_edge<OWN>(causal, ss0, lo, A.n_str);
+          int wlo, whi;
+          fm_tile_window<OWN>(causal, ss0, lo, lr, A.n_str, wlo, whi);
+          fm_f32x16 dp = fm_zero16();
+          const E* yrow = Ys + (32 * st + lr) * PQ + lh * M::KPL + (QT > 1 ? FM_OPAQUE_ZERO() : 0);
 #pragma unroll
-              for (int ss = 0; ss < M::ACC_KSTEPS; ++ss) crow[ss] = M::load_perm(cs + 32 * st, ss, lh);
-              TM::dsr(s, dp, crow, coef, edge, wlo, whi, lh, db);
-            }
+          for (int ks = 0; ks < NKS; ++ks) dp = M::mma(M::load(yrow + ks * M::KSTEP), of2[j][ks], dp);
+          frag db[M::ACC_KSTEPS];
+          if (OWN == FM_OWN_Q) TM::dsc(s[j], dp, cs_own[j], coef, edge, wlo, whi, lh, db);
+          else TM::dsr(s[j], dp, crow, coef, edge, wlo, whi, lh, db);
 #pragma unroll
-            for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
+          for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
 #pragma unroll
-              for (int mt = 0; mt < NT; ++mt)
-                acc[j][mt] = M::mma(M::load_perm(Zt + (32 * mt + lr) * PV + 32 * st, ss, lh), db[ss], acc[j][mt]);
-          }
+            for (int mt = 0; mt < NT; ++mt) acc[j][mt] = M::mma(zf[mt][ss], db[ss], acc[j][mt]);
+        }
       }
       if (NBUF == 1) FM_SYNC(); else buf ^= 1;
     }
