@@ -285,18 +285,25 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
     TileRegs<E, DH, KT> rz;
     const E* xb = A.xr + int64_t(bh) * A.npad_str * DH;
     const E* zb = A.zt + int64_t(bh) * DH * A.npad_str;
-    rx.load(xb + int64_t(G.sbeg) * DH, DH, tid);
-    rz.load(zb + G.sbeg, A.npad_str, tid);
+    // Stages are walked so that all blocks of a batch*head start at the same end of the stream
+    // (queries start at the first key of the segment, keys at its last query): blocks that run at
+    // the same time then read the same tiles at about the same time and share them in the L2.
+    const int nst = (G.send - G.sbeg + KT - 1) / KT;
+    const int s_first = OWN == FM_OWN_Q ? G.sbeg : G.sbeg + KT * (nst - 1);
+    const int s_step = OWN == FM_OWN_Q ? KT : -KT;
+    rx.load(xb + int64_t(s_first) * DH, DH, tid);
+    rz.load(zb + s_first, A.npad_str, tid);
     int buf = 0;
-    for (int s0 = G.sbeg; s0 < G.send; s0 += KT) {
+    for (int s0 = s_first; OWN == FM_OWN_Q ? (s0 < G.send) : (s0 >= G.sbeg); s0 += s_step) {
       E* Xs = Own + buf * STAGE;                        // the own rows and the slabs are spent
       E* Zt = Xs + KT * PQ;
       rx.store(Xs, PQ, tid);
       rz.store(Zt, PV, tid);
       FM_SYNC();
-      if (s0 + KT < G.send) {
-        rx.load(xb + int64_t(s0 + KT) * DH, DH, tid);
-        rz.load(zb + s0 + KT, A.npad_str, tid);
+      const int sn = s0 + s_step;
+      if (OWN == FM_OWN_Q ? (sn < G.send) : (sn >= G.sbeg)) {
+        rx.load(xb + int64_t(sn) * DH, DH, tid);
+        rz.load(zb + sn, A.npad_str, tid);
       }
       // One code path for every tile: the products always run, and a tile that touches the mask
       // or the end of the sequence (a wavefront-uniform test) zeroes the entries outside its row
@@ -461,23 +468,30 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_DS)) k_ds(T
     const E* yb = A.yr + int64_t(bh) * A.npad_str * DH;
     const E* zb = A.zt + int64_t(bh) * DH * A.npad_str;
     const E* cvb = A.cv + int64_t(bh) * A.npad_str;    // own = keys: c of the streamed queries
+    // stage order: see k_pv
+    const int nst = (G.send - G.sbeg + KT - 1) / KT;
+    const int s_first = OWN == FM_OWN_Q ? G.sbeg : G.sbeg + KT * (nst - 1);
+    const int s_step = OWN == FM_OWN_Q ? KT : -KT;
+    TileRegs<E, KT, DH> rx, ry;
+    TileRegs<E, DH, KT> rz;
+    E creg = E(0.f);
+    rx.load(xb + int64_t(s_first) * DH, DH, tid);
+    ry.load(yb + int64_t(s_first) * DH, DH, tid);
+    rz.load(zb + s_first, A.npad_str, tid);
+    if (OWN == FM_OWN_K && tid < KT) creg = cvb[s_first + tid];
     int buf = 0;
-    for (int s0 = G.sbeg; s0 < G.send; s0 += KT) {
-      // no register prefetch across the products: the second workgroup of the CU covers the
-      // load latency, and the registers go to the fragments of both own tiles instead
+    for (int s0 = s_first; OWN == FM_OWN_Q ? (s0 < G.send) : (s0 >= G.sbeg); s0 += s_step) {
       E* Xs = Own + buf * STAGE; E* Ys = Xs + KT * PQ; E* Zt = Ys + KT * PQ; E* cs = Zt + DH * PV;
-      {
-        TileRegs<E, KT, DH> rx, ry;
-        TileRegs<E, DH, KT> rz;
-        E creg = E(0.f);
-        rx.load(xb + int64_t(s0) * DH, DH, tid);
-        ry.load(yb + int64_t(s0) * DH, DH, tid);
-        rz.load(zb + s0, A.npad_str, tid);
-        if (OWN == FM_OWN_K && tid < KT) creg = cvb[s0 + tid];
-        rx.store(Xs, PQ, tid); ry.store(Ys, PQ, tid); rz.store(Zt, PV, tid);
-        if (OWN == FM_OWN_K && tid < KT) cs[tid] = creg;
-      }
+      rx.store(Xs, PQ, tid); ry.store(Ys, PQ, tid); rz.store(Zt, PV, tid);
+      if (OWN == FM_OWN_K && tid < KT) cs[tid] = creg;
       FM_SYNC();
+      const int sn = s0 + s_step;
+      if (OWN == FM_OWN_Q ? (sn < G.send) : (sn >= G.sbeg)) {
+        rx.load(xb + int64_t(sn) * DH, DH, tid);
+        ry.load(yb + int64_t(sn) * DH, DH, tid);
+        rz.load(zb + sn, A.npad_str, tid);
+        if (OWN == FM_OWN_K && tid < KT) creg = cvb[sn + tid];
+      }
       // One code path for every tile (see k_pv).  The score fragments and the transposed fragments
       // serve all own tiles of the wavefront; gh.v is formed per own tile.
 #pragma unroll
