@@ -504,13 +504,8 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 ? 2 : 1)
 // ------------------------------------------------------------------------------
 // LDS sizes (in elements of E) used by k_pv / k_ds; the host computes the dynamic LDS
 // bytes from the same struct.
-// Tuning knobs of the _Float16 token kernels (the values are the ones measured best on MI355X).
-#ifndef FM_TUNE_OCC_PV
-#define FM_TUNE_OCC_PV 4
-#endif
-#ifndef FM_TUNE_OCC_DS
-#define FM_TUNE_OCC_DS 3
-#endif
+// Stream tokens per stage of the dense loops of the _Float16 token kernels (64-token stages
+// measured slower on MI355X: the larger tile movers cost registers).
 #ifndef FM_TUNE_KT_PV
 #define FM_TUNE_KT_PV 32
 #endif
@@ -525,14 +520,16 @@ struct TokCfg {
   static constexpr int QW = 4 * QT * 32;            // tokens per workgroup
   static constexpr int PQ = DH + M::PAD;            // pitch of row-major token tiles
   static constexpr int PS = DH + M::PAD;            // pitch of state rows
-  // _Float16: one tile per wavefront, small slabs and stages, so that four (k_pv) or three
-  // (k_ds) workgroups share a CU: 12 to 16 wavefronts hide each other's LDS and MFMA latency.
-  // On MI355X at B*H = 32, N = 4096, D = 64 this measured faster than two tiles per wavefront
-  // at two workgroups per CU, dense tiles 0.47 vs 0.56 ms for the four kernels together.
-  static constexpr int OCC_PV = sizeof(E) == 2 ? FM_TUNE_OCC_PV : 1;   // workgroups per CU the kernels are sized for
-  static constexpr int OCC_DS = sizeof(E) == 2 ? FM_TUNE_OCC_DS : 1;
-  static constexpr int SA = sizeof(E) == 2 ? 1 : 2;       // values of a per state slab
-  // (64-token stages for _Float16 measured slower on MI355X: the larger tile movers cost registers)
+  // _Float16, QT = 1: one tile per wavefront, small slabs and stages, so that four (k_pv) or three
+  // (k_ds) workgroups share a CU: 12 to 16 wavefronts hide each other's LDS and MFMA latency.  On
+  // MI355X at B*H = 32, N = 4096, D = 64 this measured faster on dense tiles than two tiles per
+  // wavefront at two workgroups per CU (0.47 vs 0.56 ms for the four kernels together).
+  // _Float16, QT = 2: two tiles per wavefront share every state fragment read from LDS and halve
+  // the state bytes staged per token; used by k_ds when there are states to read (dQ + dK
+  // 0.20 vs 0.23 ms at the same shape with 1024-token segments).
+  static constexpr int OCC_PV = sizeof(E) == 2 ? (QT == 1 ? 4 : 2) : 1;   // workgroups per CU the kernels are sized for
+  static constexpr int OCC_DS = sizeof(E) == 2 ? (QT == 1 ? 3 : 2) : 1;
+  static constexpr int SA = sizeof(E) == 2 ? QT : 2;                      // values of a per state slab
   static constexpr int KT_PV = sizeof(E) == 2 ? FM_TUNE_KT_PV : 64;   // stream tokens per stage of the dense loop, k_pv
   static constexpr int KT_DS = sizeof(E) == 2 ? FM_TUNE_KT_DS : 64;   //                                           k_ds
   static constexpr int PV_PV = KT_PV + M::PAD;      // pitch of the transposed token tiles
