@@ -45,9 +45,9 @@ WORKLOAD = dict(name="configs[1]: causal order-2 fwd+bwd", B=4, H=8, N=4096, D=6
 # each, and dQ also carries the unit of the prefix rebuild it is spared by reading the forward's.
 # Without (a sequence short enough for one segment) each kernel carries its walk as well.
 UNITS_STATE = {"build": 1, "fwd": 1, "dq": 2, "dk": 1, "dv": 1}
-UNITS_DENSE = {"fwd": 2, "dq": 2, "dk": 2, "dv": 1}
+UNITS_DENSE = {"fwd": 2, "dq": 2, "dk": 2, "dv": 1, "dkv": 3}
 # 32x32x16 MFMA instructions per 32x32 score tile in the dense loops of each kernel
-MFMA_PER_TILE = {"fwd": 8, "dv": 8, "dq": 12, "dk": 12}
+MFMA_PER_TILE = {"fwd": 8, "dv": 8, "dq": 12, "dk": 12, "dkv": 16}
 
 
 def alg_flops_unit(bh: int, n: int, d: int, p: int) -> float:
@@ -163,7 +163,7 @@ def main() -> int:
         # what the matrix cores actually execute when one segment covers the sequence: causal 32x32 tiles only
         nt = (N + 31) // 32
         tiles = bh * nt * (nt + 1) // 2
-        executed = sum(MFMA_PER_TILE.values()) * tiles * 2.0 * 32 * 32 * 16
+        executed = sum(MFMA_PER_TILE[nme] for nme in per_kernel if nme in MFMA_PER_TILE) * tiles * 2.0 * 32 * 32 * 16
         roofline["executed_mfma"] = {"flop_per_step": executed,
                                      "achieved": executed / (ms_per_step * 1e-3) / 1e12,
                                      "frac": executed / (ms_per_step * 1e-3) / 1e12 / peak}

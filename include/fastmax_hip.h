@@ -121,7 +121,8 @@ int fastmax_version(void);
 /* Per-kernel timing for benchmarks (no counterpart in the reference).  Between begin and end the
  * library brackets every kernel it launches with HIP events on the launch stream; end waits for
  * them and returns how many launches were recorded, filling up to `capacity` entries with the
- * kernel id (0 transpose, 1 backward prep, 2 state build, 3 forward, 4 dQ, 5 dK, 6 normalise, 7 dV)
+ * kernel id (0 transpose, 1 backward prep, 2 state build, 3 forward, 4 dQ, 5 dK, 6 normalise, 7 dV,
+ * 8 dK and dV in one pass)
  * and its duration.  Process-global and not re-entrant: do not use from concurrent threads. */
 int fastmax_profile_begin(void);
 int fastmax_profile_end(int* kernel_ids, float* milliseconds, int capacity);

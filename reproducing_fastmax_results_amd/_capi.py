@@ -212,7 +212,7 @@ class FastmaxLib:
         self.check(st, "fastmax_normalize")
         return out
 
-    KERNEL_NAMES = ("transpose", "prep_bwd", "build", "fwd", "dq", "dk", "normalize", "dv")
+    KERNEL_NAMES = ("transpose", "prep_bwd", "build", "fwd", "dq", "dk", "normalize", "dv", "dkv")
 
     def profile_begin(self) -> None:
         self.lib.fastmax_profile_begin()

@@ -21,7 +21,7 @@ inline void fm_allow_lds(const void* fn, size_t bytes) {
 #endif
 
 // ---- optional per-kernel timing (used by the benchmark; not re-entrant) --------
-enum { FM_K_TRANSPOSE = 0, FM_K_PREP_BWD = 1, FM_K_BUILD = 2, FM_K_FWD = 3, FM_K_DQ = 4, FM_K_DK = 5, FM_K_NORM = 6, FM_K_DV = 7 };
+enum { FM_K_TRANSPOSE = 0, FM_K_PREP_BWD = 1, FM_K_BUILD = 2, FM_K_FWD = 3, FM_K_DQ = 4, FM_K_DK = 5, FM_K_NORM = 6, FM_K_DV = 7, FM_K_DKV = 8 };
 #if defined(FM_HOSTSIM)
 struct ProfScope { ProfScope(int, fm_stream_t) {} };
 #else
@@ -47,7 +47,6 @@ inline size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
 struct Plan {
   bool half;            // compute type: _Float16 (bf16 interface) or float
   int esz;              // sizeof compute element
-  int qw;               // tokens per workgroup of the token-side kernels
   int L, nseg, nslots;
   bool use_state, quad;
   int npad_q, npad_k;
@@ -86,7 +85,6 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   if (st != FASTMAX_OK) return st;
   p.half = d->dtype == FASTMAX_BF16;
   p.esz = p.half ? 2 : 4;
-  p.qw = 128;
   p.npad_q = int(round_up(d->nq, 256));
   p.npad_k = int(round_up(d->nk, 256));
   p.quad = d->p == 2 && d->a2 != 0.0f;
@@ -201,7 +199,7 @@ template <typename E, int DH, int QT> size_t tok_lds_bytes() {
   size_t body = size_t(C::QW) * C::PQ * sizeof(E) + region;
   const size_t outst = size_t(C::QW) * (DH + 1) * 4;
   const size_t pv = size_t(2) * C::PV_STAGE * sizeof(E);
-  const size_t ds = size_t(C::DS_NBUF) * C::DS_STAGE * sizeof(E);
+  const size_t ds = size_t(C::DS_NBUF) * C::DS_STAGE2 * sizeof(E);
   if (outst > body) body = outst;
   if (pv > body) body = pv;
   if (ds > body) body = ds;
@@ -210,7 +208,8 @@ template <typename E, int DH, int QT> size_t tok_lds_bytes() {
 
 template <typename TIO, typename E> void tok_common(TokArgs<TIO, E>& a, const FastmaxDesc* d, const Plan& p) {
   a.own_io = TRef<const TIO>{nullptr, 0, 0, 0};
-  a.own_r = nullptr; a.own2_r = nullptr; a.cv = nullptr; a.xr = nullptr; a.yr = nullptr; a.zt = nullptr;
+  a.own_r = nullptr; a.own2_r = nullptr; a.cv = nullptr; a.xr = nullptr; a.yr = nullptr; a.zt = nullptr; a.zt2 = nullptr;
+  a.out2 = TRef<TIO>{nullptr, 0, 0, 0}; a.out2_scale = 1.0f;
   a.g = nullptr; a.g_s_bh = 0; a.g_s_n = 0;
   a.nslots = p.nslots; a.L = p.L; a.nseg = p.nseg; a.causal = d->mask != 0; a.use_state = p.use_state;
   a.quad = p.quad; a.a0 = p.a0; a.a1 = p.a1; a.a2 = p.a2; a.sc = p.sc; a.out_scale = 1.0f; a.zscale = 1.0f;
@@ -227,13 +226,13 @@ int launch_pv(const TokArgs<TIO, E>& a, int bh, int kernel_id, fm_stream_t strea
   return fm_after_launch();
 }
 
-template <typename TIO, typename E, int DH, int QT, int OWN>
+template <typename TIO, typename E, int DH, int QT, int OWN, int DV = 0>
 int launch_ds(const TokArgs<TIO, E>& a, int bh, int kernel_id, fm_stream_t stream) {
   typedef TokCfg<E, DH, QT> C;
   const size_t lds = tok_lds_bytes<E, DH, QT>();
-  fm_allow_lds(reinterpret_cast<const void*>(&k_ds<TIO, E, DH, QT, OWN>), lds);
+  fm_allow_lds(reinterpret_cast<const void*>(&k_ds<TIO, E, DH, QT, OWN, DV>), lds);
   ProfScope prof(kernel_id, stream);
-  FM_KERNEL_LAUNCH((k_ds<TIO, E, DH, QT, OWN>), fm_dim3((a.n_own + C::QW - 1) / C::QW, bh), fm_dim3(FM_THREADS), lds,
+  FM_KERNEL_LAUNCH((k_ds<TIO, E, DH, QT, OWN, DV>), fm_dim3((a.n_own + C::QW - 1) / C::QW, bh), fm_dim3(FM_THREADS), lds,
                    stream, a);
   return fm_after_launch();
 }

@@ -157,7 +157,8 @@ k_transpose(const TIO* FM_RESTRICT x, int64_t s_bh, int64_t s_n, int vec, int n,
 // ------------------------------------------------------------------------------
 // k_prep_bwd: per token  gh = gscale * dO / g,  c = gh . o,  q' = qscale * q ; writes
 //   gh  [bh][npad][DH]  (row-major, compute type)      ght [bh][DH][npad]
-//   qt  [bh][DH][npad]  (q' transposed)                 qct [bh][DH][npad]  (c_i q'_i)
+//   qt  [bh][DH][npad]  (q' transposed)                 qct [bh][DH][npad]  (c_i q'_i; skipped when null:
+//                                                        only the state walk reads it)
 //   qr  [bh][npad][DH]  (q' row-major)
 //   cv  [bh][npad]      (c, compute type)
 // gscale is a power of two that keeps gh inside the _Float16 range for long sequences
@@ -224,7 +225,7 @@ k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, const floa
     const int64_t off = ob + int64_t(d) * npad + tk;
     *reinterpret_cast<fm_u32x4*>(ght + off) = *reinterpret_cast<const fm_u32x4*>(&tg[d * PT + tk]);
     *reinterpret_cast<fm_u32x4*>(qt + off) = *reinterpret_cast<const fm_u32x4*>(&tq[d * PT + tk]);
-    *reinterpret_cast<fm_u32x4*>(qct + off) = *reinterpret_cast<const fm_u32x4*>(&tc[d * PT + tk]);
+    if (qct) *reinterpret_cast<fm_u32x4*>(qct + off) = *reinterpret_cast<const fm_u32x4*>(&tc[d * PT + tk]);
   }
 }
 
@@ -538,6 +539,7 @@ struct TokCfg {
   static constexpr int SLAB = SA * DH * PS;         // elements per slab buffer
   static constexpr int PV_STAGE = KT_PV * PQ + DH * PV_PV;                // k_pv: stream rows, stream transposed
   static constexpr int DS_STAGE = 2 * KT_DS * PQ + DH * PV_DS + KT_DS;    // k_ds: two row tiles, transposed tile, c values
+  static constexpr int DS_STAGE2 = DS_STAGE + DH * PV_DS;                 // k_ds with dV: + gh transposed
   static constexpr int DS_NBUF = sizeof(E) == 2 ? 2 : 1;
 };
 

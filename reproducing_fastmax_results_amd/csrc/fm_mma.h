@@ -161,6 +161,7 @@ template <> struct CE<float> {
 //   fwd : P  = a0 + s (a1 + a2 s)                      and the lane's partial row-sum of P
 //   dsc : dS = (a1 + 2 a2 s) (dp - c),  c one scalar per lane
 //   dsr : the same with c per accumulator row (given as fragments in accumulator order)
+//   both: P and dS (c per accumulator row) from one conversion of the score tile
 // The _Float16 instantiation evaluates the polynomials on packed halves (v_pk_fma_f16)
 // and sums with v_dot2_f32_f16, which keeps the vector pipe off the critical path.
 template <typename E> struct TileMath;
@@ -198,6 +199,18 @@ template <> struct TileMath<float> {
     for (int e = 0; e < 16; ++e) {
       float ds = (k.a1 + k.ta2 * s[e]) * (dp[e] - crow[e]);
       if (edge) { const int r = fm_acc_row(e, lh); if (r < lo || r > hi) ds = 0.f; }
+      db[e] = ds;
+    }
+  }
+  static FM_DEVICE void both(const fm_f32x16& s, const fm_f32x16& dp, const frag* crow, const Coef& k, bool edge, int lo,
+                             int hi, int lh, frag* pb, frag* db) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const float x = s[e];
+      float pv = k.a0 + x * (k.a1 + k.a2 * x);
+      float ds = (k.a1 + k.ta2 * x) * (dp[e] - crow[e]);
+      if (edge) { const int r = fm_acc_row(e, lh); if (r < lo || r > hi) { pv = 0.f; ds = 0.f; } }
+      pb[e] = pv;
       db[e] = ds;
     }
   }
@@ -276,5 +289,18 @@ template <> struct TileMath<fm_half> {
         put2(db[ss], i, (x * k.ta2 + k.a1) * (cvt2(dp[e], dp[e + 1]) - get2(crow[ss], i)));
       }
     if (edge) { FM_KEEP_BRANCH(); window_frags(db, lo, hi, lh); }
+  }
+  static FM_DEVICE void both(const fm_f32x16& s, const fm_f32x16& dp, const frag* crow, const Coef& k, bool edge, int lo,
+                             int hi, int lh, frag* pb, frag* db) {
+#pragma unroll
+    for (int ss = 0; ss < 2; ++ss)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int e = 8 * ss + 2 * i;
+        const fm_half2 x = cvt2(s[e], s[e + 1]);
+        put2(pb[ss], i, (x * k.a2 + k.a1) * x + k.a0);
+        put2(db[ss], i, (x * k.ta2 + k.a1) * (cvt2(dp[e], dp[e + 1]) - get2(crow[ss], i)));
+      }
+    if (edge) { FM_KEEP_BRANCH(); window_frags(pb, lo, hi, lh); window_frags(db, lo, hi, lh); }
   }
 };

@@ -32,14 +32,17 @@ template <typename TIO, typename E> struct TokArgs {
   const E* xr;              // stream rows that form the scores      [bh][npad_str][DH]
   const E* yr;              // k_ds: stream rows that form gh.v      [bh][npad_str][DH]
   const E* zt;              // stream tokens, transposed             [bh][DH][npad_str]
+  const E* zt2;             // k_ds with dV: gh transposed           [bh][DH][npad_str]
   int npad_own, npad_str;
   const E* big; const float* small; int nslots;
   TRef<TIO> out;
+  TRef<TIO> out2;           // k_ds with dV: dV
   float* g; int64_t g_s_bh, g_s_n;      // k_pv, own = queries: denominators
   int n_own, n_str, L, nseg, causal, use_state, quad;
   float a0, a1, a2;                     // f(x) = a0 + a1 x + a2 x^2
   float sc;                             // sqrt(1/tau)
   float out_scale;                      // factor on the stored gradient
+  float out2_scale;                     // k_ds with dV: factor on dV
   float zscale;                         // factor on the Z of the state (k_ds)
 };
 
@@ -389,16 +392,19 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
 // LDS: va, vb | own rows [QW][PQ] | region (Z, then state slabs); the dense stages
 // (stream rows for the scores, stream rows for gh.v, stream transposed, c values)
 // and the output staging lie over the own rows and the region once they are spent.
+// DV = 1 (own = keys, sequences of one segment): the same pass also forms dV from the
+// score tiles it already has, P = f(S), dV^T += gh^T P, which saves the four score
+// products per tile that a separate k_pv launch would repeat.
 // ------------------------------------------------------------------------------
-template <typename TIO, typename E, int DH, int QT, int OWN>
-FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_DS)) k_ds(TokArgs<TIO, E> A) {
+template <typename TIO, typename E, int DH, int QT, int OWN, int DV>
+FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS)) k_ds(TokArgs<TIO, E> A) {
   typedef TokCfg<E, DH, QT> C;
   typedef Mma<E> M;
   typedef TileMath<E> TM;
   typedef typename M::frag frag;
   constexpr int NT = C::NT, NKS = C::NKS, QW = C::QW, PQ = C::PQ, KT = C::KT_DS, PV = C::PV_DS;
   constexpr int NBUF = C::DS_NBUF;
-  constexpr int STAGE = C::DS_STAGE;
+  constexpr int STAGE = DV ? C::DS_STAGE2 : C::DS_STAGE;
   FM_DYN_SMEM(smem);
   float* vecs = reinterpret_cast<float*>(smem);
   E* Own = reinterpret_cast<E*>(vecs + 2 * DH);       // [QW][PQ]
@@ -439,11 +445,15 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_DS)) k_ds(T
       of2[j][ks] = M::load(o2 + ks * M::KSTEP);
     }
   }
-  fm_f32x16 acc[QT][NT];
+  fm_f32x16 acc[QT][NT], av[DV ? QT : 1][NT];
 #pragma unroll
   for (int j = 0; j < QT; ++j)
 #pragma unroll
     for (int mt = 0; mt < NT; ++mt) acc[j][mt] = fm_zero16();
+#pragma unroll
+  for (int j = 0; j < (DV ? QT : 1); ++j)
+#pragma unroll
+    for (int mt = 0; mt < NT; ++mt) av[j][mt] = fm_zero16();
 
   if (G.use_state) {
     // - c * (va[m] + sum_l Z[m][l] own_l)   (c = c_i for own = queries; folded into Z and va for own = keys)
@@ -468,21 +478,25 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_DS)) k_ds(T
     const E* yb = A.yr + int64_t(bh) * A.npad_str * DH;
     const E* zb = A.zt + int64_t(bh) * DH * A.npad_str;
     const E* cvb = A.cv + int64_t(bh) * A.npad_str;    // own = keys: c of the streamed queries
+    const E* z2b = DV ? A.zt2 + int64_t(bh) * DH * A.npad_str : nullptr;
     // stage order: see k_pv
     const int nst = (G.send - G.sbeg + KT - 1) / KT;
     const int s_first = OWN == FM_OWN_Q ? G.sbeg : G.sbeg + KT * (nst - 1);
     const int s_step = OWN == FM_OWN_Q ? KT : -KT;
     TileRegs<E, KT, DH> rx, ry;
-    TileRegs<E, DH, KT> rz;
+    TileRegs<E, DH, KT> rz, rz2;
     E creg = E(0.f);
     rx.load(xb + int64_t(s_first) * DH, DH, tid);
     ry.load(yb + int64_t(s_first) * DH, DH, tid);
     rz.load(zb + s_first, A.npad_str, tid);
+    if (DV) rz2.load(z2b + s_first, A.npad_str, tid);
     if (OWN == FM_OWN_K && tid < KT) creg = cvb[s_first + tid];
     int buf = 0;
     for (int s0 = s_first; OWN == FM_OWN_Q ? (s0 < G.send) : (s0 >= G.sbeg); s0 += s_step) {
       E* Xs = Own + buf * STAGE; E* Ys = Xs + KT * PQ; E* Zt = Ys + KT * PQ; E* cs = Zt + DH * PV;
+      E* Zt2 = cs + KT;
       rx.store(Xs, PQ, tid); ry.store(Ys, PQ, tid); rz.store(Zt, PV, tid);
+      if (DV) rz2.store(Zt2, PV, tid);
       if (OWN == FM_OWN_K && tid < KT) cs[tid] = creg;
       FM_SYNC();
       const int sn = s0 + s_step;
@@ -490,6 +504,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_DS)) k_ds(T
         rx.load(xb + int64_t(sn) * DH, DH, tid);
         ry.load(yb + int64_t(sn) * DH, DH, tid);
         rz.load(zb + sn, A.npad_str, tid);
+        if (DV) rz2.load(z2b + sn, A.npad_str, tid);
         if (OWN == FM_OWN_K && tid < KT) creg = cvb[sn + tid];
       }
       // One code path for every tile (see k_pv).  The score fragments and the transposed fragments
@@ -522,13 +537,18 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_DS)) k_ds(T
           const E* yrow = Ys + (32 * st + lr) * PQ + lh * M::KPL + (QT > 1 ? FM_OPAQUE_ZERO() : 0);
 #pragma unroll
           for (int ks = 0; ks < NKS; ++ks) dp = M::mma(M::load(yrow + ks * M::KSTEP), of2[j][ks], dp);
-          frag db[M::ACC_KSTEPS];
-          if (OWN == FM_OWN_Q) TM::dsc(s[j], dp, cs_own[j], coef, edge, wlo, whi, lh, db);
+          frag db[M::ACC_KSTEPS], pb[M::ACC_KSTEPS];
+          if (DV) TM::both(s[j], dp, crow, coef, edge, wlo, whi, lh, pb, db);
+          else if (OWN == FM_OWN_Q) TM::dsc(s[j], dp, cs_own[j], coef, edge, wlo, whi, lh, db);
           else TM::dsr(s[j], dp, crow, coef, edge, wlo, whi, lh, db);
 #pragma unroll
           for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
 #pragma unroll
-            for (int mt = 0; mt < NT; ++mt) acc[j][mt] = M::mma(zf[mt][ss], db[ss], acc[j][mt]);
+            for (int mt = 0; mt < NT; ++mt) {
+              acc[j][mt] = M::mma(zf[mt][ss], db[ss], acc[j][mt]);
+              if (DV)
+                av[j][mt] = M::mma(M::load_perm(Zt2 + (32 * mt + lr) * PV + 32 * st, ss, lh), pb[ss], av[j][mt]);
+            }
         }
       }
       if (NBUF == 1) FM_SYNC(); else buf ^= 1;
@@ -537,4 +557,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_DS)) k_ds(T
   }
   fm_store_tokens<TIO, E, DH, QT>(acc, xrow, nullptr, A.out_scale, reinterpret_cast<float*>(Own), A.out, bh, t0,
                                   A.n_own, tid);
+  if (DV)
+    fm_store_tokens<TIO, E, DH, QT>(av, xrow, nullptr, A.out2_scale, reinterpret_cast<float*>(Own), A.out2, bh, t0,
+                                    A.n_own, tid);
 }
