@@ -371,6 +371,7 @@ int fastmax_backward_saved(const FastmaxDesc* desc, const void* q, const void* k
 }
 
 int fastmax_normalize(const FastmaxNormDesc* desc, const void* x, void* y, float* stats, void* hip_stream) {
+  ProfScope prof(FM_K_NORM, static_cast<fm_stream_t>(hip_stream));   // the whole pass (its kernels together)
   return fm_normalize_dispatch(desc, x, y, stats, static_cast<fm_stream_t>(hip_stream));
 }
 

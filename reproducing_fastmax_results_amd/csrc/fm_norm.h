@@ -21,23 +21,33 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_clear(float* stats) {
   (void)i;
 }
 
-// token mean per feature: one workgroup per batch*head, deterministic tree.
+// token mean per feature: one workgroup per (8 features, batch*head), 16-byte loads, a fixed
+// reduction tree (the same sum order on every run).  grid (DH / 8, bh).
 template <typename TIO, int DH>
-FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_colmean(const TIO* FM_RESTRICT x, int64_t s_bh, int64_t s_n, int n,
+FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_colmean(const TIO* FM_RESTRICT x, int64_t s_bh, int64_t s_n, int vec, int n,
                                                     float* FM_RESTRICT stats) {
-  FM_SHARED float part[256];
-  const int tid = FM_TID_X, bh = FM_BID_X;
-  const int d = tid % DH, r0 = tid / DH;
-  constexpr int RPB = 256 / DH;
-  float s = 0.f;
-  for (int t = r0; t < n; t += RPB) s += IO<TIO>::ld(x + int64_t(bh) * s_bh + int64_t(t) * s_n + d);
-  part[tid] = s;
-  FM_SYNC();
-  if (tid < DH) {
-    float tot = 0.f;
-    for (int r = 0; r < RPB; ++r) tot += part[r * DH + tid];
-    stats[bh * NormStats<DH>::N + 2 + tid] = tot / float(n);
+  FM_SHARED float part[8 * 256];
+  const int tid = FM_TID_X, d0 = FM_BID_X * 8, bh = FM_BID_Y;
+  float s[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) s[j] = 0.f;
+  for (int t = tid; t < n; t += 256) {
+    float v[8];
+    IO<TIO>::ld8(x + int64_t(bh) * s_bh + int64_t(t) * s_n + d0, vec != 0, v);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s[j] += v[j];
   }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) part[j * 256 + tid] = s[j];
+  FM_SYNC();
+  for (int stride = 128; stride > 0; stride >>= 1) {
+    if (tid < stride) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) part[j * 256 + tid] += part[j * 256 + tid + stride];
+    }
+    FM_SYNC();
+  }
+  if (tid < 8) stats[bh * NormStats<DH>::N + 2 + d0 + tid] = part[tid * 256] / float(n);
 }
 
 template <typename TIO, int DH>
@@ -124,7 +134,8 @@ int fm_normalize_run(const FastmaxNormDesc* d, const void* x, void* y, float* st
   if (d->max_norm || d->centre == 2) {
     FM_KERNEL_LAUNCH((k_norm_clear<DH>), fm_dim3(d->bh), fm_dim3(256), 0, stream, stats);
     if (d->centre == 2)
-      FM_KERNEL_LAUNCH((k_norm_colmean<TIO, DH>), fm_dim3(d->bh), fm_dim3(256), 0, stream, xp, d->sx.bh, d->sx.n, d->n, stats);
+      FM_KERNEL_LAUNCH((k_norm_colmean<TIO, DH>), fm_dim3(DH / 8, d->bh), fm_dim3(256), 0, stream, xp, d->sx.bh, d->sx.n,
+                       vx, d->n, stats);
     if (d->max_norm)
       FM_KERNEL_LAUNCH((k_norm_maxnorm<TIO, DH>), grid, fm_dim3(256), 0, stream, xp, d->sx.bh, d->sx.n, vx, d->n,
                        d->centre, stats);
