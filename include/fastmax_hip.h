@@ -40,9 +40,18 @@ enum {
                                         forward_bytes grows accordingly */
 };
 
+/* Where slice i of the batch*head axis, token t, feature f of a tensor lives:
+ *   heads <= 1:  i * bh + t * n + f
+ *   heads  > 1:  (i / heads) * b + (i % heads) * bh + t * n + f      (i = batch * heads + head)
+ * The second form takes the (b, n, h*d) output of a projection, viewed as (b, h, n, d), as it is:
+ * b = n*h*d, bh = d, n = h*d (reference transformer/model.py:283-285 makes that view and the
+ * reference wrapper then copies it, model.py:29-32). */
 typedef struct FastmaxStrides {
-  int64_t bh;   /* elements between consecutive batch*head slices */
-  int64_t n;    /* elements between consecutive tokens */
+  int64_t bh;     /* elements between consecutive batch*head slices (heads <= 1) or heads (heads > 1) */
+  int64_t n;      /* elements between consecutive tokens */
+  int64_t b;      /* elements between consecutive batches; read only when heads > 1 */
+  int32_t heads;  /* heads per batch for the two-level form; 0 or 1: one stride for the whole axis */
+  int32_t reserved;
 } FastmaxStrides;
 
 /* Problem description shared by forward and backward.

@@ -23,7 +23,11 @@ STATUS_OK = 0
 
 
 class Strides(C.Structure):
-    _fields_ = [("bh", C.c_int64), ("n", C.c_int64)]
+    """FastmaxStrides: one stride for the batch*head axis, or batch and head strides (heads > 1)."""
+    _fields_ = [("bh", C.c_int64), ("n", C.c_int64), ("b", C.c_int64), ("heads", C.c_int32), ("reserved", C.c_int32)]
+
+    def __init__(self, bh=0, n=0, b=0, heads=0):
+        super().__init__(bh, n, b, heads, 0)
 
 
 class Desc(C.Structure):
@@ -65,11 +69,29 @@ def _dtype_code(t: torch.Tensor) -> int:
 
 
 def _strides(t: torch.Tensor) -> Strides:
-    if t.dim() != 3:
-        raise FastmaxError("fastmax: expected a (bh, n, d) view")
-    if t.shape[2] > 1 and t.stride(2) != 1:
+    """(bh, n, d) view: one stride for the batch*head axis; (b, h, n, d) view: batch and head strides,
+    so the transposed view of a (b, n, h*d) projection output is taken as it is."""
+    if t.dim() not in (3, 4):
+        raise FastmaxError("fastmax: expected a (bh, n, d) or (b, h, n, d) view")
+    if t.shape[-1] > 1 and t.stride(-1) != 1:
         raise FastmaxError("fastmax: the feature axis must be contiguous")
-    return Strides(t.stride(0), t.stride(1))
+    if t.dim() == 3:
+        return Strides(t.stride(0), t.stride(1))
+    return Strides(t.stride(1), t.stride(2), t.stride(0), t.shape[1])
+
+
+def _dims(t: torch.Tensor):
+    """(batch*heads, tokens, features) of a 3-D or 4-D view."""
+    if t.dim() == 4:
+        return t.shape[0] * t.shape[1], t.shape[2], t.shape[3]
+    return tuple(t.shape)
+
+
+def _gstrides(g: torch.Tensor) -> Strides:
+    """Strides of the denominators: (bh, n) or (b, h, n)."""
+    if g.dim() == 3:
+        return Strides(g.stride(1), g.stride(2), g.stride(0), g.shape[1])
+    return Strides(g.stride(0), g.stride(1))
 
 
 class FastmaxLib:
@@ -119,9 +141,9 @@ class FastmaxLib:
 
     def make_desc(self, q, k, v, *, mask, inv_tau, a0, a1, a2, p, chunk=0, flags=0) -> Desc:
         d = Desc()
-        d.bh, d.nq, d.d = q.shape
-        d.nk = k.shape[1]
-        if k.shape[0] != d.bh or v.shape[0] != d.bh or k.shape[2] != d.d or v.shape[2] != d.d or v.shape[1] != d.nk:
+        d.bh, d.nq, d.d = _dims(q)
+        kb, d.nk, kd = _dims(k)
+        if kb != d.bh or kd != d.d or _dims(v) != (d.bh, d.nk, d.d):
             raise FastmaxError("fastmax: q, k, v must be (bh, nq, d), (bh, nk, d), (bh, nk, d)")
         d.dtype = _dtype_code(q)
         if k.dtype != q.dtype or v.dtype != q.dtype:
@@ -148,18 +170,19 @@ class FastmaxLib:
     # -- entry points ------------------------------------------------------------
     def forward(self, q, k, v, *, mask, inv_tau, a0=1.0, a1=1.0, a2=0.5, p=2, chunk=0, flags=0,
                 out: Optional[torch.Tensor] = None, g: Optional[torch.Tensor] = None, save: bool = False):
-        """q (bh, nq, d), k, v (bh, nk, d) views with contiguous features.
-        Returns (o, g): o like q, g (bh, nq) float32; with ``save`` also the workspace
-        tensor that ``backward(..., saved=...)`` can reuse."""
+        """q (bh, nq, d), k, v (bh, nk, d) views with contiguous features, or (b, h, n, d) views.
+        Returns (o, g): o shaped like q, g (bh, nq) or (b, h, nq) float32; with ``save`` also the
+        workspace tensor that ``backward(..., saved=...)`` can reuse."""
         if save:
             flags |= FLAG_SAVE_FOR_BACKWARD
         desc = self.make_desc(q, k, v, mask=mask, inv_tau=inv_tau, a0=a0, a1=a1, a2=a2, p=p, chunk=chunk, flags=flags)
+        lead = tuple(q.shape[:-2])
         if out is None:
-            out = torch.empty((desc.bh, desc.nq, desc.d), dtype=q.dtype, device=q.device)
+            out = torch.empty(lead + (desc.nq, desc.d), dtype=q.dtype, device=q.device)
         if g is None:
-            g = torch.empty((desc.bh, desc.nq), dtype=torch.float32, device=q.device)
+            g = torch.empty(lead + (desc.nq,), dtype=torch.float32, device=q.device)
         desc.so = _strides(out)
-        desc.sg = Strides(g.stride(0), g.stride(1))
+        desc.sg = _gstrides(g)
         fwd, _ = self.workspace_bytes(desc)
         ws = self._workspace(fwd, q.device)
         st = self.lib.fastmax_forward(C.byref(desc), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
@@ -178,11 +201,12 @@ class FastmaxLib:
         desc = self.make_desc(q, k, v, mask=mask, inv_tau=inv_tau, a0=a0, a1=a1, a2=a2, p=p, chunk=chunk, flags=flags)
         if o.dtype != q.dtype or d_o.dtype != q.dtype or g.dtype != torch.float32:
             raise FastmaxError("fastmax: o and d_o must have q's dtype and g must be float32")
-        dq = torch.empty((desc.bh, desc.nq, desc.d), dtype=q.dtype, device=q.device)
-        dk = torch.empty((desc.bh, desc.nk, desc.d), dtype=q.dtype, device=q.device)
-        dv = torch.empty((desc.bh, desc.nk, desc.d), dtype=q.dtype, device=q.device)
+        lead = tuple(q.shape[:-2])
+        dq = torch.empty(lead + (desc.nq, desc.d), dtype=q.dtype, device=q.device)
+        dk = torch.empty(lead + (desc.nk, desc.d), dtype=q.dtype, device=q.device)
+        dv = torch.empty(lead + (desc.nk, desc.d), dtype=q.dtype, device=q.device)
         desc.so, desc.sdo = _strides(o), _strides(d_o)
-        desc.sg = Strides(g.stride(0), g.stride(1))
+        desc.sg = _gstrides(g)
         desc.sdq, desc.sdk, desc.sdv = _strides(dq), _strides(dk), _strides(dv)
         _, bwd = self.workspace_bytes(desc)
         ws = self._workspace(bwd, q.device)
@@ -201,7 +225,7 @@ class FastmaxLib:
     def normalize(self, x, *, centre=0, max_norm=True, scale=1.0, out: Optional[torch.Tensor] = None):
         """x (bh, n, d) view; returns y = scale * (x - centre) / max_n ||.|| (see the header)."""
         nd = NormDesc()
-        nd.bh, nd.n, nd.d = x.shape
+        nd.bh, nd.n, nd.d = _dims(x)
         nd.dtype = _dtype_code(x)
         nd.centre, nd.max_norm, nd.scale = int(centre), int(bool(max_norm)), float(scale)
         if out is None:

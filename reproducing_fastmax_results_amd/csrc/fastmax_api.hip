@@ -61,7 +61,13 @@ struct Plan {
 
 bool strides_ok(const FastmaxStrides& s, int bh, int n, int d) {
   if (s.n < d && n > 1) return false;
-  if (s.bh <= 0 && bh > 1) return false;
+  if (s.heads > 1) {                                   // batch and head strides
+    if (bh % s.heads != 0) return false;
+    if (s.bh <= 0) return false;
+    if (s.b <= 0 && bh > s.heads) return false;
+  } else if (s.bh <= 0 && bh > 1) {
+    return false;
+  }
   return s.n > 0 || n <= 1;
 }
 
@@ -142,24 +148,18 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   return FASTMAX_OK;
 }
 
-template <typename T> bool vec_ok(const void* ptr, const FastmaxStrides& s) {
-  const int64_t a = 16 / int64_t(sizeof(T));          // elements per 16 bytes
-  return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && (s.n % a == 0) && (s.bh % a == 0);
-}
 template <typename T> TRef<const T> cref(const void* ptr, const FastmaxStrides& s) {
-  TRef<const T> r; r.p = static_cast<const T*>(ptr); r.s_bh = s.bh; r.s_n = s.n; r.vec = vec_ok<T>(ptr, s); return r;
+  return fm_ref<const T>(static_cast<const T*>(ptr), s);
 }
-template <typename T> TRef<T> mref(void* ptr, const FastmaxStrides& s) {
-  TRef<T> r; r.p = static_cast<T*>(ptr); r.s_bh = s.bh; r.s_n = s.n; r.vec = vec_ok<T>(ptr, s); return r;
-}
+template <typename T> TRef<T> mref(void* ptr, const FastmaxStrides& s) { return fm_ref<T>(static_cast<T*>(ptr), s); }
 
 template <typename TIO, typename E, int DH>
 int launch_transpose(const void* x, const FastmaxStrides& s, int bh, int n, int npad, E* xt, E* xr, float scale,
                      fm_stream_t stream) {
   TRef<const TIO> r = cref<TIO>(x, s);
   ProfScope prof(FM_K_TRANSPOSE, stream);
-  FM_KERNEL_LAUNCH((k_transpose<TIO, E, DH>), fm_dim3(npad / 64, bh), fm_dim3(FM_THREADS), 0, stream,
-                   r.p, r.s_bh, r.s_n, r.vec, n, npad, xt, xr, scale);
+  FM_KERNEL_LAUNCH((k_transpose<TIO, E, DH>), fm_dim3(npad / 64, bh), fm_dim3(FM_THREADS), 0, stream, r, n, npad, xt,
+                   xr, scale);
   return fm_after_launch();
 }
 
@@ -207,10 +207,10 @@ template <typename E, int DH, int QT> size_t tok_lds_bytes() {
 }
 
 template <typename TIO, typename E> void tok_common(TokArgs<TIO, E>& a, const FastmaxDesc* d, const Plan& p) {
-  a.own_io = TRef<const TIO>{nullptr, 0, 0, 0};
+  a.own_io = TRef<const TIO>{nullptr, 0, 0, 0, 0, 0};
   a.own_r = nullptr; a.own2_r = nullptr; a.cv = nullptr; a.xr = nullptr; a.yr = nullptr; a.zt = nullptr; a.zt2 = nullptr;
-  a.out2 = TRef<TIO>{nullptr, 0, 0, 0}; a.out2_scale = 1.0f;
-  a.g = nullptr; a.g_s_bh = 0; a.g_s_n = 0;
+  a.out2 = TRef<TIO>{nullptr, 0, 0, 0, 0, 0}; a.out2_scale = 1.0f;
+  a.g = TRef<float>{nullptr, 0, 0, 0, 0, 0};
   a.nslots = p.nslots; a.L = p.L; a.nseg = p.nseg; a.causal = d->mask != 0; a.use_state = p.use_state;
   a.quad = p.quad; a.a0 = p.a0; a.a1 = p.a1; a.a2 = p.a2; a.sc = p.sc; a.out_scale = 1.0f; a.zscale = 1.0f;
 }
@@ -268,7 +268,7 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   a.xr = kr; a.zt = vt; a.npad_own = p.npad_q; a.npad_str = p.npad_k;
   a.big = big; a.small = small;
   a.out = mref<TIO>(o, d->so);
-  a.g = g; a.g_s_bh = d->sg.bh; a.g_s_n = d->sg.n;
+  a.g = mref<float>(g, d->sg);
   a.n_own = d->nq; a.n_str = d->nk;
   return launch_pv<TIO, E, DH, QT, FM_OWN_Q>(a, d->bh, FM_K_FWD, stream);
 }
@@ -279,7 +279,7 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
 
 extern "C" {
 
-int fastmax_version(void) { return 100; }
+int fastmax_version(void) { return 101; }
 
 const char* fastmax_status_string(int status) {
   switch (status) {

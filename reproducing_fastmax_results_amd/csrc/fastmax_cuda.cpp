@@ -153,53 +153,79 @@ std::vector<torch::Tensor> backwardpass(torch::Tensor q, torch::Tensor k, torch:
 }
 
 // ---------------------------------------------------------------------------------
-// Stride-aware entry points: any (bh, n, d) view (3-D) or (b, h, n, d) tensor whose
-// feature axis is contiguous and whose batch and head axes collapse to one stride.
+// Stride-aware entry points: any (bh, n, d) view (3-D) or (b, h, n, d) view (4-D) whose
+// feature axis is contiguous is handed to the library as it lies in memory: a 3-D view with
+// one stride for its first axis, a 4-D view with batch and head strides, so the transposed
+// view of a (b, n, h*d) projection output needs no copy.
 // ---------------------------------------------------------------------------------
-torch::Tensor as_bhnd(const torch::Tensor& t, const char* name) {
-  TORCH_CHECK(t.dim() == 3 || t.dim() == 4, name, " must be (bh, n, d) or (b, h, n, d)");
-  torch::Tensor x = t;
-  if (x.size(-1) > 1 && x.stride(-1) != 1) x = x.contiguous();
-  if (x.dim() == 4) {
-    if (x.size(0) > 1 && x.size(1) > 1 && x.stride(0) != x.size(1) * x.stride(1)) x = x.contiguous();
-    const int64_t sbh = x.size(1) > 1 ? x.stride(1) : x.stride(0);
-    x = x.as_strided({x.size(0) * x.size(1), x.size(2), x.size(3)}, {sbh, x.stride(2), x.stride(3)}, x.storage_offset());
+struct View {
+  torch::Tensor t;
+  FastmaxStrides s;
+  int64_t bh, n, d;
+};
+
+View view_of(const torch::Tensor& t_, const char* name) {
+  TORCH_CHECK(t_.dim() == 3 || t_.dim() == 4, name, " must be (bh, n, d) or (b, h, n, d)");
+  View w;
+  w.t = (t_.size(-1) > 1 && t_.stride(-1) != 1) ? t_.contiguous() : t_;
+  const torch::Tensor& x = w.t;
+  if (x.dim() == 3) {
+    w.s = FastmaxStrides{x.stride(0), x.stride(1), 0, 0, 0};
+    w.bh = x.size(0); w.n = x.size(1); w.d = x.size(2);
+  } else {
+    w.s = FastmaxStrides{x.stride(1), x.stride(2), x.stride(0), static_cast<int32_t>(x.size(1)), 0};
+    w.bh = x.size(0) * x.size(1); w.n = x.size(2); w.d = x.size(3);
   }
-  return x;
+  return w;
 }
 
-FastmaxStrides strides_of(const torch::Tensor& t) { return FastmaxStrides{t.stride(0), t.stride(1)}; }
+// A new tensor shaped like `like` with n tokens; a 4-D view whose tokens lie outside its heads in
+// memory (the projection layout (b, n, h, d)) gets its result in the same order, so the caller's
+// transpose back to (b, n, h*d) is a view as well.
+torch::Tensor empty_like_layout(const torch::Tensor& like, int64_t n, torch::ScalarType dtype) {
+  if (like.dim() == 3) return torch::empty({like.size(0), n, like.size(2)}, like.options().dtype(dtype));
+  const int64_t b = like.size(0), h = like.size(1), d = like.size(3);
+  if (h > 1 && like.stride(2) > like.stride(1))
+    return torch::empty({b, n, h, d}, like.options().dtype(dtype)).permute({0, 2, 1, 3});
+  return torch::empty({b, h, n, d}, like.options().dtype(dtype));
+}
 
-FastmaxDesc ex_desc(const torch::Tensor& q, const torch::Tensor& k, const torch::Tensor& v, bool mask, double inv_tau,
-                    double a0, double a1, double a2, int64_t p, int64_t chunk, int64_t flags) {
-  FM_CHECK_CUDA(q); FM_CHECK_CUDA(k); FM_CHECK_CUDA(v);
-  TORCH_CHECK(k.size(0) == q.size(0) && v.size(0) == q.size(0) && k.size(2) == q.size(2) && v.size(2) == q.size(2) &&
-                  v.size(1) == k.size(1), "q, k, v must be (bh, nq, d), (bh, nk, d), (bh, nk, d)");
-  TORCH_CHECK(k.scalar_type() == q.scalar_type() && v.scalar_type() == q.scalar_type(), "q, k, v must share one dtype");
+FastmaxStrides gstrides_of(const torch::Tensor& g) {
+  if (g.dim() == 3) return FastmaxStrides{g.stride(1), g.stride(2), g.stride(0), static_cast<int32_t>(g.size(1)), 0};
+  return FastmaxStrides{g.stride(0), g.stride(1), 0, 0, 0};
+}
+
+FastmaxDesc ex_desc(const View& q, const View& k, const View& v, bool mask, double inv_tau, double a0, double a1,
+                    double a2, int64_t p, int64_t chunk, int64_t flags) {
+  FM_CHECK_CUDA(q.t); FM_CHECK_CUDA(k.t); FM_CHECK_CUDA(v.t);
+  TORCH_CHECK(k.bh == q.bh && v.bh == q.bh && k.d == q.d && v.d == q.d && v.n == k.n,
+              "q, k, v must be (bh, nq, d), (bh, nk, d), (bh, nk, d)");
+  TORCH_CHECK(k.t.scalar_type() == q.t.scalar_type() && v.t.scalar_type() == q.t.scalar_type(),
+              "q, k, v must share one dtype");
   FastmaxDesc d{};
-  d.bh = static_cast<int32_t>(q.size(0)); d.nq = static_cast<int32_t>(q.size(1)); d.nk = static_cast<int32_t>(k.size(1));
-  d.d = static_cast<int32_t>(q.size(2)); d.dtype = dtype_code(q);
+  d.bh = static_cast<int32_t>(q.bh); d.nq = static_cast<int32_t>(q.n); d.nk = static_cast<int32_t>(k.n);
+  d.d = static_cast<int32_t>(q.d); d.dtype = dtype_code(q.t);
   d.mask = mask ? 1 : 0; d.p = static_cast<int32_t>(p);
   d.a0 = float(a0); d.a1 = float(a1); d.a2 = float(a2); d.inv_tau = float(inv_tau);
   d.chunk = static_cast<int32_t>(chunk); d.flags = static_cast<int32_t>(flags);
-  d.sq = strides_of(q); d.sk = strides_of(k); d.sv = strides_of(v);
+  d.sq = q.s; d.sk = k.s; d.sv = v.s;
   return d;
 }
 
 std::vector<torch::Tensor> forward_any(torch::Tensor q_, torch::Tensor k_, torch::Tensor v_, bool mask, double inv_tau,
                                        double a0, double a1, double a2, int64_t p, int64_t chunk, int64_t flags) {
-  torch::Tensor q = as_bhnd(q_, "q"), k = as_bhnd(k_, "k"), v = as_bhnd(v_, "v");
+  const View q = view_of(q_, "q"), k = view_of(k_, "k"), v = view_of(v_, "v");
   FastmaxDesc d = ex_desc(q, k, v, mask, inv_tau, a0, a1, a2, p, chunk, flags);
-  torch::Tensor o = torch::empty({d.bh, d.nq, d.d}, q.options());
-  torch::Tensor g = torch::empty({d.bh, d.nq}, q.options().dtype(torch::kFloat32));
-  d.so = strides_of(o);
-  d.sg = FastmaxStrides{g.stride(0), g.stride(1)};
+  torch::Tensor o = empty_like_layout(q.t, q.n, q.t.scalar_type());
+  torch::Tensor g = q.t.dim() == 4 ? torch::empty({q.t.size(0), q.t.size(1), q.n}, q.t.options().dtype(torch::kFloat32))
+                                   : torch::empty({q.bh, q.n}, q.t.options().dtype(torch::kFloat32));
+  d.so = view_of(o, "o").s;
+  d.sg = gstrides_of(g);
   size_t fwd = 0, bwd = 0;
   check_status(fastmax_workspace_bytes(&d, &fwd, &bwd), "fastmax_workspace_bytes");
-  torch::Tensor ws = workspace(fwd, q);
-  check_status(fastmax_forward(&d, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), g.data_ptr<float>(),
-                               ws.data_ptr(), fwd, stream_of(q)), "fastmax_forward");
-  if (q_.dim() == 4) return {o.view({q_.size(0), q_.size(1), d.nq, d.d}), g.view({q_.size(0), q_.size(1), d.nq}), ws};
+  torch::Tensor ws = workspace(fwd, q.t);
+  check_status(fastmax_forward(&d, q.t.data_ptr(), k.t.data_ptr(), v.t.data_ptr(), o.data_ptr(), g.data_ptr<float>(),
+                               ws.data_ptr(), fwd, stream_of(q.t)), "fastmax_forward");
   return {o, g, ws};
 }
 
@@ -224,36 +250,36 @@ std::vector<torch::Tensor> backward_any(torch::Tensor q_, torch::Tensor k_, torc
                                         torch::Tensor g_, torch::Tensor go_, const torch::Tensor* saved, bool mask,
                                         double inv_tau, double a0, double a1, double a2, int64_t p, int64_t chunk,
                                         int64_t flags) {
-  torch::Tensor q = as_bhnd(q_, "q"), k = as_bhnd(k_, "k"), v = as_bhnd(v_, "v");
-  torch::Tensor o = as_bhnd(o_, "o"), go = as_bhnd(go_, "grad_output");
+  const View q = view_of(q_, "q"), k = view_of(k_, "k"), v = view_of(v_, "v");
+  const View o = view_of(o_, "o"), go = view_of(go_, "grad_output");
   FastmaxDesc d = ex_desc(q, k, v, mask, inv_tau, a0, a1, a2, p, chunk, flags);
-  TORCH_CHECK(o.scalar_type() == q.scalar_type() && go.scalar_type() == q.scalar_type(), "o and grad_output must match q");
+  TORCH_CHECK(o.t.scalar_type() == q.t.scalar_type() && go.t.scalar_type() == q.t.scalar_type(),
+              "o and grad_output must match q");
+  TORCH_CHECK(o.bh == q.bh && o.n == q.n && o.d == q.d && go.bh == q.bh && go.n == q.n && go.d == q.d,
+              "o and grad_output must be shaped like q");
   TORCH_CHECK(g_.scalar_type() == torch::kFloat32 && g_.numel() == int64_t(d.bh) * d.nq, "g must be float32 (bh, nq)");
-  torch::Tensor g = g_.contiguous().view({d.bh, d.nq});
-  torch::Tensor dq = torch::empty({d.bh, d.nq, d.d}, q.options());
-  torch::Tensor dk = torch::empty({d.bh, d.nk, d.d}, q.options());
-  torch::Tensor dv = torch::empty({d.bh, d.nk, d.d}, q.options());
-  d.so = strides_of(o); d.sdo = strides_of(go);
-  d.sg = FastmaxStrides{g.stride(0), g.stride(1)};
-  d.sdq = strides_of(dq); d.sdk = strides_of(dk); d.sdv = strides_of(dv);
+  torch::Tensor g = g_.dim() == 3 ? g_ : g_.contiguous().view({d.bh, d.nq});
+  torch::Tensor dq = empty_like_layout(q.t, q.n, q.t.scalar_type());
+  torch::Tensor dk = empty_like_layout(k.t, k.n, q.t.scalar_type());
+  torch::Tensor dv = empty_like_layout(v.t, v.n, q.t.scalar_type());
+  d.so = o.s; d.sdo = go.s;
+  d.sg = gstrides_of(g);
+  d.sdq = view_of(dq, "dq").s; d.sdk = view_of(dk, "dk").s; d.sdv = view_of(dv, "dv").s;
   size_t fwd = 0, bwd = 0;
   check_status(fastmax_workspace_bytes(&d, &fwd, &bwd), "fastmax_workspace_bytes");
-  torch::Tensor ws = workspace(bwd, q);
+  torch::Tensor ws = workspace(bwd, q.t);
   if (saved) {
     TORCH_CHECK(saved->is_cuda() && saved->scalar_type() == torch::kUInt8 && saved->is_contiguous(),
                 "saved workspace must be the uint8 tensor returned by forward_save");
-    check_status(fastmax_backward_saved(&d, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), g.data_ptr<float>(),
-                                        go.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), saved->data_ptr(),
-                                        size_t(saved->numel()), ws.data_ptr(), bwd, stream_of(q)),
+    check_status(fastmax_backward_saved(&d, q.t.data_ptr(), k.t.data_ptr(), v.t.data_ptr(), o.t.data_ptr(),
+                                        g.data_ptr<float>(), go.t.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                                        dv.data_ptr(), saved->data_ptr(), size_t(saved->numel()), ws.data_ptr(), bwd,
+                                        stream_of(q.t)),
                  "fastmax_backward_saved");
   } else {
-    check_status(fastmax_backward(&d, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), g.data_ptr<float>(),
-                                  go.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), bwd,
-                                  stream_of(q)), "fastmax_backward");
-  }
-  if (q_.dim() == 4) {
-    const int64_t b = q_.size(0), h = q_.size(1);
-    return {dq.view({b, h, d.nq, d.d}), dk.view({b, h, d.nk, d.d}), dv.view({b, h, d.nk, d.d})};
+    check_status(fastmax_backward(&d, q.t.data_ptr(), k.t.data_ptr(), v.t.data_ptr(), o.t.data_ptr(),
+                                  g.data_ptr<float>(), go.t.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                                  ws.data_ptr(), bwd, stream_of(q.t)), "fastmax_backward");
   }
   return {dq, dk, dv};
 }
@@ -276,18 +302,18 @@ std::vector<torch::Tensor> backward_saved(torch::Tensor q, torch::Tensor k, torc
 
 // y = scale * (x - centre) / max_n ||x_n - centre||  (see fastmax_normalize in the C header)
 torch::Tensor normalize(torch::Tensor x_, int64_t centre, bool max_norm, double scale) {
-  torch::Tensor x = as_bhnd(x_, "x");
-  FM_CHECK_CUDA(x);
+  const View x = view_of(x_, "x");
+  FM_CHECK_CUDA(x.t);
   FastmaxNormDesc nd{};
-  nd.bh = static_cast<int32_t>(x.size(0)); nd.n = static_cast<int32_t>(x.size(1)); nd.d = static_cast<int32_t>(x.size(2));
-  nd.dtype = dtype_code(x); nd.centre = static_cast<int32_t>(centre); nd.max_norm = max_norm ? 1 : 0;
+  nd.bh = static_cast<int32_t>(x.bh); nd.n = static_cast<int32_t>(x.n); nd.d = static_cast<int32_t>(x.d);
+  nd.dtype = dtype_code(x.t); nd.centre = static_cast<int32_t>(centre); nd.max_norm = max_norm ? 1 : 0;
   nd.scale = float(scale);
-  torch::Tensor y = torch::empty({nd.bh, nd.n, nd.d}, x.options());
-  nd.sx = strides_of(x); nd.sy = strides_of(y);
-  torch::Tensor stats = torch::empty({int64_t(nd.bh) * (nd.d + 2)}, x.options().dtype(torch::kFloat32));
-  check_status(fastmax_normalize(&nd, x.data_ptr(), y.data_ptr(), stats.data_ptr<float>(), stream_of(x)),
+  torch::Tensor y = empty_like_layout(x.t, x.n, x.t.scalar_type());
+  nd.sx = x.s; nd.sy = view_of(y, "y").s;
+  torch::Tensor stats = torch::empty({int64_t(nd.bh) * (nd.d + 2)}, x.t.options().dtype(torch::kFloat32));
+  check_status(fastmax_normalize(&nd, x.t.data_ptr(), y.data_ptr(), stats.data_ptr<float>(), stream_of(x.t)),
                "fastmax_normalize");
-  return x_.dim() == 4 ? y.view(x_.sizes()) : y;
+  return y;
 }
 
 }  // namespace

@@ -13,6 +13,7 @@
 // the token, the accumulator rows are features.  That keeps one token per lane,
 // so a per-token scalar (q_ia, 1/g_i, c_i) is a per-lane scalar.
 #pragma once
+#include "fastmax_hip.h"
 #include "fm_mma.h"
 
 #if defined(FM_HOSTSIM)
@@ -115,6 +116,28 @@ struct RowRegs {
   }
 };
 
+// A caller tensor: base pointer, strides in elements, whether 16-byte accesses are aligned.
+template <typename TIO> struct TRef {
+  TIO* p; int64_t s_bh, s_n; int vec; int64_t s_b; int heads;
+  // first element of batch*head slice bh (one stride, or batch and head strides when heads > 1)
+  FM_DEVICE TIO* base(int bh) const {
+    return heads > 1 ? p + int64_t(bh / heads) * s_b + int64_t(bh % heads) * s_bh : p + int64_t(bh) * s_bh;
+  }
+};
+
+// host side: TRef of a caller pointer and its FastmaxStrides
+template <typename T> inline bool fm_vec_ok(const void* ptr, const FastmaxStrides& s) {
+  const int64_t a = 16 / int64_t(sizeof(T));          // elements per 16 bytes
+  return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && (s.n % a == 0) && (s.bh % a == 0) &&
+         (s.heads <= 1 || s.b % a == 0);
+}
+template <typename T> inline TRef<T> fm_ref(T* ptr, const FastmaxStrides& s) {
+  TRef<T> r;
+  r.p = ptr; r.s_bh = s.bh; r.s_n = s.n; r.vec = fm_vec_ok<T>(ptr, s) ? 1 : 0;
+  r.s_b = s.heads > 1 ? s.b : 0; r.heads = s.heads > 1 ? s.heads : 0;
+  return r;
+}
+
 // ------------------------------------------------------------------------------
 // k_transpose: x (bh, n, DH) strided, interface type  ->  compute type, multiplied by
 // `scale`, zero for tokens >= n:  xt [bh][DH][npad] (transposed) and, when xr is not
@@ -123,13 +146,14 @@ struct RowRegs {
 // ------------------------------------------------------------------------------
 template <typename TIO, typename E, int DH>
 FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS)
-k_transpose(const TIO* FM_RESTRICT x, int64_t s_bh, int64_t s_n, int vec, int n, int npad,
-            E* FM_RESTRICT xt, E* FM_RESTRICT xr, float scale) {
+k_transpose(TRef<const TIO> x, int n, int npad, E* FM_RESTRICT xt, E* FM_RESTRICT xr, float scale) {
   constexpr int PT = 64 + Mma<E>::PAD;
   constexpr int VEC = Mma<E>::VEC;
   FM_SHARED E tile[DH * PT];
   const int tid = FM_TID_X, t0 = FM_BID_X * 64, bh = FM_BID_Y;
-  const TIO* xb = x + int64_t(bh) * s_bh;
+  const TIO* xb = x.base(bh);
+  const int64_t s_n = x.s_n;
+  const int vec = x.vec;
   for (int c = tid; c < 64 * (DH / 8); c += FM_THREADS) {
     const int tok = c / (DH / 8), d0 = (c % (DH / 8)) * 8;
     float v[8];
@@ -168,12 +192,9 @@ k_transpose(const TIO* FM_RESTRICT x, int64_t s_bh, int64_t s_n, int vec, int n,
 // Reference: div_grad_output, fastmax_cuda_backward.cu:494-501, and the
 // "grad * o" row sums of fastattention_einops.py:405-407.
 // ------------------------------------------------------------------------------
-template <typename TIO> struct TRef { TIO* p; int64_t s_bh, s_n; int vec; };
-
 template <typename TIO, typename E, int DH>
 FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS)
-k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, const float* FM_RESTRICT g,
-           int64_t g_s_bh, int64_t g_s_n, int n, int npad, E* FM_RESTRICT gh, E* FM_RESTRICT ght,
+k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, TRef<const float> g, int n, int npad, E* FM_RESTRICT gh, E* FM_RESTRICT ght,
            E* FM_RESTRICT qt, E* FM_RESTRICT qct, E* FM_RESTRICT qr, E* FM_RESTRICT cv, float qscale, float gscale) {
   constexpr int PT = 64 + Mma<E>::PAD;
   constexpr int VEC = Mma<E>::VEC;
@@ -187,13 +208,13 @@ k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, const floa
   float vg[EPT], vq[EPT];
   float csum = 0.f;
   if (row < n) {
-    const float ginv = gscale / g[int64_t(bh) * g_s_bh + int64_t(row) * g_s_n];
+    const float ginv = gscale / g.base(bh)[int64_t(row) * g.s_n];
 #pragma unroll
     for (int j = 0; j < EPT; j += 8) {
       float a[8], b[8], c[8];
-      IO<TIO>::ld8(d_o.p + int64_t(bh) * d_o.s_bh + int64_t(row) * d_o.s_n + d0 + j, d_o.vec != 0, a);
-      IO<TIO>::ld8(o.p + int64_t(bh) * o.s_bh + int64_t(row) * o.s_n + d0 + j, o.vec != 0, b);
-      IO<TIO>::ld8(q.p + int64_t(bh) * q.s_bh + int64_t(row) * q.s_n + d0 + j, q.vec != 0, c);
+      IO<TIO>::ld8(d_o.base(bh) + int64_t(row) * d_o.s_n + d0 + j, d_o.vec != 0, a);
+      IO<TIO>::ld8(o.base(bh) + int64_t(row) * o.s_n + d0 + j, o.vec != 0, b);
+      IO<TIO>::ld8(q.base(bh) + int64_t(row) * q.s_n + d0 + j, q.vec != 0, c);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         vg[j + i] = a[i] * ginv;

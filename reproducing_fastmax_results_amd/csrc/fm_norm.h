@@ -9,7 +9,7 @@
 // non-negative float, which is order independent.
 #pragma once
 #include "fastmax_hip.h"
-#include "fm_mma.h"
+#include "fm_kernels.h"
 
 // stats layout per batch*head: [0] max squared norm (as float bits), [1] unused, [2..2+d) token mean
 template <int DH> struct NormStats { static constexpr int N = DH + 2; };
@@ -24,8 +24,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_clear(float* stats) {
 // token mean per feature: one workgroup per (8 features, batch*head), 16-byte loads, a fixed
 // reduction tree (the same sum order on every run).  grid (DH / 8, bh).
 template <typename TIO, int DH>
-FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_colmean(const TIO* FM_RESTRICT x, int64_t s_bh, int64_t s_n, int vec, int n,
-                                                    float* FM_RESTRICT stats) {
+FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_colmean(TRef<const TIO> x, int n, float* FM_RESTRICT stats) {
   FM_SHARED float part[8 * 256];
   const int tid = FM_TID_X, d0 = FM_BID_X * 8, bh = FM_BID_Y;
   float s[8];
@@ -33,7 +32,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_colmean(const TIO* FM_RESTRICT x, in
   for (int j = 0; j < 8; ++j) s[j] = 0.f;
   for (int t = tid; t < n; t += 256) {
     float v[8];
-    IO<TIO>::ld8(x + int64_t(bh) * s_bh + int64_t(t) * s_n + d0, vec != 0, v);
+    IO<TIO>::ld8(x.base(bh) + int64_t(t) * x.s_n + d0, x.vec != 0, v);
 #pragma unroll
     for (int j = 0; j < 8; ++j) s[j] += v[j];
   }
@@ -72,8 +71,7 @@ FM_DEVICE void fm_norm_load_centred(const TIO* row, bool vec, int d0, int centre
 
 // grid (ceil(n/64), bh); four threads per token
 template <typename TIO, int DH>
-FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_maxnorm(const TIO* FM_RESTRICT x, int64_t s_bh, int64_t s_n, int vec, int n,
-                                                    int centre, float* FM_RESTRICT stats) {
+FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_maxnorm(TRef<const TIO> x, int n, int centre, float* FM_RESTRICT stats) {
   constexpr int EPT = DH / 4;
   const int tid = FM_TID_X, bh = FM_BID_Y;
   const int tok = FM_BID_X * 64 + (tid >> 2), d0 = (tid & 3) * EPT;
@@ -82,7 +80,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_maxnorm(const TIO* FM_RESTRICT x, in
   // every lane takes part in the shuffles; rows past the end contribute zero
   const int tk = tok < n ? tok : n - 1;
   float v[EPT];
-  fm_norm_load_centred<TIO, DH>(x + int64_t(bh) * s_bh + int64_t(tk) * s_n, vec != 0, d0, centre, st + 2, v);
+  fm_norm_load_centred<TIO, DH>(x.base(bh) + int64_t(tk) * x.s_n, x.vec != 0, d0, centre, st + 2, v);
 #pragma unroll
   for (int j = 0; j < EPT; ++j) nrm += v[j] * v[j];
   nrm += fm_shfl_xor(nrm, 1);
@@ -103,45 +101,39 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_maxnorm(const TIO* FM_RESTRICT x, in
 }
 
 template <typename TIO, int DH>
-FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_apply(const TIO* FM_RESTRICT x, int64_t s_bh, int64_t s_n, int vecx,
-                                                  TIO* FM_RESTRICT y, int64_t y_bh, int64_t y_n, int vecy, int n,
-                                                  int centre, int max_norm, float scale, const float* FM_RESTRICT stats) {
+FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_apply(TRef<const TIO> x, TRef<TIO> y, int n, int centre, int max_norm, float scale,
+                                                  const float* FM_RESTRICT stats) {
   constexpr int EPT = DH / 4;
   const int tid = FM_TID_X, bh = FM_BID_Y;
   const int tok = FM_BID_X * 64 + (tid >> 2), d0 = (tid & 3) * EPT;
   const float* st = stats ? stats + bh * NormStats<DH>::N : nullptr;
   const int tk = tok < n ? tok : n - 1;
   float v[EPT];
-  fm_norm_load_centred<TIO, DH>(x + int64_t(bh) * s_bh + int64_t(tk) * s_n, vecx != 0, d0, centre, st ? st + 2 : nullptr, v);
+  fm_norm_load_centred<TIO, DH>(x.base(bh) + int64_t(tk) * x.s_n, x.vec != 0, d0, centre, st ? st + 2 : nullptr, v);
   float f = scale;
   if (max_norm) f = scale / fm_sqrtf(st[0]);
   if (tok < n) {
 #pragma unroll
     for (int j = 0; j < EPT; ++j) v[j] *= f;
 #pragma unroll
-    for (int j = 0; j < EPT; j += 8) IO<TIO>::st8(y + int64_t(bh) * y_bh + int64_t(tok) * y_n + d0 + j, vecy != 0, &v[j]);
+    for (int j = 0; j < EPT; j += 8) IO<TIO>::st8(y.base(bh) + int64_t(tok) * y.s_n + d0 + j, y.vec != 0, &v[j]);
   }
 }
 
 template <typename TIO, int DH>
 int fm_normalize_run(const FastmaxNormDesc* d, const void* x, void* y, float* stats, fm_stream_t stream) {
-  const TIO* xp = static_cast<const TIO*>(x);
-  TIO* yp = static_cast<TIO*>(y);
-  const int a = 16 / int(sizeof(TIO));
-  const int vx = (reinterpret_cast<uintptr_t>(x) % 16 == 0) && d->sx.n % a == 0 && d->sx.bh % a == 0;
-  const int vy = (reinterpret_cast<uintptr_t>(y) % 16 == 0) && d->sy.n % a == 0 && d->sy.bh % a == 0;
+  const TRef<const TIO> xr = fm_ref<const TIO>(static_cast<const TIO*>(x), d->sx);
+  const TRef<TIO> yr = fm_ref<TIO>(static_cast<TIO*>(y), d->sy);
   const fm_dim3 grid((d->n + 63) / 64, d->bh);
   if (d->max_norm || d->centre == 2) {
     FM_KERNEL_LAUNCH((k_norm_clear<DH>), fm_dim3(d->bh), fm_dim3(256), 0, stream, stats);
     if (d->centre == 2)
-      FM_KERNEL_LAUNCH((k_norm_colmean<TIO, DH>), fm_dim3(DH / 8, d->bh), fm_dim3(256), 0, stream, xp, d->sx.bh, d->sx.n,
-                       vx, d->n, stats);
+      FM_KERNEL_LAUNCH((k_norm_colmean<TIO, DH>), fm_dim3(DH / 8, d->bh), fm_dim3(256), 0, stream, xr, d->n, stats);
     if (d->max_norm)
-      FM_KERNEL_LAUNCH((k_norm_maxnorm<TIO, DH>), grid, fm_dim3(256), 0, stream, xp, d->sx.bh, d->sx.n, vx, d->n,
-                       d->centre, stats);
+      FM_KERNEL_LAUNCH((k_norm_maxnorm<TIO, DH>), grid, fm_dim3(256), 0, stream, xr, d->n, d->centre, stats);
   }
-  FM_KERNEL_LAUNCH((k_norm_apply<TIO, DH>), grid, fm_dim3(256), 0, stream, xp, d->sx.bh, d->sx.n, vx, yp, d->sy.bh,
-                   d->sy.n, vy, d->n, d->centre, d->max_norm, d->scale, stats);
+  FM_KERNEL_LAUNCH((k_norm_apply<TIO, DH>), grid, fm_dim3(256), 0, stream, xr, yr, d->n, d->centre, d->max_norm,
+                   d->scale, stats);
 #if defined(FM_HOSTSIM)
   return FASTMAX_OK;
 #else

@@ -37,7 +37,7 @@ template <typename TIO, typename E> struct TokArgs {
   const E* big; const float* small; int nslots;
   TRef<TIO> out;
   TRef<TIO> out2;           // k_ds with dV: dV
-  float* g; int64_t g_s_bh, g_s_n;      // k_pv, own = queries: denominators
+  TRef<float> g;                        // k_pv, own = queries: denominators (bh, n)
   int n_own, n_str, L, nseg, causal, use_state, quad;
   float a0, a1, a2;                     // f(x) = a0 + a1 x + a2 x^2
   float sc;                             // sqrt(1/tau)
@@ -91,7 +91,7 @@ FM_DEVICE void fm_store_tokens(fm_f32x16 (*acc)[DH / 32], const int* xrow, const
         Os[xrow[j] * (DH + 1) + c] = scale * (acc[j][ct][e] + (addvec ? addvec[c] : 0.f));
       }
   FM_SYNC();
-  TIO* ob = out.p + int64_t(bh) * out.s_bh;
+  TIO* ob = out.base(bh);
   for (int c = tid; c < C::QW * (DH / 8); c += FM_THREADS) {
     const int row = c / (DH / 8), col = (c % (DH / 8)) * 8;
     if (row0 + row < nrows) {
@@ -224,7 +224,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
   // ---- stage the own rows (and the small states) ----
   if (OWN == FM_OWN_Q) {
     RowRegs<TIO, E, QW, DH> rq;
-    rq.load(A.own_io.p + int64_t(bh) * A.own_io.s_bh, A.own_io.s_n, A.own_io.vec != 0, t0, A.n_own, tid);
+    rq.load(A.own_io.base(bh), A.own_io.s_n, A.own_io.vec != 0, t0, A.n_own, tid);
     rq.store(Own, PQ, tid, A.sc);
   } else {
     TileRegs<E, QW, DH> ro;
@@ -367,10 +367,10 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
           Os[xrow[j] * (DH + 1) + c] = f * ginv;
         }
       const int qi = t0 + xrow[j];
-      if (lh == 0 && qi < A.n_own) A.g[int64_t(bh) * A.g_s_bh + int64_t(qi) * A.g_s_n] = gt;
+      if (lh == 0 && qi < A.n_own) A.g.base(bh)[int64_t(qi) * A.g.s_n] = gt;
     }
     FM_SYNC();
-    TIO* ob = A.out.p + int64_t(bh) * A.out.s_bh;
+    TIO* ob = A.out.base(bh);
     for (int c = tid; c < QW * (DH / 8); c += FM_THREADS) {
       const int row = c / (DH / 8), col = (c % (DH / 8)) * 8;
       if (t0 + row < A.n_own) {

@@ -66,3 +66,24 @@ def check_forward_backward(lib, bh, nq, d, dtype, device, *, mask, p, nk=None, c
     for n, e in errs.items():
         assert e < TOL[dtype], f"{n} rel-L2 {e:.3e} (all: {errs})"
     return errs
+
+
+def check_batch_head_strides(lib, b, h, n, d, dtype, device, *, mask, p, chunk=0, seed=0):
+    """q, k, v, dO as transposed views of (b, n, h*d) tensors, handed over with batch and head
+    strides (FastmaxStrides.heads > 1), outputs written into the same memory order: bit-identical
+    to the run on contiguous (b*h, n, d) copies."""
+    gen = torch.Generator().manual_seed(seed)
+    base = [torch.randn(b, n, h * d, generator=gen).to(dtype).to(device) for _ in range(4)]
+    q4, k4, v4, go4 = (x.view(b, n, h, d).transpose(1, 2) for x in base)
+    tau = 8.0 * math.sqrt(d)
+    kw = dict(mask=mask, inv_tau=1.0 / tau, p=p, chunk=chunk)
+    out = torch.empty(b, n, h, d, dtype=dtype, device=device).transpose(1, 2)
+    o4, g4, ws = lib.forward(q4, k4, v4, save=True, out=out, **kw)
+    q3, k3, v3, go3 = (x.contiguous().view(b * h, n, d) for x in (q4, k4, v4, go4))
+    o3, g3, ws3 = lib.forward(q3, k3, v3, save=True, **kw)
+    assert torch.equal(o4.contiguous().view(b * h, n, d), o3) and torch.equal(g4.reshape(b * h, n), g3)
+    d4 = lib.backward(q4, k4, v4, o4, g4, go4, saved=ws, **kw)
+    d3 = lib.backward(q3, k3, v3, o3, g3, go3, saved=ws3, **kw)
+    for x4, x3 in zip(d4, d3):
+        assert torch.equal(x4.contiguous().view(b * h, n, d), x3)
+    return True

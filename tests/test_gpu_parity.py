@@ -4,7 +4,7 @@ bf16-rounded inputs)."""
 import pytest
 import torch
 
-from tests.parity import check_forward, check_forward_backward
+from tests.parity import check_batch_head_strides, check_forward, check_forward_backward
 from reproducing_fastmax_results_amd._capi import FLAG_FORCE_DENSE, FLAG_FORCE_MOMENTS
 
 pytestmark = pytest.mark.gpu
@@ -141,3 +141,11 @@ def test_backward_on_saved_forward_workspace(lib, dtype, mask, p):
                            seed=18, saved=True)
     check_forward_backward(lib, 3, 333, 32, dtype, DEV, mask=mask, p=p, flags=FLAG_FORCE_DENSE, seed=19, saved=True)
     check_forward_backward(lib, 2, 2500, 64, dtype, DEV, mask=mask, p=p, seed=20, saved=True, chunk=1024)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mask,chunk", [(True, 0), (True, 256), (False, 0)])
+def test_batch_and_head_strides(lib, dtype, mask, chunk):
+    print(f"case two-level strides dtype={dtype} mask={mask} chunk={chunk}", flush=True)
+    check_batch_head_strides(lib, 3, 4, 700, 64, dtype, DEV, mask=mask, p=2, chunk=chunk, seed=30)
+    check_batch_head_strides(lib, 2, 8, 130, 32, dtype, DEV, mask=mask, p=1, chunk=chunk, seed=31)

@@ -15,7 +15,7 @@ import pytest
 import torch
 
 from reproducing_fastmax_results_amd import _capi
-from tests.parity import check_forward, check_forward_backward
+from tests.parity import check_batch_head_strides, check_forward, check_forward_backward
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CLANG = shutil.which("clang++", path="/opt/rocm/llvm/bin:" + os.environ.get("PATH", ""))
@@ -54,6 +54,12 @@ def test_moment_path_forward_backward_bf16(sim):
     check_forward_backward(sim, 1, 300, 32, torch.bfloat16, "cpu", mask=True, p=2, chunk=256, seed=3, saved=True)
     check_forward_backward(sim, 1, 40, 32, torch.bfloat16, "cpu", mask=False, p=2, nk=260,
                            flags=_capi.FLAG_FORCE_MOMENTS, seed=4)
+
+
+def test_batch_and_head_strides(sim):
+    # (b, n, h*d) projections viewed as (b, h, n, d): FastmaxStrides with heads > 1
+    check_batch_head_strides(sim, 2, 2, 70, 32, torch.bfloat16, "cpu", mask=True, p=2, seed=7)
+    check_batch_head_strides(sim, 2, 2, 40, 32, torch.float32, "cpu", mask=False, p=1, seed=8)
 
 
 def test_moment_path_forward_fp32_d64(sim):
