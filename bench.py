@@ -80,6 +80,51 @@ def cpu_baseline(n: int, d: int, p: int, tokens_per_step: int, heads_total: int,
     return {"value": tokens_per_step / t_step, "unit": "tokens/s", "cores": threads, "kind": "port", "sample": sample}
 
 
+def model_step(args, dev):
+    """One optimiser step of the model counterparts (the callers of the operator), synthetic data."""
+    import torch
+    from reproducing_fastmax_results_amd.transformer.model import gpt_for_c5, vit_for_c4
+    torch.manual_seed(0)
+    if args.model_step == "vit":
+        model = vit_for_c4().to(dev)
+        x = torch.rand(256, 1, 28, 28, device=dev)
+        y = torch.randint(0, 10, (256,), device=dev)
+        tokens, dtype, name = 256 * 50, "f32", "ViT 4 layers d_model=128 4 heads of 32, 256 images 28x28 in 4x4 patches + class token"
+
+        def loss_of():
+            return torch.nn.functional.cross_entropy(model(x), y)
+    else:
+        model = gpt_for_c5().to(dev).to(torch.bfloat16)
+        x = torch.randint(0, 50257, (16, 1024), device=dev)
+        y = torch.randint(0, 50257, (16, 1024), device=dev)
+        tokens, dtype, name = 16 * 1024, "bf16", "decoder-only LM 6 layers d_model=512 8 heads of 64, 16 x 1024 tokens, vocabulary 50257"
+
+        def loss_of():
+            return torch.nn.functional.cross_entropy(model(x).float().view(-1, 50257), y.view(-1))
+    opt = torch.optim.AdamW(model.parameters(), lr=1e-4)
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        loss = loss_of()
+        loss.backward()
+        opt.step()
+        return loss
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss = step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    return {"metric": f"{args.model_step} training step tokens/s", "value": tokens / dt, "unit": "tokens/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": 1e3 * dt, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
+            "config": {"workload": name, "optimizer": "AdamW", "attention": "Fastmax order 2, normalised q and k"},
+            "final_loss": float(loss)}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -89,6 +134,9 @@ def main() -> int:
     ap.add_argument("--chunk", type=int, default=0, help="segment length of the causal moment scan (0 = library default)")
     ap.add_argument("--independent-backward", action="store_true",
                     help="backward rebuilds the key-side copies and states instead of taking them from the forward")
+    ap.add_argument("--model-step", choices=["vit", "gpt"], default=None,
+                    help="instead of the operator benchmark, time one training step (forward, backward, AdamW) of "
+                         "the minimal ViT (fp32, 256 images of 28x28) or decoder-only LM (bf16, 16 x 1024 tokens)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device copy, the yardstick for the HBM traffic counters")
@@ -107,6 +155,9 @@ def main() -> int:
         return 3
     lib = get_lib()
     dev = torch.device("cuda:0")
+    if args.model_step:
+        print(json.dumps(model_step(args, dev)))
+        return 0
     W = WORKLOAD
     B, H, N, D, p = W["B"], W["H"], W["N"], W["D"], W["p"]
     bh = B * H
