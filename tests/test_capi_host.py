@@ -87,6 +87,20 @@ def test_forward_backward_reject_bad_arguments_before_launching(lib):
     args = [one] * 9
     assert lib.lib.fastmax_backward(C.byref(d), *args, None, 0, None) == 4
     assert lib.lib.fastmax_backward(C.byref(d), None, *args[1:], one, 1 << 30, None) == 1
+    # backward on a saved forward workspace: the workspace, its size and the flag are checked
+    big = 1 << 30
+    assert lib.lib.fastmax_backward_saved(C.byref(d), *args, None, big, one, big, None) == 1          # no forward workspace
+    assert lib.lib.fastmax_backward_saved(C.byref(d), *args, one, big, one, big, None) == 2           # flag not set
+    ds = base_desc()
+    ds.flags = _capi.FLAG_SAVE_FOR_BACKWARD
+    assert lib.lib.fastmax_backward_saved(C.byref(ds), *args, one, 16, one, big, None) == 4           # too small
+    assert lib.lib.fastmax_backward_saved(C.byref(ds), *args, C.c_void_p(264), big, one, big, None) == 4  # misaligned
+    # batch and head strides: heads must divide bh, both strides must be positive
+    two = base_desc(bh=8)
+    two.sq = _capi.Strides(64, 8 * 64, 128 * 8 * 64, 3)
+    assert lib.lib.fastmax_forward(C.byref(two), one, one, one, one, one, one, big, None) == 2
+    two.sq = _capi.Strides(64, 8 * 64, 0, 4)
+    assert lib.lib.fastmax_forward(C.byref(two), one, one, one, one, one, one, big, None) == 2
     nd = _capi.NormDesc()
     nd.bh, nd.n, nd.d, nd.dtype, nd.centre, nd.max_norm, nd.scale = 2, 10, 40, 0, 0, 1, 1.0
     assert lib.lib.fastmax_normalize(C.byref(nd), one, one, one, None) == 3
@@ -96,4 +110,4 @@ def test_forward_backward_reject_bad_arguments_before_launching(lib):
     nd.sx = nd.sy = _capi.Strides(640, 64)
     assert lib.lib.fastmax_normalize(C.byref(nd), one, one, None, None) == 4   # max_norm needs stats scratch
     assert lib.lib.fastmax_probe_mfma(None, None, None) == 1
-    assert lib.lib.fastmax_version() >= 100
+    assert lib.lib.fastmax_version() >= 101
