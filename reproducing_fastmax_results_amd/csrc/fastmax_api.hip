@@ -163,30 +163,49 @@ int launch_transpose(const void* x, const FastmaxStrides& s, int bh, int n, int 
   return fm_after_launch();
 }
 
-template <typename E, int DH, int NA, int TT>
-int launch_build_cfg(const BuildArgs<E>& a, int bh, fm_stream_t stream) {
+template <typename E, int DH, int NA, int TT, int SPW, bool QUAD>
+int launch_build_cfg(const BuildArgs<E>& a, int groups, int bh, int nsteps, fm_stream_t stream) {
   constexpr int PT = TT + Mma<E>::PAD;
   constexpr int AW = 4 * NA;
   size_t lds = size_t(3 * DH + AW) * PT * sizeof(E);                        // staged token tiles
-  const size_t red = size_t(2) * 4 * 64 * 16 * 4;                            // reduction scratch of the lower-order tiles
+  const size_t red = size_t(SPW) * 4 * 64 * 16 * 4;                          // reduction scratch of the lower-order tiles
   const size_t snap = size_t(AW) * DH * (DH + Mma<E>::PAD) * sizeof(E);      // snapshot staging
   if (lds < red) lds = red;
-  if (lds < snap) lds = snap;
-  fm_allow_lds(reinterpret_cast<const void*>(&k_build<E, DH, NA, TT>), lds);
-  FM_KERNEL_LAUNCH((k_build<E, DH, NA, TT>), fm_dim3(DH / AW, bh), fm_dim3(FM_THREADS), lds, stream, a);
+  if (QUAD && lds < snap) lds = snap;
+  fm_allow_lds(reinterpret_cast<const void*>(&k_build<E, DH, NA, TT, SPW, QUAD>), lds);
+  FM_KERNEL_LAUNCH((k_build<E, DH, NA, TT, SPW, QUAD>), fm_dim3(groups, bh, a.seg_parallel ? nsteps : 1),
+                   fm_dim3(FM_THREADS), lds, stream, a);
+  int st = fm_after_launch();
+  if (st || !a.seg_parallel || nsteps < 2) return st;
+  const int64_t nbig = a.quad ? int64_t(DH + 1) * DH * DH : int64_t(DH) * DH;
+  const int64_t total = nbig * (a.big2 ? 2 : 1) + StateDims<DH>::SMALL;
+  FM_KERNEL_LAUNCH((k_state_scan<E, DH>), fm_dim3(int((total + 255) / 256), bh), fm_dim3(256), 0, stream, a.big, a.big2,
+                   a.small, a.nslots, nsteps, a.mode, a.nseg, a.quad);
   return fm_after_launch();
 }
 
 template <typename E, int DH>
-int launch_build(const BuildArgs<E>& a, int bh, fm_stream_t stream) {
-  const int nsteps = a.mode == FM_WALK_TOTAL ? 1 : a.nseg - 1;
+int launch_build(const BuildArgs<E>& args, int bh, fm_stream_t stream) {
+  const int nsteps = args.mode == FM_WALK_TOTAL ? 1 : args.nseg - 1;
   if (nsteps <= 0) return FASTMAX_OK;
   ProfScope prof(FM_K_BUILD, stream);
-  // One value of `a` per wavefront (4 per workgroup) and 64-token tiles: 64 accumulator
-  // registers per wavefront leave room for two workgroups per CU, which measured faster on
-  // MI355X than two values per wavefront at one workgroup per CU (0.092 vs 0.115 ms at
-  // B*H = 32, N = 4096, D = 64).
-  return launch_build_cfg<E, DH, 1, 64>(a, bh, stream);
+  constexpr int NT = DH / 32, NSMALL = 2 * NT * NT + 2 * NT;
+  BuildArgs<E> a = args;
+  if (a.quad) {
+    // One value of `a` per wavefront (4 per workgroup) and 64-token tiles: 64 accumulator
+    // registers per wavefront leave room for two workgroups per CU, which measured faster on
+    // MI355X than two values per wavefront at one workgroup per CU (0.092 vs 0.115 ms at
+    // B*H = 32, N = 4096, D = 64).
+    constexpr int G = DH / 4;
+    a.seg_parallel = 0;
+    return launch_build_cfg<E, DH, 1, 64, (NSMALL + G - 1) / G, true>(a, G, bh, nsteps, stream);
+  }
+  // Order 1: the sums are a few 32x32 tiles per segment, so a serial walk is all latency.  Four
+  // workgroups per (segment, batch*head) share the tiles, every segment is summed on its own and a
+  // scan over the segments follows.
+  constexpr int SPW = (NSMALL + 3) / 4;
+  a.seg_parallel = nsteps > 1;
+  return launch_build_cfg<E, DH, 1, 64, SPW, false>(a, (NSMALL + SPW - 1) / SPW, bh, nsteps, stream);
 }
 
 // Dynamic LDS of k_pv and k_ds (one size for both): va, vb | own rows | region, where the
@@ -252,6 +271,7 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   if (st) return st;
   if (p.use_state) {
     BuildArgs<E> b;
+    b.seg_parallel = 0;
     b.xt = kt; b.pt = vt; b.rt = kt; b.zt = nullptr; b.za_sel = FM_SRC_R; b.zb_sel = FM_SRC_R;
     b.npad = p.npad_k; b.nseg = p.nseg; b.L = p.L; b.mode = d->mask ? FM_WALK_PREFIX : FM_WALK_TOTAL;
     b.quad = p.quad; b.big = big; b.small = small; b.nslots = p.nslots;

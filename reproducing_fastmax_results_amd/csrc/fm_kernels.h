@@ -282,6 +282,8 @@ template <typename E> struct BuildArgs {
   int vb_from_r;                           // vb sums the r operand instead of p
   float coef2, coef1, coefz, coefva, coefvb;
   float coef2b, coef1b;                    // coefficients of the transposed copy
+  int seg_parallel;                        // grid z = walk step: every workgroup sums one segment only and
+                                           // k_state_scan turns the per-segment sums into prefix / suffix states
 };
 
 FM_DEVICE void fm_walk_step(int mode, int nseg, int L, int npad, int w, int& tb, int& te, int& slot) {
@@ -298,20 +300,21 @@ FM_DEVICE void fm_walk_step(int mode, int nseg, int L, int npad, int w, int& tb,
 // The order-1 state, the denominator matrix Z and the two vector sums are 2*NT*NT + 2*NT
 // further 32x32 tiles; they are dealt round-robin to the workgroups of a batch*head, and
 // inside a workgroup each wavefront adds its quarter of the k-steps, so every workgroup
-// does the same amount of work and the grid is exactly (DH / (4*NA)) x bh.
+// does the same amount of work and the grid is exactly (DH / (4*NA)) x bh.  Order 1 has only the
+// lower-order tiles: QUAD = false drops the order-2 code and the grid shrinks to
+// ceil(tiles / SPW) workgroups per batch*head, each taking SPW tiles, so that the token tiles are
+// staged by four workgroups instead of sixteen.
 // Replaces the running sums of fastmax_cuda_forward.cu:165-276 (one thread per feature,
 // serial over tokens) and the cumsum of materialised outer products of
 // fastattention_einops.py:237-248.
-template <typename E, int DH, int NA, int TT>
+template <typename E, int DH, int NA, int TT, int SPW, bool QUAD>
 FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 ? 2 : 1)) k_build(BuildArgs<E> A) {
   typedef Mma<E> M;
   typedef typename M::frag frag;
   constexpr int AW = 4 * NA;
-  constexpr int G = DH / AW;                 // workgroups per batch*head
   constexpr int NT = DH / 32;                // 32-row tiles per feature axis
   constexpr int PT = TT + M::PAD;
   constexpr int NSMALL = 2 * NT * NT + 2 * NT;
-  constexpr int SPW = (NSMALL + G - 1) / G;  // small tiles per workgroup (at most)
   constexpr int NSTEP = TT / M::KSTEP;
   FM_DYN_SMEM(smem);
   E* s0 = reinterpret_cast<E*>(smem);        // p tile   [DH][PT]
@@ -321,6 +324,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 ? 2 : 1)
   const int tid = FM_TID_X, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   const int wave = FM_UNIFORM(tid >> 6);
   int grp, bh;
+  const int G = FM_GDIM_X;                   // workgroups per batch*head
   fm_xcd_map(G, FM_GDIM_Y, grp, bh);
   const int64_t tb_off = int64_t(bh) * DH * A.npad;
   const int nsteps = (A.mode == FM_WALK_TOTAL) ? 1 : A.nseg - 1;
@@ -329,7 +333,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 ? 2 : 1)
   E* big2 = A.big2 ? A.big2 + int64_t(bh) * A.nslots * StateDims<DH>::BIG : nullptr;
   float* sml = A.small + int64_t(bh) * A.nslots * StateDims<DH>::SMALL;
   const bool has_z = A.zt != nullptr;
-  const bool quad = A.quad != 0;
+  const bool quad = QUAD && A.quad != 0;
 
   // small tiles of this workgroup: offsets (elements from s0) of the operand rows in LDS for
   // the A side and the B side (-1: a column of ones)
@@ -352,8 +356,10 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 ? 2 : 1)
     sm_b[s] = pb >= 0 ? pb + lr * PT + lh * M::KPL : -1;
   }
 
-  int w = 0, tb, te, slot;
-  fm_walk_step(A.mode, A.nseg, A.L, A.npad, 0, tb, te, slot);
+  // the steps of the walk this workgroup takes: all of them in turn, or the one its grid z names
+  const int w_end = A.seg_parallel ? FM_BID_Z + 1 : nsteps;
+  int w = A.seg_parallel ? FM_BID_Z : 0, tb, te, slot;
+  fm_walk_step(A.mode, A.nseg, A.L, A.npad, w, tb, te, slot);
   int t = tb;
   const int a0 = grp * AW;
   TileRegs<E, DH, TT> rp, rr, rz;
@@ -385,7 +391,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 ? 2 : 1)
     bool has_next = true;
     if (last) {
       nw = w + 1;
-      if (nw < nsteps) { fm_walk_step(A.mode, A.nseg, A.L, A.npad, nw, ntb, nte, nslot); nt = ntb; }
+      if (nw < w_end) { fm_walk_step(A.mode, A.nseg, A.L, A.npad, nw, ntb, nte, nslot); nt = ntb; }
       else has_next = false;
     }
     if (has_next) {
@@ -518,6 +524,37 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 ? 2 : 1)
       }
     }
     t = nt; w = nw; tb = ntb; te = nte; slot = nslot; have = has_next;
+  }
+}
+
+// ------------------------------------------------------------------------------
+// k_state_scan: turns per-segment sums (k_build with seg_parallel) into the states the readers
+// expect: slot s becomes the sum over the walk up to and including its own step.  Elementwise
+// over the order-1 slab of `big` (and of `big2`), over the order-2 slabs too when quad, and over
+// `small`; the running sum is kept in fp32.  grid (ceil(elements / 256), bh).
+// ------------------------------------------------------------------------------
+template <typename E, int DH>
+FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_state_scan(E* FM_RESTRICT big, E* FM_RESTRICT big2, float* FM_RESTRICT small,
+                                                  int nslots, int nsteps, int mode, int nseg, int quad) {
+  const int bh = FM_BID_Y;
+  const int64_t nbig = quad ? int64_t(DH + 1) * DH * DH : int64_t(DH) * DH;
+  const int64_t first = quad ? 0 : int64_t(DH) * DH * DH;       // the order-1 slab is the last one
+  const int64_t nsmall = StateDims<DH>::SMALL;
+  const int64_t total = nbig * (big2 ? 2 : 1) + nsmall;
+  const int64_t i = int64_t(FM_BID_X) * 256 + FM_TID_X;
+  if (i >= total) return;
+  float run = 0.f;
+  for (int w = 0; w < nsteps; ++w) {
+    const int slot = mode == FM_WALK_PREFIX ? w + 1 : nseg - 2 - w;   // the slot k_build's step w writes
+    if (i < nbig * (big2 ? 2 : 1)) {
+      E* b = (i < nbig ? big : big2) + (int64_t(bh) * nslots + slot) * StateDims<DH>::BIG + first + (i < nbig ? i : i - nbig);
+      run += float(*b);
+      *b = CE<E>::from(run);
+    } else {
+      float* sp = small + (int64_t(bh) * nslots + slot) * nsmall + (i - nbig * (big2 ? 2 : 1));
+      run += *sp;
+      *sp = run;
+    }
   }
 }
 

@@ -56,6 +56,15 @@ def test_moment_path_forward_backward_bf16(sim):
                            flags=_capi.FLAG_FORCE_MOMENTS, seed=4)
 
 
+def test_order1_segments_summed_apart_then_scanned(sim):
+    # order 1 with three segments: each segment's sums come from its own workgroups and
+    # an elementwise scan over the segments makes the prefix and suffix states
+    check_forward_backward(sim, 1, 600, 32, torch.bfloat16, "cpu", mask=True, p=1, chunk=256, seed=9)
+    check_forward_backward(sim, 1, 600, 32, torch.float32, "cpu", mask=True, p=1, chunk=256, seed=10, saved=True)
+    check_forward_backward(sim, 1, 40, 32, torch.bfloat16, "cpu", mask=False, p=1, nk=300,
+                           flags=_capi.FLAG_FORCE_MOMENTS, seed=11)
+
+
 def test_batch_and_head_strides(sim):
     # (b, n, h*d) projections viewed as (b, h, n, d): FastmaxStrides with heads > 1
     check_batch_head_strides(sim, 2, 2, 70, 32, torch.bfloat16, "cpu", mask=True, p=2, seed=7)
