@@ -107,8 +107,11 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   if (d->mask) {
     // Segment length.  Dense tiles cost grows with L, the moment states cost the same per token
     // whatever L is (readout) plus the walk that builds them.  Measured on MI355X (D = 64, bf16):
-    // one segment (no states at all) wins up to about 6000 tokens, 1024-token segments beyond.
-    int L = d->chunk > 0 ? int(round_up(d->chunk, 256)) : (d->nq > 6144 ? 1024 : p.npad_q);
+    // order 2: one segment (no states at all) wins up to about 6000 tokens, 1024-token segments
+    // beyond; order 1 (one D x D state per segment): one segment up to about 3000 tokens,
+    // 512-token segments beyond.
+    const int auto_L = p.quad ? (d->nq > 6144 ? 1024 : p.npad_q) : (d->nq > 3072 ? 512 : p.npad_q);
+    int L = d->chunk > 0 ? int(round_up(d->chunk, 256)) : auto_L;
     if (force_dense || L > p.npad_q) L = p.npad_q;
     p.L = L;
     p.nseg = (d->nq + L - 1) / L;
@@ -168,7 +171,7 @@ int launch_build_cfg(const BuildArgs<E>& a, int groups, int bh, int nsteps, fm_s
   constexpr int PT = TT + Mma<E>::PAD;
   constexpr int AW = 4 * NA;
   size_t lds = size_t(3 * DH + AW) * PT * sizeof(E);                        // staged token tiles
-  const size_t red = size_t(SPW) * 4 * 64 * 16 * 4;                          // reduction scratch of the lower-order tiles
+  const size_t red = size_t(SPW < 4 ? SPW : 4) * 4 * 64 * 16 * 4;                // reduction scratch of the lower-order tiles
   const size_t snap = size_t(AW) * DH * (DH + Mma<E>::PAD) * sizeof(E);      // snapshot staging
   if (lds < red) lds = red;
   if (QUAD && lds < snap) lds = snap;
@@ -200,10 +203,14 @@ int launch_build(const BuildArgs<E>& args, int bh, fm_stream_t stream) {
     a.seg_parallel = 0;
     return launch_build_cfg<E, DH, 1, 64, (NSMALL + G - 1) / G, true>(a, G, bh, nsteps, stream);
   }
-  // Order 1: the sums are a few 32x32 tiles per segment, so a serial walk is all latency.  Four
-  // workgroups per (segment, batch*head) share the tiles, every segment is summed on its own and a
-  // scan over the segments follows.
-  constexpr int SPW = (NSMALL + 3) / 4;
+  // Order 1: the sums are a few 32x32 tiles per segment, so a serial walk is all latency and
+  // splitting the tiles over workgroups only multiplies the reads of the token tiles.  One
+  // workgroup per (segment, batch*head) sums all the tiles of its segment and a scan over the
+  // segments follows.
+#ifndef FM_TUNE_P1_G
+#define FM_TUNE_P1_G 1
+#endif
+  constexpr int SPW = (NSMALL + FM_TUNE_P1_G - 1) / FM_TUNE_P1_G;
   a.seg_parallel = nsteps > 1;
   return launch_build_cfg<E, DH, 1, 64, SPW, false>(a, (NSMALL + SPW - 1) / SPW, bh, nsteps, stream);
 }

@@ -308,7 +308,7 @@ FM_DEVICE void fm_walk_step(int mode, int nseg, int L, int npad, int w, int& tb,
 // serial over tokens) and the cumsum of materialised outer products of
 // fastattention_einops.py:237-248.
 template <typename E, int DH, int NA, int TT, int SPW, bool QUAD>
-FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 ? 2 : 1)) k_build(BuildArgs<E> A) {
+FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <= 4 ? 2 : 1)) k_build(BuildArgs<E> A) {
   typedef Mma<E> M;
   typedef typename M::frag frag;
   constexpr int AW = 4 * NA;
@@ -341,7 +341,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 ? 2 : 1)
 #pragma unroll
   for (int s = 0; s < SPW; ++s) {
     const int t = grp + s * G;
-    sm_id[s] = t < NSMALL ? t : -1;
+    sm_id[s] = (t < NSMALL && (quad || t < NT * NT || t >= 2 * NT * NT)) ? t : -1;   // order 1 has no Z
     const int o0 = 0, o1 = DH * PT, o3 = (2 * DH + AW) * PT;
     const int oza = A.za_sel == FM_SRC_P ? o0 : (A.za_sel == FM_SRC_R ? o1 : o3);
     const int ozb = A.zb_sel == FM_SRC_P ? o0 : (A.zb_sel == FM_SRC_R ? o1 : o3);
@@ -488,37 +488,50 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 ? 2 : 1)
           }
         }
       }
-      // reduce the four wavefronts' partial lower-order tiles through LDS (the token tiles are spent)
-      FM_SYNC();
-      float* red = reinterpret_cast<float*>(smem);           // [SPW][4 waves][64 lanes][16]
+      // reduce the four wavefronts' partial lower-order tiles through LDS (the token tiles are
+      // spent), RC tiles per pass: every wavefront stores its part of each, then wavefront u adds
+      // the four parts of tile u and writes it
+      constexpr int RC = SPW < 4 ? SPW : 4;
+      float* red = reinterpret_cast<float*>(smem);           // [RC][4 waves][16][64 lanes]
+      float* ds = sml + int64_t(slot) * StateDims<DH>::SMALL;
 #pragma unroll
-      for (int s = 0; s < SPW; ++s)
+      for (int sb = 0; sb < SPW; sb += RC) {
+        FM_SYNC();
 #pragma unroll
-        for (int e = 0; e < 16; ++e) red[((s * 4 + wave) * 16 + e) * 64 + lane] = sacc[s][e];
-      FM_SYNC();
-      if (wave == 0) {
-        float* ds = sml + int64_t(slot) * StateDims<DH>::SMALL;
+        for (int u = 0; u < RC; ++u)
+          if (sb + u < SPW) {
 #pragma unroll
-        for (int s = 0; s < SPW; ++s) {
-          const int tl = sm_id[s];
-          if (tl < 0) continue;
+            for (int e = 0; e < 16; ++e) red[((u * 4 + wave) * 16 + e) * 64 + lane] = sacc[sb + u][e];
+          }
+        FM_SYNC();
+        const int tl = grp + (sb + wave) * G;
+        if (wave < RC && sb + wave < SPW && tl < NSMALL && (quad || tl < NT * NT || tl >= 2 * NT * NT)) {
+          float v[16];
 #pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            const float v = red[((s * 4 + 0) * 16 + e) * 64 + lane] + red[((s * 4 + 1) * 16 + e) * 64 + lane] +
-                            red[((s * 4 + 2) * 16 + e) * 64 + lane] + red[((s * 4 + 3) * 16 + e) * 64 + lane];
-            const int rr_ = fm_acc_row(e, lh);
-            if (tl < NT * NT) {
-              const int r = 32 * (tl / NT) + rr_, c = 32 * (tl % NT) + lr;
-              big[int64_t(slot) * StateDims<DH>::BIG + int64_t(DH) * DH * DH + r * DH + c] = CE<E>::from(A.coef1 * v);
-              if (big2)
-                big2[int64_t(slot) * StateDims<DH>::BIG + int64_t(DH) * DH * DH + c * DH + r] = CE<E>::from(A.coef1b * v);
-            } else if (tl < 2 * NT * NT) {
-              const int u = tl - NT * NT;
-              ds[(32 * (u / NT) + rr_) * DH + 32 * (u % NT) + lr] = A.coefz * v;
-            } else if (lr == 0) {
-              if (tl < 2 * NT * NT + NT) ds[DH * DH + 32 * (tl - 2 * NT * NT) + rr_] = A.coefva * v;
-              else ds[DH * DH + DH + 32 * (tl - 2 * NT * NT - NT) + rr_] = A.coefvb * v;
+          for (int e = 0; e < 16; ++e)
+            v[e] = red[((wave * 4 + 0) * 16 + e) * 64 + lane] + red[((wave * 4 + 1) * 16 + e) * 64 + lane] +
+                   red[((wave * 4 + 2) * 16 + e) * 64 + lane] + red[((wave * 4 + 3) * 16 + e) * 64 + lane];
+          if (tl < NT * NT) {
+            const int r0 = 32 * (tl / NT), c = 32 * (tl % NT) + lr;
+            E* d1 = big + int64_t(slot) * StateDims<DH>::BIG + int64_t(DH) * DH * DH;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) d1[(r0 + fm_acc_row(e, lh)) * DH + c] = CE<E>::from(A.coef1 * v[e]);
+            if (big2) {
+              E* d2 = big2 + int64_t(slot) * StateDims<DH>::BIG + int64_t(DH) * DH * DH;
+#pragma unroll
+              for (int e = 0; e < 16; ++e) d2[c * DH + r0 + fm_acc_row(e, lh)] = CE<E>::from(A.coef1b * v[e]);
             }
+          } else if (tl < 2 * NT * NT) {
+            const int u = tl - NT * NT;
+            float* dz = ds + 32 * (u / NT) * DH + 32 * (u % NT) + lr;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) dz[fm_acc_row(e, lh) * DH] = A.coefz * v[e];
+          } else if (lr == 0) {
+            const bool is_va = tl < 2 * NT * NT + NT;
+            float* dv = ds + DH * DH + (is_va ? 32 * (tl - 2 * NT * NT) : DH + 32 * (tl - 2 * NT * NT - NT));
+            const float cf = is_va ? A.coefva : A.coefvb;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) dv[fm_acc_row(e, lh)] = cf * v[e];
           }
         }
       }
@@ -533,6 +546,22 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 ? 2 : 1)
 // over the order-1 slab of `big` (and of `big2`), over the order-2 slabs too when quad, and over
 // `small`; the running sum is kept in fp32.  grid (ceil(elements / 256), bh).
 // ------------------------------------------------------------------------------
+// One element's running sum over the walk: `stride` elements lie between the slots of two
+// consecutive steps.  Sixteen steps are loaded before any is added and stored, so the chain of
+// dependent memory round trips is a sixteenth as long as the walk.
+template <typename T> FM_DEVICE void fm_scan_run(T* p, int64_t stride, int nsteps) {
+  constexpr int UB = 16;
+  float run = 0.f;
+  for (int w0 = 0; w0 < nsteps; w0 += UB) {
+    float v[UB];
+#pragma unroll
+    for (int u = 0; u < UB; ++u) v[u] = (w0 + u < nsteps) ? float(p[(w0 + u) * stride]) : 0.f;
+#pragma unroll
+    for (int u = 0; u < UB; ++u)
+      if (w0 + u < nsteps) { run += v[u]; p[(w0 + u) * stride] = CE<T>::from(run); }
+  }
+}
+
 template <typename E, int DH>
 FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_state_scan(E* FM_RESTRICT big, E* FM_RESTRICT big2, float* FM_RESTRICT small,
                                                   int nslots, int nsteps, int mode, int nseg, int quad) {
@@ -540,21 +569,18 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_state_scan(E* FM_RESTRICT big, E* FM_REST
   const int64_t nbig = quad ? int64_t(DH + 1) * DH * DH : int64_t(DH) * DH;
   const int64_t first = quad ? 0 : int64_t(DH) * DH * DH;       // the order-1 slab is the last one
   const int64_t nsmall = StateDims<DH>::SMALL;
-  const int64_t total = nbig * (big2 ? 2 : 1) + nsmall;
+  const int64_t nb2 = nbig * (big2 ? 2 : 1);
   const int64_t i = int64_t(FM_BID_X) * 256 + FM_TID_X;
-  if (i >= total) return;
-  float run = 0.f;
-  for (int w = 0; w < nsteps; ++w) {
-    const int slot = mode == FM_WALK_PREFIX ? w + 1 : nseg - 2 - w;   // the slot k_build's step w writes
-    if (i < nbig * (big2 ? 2 : 1)) {
-      E* b = (i < nbig ? big : big2) + (int64_t(bh) * nslots + slot) * StateDims<DH>::BIG + first + (i < nbig ? i : i - nbig);
-      run += float(*b);
-      *b = CE<E>::from(run);
-    } else {
-      float* sp = small + (int64_t(bh) * nslots + slot) * nsmall + (i - nbig * (big2 ? 2 : 1));
-      run += *sp;
-      *sp = run;
-    }
+  if (i >= nb2 + nsmall) return;
+  // the slot k_build's step w writes is slot0 + w * dir
+  const int slot0 = mode == FM_WALK_PREFIX ? 1 : nseg - 2;
+  const int dir = mode == FM_WALK_PREFIX ? 1 : -1;
+  if (i < nb2) {
+    E* b = (i < nbig ? big : big2) + (int64_t(bh) * nslots + slot0) * StateDims<DH>::BIG + first + (i < nbig ? i : i - nbig);
+    fm_scan_run<E>(b, int64_t(dir) * StateDims<DH>::BIG, nsteps);
+  } else {
+    float* sp = small + (int64_t(bh) * nslots + slot0) * nsmall + (i - nb2);
+    fm_scan_run<float>(sp, int64_t(dir) * nsmall, nsteps);
   }
 }
 

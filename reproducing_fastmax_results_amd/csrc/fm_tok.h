@@ -233,7 +233,8 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
   }
   const float* sml = A.small + (int64_t(bh) * A.nslots + G.slot) * StateDims<DH>::SMALL;
   if (G.use_state) {
-    if (OWN == FM_OWN_Q) fm_stage_small<E, DH, QT>(sml, R, vecs, tid, 1.0f);
+    // order 1 has no Z (its coefficient is the order-2 one): only the two vectors are staged
+    if (OWN == FM_OWN_Q && A.quad) fm_stage_small<E, DH, QT>(sml, R, vecs, tid, 1.0f);
     else if (tid < 2 * DH) vecs[tid] = sml[DH * DH + tid];
   }
   FM_SYNC();
@@ -266,7 +267,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
       for (int j = 0; j < QT; ++j)
 #pragma unroll
         for (int mt = 0; mt < NT; ++mt) {
-          const fm_f32x16 y = fm_zy<E, DH, QT>(R, of[j], mt, lr, lh);
+          const fm_f32x16 y = A.quad ? fm_zy<E, DH, QT>(R, of[j], mt, lr, lh) : fm_zero16();
 #pragma unroll
           for (int e = 0; e < 16; ++e) {
             const int m = 32 * mt + fm_acc_row(e, lh);
@@ -421,8 +422,11 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
     ro.load(A.own_r + (int64_t(bh) * A.npad_own + t0) * DH, DH, tid);
     ro.store(Own, PQ, tid);
   }
-  if (G.use_state)
-    fm_stage_small<E, DH, QT>(A.small + (int64_t(bh) * A.nslots + G.slot) * StateDims<DH>::SMALL, R, vecs, tid, A.zscale);
+  if (G.use_state) {
+    const float* sml = A.small + (int64_t(bh) * A.nslots + G.slot) * StateDims<DH>::SMALL;
+    if (A.quad) fm_stage_small<E, DH, QT>(sml, R, vecs, tid, A.zscale);
+    else if (tid < 2 * DH) vecs[tid] = sml[DH * DH + tid];   // order 1 has no Z
+  }
   FM_SYNC();
 
   int tw[QT], xrow[QT];
@@ -461,7 +465,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
     for (int j = 0; j < QT; ++j)
 #pragma unroll
       for (int mt = 0; mt < NT; ++mt) {
-        const fm_f32x16 y = fm_zy<E, DH, QT>(R, of[j], mt, lr, lh);
+        const fm_f32x16 y = A.quad ? fm_zy<E, DH, QT>(R, of[j], mt, lr, lh) : fm_zero16();
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[j][mt][e] = -ci[j] * (y[e] + vecs[32 * mt + fm_acc_row(e, lh)]);
       }
