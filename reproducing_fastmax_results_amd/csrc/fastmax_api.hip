@@ -108,9 +108,9 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
     // Segment length.  Dense tiles cost grows with L, the moment states cost the same per token
     // whatever L is (readout) plus the walk that builds them.  Measured on MI355X (D = 64, bf16):
     // order 2: one segment (no states at all) wins up to about 6000 tokens, 1024-token segments
-    // beyond; order 1 (one D x D state per segment): one segment up to about 3000 tokens,
-    // 512-token segments beyond.
-    const int auto_L = p.quad ? (d->nq > 6144 ? 1024 : p.npad_q) : (d->nq > 3072 ? 512 : p.npad_q);
+    // beyond; order 1 (one D x D state per segment): one segment up to about 1500 tokens,
+    // 256-token segments beyond.
+    const int auto_L = p.quad ? (d->nq > 6144 ? 1024 : p.npad_q) : (d->nq > 1536 ? 256 : p.npad_q);
     int L = d->chunk > 0 ? int(round_up(d->chunk, 256)) : auto_L;
     if (force_dense || L > p.npad_q) L = p.npad_q;
     p.L = L;
@@ -166,6 +166,17 @@ int launch_transpose(const void* x, const FastmaxStrides& s, int bh, int n, int 
   return fm_after_launch();
 }
 
+// per-segment sums -> prefix / suffix states (after a build whose workgroups took one step each)
+template <typename E, int DH>
+int launch_scan(const BuildArgs<E>& a, int bh, int nsteps, fm_stream_t stream) {
+  constexpr int VE = 16 / sizeof(E);                            // 16-byte items, as k_state_scan counts them
+  const int64_t nbig = (a.quad ? int64_t(DH + 1) * DH * DH : int64_t(DH) * DH) / VE;
+  const int64_t total = nbig * (a.big2 ? 2 : 1) + (StateDims<DH>::SMALL - (a.quad ? 0 : DH * DH)) / 4;
+  FM_KERNEL_LAUNCH((k_state_scan<E, DH>), fm_dim3(int((total + 255) / 256), bh), fm_dim3(256), 0, stream, a.big, a.big2,
+                   a.small, a.nslots, nsteps, a.mode, a.nseg, a.quad);
+  return fm_after_launch();
+}
+
 template <typename E, int DH, int NA, int TT, int SPW, bool QUAD>
 int launch_build_cfg(const BuildArgs<E>& a, int groups, int bh, int nsteps, fm_stream_t stream) {
   constexpr int PT = TT + Mma<E>::PAD;
@@ -180,11 +191,7 @@ int launch_build_cfg(const BuildArgs<E>& a, int groups, int bh, int nsteps, fm_s
                    fm_dim3(FM_THREADS), lds, stream, a);
   int st = fm_after_launch();
   if (st || !a.seg_parallel || nsteps < 2) return st;
-  const int64_t nbig = a.quad ? int64_t(DH + 1) * DH * DH : int64_t(DH) * DH;
-  const int64_t total = nbig * (a.big2 ? 2 : 1) + StateDims<DH>::SMALL;
-  FM_KERNEL_LAUNCH((k_state_scan<E, DH>), fm_dim3(int((total + 255) / 256), bh), fm_dim3(256), 0, stream, a.big, a.big2,
-                   a.small, a.nslots, nsteps, a.mode, a.nseg, a.quad);
-  return fm_after_launch();
+  return launch_scan<E, DH>(a, bh, nsteps, stream);
 }
 
 template <typename E, int DH>
@@ -203,16 +210,16 @@ int launch_build(const BuildArgs<E>& args, int bh, fm_stream_t stream) {
     a.seg_parallel = 0;
     return launch_build_cfg<E, DH, 1, 64, (NSMALL + G - 1) / G, true>(a, G, bh, nsteps, stream);
   }
-  // Order 1: the sums are a few 32x32 tiles per segment, so a serial walk is all latency and
-  // splitting the tiles over workgroups only multiplies the reads of the token tiles.  One
-  // workgroup per (segment, batch*head) sums all the tiles of its segment and a scan over the
-  // segments follows.
-#ifndef FM_TUNE_P1_G
-#define FM_TUNE_P1_G 1
-#endif
-  constexpr int SPW = (NSMALL + FM_TUNE_P1_G - 1) / FM_TUNE_P1_G;
-  a.seg_parallel = nsteps > 1;
-  return launch_build_cfg<E, DH, 1, 64, SPW, false>(a, (NSMALL + SPW - 1) / SPW, bh, nsteps, stream);
+  // Order 1: the sums are a few 32x32 tiles per segment, far too little work per token tile for
+  // a staged walk.  One workgroup per (segment, batch*head) sums its segment from fragments loaded
+  // straight from the operands, and a scan over the segments follows.
+  a.seg_parallel = 1;
+  const size_t lds = size_t(4) * 4 * 64 * 16 * 4;
+  fm_allow_lds(reinterpret_cast<const void*>(&k_build1<E, DH>), lds);
+  FM_KERNEL_LAUNCH((k_build1<E, DH>), fm_dim3(1, bh, nsteps), fm_dim3(FM_THREADS), lds, stream, a);
+  const int st = fm_after_launch();
+  if (st || nsteps < 2) return st;
+  return launch_scan<E, DH>(a, bh, nsteps, stream);
 }
 
 // Dynamic LDS of k_pv and k_ds (one size for both): va, vb | own rows | region, where the

@@ -294,6 +294,37 @@ FM_DEVICE void fm_walk_step(int mode, int nseg, int L, int npad, int w, int& tb,
   } else { tb = 0; te = npad; slot = 0; }
 }
 
+// One reduced lower-order 32x32 tile (v: the lane's 16 accumulator values) to its place in the
+// state of `slot`: tl < NT*NT the order-1 tile (and its transposed copy), then the Z tiles, then
+// the two vector sums (column 0 of their tiles).
+template <typename E, int DH>
+FM_DEVICE void fm_put_small(const BuildArgs<E>& A, E* big, E* big2, float* ds, int slot, int tl, const float* v, int lr,
+                            int lh) {
+  constexpr int NT = DH / 32;
+  if (tl < NT * NT) {
+    const int r0 = 32 * (tl / NT), c = 32 * (tl % NT) + lr;
+    E* d1 = big + int64_t(slot) * StateDims<DH>::BIG + int64_t(DH) * DH * DH;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) d1[(r0 + fm_acc_row(e, lh)) * DH + c] = CE<E>::from(A.coef1 * v[e]);
+    if (big2) {
+      E* d2 = big2 + int64_t(slot) * StateDims<DH>::BIG + int64_t(DH) * DH * DH;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) d2[c * DH + r0 + fm_acc_row(e, lh)] = CE<E>::from(A.coef1b * v[e]);
+    }
+  } else if (tl < 2 * NT * NT) {
+    const int u = tl - NT * NT;
+    float* dz = ds + 32 * (u / NT) * DH + 32 * (u % NT) + lr;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) dz[fm_acc_row(e, lh) * DH] = A.coefz * v[e];
+  } else if (lr == 0) {
+    const bool is_va = tl < 2 * NT * NT + NT;
+    float* dv = ds + DH * DH + (is_va ? 32 * (tl - 2 * NT * NT) : DH + 32 * (tl - 2 * NT * NT - NT));
+    const float cf = is_va ? A.coefva : A.coefvb;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) dv[fm_acc_row(e, lh)] = cf * v[e];
+  }
+}
+
 // k_build: one workgroup per (group of 4*NA values of a, batch*head) walks the tokens
 // once, keeping its slice of the order-2 state in accumulators and writing a snapshot at
 // every segment boundary, so the prefix (or suffix) scan over segments is implicit.
@@ -511,28 +542,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <
           for (int e = 0; e < 16; ++e)
             v[e] = red[((wave * 4 + 0) * 16 + e) * 64 + lane] + red[((wave * 4 + 1) * 16 + e) * 64 + lane] +
                    red[((wave * 4 + 2) * 16 + e) * 64 + lane] + red[((wave * 4 + 3) * 16 + e) * 64 + lane];
-          if (tl < NT * NT) {
-            const int r0 = 32 * (tl / NT), c = 32 * (tl % NT) + lr;
-            E* d1 = big + int64_t(slot) * StateDims<DH>::BIG + int64_t(DH) * DH * DH;
-#pragma unroll
-            for (int e = 0; e < 16; ++e) d1[(r0 + fm_acc_row(e, lh)) * DH + c] = CE<E>::from(A.coef1 * v[e]);
-            if (big2) {
-              E* d2 = big2 + int64_t(slot) * StateDims<DH>::BIG + int64_t(DH) * DH * DH;
-#pragma unroll
-              for (int e = 0; e < 16; ++e) d2[c * DH + r0 + fm_acc_row(e, lh)] = CE<E>::from(A.coef1b * v[e]);
-            }
-          } else if (tl < 2 * NT * NT) {
-            const int u = tl - NT * NT;
-            float* dz = ds + 32 * (u / NT) * DH + 32 * (u % NT) + lr;
-#pragma unroll
-            for (int e = 0; e < 16; ++e) dz[fm_acc_row(e, lh) * DH] = A.coefz * v[e];
-          } else if (lr == 0) {
-            const bool is_va = tl < 2 * NT * NT + NT;
-            float* dv = ds + DH * DH + (is_va ? 32 * (tl - 2 * NT * NT) : DH + 32 * (tl - 2 * NT * NT - NT));
-            const float cf = is_va ? A.coefva : A.coefvb;
-#pragma unroll
-            for (int e = 0; e < 16; ++e) dv[fm_acc_row(e, lh)] = cf * v[e];
-          }
+          fm_put_small<E, DH>(A, big, big2, ds, slot, tl, v, lr, lh);
         }
       }
     }
@@ -540,35 +550,132 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <
   }
 }
 
+// k_build1: the order-1 states (the D x D sum and the two vector sums, no Z) of one walk step per
+// workgroup; grid (1, bh, steps), k_state_scan follows when there are several steps.  The sums are
+// 8 tiles for D = 64, far too little work per token tile to pay for staging and barriers: each
+// wavefront takes a quarter of the step's tokens and loads its MFMA fragments straight from the
+// transposed operands (16 bytes per lane, four k-steps in flight), and the four partial sums meet
+// in LDS once at the end.  Needs (te - tb) to be a multiple of 4 * 4 * KSTEP tokens (segments and
+// padded lengths are multiples of 256).
+template <typename E, int DH>
+FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_build1(BuildArgs<E> A) {
+  typedef Mma<E> M;
+  typedef typename M::frag frag;
+  constexpr int NT = DH / 32, NTILE = NT * NT + 2 * NT, UB = 4;
+  FM_DYN_SMEM(smem);
+  const int tid = FM_TID_X, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int wave = FM_UNIFORM(tid >> 6);
+  const int bh = FM_BID_Y;
+  int tb, te, slot;
+  fm_walk_step(A.mode, A.nseg, A.L, A.npad, FM_BID_Z, tb, te, slot);
+  E* big = A.big + int64_t(bh) * A.nslots * StateDims<DH>::BIG;
+  E* big2 = A.big2 ? A.big2 + int64_t(bh) * A.nslots * StateDims<DH>::BIG : nullptr;
+  float* ds = A.small + (int64_t(bh) * A.nslots + slot) * StateDims<DH>::SMALL;
+  const int per_wave = (te - tb) / 4;                  // tokens of this wavefront
+  const int64_t row = (int64_t(bh) * DH + lr) * A.npad + tb + wave * per_wave + lh * M::KPL;
+  const E* pp = A.pt + row;
+  const E* rp = A.rt + row;
+  const bool has_z = A.zt != nullptr;
+  const E* zp = has_z ? A.zt + row : pp;
+  const int za = A.za_sel;
+  const bool vb_r = A.vb_from_r != 0;
+  const int64_t tile = int64_t(32) * A.npad;           // 32 feature rows further
+  fm_f32x16 acc[NTILE];
+#pragma unroll
+  for (int i = 0; i < NTILE; ++i) acc[i] = fm_zero16();
+  const frag ones = M::splat(E(1.0f));
+  for (int t = 0; t < per_wave; t += UB * M::KSTEP) {
+    frag fp[UB][NT], fr[UB][NT], fz[UB][NT];
+#pragma unroll
+    for (int u = 0; u < UB; ++u)
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        fp[u][j] = M::load(pp + j * tile + t + u * M::KSTEP);
+        fr[u][j] = M::load(rp + j * tile + t + u * M::KSTEP);
+        fz[u][j] = has_z ? M::load(zp + j * tile + t + u * M::KSTEP) : fp[u][j];
+      }
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+#pragma unroll
+      for (int i = 0; i < NT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) acc[i * NT + j] = M::mma(fp[u][i], fr[u][j], acc[i * NT + j]);
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        const frag fa = za == FM_SRC_P ? fp[u][j] : (za == FM_SRC_R ? fr[u][j] : fz[u][j]);
+        acc[NT * NT + j] = M::mma(fa, ones, acc[NT * NT + j]);
+        acc[NT * NT + NT + j] = M::mma(vb_r ? fr[u][j] : fp[u][j], ones, acc[NT * NT + NT + j]);
+      }
+    }
+  }
+  // the four wavefronts' partial tiles meet in LDS, RC tiles per pass; wavefront u adds and writes tile u
+  constexpr int RC = 4;
+  float* red = reinterpret_cast<float*>(smem);         // [RC][4 waves][16][64 lanes]
+#pragma unroll
+  for (int sb = 0; sb < NTILE; sb += RC) {
+    if (sb) FM_SYNC();
+#pragma unroll
+    for (int u = 0; u < RC; ++u)
+      if (sb + u < NTILE) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) red[((u * 4 + wave) * 16 + e) * 64 + lane] = acc[sb + u][e];
+      }
+    FM_SYNC();
+    const int i = sb + wave;
+    if (i < NTILE) {
+      float v[16];
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+        v[e] = red[((wave * 4 + 0) * 16 + e) * 64 + lane] + red[((wave * 4 + 1) * 16 + e) * 64 + lane] +
+               red[((wave * 4 + 2) * 16 + e) * 64 + lane] + red[((wave * 4 + 3) * 16 + e) * 64 + lane];
+      fm_put_small<E, DH>(A, big, big2, ds, slot, i < NT * NT ? i : i + NT * NT, v, lr, lh);
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------
 // k_state_scan: turns per-segment sums (k_build with seg_parallel) into the states the readers
 // expect: slot s becomes the sum over the walk up to and including its own step.  Elementwise
 // over the order-1 slab of `big` (and of `big2`), over the order-2 slabs too when quad, and over
-// `small`; the running sum is kept in fp32.  grid (ceil(elements / 256), bh).
+// the vector sums (and Z when quad) of `small`; the running sum is kept in fp32.
 // ------------------------------------------------------------------------------
-// One element's running sum over the walk: `stride` elements lie between the slots of two
-// consecutive steps.  Sixteen steps are loaded before any is added and stored, so the chain of
-// dependent memory round trips is a sixteenth as long as the walk.
+// Running sums over the walk of the 16 bytes at p: `stride` elements lie between the slots of two
+// consecutive steps.  Eight steps are loaded before any is added and stored, so the chain of
+// dependent memory round trips is an eighth as long as the walk.
 template <typename T> FM_DEVICE void fm_scan_run(T* p, int64_t stride, int nsteps) {
-  constexpr int UB = 16;
-  float run = 0.f;
-  for (int w0 = 0; w0 < nsteps; w0 += UB) {
-    float v[UB];
+  constexpr int UB = 8, VE = 16 / sizeof(T);
+  float run[VE];
 #pragma unroll
-    for (int u = 0; u < UB; ++u) v[u] = (w0 + u < nsteps) ? float(p[(w0 + u) * stride]) : 0.f;
+  for (int i = 0; i < VE; ++i) run[i] = 0.f;
+  for (int w0 = 0; w0 < nsteps; w0 += UB) {
+    fm_u32x4 raw[UB];
 #pragma unroll
     for (int u = 0; u < UB; ++u)
-      if (w0 + u < nsteps) { run += v[u]; p[(w0 + u) * stride] = CE<T>::from(run); }
+      if (w0 + u < nsteps) raw[u] = *reinterpret_cast<const fm_u32x4*>(p + (w0 + u) * stride);
+#pragma unroll
+    for (int u = 0; u < UB; ++u)
+      if (w0 + u < nsteps) {
+        T v[VE];
+        __builtin_memcpy(v, &raw[u], 16);
+#pragma unroll
+        for (int i = 0; i < VE; ++i) { run[i] += float(v[i]); v[i] = CE<T>::from(run[i]); }
+        fm_u32x4 out;
+        __builtin_memcpy(&out, v, 16);
+        *reinterpret_cast<fm_u32x4*>(p + (w0 + u) * stride) = out;
+      }
   }
 }
 
+// grid (ceil(items / 256), bh); an item is 16 bytes of one state array.
 template <typename E, int DH>
 FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_state_scan(E* FM_RESTRICT big, E* FM_RESTRICT big2, float* FM_RESTRICT small,
                                                   int nslots, int nsteps, int mode, int nseg, int quad) {
+  constexpr int VE = 16 / sizeof(E);
   const int bh = FM_BID_Y;
-  const int64_t nbig = quad ? int64_t(DH + 1) * DH * DH : int64_t(DH) * DH;
+  const int64_t nbig = (quad ? int64_t(DH + 1) * DH * DH : int64_t(DH) * DH) / VE;   // items of big
   const int64_t first = quad ? 0 : int64_t(DH) * DH * DH;       // the order-1 slab is the last one
-  const int64_t nsmall = StateDims<DH>::SMALL;
+  const int64_t sfirst = quad ? 0 : int64_t(DH) * DH;           // order 1 has no Z: only the two vectors
+  const int64_t nsmall = (StateDims<DH>::SMALL - sfirst) / 4;
   const int64_t nb2 = nbig * (big2 ? 2 : 1);
   const int64_t i = int64_t(FM_BID_X) * 256 + FM_TID_X;
   if (i >= nb2 + nsmall) return;
@@ -576,11 +683,11 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_state_scan(E* FM_RESTRICT big, E* FM_REST
   const int slot0 = mode == FM_WALK_PREFIX ? 1 : nseg - 2;
   const int dir = mode == FM_WALK_PREFIX ? 1 : -1;
   if (i < nb2) {
-    E* b = (i < nbig ? big : big2) + (int64_t(bh) * nslots + slot0) * StateDims<DH>::BIG + first + (i < nbig ? i : i - nbig);
+    E* b = (i < nbig ? big : big2) + (int64_t(bh) * nslots + slot0) * StateDims<DH>::BIG + first + (i < nbig ? i : i - nbig) * VE;
     fm_scan_run<E>(b, int64_t(dir) * StateDims<DH>::BIG, nsteps);
   } else {
-    float* sp = small + (int64_t(bh) * nslots + slot0) * nsmall + (i - nb2);
-    fm_scan_run<float>(sp, int64_t(dir) * nsmall, nsteps);
+    float* sp = small + (int64_t(bh) * nslots + slot0) * StateDims<DH>::SMALL + sfirst + (i - nb2) * 4;
+    fm_scan_run<float>(sp, int64_t(dir) * StateDims<DH>::SMALL, nsteps);
   }
 }
 
