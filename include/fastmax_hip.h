@@ -122,6 +122,22 @@ typedef struct FastmaxNormDesc {
 int fastmax_normalize(const FastmaxNormDesc* desc, const void* x, void* y, float* stats,
                       void* hip_stream);
 
+/* Gradient of fastmax_normalize with respect to x, given dy (the gradient with respect to y).
+ * The reference's extension has no counterpart: fastmax_cuda_backward.cu:518-613 returns the
+ * gradients with respect to the already normalised q and k and the normalisation's own Jacobian
+ * is dropped; its Python variants get it from autograd (score_function.py:40-55,
+ * fastattention_einops.py:327-334), which this entry point reproduces:
+ *   dx_n = (scale / m) * ( C(dy)_n - ([n == n*] - [centre == 2] / N) * (B / m^2) * c_{n*} )
+ * with c = x - centre, m = max_n ||c_n|| reached at token n* (the first one among equal norms),
+ * B = sum dy * c, and C(.) the same centring applied to dy; dx = scale * C(dy) when max_norm == 0.
+ * desc->sx: strides of x and of dx; desc->sy: strides of dy.  dx may be the same buffer as dy
+ * when their strides agree; it must not overlap x.
+ * stats: device scratch of fastmax_normalize_backward_stats_bytes(desc) bytes (8-byte aligned),
+ * or null when max_norm == 0 and centre != 2. */
+size_t fastmax_normalize_backward_stats_bytes(const FastmaxNormDesc* desc);
+int fastmax_normalize_backward(const FastmaxNormDesc* desc, const void* x, const void* dy, void* dx,
+                               float* stats, void* hip_stream);
+
 const char* fastmax_status_string(int status);
 
 /* Library version: major * 10000 + minor * 100 + patch. */

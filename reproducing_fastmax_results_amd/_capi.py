@@ -51,6 +51,7 @@ class NormDesc(C.Structure):
 
 EXPORTS = (
     "fastmax_workspace_bytes", "fastmax_forward", "fastmax_backward", "fastmax_backward_saved", "fastmax_normalize",
+    "fastmax_normalize_backward", "fastmax_normalize_backward_stats_bytes",
     "fastmax_status_string", "fastmax_version", "fastmax_probe_mfma",
     "fastmax_profile_begin", "fastmax_profile_end",
 )
@@ -116,6 +117,11 @@ class FastmaxLib:
         L.fastmax_backward_saved.restype = C.c_int
         L.fastmax_normalize.argtypes = [C.POINTER(NormDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         L.fastmax_normalize.restype = C.c_int
+        L.fastmax_normalize_backward.argtypes = [C.POINTER(NormDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                                 C.c_void_p]
+        L.fastmax_normalize_backward.restype = C.c_int
+        L.fastmax_normalize_backward_stats_bytes.argtypes = [C.POINTER(NormDesc)]
+        L.fastmax_normalize_backward_stats_bytes.restype = C.c_size_t
         L.fastmax_status_string.argtypes = [C.c_int]
         L.fastmax_status_string.restype = C.c_char_p
         L.fastmax_version.restype = C.c_int
@@ -235,6 +241,22 @@ class FastmaxLib:
         st = self.lib.fastmax_normalize(C.byref(nd), x.data_ptr(), out.data_ptr(), stats.data_ptr(), self._stream(x))
         self.check(st, "fastmax_normalize")
         return out
+
+    def normalize_backward(self, x, dy, *, centre=0, max_norm=True, scale=1.0):
+        """Gradient of normalize() with respect to x; x and dy are (bh, n, d) views."""
+        nd = NormDesc()
+        nd.bh, nd.n, nd.d = _dims(x)
+        nd.dtype = _dtype_code(x)
+        nd.centre, nd.max_norm, nd.scale = int(centre), int(bool(max_norm)), float(scale)
+        x = x.contiguous()                 # dx is written with x's strides
+        dx = torch.empty_like(x)
+        nd.sx, nd.sy = _strides(x), _strides(dy)
+        nbytes = self.lib.fastmax_normalize_backward_stats_bytes(C.byref(nd))
+        stats = torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device=x.device)
+        st = self.lib.fastmax_normalize_backward(C.byref(nd), x.data_ptr(), dy.data_ptr(), dx.data_ptr(), stats.data_ptr(),
+                                                 self._stream(x))
+        self.check(st, "fastmax_normalize_backward")
+        return dx
 
     KERNEL_NAMES = ("transpose", "prep_bwd", "build", "fwd", "dq", "dk", "normalize", "dv", "dkv")
 

@@ -35,21 +35,11 @@ __all__ = [
 CENTRE_NONE, CENTRE_FEATURE, CENTRE_TOKEN = 0, 1, 2
 
 
-def _torch_normalize(x, centre: int, scale: float):
-    """Differentiable restatement of the normalisation kernel (used for its backward)."""
-    if centre == CENTRE_FEATURE:
-        x = x - x.mean(-1, keepdim=True)
-    elif centre == CENTRE_TOKEN:
-        x = x - x.mean(-2, keepdim=True)
-    m = torch.linalg.vector_norm(x.float(), dim=-1).amax(-1)
-    return (scale * x.float() / m[..., None, None]).to(x.dtype)
-
-
 class FastmaxNormalize(torch.autograd.Function):
-    """``y = scale * (x - centre) / max_n ||x_n - centre||_2`` per (b, h): forward on the
-    fused HIP pass, backward by differentiating the same formula (the reference's
-    extension drops this gradient; its Python variants carry it through autograd,
-    ``score_function.py:40-55``)."""
+    """``y = scale * (x - centre) / max_n ||x_n - centre||_2`` per (b, h), forward and
+    backward on the HIP passes.  The reference's extension drops this gradient; its
+    Python variants carry it through autograd (``score_function.py:40-55``,
+    ``fastattention_einops.py:327-334``), which the backward pass reproduces."""
 
     @staticmethod
     def forward(ctx, x, centre: int = CENTRE_NONE, scale: float = 1.0):
@@ -60,11 +50,7 @@ class FastmaxNormalize(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_y):
         (x,) = ctx.saved_tensors
-        with torch.enable_grad():
-            xr = x.detach().requires_grad_(True)
-            y = _torch_normalize(xr, ctx.centre, ctx.scale)
-            (gx,) = torch.autograd.grad(y, xr, grad_y)
-        return gx, None, None
+        return _ext.normalize_backward(x, grad_y, ctx.centre, True, ctx.scale), None, None
 
 
 class FASTMultiHeadAttention_Function(torch.autograd.Function):

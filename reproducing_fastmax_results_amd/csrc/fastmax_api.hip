@@ -313,7 +313,7 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
 
 extern "C" {
 
-int fastmax_version(void) { return 101; }
+int fastmax_version(void) { return 102; }
 
 const char* fastmax_status_string(int status) {
   switch (status) {
@@ -407,6 +407,17 @@ int fastmax_backward_saved(const FastmaxDesc* desc, const void* q, const void* k
 int fastmax_normalize(const FastmaxNormDesc* desc, const void* x, void* y, float* stats, void* hip_stream) {
   ProfScope prof(FM_K_NORM, static_cast<fm_stream_t>(hip_stream));   // the whole pass (its kernels together)
   return fm_normalize_dispatch(desc, x, y, stats, static_cast<fm_stream_t>(hip_stream));
+}
+
+size_t fastmax_normalize_backward_stats_bytes(const FastmaxNormDesc* desc) {
+  if (!desc || desc->bh <= 0 || desc->n <= 0 || desc->d <= 0) return 0;
+  return size_t(desc->bh) * size_t(fm_normb_stride(desc->d, desc->n)) * sizeof(float);
+}
+
+int fastmax_normalize_backward(const FastmaxNormDesc* desc, const void* x, const void* dy, void* dx, float* stats,
+                               void* hip_stream) {
+  ProfScope prof(FM_K_NORM, static_cast<fm_stream_t>(hip_stream));
+  return fm_normalize_bwd_dispatch(desc, x, dy, dx, stats, static_cast<fm_stream_t>(hip_stream));
 }
 
 int fastmax_profile_begin(void) {

@@ -316,6 +316,36 @@ torch::Tensor normalize(torch::Tensor x_, int64_t centre, bool max_norm, double 
   return y;
 }
 
+// gradient of normalize() with respect to x (see fastmax_normalize_backward in the C header)
+torch::Tensor normalize_backward(torch::Tensor x_, torch::Tensor dy_, int64_t centre, bool max_norm, double scale) {
+  const View x = view_of(x_, "x");
+  const View dy = view_of(dy_, "dy");
+  FM_CHECK_CUDA(x.t);
+  FM_CHECK_CUDA(dy.t);
+  TORCH_CHECK(dy.bh == x.bh && dy.n == x.n && dy.d == x.d && dy.t.scalar_type() == x.t.scalar_type(),
+              "dy must have x's shape and dtype");
+  FastmaxNormDesc nd{};
+  nd.bh = static_cast<int32_t>(x.bh); nd.n = static_cast<int32_t>(x.n); nd.d = static_cast<int32_t>(x.d);
+  nd.dtype = dtype_code(x.t); nd.centre = static_cast<int32_t>(centre); nd.max_norm = max_norm ? 1 : 0;
+  nd.scale = float(scale);
+  // dx shares x's strides: lay it out like x, and if that is not possible take a packed copy of x
+  torch::Tensor xs = x.t;
+  torch::Tensor dx = empty_like_layout(xs, x.n, xs.scalar_type());
+  View dxv = view_of(dx, "dx");
+  View xv = x;
+  if (dxv.s.bh != x.s.bh || dxv.s.n != x.s.n || dxv.s.b != x.s.b || dxv.s.heads != x.s.heads) {
+    xs = x.t.contiguous();
+    xv = view_of(xs, "x");
+    dx = torch::empty_like(xs);
+  }
+  nd.sx = xv.s; nd.sy = dy.s;
+  const size_t nbytes = fastmax_normalize_backward_stats_bytes(&nd);
+  torch::Tensor stats = torch::empty({int64_t(nbytes / 4 + 1)}, x.t.options().dtype(torch::kFloat32));
+  check_status(fastmax_normalize_backward(&nd, xs.data_ptr(), dy.t.data_ptr(), dx.data_ptr(), stats.data_ptr<float>(),
+                                          stream_of(x.t)), "fastmax_normalize_backward");
+  return dx;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(fastmax_cuda, m) {
@@ -326,5 +356,6 @@ PYBIND11_MODULE(fastmax_cuda, m) {
   m.def("forward_save", &forward_save, "strided forward keeping its workspace: returns (o, g, saved)");
   m.def("backward_saved", &backward_saved, "strided backward on a saved forward workspace: returns [dq, dk, dv]");
   m.def("normalize", &normalize, "fused normalisation pass");
+  m.def("normalize_backward", &normalize_backward, "gradient of the normalisation pass with respect to its input");
   m.def("version", []() { return fastmax_version(); });
 }

@@ -24,7 +24,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_clear(float* stats) {
 // token mean per feature: one workgroup per (8 features, batch*head), 16-byte loads, a fixed
 // reduction tree (the same sum order on every run).  grid (DH / 8, bh).
 template <typename TIO, int DH>
-FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_colmean(TRef<const TIO> x, int n, float* FM_RESTRICT stats) {
+FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_colmean(TRef<const TIO> x, int n, float* FM_RESTRICT out, int64_t out_stride) {
   FM_SHARED float part[8 * 256];
   const int tid = FM_TID_X, d0 = FM_BID_X * 8, bh = FM_BID_Y;
   float s[8];
@@ -46,7 +46,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_colmean(TRef<const TIO> x, int n, fl
     }
     FM_SYNC();
   }
-  if (tid < 8) stats[bh * NormStats<DH>::N + 2 + d0 + tid] = part[tid * 256] / float(n);
+  if (tid < 8) out[bh * out_stride + d0 + tid] = part[tid * 256] / float(n);   // out: DH means per batch*head
 }
 
 template <typename TIO, int DH>
@@ -128,7 +128,8 @@ int fm_normalize_run(const FastmaxNormDesc* d, const void* x, void* y, float* st
   if (d->max_norm || d->centre == 2) {
     FM_KERNEL_LAUNCH((k_norm_clear<DH>), fm_dim3(d->bh), fm_dim3(256), 0, stream, stats);
     if (d->centre == 2)
-      FM_KERNEL_LAUNCH((k_norm_colmean<TIO, DH>), fm_dim3(DH / 8, d->bh), fm_dim3(256), 0, stream, xr, d->n, stats);
+      FM_KERNEL_LAUNCH((k_norm_colmean<TIO, DH>), fm_dim3(DH / 8, d->bh), fm_dim3(256), 0, stream, xr, d->n, stats + 2,
+                       int64_t(NormStats<DH>::N));
     if (d->max_norm)
       FM_KERNEL_LAUNCH((k_norm_maxnorm<TIO, DH>), grid, fm_dim3(256), 0, stream, xr, d->n, d->centre, stats);
   }
@@ -153,4 +154,159 @@ inline int fm_normalize_dispatch(const FastmaxNormDesc* d, const void* x, void* 
     return d->d == 64 ? fm_normalize_run<fm_bf16, 64>(d, x, y, stats, stream) : fm_normalize_run<fm_bf16, 32>(d, x, y, stats, stream);
   }
   return d->d == 64 ? fm_normalize_run<float, 64>(d, x, y, stats, stream) : fm_normalize_run<float, 32>(d, x, y, stats, stream);
+}
+
+// ------------------------------------------------------------------------------
+// Backward of the pass above.  With c = x - centre, m = max_n ||c_n|| reached at token n*
+// (the first one among equal norms), B = sum_{n,d} dy * c and C(.) the same centring applied to dy:
+//   dx_n = (scale / m) * ( C(dy)_n - ([n == n*] - [centre == 2] / N) * (B / m^2) * c_{n*} )
+// and dx = scale * C(dy) without max_norm.  The reference's extension drops this gradient
+// (fastmax_cuda_backward.cu returns the gradients with respect to the normalised tensors); its
+// Python variants carry it through autograd (score_function.py:40-55, fastattention_einops.py:327-334).
+//
+// stats per batch*head, fm_normb_stride(d, n) floats: [0..1] one 64-bit word, the bit pattern of the
+// largest squared norm in the high half and ~token in the low half (an integer atomicMax finds
+// the largest norm and, among equal ones, the first token); [2], [3] unused; [4 .. 4+d) token mean
+// of x; [4+d .. 4+2d) token mean of dy; then one partial sum of dy * c per 64-token block, added
+// in a fixed order by every workgroup of the second kernel (no floating-point atomics).
+// ------------------------------------------------------------------------------
+inline int64_t fm_normb_stride(int dh, int n) { return 4 + 2 * int64_t(dh) + ((n + 63) / 64 + 1) / 2 * 2; }
+
+FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_normb_clear(float* stats, int64_t stride) {
+  if (FM_TID_X < 4) stats[FM_BID_X * stride + FM_TID_X] = 0.f;
+}
+
+// grid (ceil(n/64), bh); four threads per token
+template <typename TIO, int DH>
+FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_normb_stats(TRef<const TIO> x, TRef<const TIO> dy, int n, int centre, int max_norm,
+                                                   float* FM_RESTRICT stats, int64_t stride) {
+  constexpr int EPT = DH / 4;
+  FM_SHARED float wsum[4];
+  const int tid = FM_TID_X, bh = FM_BID_Y;
+  const int tok = FM_BID_X * 64 + (tid >> 2), d0 = (tid & 3) * EPT;
+  float* st = stats + bh * stride;
+  const int tk = tok < n ? tok : n - 1;
+  float c[EPT], g[EPT];
+  fm_norm_load_centred<TIO, DH>(x.base(bh) + int64_t(tk) * x.s_n, x.vec != 0, d0, centre, st + 4, c);
+  fm_norm_load_centred<TIO, DH>(dy.base(bh) + int64_t(tk) * dy.s_n, dy.vec != 0, d0, 0, nullptr, g);
+  float nrm = 0.f, b = 0.f;
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) { nrm += c[j] * c[j]; b += g[j] * c[j]; }
+  nrm += fm_shfl_xor(nrm, 1);
+  nrm += fm_shfl_xor(nrm, 2);
+  if (tok >= n) { nrm = 0.f; b = 0.f; }
+  float mx = nrm;
+#pragma unroll
+  for (int m = 4; m < 64; m <<= 1) mx = fm_fmaxf(mx, fm_shfl_xor(mx, m));
+  int cand = (tok < n && nrm == mx) ? tok : 0x7fffffff;
+#pragma unroll
+  for (int m = 4; m < 64; m <<= 1) { const int o = fm_shfl_xor_i(cand, m); cand = o < cand ? o : cand; }
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) b += fm_shfl_xor(b, m);
+  if ((tid & 63) == 0) {
+    wsum[tid >> 6] = b;
+    if (max_norm && cand != 0x7fffffff) {
+      uint32_t bits;
+      __builtin_memcpy(&bits, &mx, 4);
+      const unsigned long long key = (static_cast<unsigned long long>(bits) << 32) | uint32_t(~uint32_t(cand));
+      unsigned long long* p = reinterpret_cast<unsigned long long*>(st);
+#if defined(FM_HOSTSIM)
+      if (key > *p) *p = key;            // workgroups run one after another in the simulator
+#else
+      atomicMax(p, key);
+#endif
+    }
+  }
+  FM_SYNC();
+  if (tid == 0) st[4 + 2 * DH + FM_BID_X] = (wsum[0] + wsum[1]) + (wsum[2] + wsum[3]);
+}
+
+template <typename TIO, int DH>
+FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_normb_apply(TRef<const TIO> x, TRef<const TIO> dy, TRef<TIO> dx, int n, int centre,
+                                                   int max_norm, float scale, const float* FM_RESTRICT stats, int64_t stride) {
+  constexpr int EPT = DH / 4;
+  FM_SHARED float red[256];
+  const int tid = FM_TID_X, bh = FM_BID_Y;
+  const int tok = FM_BID_X * 64 + (tid >> 2), d0 = (tid & 3) * EPT;
+  const float* st = stats ? stats + bh * stride : nullptr;
+  float f = scale, kf = 0.f;
+  int nstar = -1;
+  if (max_norm) {
+    const int nblk = (n + 63) / 64;
+    float s = 0.f;
+    for (int i = tid; i < nblk; i += 256) s += st[4 + 2 * DH + i];
+    red[tid] = s;
+    FM_SYNC();
+    for (int w = 128; w > 0; w >>= 1) {
+      if (tid < w) red[tid] += red[tid + w];
+      FM_SYNC();
+    }
+    const unsigned long long key = *reinterpret_cast<const unsigned long long*>(st);
+    const uint32_t bits = uint32_t(key >> 32);
+    float m2;
+    __builtin_memcpy(&m2, &bits, 4);
+    nstar = int(~uint32_t(key));
+    if (nstar < 0 || nstar >= n) nstar = 0;            // no token won (every norm is a NaN)
+    f = scale / fm_sqrtf(m2);
+    kf = red[0] / m2;
+  }
+  const int tk = tok < n ? tok : n - 1;
+  float g[EPT], cs[EPT];
+  fm_norm_load_centred<TIO, DH>(dy.base(bh) + int64_t(tk) * dy.s_n, dy.vec != 0, d0, centre, st ? st + 4 + DH : nullptr, g);
+  const float w = max_norm ? kf * ((tok == nstar ? 1.0f : 0.0f) - (centre == 2 ? 1.0f / float(n) : 0.0f)) : 0.0f;
+  if (max_norm) {                        // every lane takes part in the shuffles of the centring
+    fm_norm_load_centred<TIO, DH>(x.base(bh) + int64_t(nstar) * x.s_n, x.vec != 0, d0, centre, st + 4, cs);
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) g[j] -= w * cs[j];
+  }
+  if (tok < n) {
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) g[j] *= f;
+#pragma unroll
+    for (int j = 0; j < EPT; j += 8) IO<TIO>::st8(dx.base(bh) + int64_t(tok) * dx.s_n + d0 + j, dx.vec != 0, &g[j]);
+  }
+}
+
+template <typename TIO, int DH>
+int fm_normalize_bwd_run(const FastmaxNormDesc* d, const void* x, const void* dy, void* dx, float* stats, fm_stream_t stream) {
+  const TRef<const TIO> xr = fm_ref<const TIO>(static_cast<const TIO*>(x), d->sx);
+  const TRef<const TIO> gr = fm_ref<const TIO>(static_cast<const TIO*>(dy), d->sy);
+  const TRef<TIO> dxr = fm_ref<TIO>(static_cast<TIO*>(dx), d->sx);
+  const fm_dim3 grid((d->n + 63) / 64, d->bh);
+  const int64_t stride = fm_normb_stride(DH, d->n);
+  if (d->max_norm || d->centre == 2) {
+    FM_KERNEL_LAUNCH(k_normb_clear, fm_dim3(d->bh), fm_dim3(64), 0, stream, stats, stride);
+    if (d->centre == 2) {
+      FM_KERNEL_LAUNCH((k_norm_colmean<TIO, DH>), fm_dim3(DH / 8, d->bh), fm_dim3(256), 0, stream, xr, d->n, stats + 4, stride);
+      FM_KERNEL_LAUNCH((k_norm_colmean<TIO, DH>), fm_dim3(DH / 8, d->bh), fm_dim3(256), 0, stream, gr, d->n, stats + 4 + DH,
+                       stride);
+    }
+    if (d->max_norm)
+      FM_KERNEL_LAUNCH((k_normb_stats<TIO, DH>), grid, fm_dim3(256), 0, stream, xr, gr, d->n, d->centre, d->max_norm, stats,
+                       stride);
+  }
+  FM_KERNEL_LAUNCH((k_normb_apply<TIO, DH>), grid, fm_dim3(256), 0, stream, xr, gr, dxr, d->n, d->centre, d->max_norm,
+                   d->scale, stats, stride);
+#if defined(FM_HOSTSIM)
+  return FASTMAX_OK;
+#else
+  return hipGetLastError() == hipSuccess ? FASTMAX_OK : FASTMAX_ERR_LAUNCH;
+#endif
+}
+
+inline int fm_normalize_bwd_dispatch(const FastmaxNormDesc* d, const void* x, const void* dy, void* dx, float* stats,
+                                     fm_stream_t stream) {
+  if (!d || !x || !dy || !dx) return FASTMAX_ERR_NULL;
+  if (d->dtype != FASTMAX_F32 && d->dtype != FASTMAX_BF16) return FASTMAX_ERR_DTYPE;
+  if (d->bh <= 0 || d->n <= 0 || d->bh > 65535) return FASTMAX_ERR_SHAPE;
+  if (d->d != 32 && d->d != 64) return FASTMAX_ERR_UNSUPPORTED;
+  if (d->centre < 0 || d->centre > 2) return FASTMAX_ERR_UNSUPPORTED;
+  if ((d->max_norm || d->centre == 2) && !stats) return FASTMAX_ERR_WORKSPACE;
+  if (d->sx.n < d->d || d->sy.n < d->d) return FASTMAX_ERR_SHAPE;
+  if (d->dtype == FASTMAX_BF16) {
+    return d->d == 64 ? fm_normalize_bwd_run<fm_bf16, 64>(d, x, dy, dx, stats, stream)
+                      : fm_normalize_bwd_run<fm_bf16, 32>(d, x, dy, dx, stats, stream);
+  }
+  return d->d == 64 ? fm_normalize_bwd_run<float, 64>(d, x, dy, dx, stats, stream)
+                    : fm_normalize_bwd_run<float, 32>(d, x, dy, dx, stats, stream);
 }

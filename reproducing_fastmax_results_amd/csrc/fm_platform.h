@@ -61,6 +61,7 @@ FM_DEVICE fm_f32x16 fm_mfma_f32(float a, float b, fm_f32x16 c) {
   return c;
 }
 FM_DEVICE float fm_shfl_xor(float v, int m) { return hostsim::shfl(v, hostsim::g_t.lane ^ m); }
+FM_DEVICE int fm_shfl_xor_i(int v, int m) { return hostsim::shfl(v, hostsim::g_t.lane ^ m); }
 FM_DEVICE float fm_dot2(fm_half2 a, fm_half2 b, float c) { return float(a[0]) * float(b[0]) + float(a[1]) * float(b[1]) + c; }
 FM_DEVICE float fm_fmaxf(float a, float b) { return a > b ? a : b; }
 FM_DEVICE float fm_clampf(float x, float lim) { return x > lim ? lim : (x < -lim ? -lim : x); }
@@ -107,6 +108,7 @@ FM_DEVICE fm_f32x16 fm_mfma_f32(float a, float b, fm_f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }
 FM_DEVICE float fm_shfl_xor(float v, int m) { return __shfl_xor(v, m, 64); }
+FM_DEVICE int fm_shfl_xor_i(int v, int m) { return __shfl_xor(v, m, 64); }
 FM_DEVICE float fm_dot2(fm_half2 a, fm_half2 b, float c) { return __builtin_amdgcn_fdot2(a, b, c, false); }
 FM_DEVICE float fm_fmaxf(float a, float b) { return fmaxf(a, b); }
 // clamp to [-lim, lim] in one instruction (v_med3_f32)

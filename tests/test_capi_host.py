@@ -111,3 +111,20 @@ def test_forward_backward_reject_bad_arguments_before_launching(lib):
     assert lib.lib.fastmax_normalize(C.byref(nd), one, one, None, None) == 4   # max_norm needs stats scratch
     assert lib.lib.fastmax_probe_mfma(None, None, None) == 1
     assert lib.lib.fastmax_version() >= 101
+
+
+def test_normalize_backward_arguments(lib):
+    nd = _capi.NormDesc()
+    nd.bh, nd.n, nd.d, nd.dtype, nd.centre, nd.max_norm, nd.scale = 4, 130, 64, _capi.F32, 2, 1, 1.0
+    nd.sx = nd.sy = _capi.Strides(130 * 64, 64)
+    # per batch*head: 4 header floats, the token means of x and dy, one partial sum per 64 tokens (even count)
+    assert lib.lib.fastmax_normalize_backward_stats_bytes(C.byref(nd)) == 4 * 4 * (4 + 2 * 64 + 4)
+    assert lib.lib.fastmax_normalize_backward_stats_bytes(None) == 0
+    one = C.c_void_p(256)     # never dereferenced: validation fails first
+    assert lib.lib.fastmax_normalize_backward(C.byref(nd), None, one, one, one, None) == 1
+    assert lib.lib.fastmax_normalize_backward(C.byref(nd), one, one, one, None, None) == 4   # needs its scratch
+    nd.d = 48
+    assert lib.lib.fastmax_normalize_backward(C.byref(nd), one, one, one, one, None) == 3
+    nd.d, nd.centre = 64, 5
+    assert lib.lib.fastmax_normalize_backward(C.byref(nd), one, one, one, one, None) == 3
+

@@ -144,7 +144,7 @@ def test_score_function_front(sf, normalize, mask, p):
     oref.backward(go.double())
     assert rel_err(o, oref) < 1e-5
     for got, want in ((qd.grad, qr.grad), (kd.grad, kr.grad), (vd.grad, vr.grad)):
-        assert rel_err(got, want) < 2e-5      # torch fp32 normalisation backward on top of the kernels
+        assert rel_err(got, want) < 2e-5      # the fp32 normalisation backward pass on top of the kernels
 
 
 def test_create_attn_matrix_debug_path(sf):
@@ -169,3 +169,44 @@ def test_normalize_kernel(ext, centre, dtype):
     else:
         ref = O.normalize_lim(xd, 2.0)
     assert rel_err(y, ref) < (1e-5 if dtype == torch.float32 else 1e-2)
+
+
+def _normalize_ref(xd, centre, scale):
+    if centre == 1:
+        return O.normalize_feature_mean(xd, xd)[0] * scale
+    if centre == 2:
+        return O.normalize_token_mean(xd, xd)[0] * scale
+    return O.normalize_lim(xd, scale)
+
+
+@pytest.mark.parametrize("centre", [0, 1, 2])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(3, 2, 333, 64), (5, 700, 32)])
+def test_normalize_backward_kernel(ext, centre, dtype, shape):
+    """Gradient of the normalisation pass against autograd (fp64) through the oracle's formula."""
+    print(f"case normalize backward centre={centre} dtype={dtype} shape={shape}", flush=True)
+    x = rnd(*shape, seed=40).to(dtype)
+    dy = rnd(*shape, seed=41).to(dtype)
+    dx = ext.normalize_backward(x.to(DEV), dy.to(DEV), centre, True, 2.0)
+    xd = x.double().requires_grad_(True)
+    _normalize_ref(xd, centre, 2.0).backward(dy.double())
+    assert dx.shape == x.shape
+    assert rel_err(dx, xd.grad) < (1e-5 if dtype == torch.float32 else 1e-2)
+    # without the max-norm division the pass is linear: dx = scale * centred dy
+    dx0 = ext.normalize_backward(x.to(DEV), dy.to(DEV), centre, False, 0.5)
+    dyd = dy.double()
+    want = 0.5 * (dyd - (dyd.mean(-1, keepdim=True) if centre == 1 else dyd.mean(-2, keepdim=True) if centre == 2 else 0))
+    assert rel_err(dx0, want) < (1e-5 if dtype == torch.float32 else 1e-2)
+
+
+def test_normalize_backward_on_projection_layout(ext):
+    """x and dy as the (b, h, n, d) views of (b, n, h*d) projections: no copies, dx in x's layout."""
+    b, h, n, d = 2, 4, 130, 64
+    xp, dyp = rnd(b, n, h * d, seed=42).to(DEV), rnd(b, n, h * d, seed=43).to(DEV)
+    x, dy = (t.view(b, n, h, d).transpose(1, 2) for t in (xp, dyp))
+    dx = ext.normalize_backward(x, dy, 2, True, 1.0)
+    assert dx.transpose(1, 2).is_contiguous()
+    xd = x.cpu().double().requires_grad_(True)
+    _normalize_ref(xd, 2, 1.0).backward(dy.cpu().double())
+    assert rel_err(dx, xd.grad) < 1e-5
+

@@ -85,3 +85,17 @@ def test_normalize(sim):
         assert O.rel_l2(y, ref) < 1e-6
     y = sim.normalize(x, centre=0, max_norm=False, scale=0.25)
     assert torch.allclose(y, 0.25 * x)
+
+
+def test_normalize_backward(sim):
+    from oracle import fastmax_oracle as O
+    g = torch.Generator().manual_seed(12)
+    x, dy = torch.randn(2, 150, 32, generator=g), torch.randn(2, 150, 32, generator=g)
+    for centre, fn in ((0, lambda t: O.normalize_lim(t, 1.5)),
+                       (1, lambda t: 1.5 * O.normalize_feature_mean(t, t)[0]),
+                       (2, lambda t: 1.5 * O.normalize_token_mean(t, t)[0])):
+        xd = x.double().requires_grad_(True)
+        fn(xd).backward(dy.double())
+        dx = sim.normalize_backward(x, dy, centre=centre, max_norm=True, scale=1.5)
+        assert O.rel_l2(dx, xd.grad) < 1e-5
+
