@@ -23,7 +23,7 @@ enum {
   FASTMAX_OK = 0,
   FASTMAX_ERR_NULL = 1,          /* a required pointer is null */
   FASTMAX_ERR_SHAPE = 2,         /* sizes or strides are not valid */
-  FASTMAX_ERR_UNSUPPORTED = 3,   /* valid, but not implemented (head size, order, masked nk != nq) */
+  FASTMAX_ERR_UNSUPPORTED = 3,   /* valid, but not implemented (head size, order, masked nq > nk) */
   FASTMAX_ERR_WORKSPACE = 4,     /* workspace missing, too small or misaligned */
   FASTMAX_ERR_LAUNCH = 5,        /* the HIP runtime refused a launch */
   FASTMAX_ERR_DTYPE = 6          /* unknown element type */
@@ -56,7 +56,10 @@ typedef struct FastmaxStrides {
 
 /* Problem description shared by forward and backward.
  * Score s_ij = (q_i . k_j) * inv_tau;  weight f(s) = a0 + a1 s + a2 s^2 (a2 ignored when p == 1);
- * mask != 0: causal, query i sees keys 0..i (requires nq == nk). */
+ * mask != 0: causal with nq <= nk, query i sees keys 0 .. nk - nq + i (the queries are aligned to
+ * the last keys, reference fastmax_cuda_forward.cu:161-172; nq == 1 is one decoding step over
+ * nk cached keys).  With nk > nq the library runs the keys every query sees and the square causal
+ * part one after the other and merges them; fastmax_backward_saved does not cover that case. */
 typedef struct FastmaxDesc {
   int32_t bh;        /* batch * heads */
   int32_t nq, nk;    /* query and key/value tokens */

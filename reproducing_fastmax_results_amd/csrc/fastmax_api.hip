@@ -4,6 +4,7 @@
 #include "fm_kernels.h"
 #include "fm_tok.h"
 #include "fm_norm.h"
+#include "fm_split.h"
 #include <cmath>
 #include <vector>
 
@@ -78,7 +79,7 @@ int validate(const FastmaxDesc* d) {
   if (d->bh > 65535) return FASTMAX_ERR_SHAPE;
   if (d->p != 1 && d->p != 2) return FASTMAX_ERR_UNSUPPORTED;
   if (d->d != 32 && d->d != 64) return FASTMAX_ERR_UNSUPPORTED;
-  if (d->mask && d->nq != d->nk) return FASTMAX_ERR_UNSUPPORTED;
+  if (d->mask && d->nq > d->nk) return FASTMAX_ERR_UNSUPPORTED;   // nk > nq: see SplitPlan
   if (d->chunk < 0) return FASTMAX_ERR_SHAPE;
   if (!(d->inv_tau > 0.0f) || !(d->inv_tau < 3.0e38f)) return FASTMAX_ERR_SHAPE;   // also rejects NaN
   return FASTMAX_OK;
@@ -307,6 +308,71 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   return launch_pv<TIO, E, DH, QT, FM_OWN_Q>(a, d->bh, FM_K_FWD, stream);
 }
 
+
+// ---- causal with more keys than queries --------------------------------------------------
+// Two ordinary problems on one workspace, one after the other on the same stream: the head
+// (all queries, keys [0, nk - nq), unmasked) and the tail (keys [nk - nq, nk), causal, square).
+struct SplitPlan {
+  int off;                         // nk - nq
+  FastmaxDesc head, head_b, tail;  // head_b: the head's backward (dq to a packed scratch tensor)
+  size_t sub_fwd, sub_bwd;         // workspace of the larger of the two parts
+  size_t off_a, off_ga, off_b;     // head's o and g (forward), head's dq (backward), after the parts' workspace
+  size_t fwd_bytes, bwd_bytes;
+};
+
+inline bool is_split(const FastmaxDesc* d) { return d->mask && d->nk > d->nq; }
+
+int make_split(const FastmaxDesc* d, SplitPlan& sp) {
+  sp.off = d->nk - d->nq;
+  const FastmaxStrides packed{int64_t(d->nq) * d->d, d->d, 0, 0, 0};
+  sp.head = *d;
+  sp.head.mask = 0; sp.head.nk = sp.off;
+  sp.head.flags &= ~FASTMAX_FLAG_SAVE_FOR_BACKWARD;
+  sp.head_b = sp.head;
+  sp.head.so = packed;
+  sp.head.sg = FastmaxStrides{d->nq, 1, 0, 0, 0};
+  sp.head_b.sdq = packed;
+  sp.tail = *d;
+  sp.tail.nk = d->nq;
+  sp.tail.flags &= ~FASTMAX_FLAG_SAVE_FOR_BACKWARD;
+  Plan ph, pt;
+  int st = make_plan(&sp.head, ph);
+  if (st) return st;
+  st = make_plan(&sp.tail, pt);
+  if (st) return st;
+  const size_t esz = d->dtype == FASTMAX_BF16 ? 2 : 4;
+  const size_t rows = align256(size_t(d->bh) * d->nq * d->d * esz);
+  sp.sub_fwd = align256(ph.fwd_bytes > pt.fwd_bytes ? ph.fwd_bytes : pt.fwd_bytes);
+  sp.sub_bwd = align256(ph.bwd_bytes > pt.bwd_bytes ? ph.bwd_bytes : pt.bwd_bytes);
+  sp.off_a = sp.sub_fwd;
+  sp.off_ga = sp.off_a + rows;
+  sp.fwd_bytes = sp.off_ga + align256(size_t(d->bh) * d->nq * 4);
+  sp.off_b = sp.sub_bwd;
+  sp.bwd_bytes = sp.off_b + rows;
+  return FASTMAX_OK;
+}
+
+template <typename TIO, int DH>
+int merge_parts(const FastmaxDesc* d, const SplitPlan& sp, const void* oa, const float* ga, void* o, float* g,
+                fm_stream_t stream) {
+  const TRef<const TIO> oar = cref<TIO>(oa, sp.head.so);
+  const TRef<const float> gar = cref<float>(ga, sp.head.sg);
+  const TRef<float> gr = mref<float>(g, d->sg);
+  const int64_t items = int64_t(d->nq) * (DH / 8);
+  FM_KERNEL_LAUNCH((k_merge_parts<TIO, DH>), fm_dim3(int((items + 255) / 256), d->bh), fm_dim3(256), 0, stream, oar, gar,
+                   mref<TIO>(o, d->so), gr, d->nq);
+  FM_KERNEL_LAUNCH(k_merge_denominators, fm_dim3((d->nq + 255) / 256, d->bh), fm_dim3(256), 0, stream, gar, gr, d->nq);
+  return fm_after_launch();
+}
+
+template <typename TIO, int DH>
+int add_rows(const FastmaxDesc* d, const SplitPlan& sp, const void* dqa, void* dq, fm_stream_t stream) {
+  const int64_t items = int64_t(d->nq) * (DH / 8);
+  FM_KERNEL_LAUNCH((k_add_rows<TIO, DH>), fm_dim3(int((items + 255) / 256), d->bh), fm_dim3(256), 0, stream,
+                   cref<TIO>(dqa, sp.head_b.sdq), mref<TIO>(dq, d->sdq), d->nq);
+  return fm_after_launch();
+}
+
 }  // namespace
 
 #include "fastmax_api_bwd.inc"
@@ -320,7 +386,7 @@ const char* fastmax_status_string(int status) {
     case FASTMAX_OK: return "ok";
     case FASTMAX_ERR_NULL: return "null pointer";
     case FASTMAX_ERR_SHAPE: return "invalid shape or strides";
-    case FASTMAX_ERR_UNSUPPORTED: return "unsupported configuration (d must be 32 or 64, p 1 or 2, masked needs nq == nk)";
+    case FASTMAX_ERR_UNSUPPORTED: return "unsupported configuration (d must be 32 or 64, p 1 or 2, masked needs nq <= nk)";
     case FASTMAX_ERR_WORKSPACE: return "workspace missing, too small or not 256-byte aligned";
     case FASTMAX_ERR_LAUNCH: return "HIP launch failed";
     case FASTMAX_ERR_DTYPE: return "unknown dtype";
@@ -329,16 +395,26 @@ const char* fastmax_status_string(int status) {
 }
 
 int fastmax_workspace_bytes(const FastmaxDesc* desc, size_t* forward_bytes, size_t* backward_bytes) {
-  Plan p;
-  const int st = make_plan(desc, p);
+  int st = validate(desc);
   if (st) return st;
-  if (forward_bytes) *forward_bytes = p.fwd_bytes;
-  if (backward_bytes) *backward_bytes = p.bwd_bytes;
+  size_t f = 0, b = 0;
+  if (is_split(desc)) {
+    SplitPlan sp;
+    st = make_split(desc, sp);
+    f = sp.fwd_bytes; b = sp.bwd_bytes;
+  } else {
+    Plan p;
+    st = make_plan(desc, p);
+    f = p.fwd_bytes; b = p.bwd_bytes;
+  }
+  if (st) return st;
+  if (forward_bytes) *forward_bytes = f;
+  if (backward_bytes) *backward_bytes = b;
   return FASTMAX_OK;
 }
 
-int fastmax_forward(const FastmaxDesc* desc, const void* q, const void* k, const void* v, void* o, float* g,
-                    void* workspace, size_t workspace_bytes, void* hip_stream) {
+static int forward_one(const FastmaxDesc* desc, const void* q, const void* k, const void* v, void* o, float* g,
+                       void* workspace, size_t workspace_bytes, void* hip_stream) {
   Plan p;
   int st = make_plan(desc, p);
   if (st) return st;
@@ -359,9 +435,39 @@ int fastmax_forward(const FastmaxDesc* desc, const void* q, const void* k, const
   return run_forward<float, float, 32, 1>(desc, p, q, k, v, o, g, ws, stream);
 }
 
-static int backward_impl(const FastmaxDesc* desc, const void* q, const void* k, const void* v, const void* o,
-                         const float* g, const void* d_o, void* dq, void* dk, void* dv, const void* fwd_ws,
-                         size_t fwd_ws_bytes, void* workspace, size_t workspace_bytes, void* hip_stream) {
+int fastmax_forward(const FastmaxDesc* desc, const void* q, const void* k, const void* v, void* o, float* g,
+                    void* workspace, size_t workspace_bytes, void* hip_stream) {
+  const int st = validate(desc);
+  if (st) return st;
+  if (!is_split(desc)) return forward_one(desc, q, k, v, o, g, workspace, workspace_bytes, hip_stream);
+  // causal with nk > nq: the keys every query sees, then the square causal part, then the merge
+  SplitPlan sp;
+  int s2 = make_split(desc, sp);
+  if (s2) return s2;
+  if (!q || !k || !v || !o || !g) return FASTMAX_ERR_NULL;
+  if (!strides_ok(desc->sk, desc->bh, desc->nk, desc->d) || !strides_ok(desc->sv, desc->bh, desc->nk, desc->d))
+    return FASTMAX_ERR_SHAPE;
+  if (!workspace || workspace_bytes < sp.fwd_bytes || reinterpret_cast<uintptr_t>(workspace) % 256)
+    return FASTMAX_ERR_WORKSPACE;
+  char* ws = static_cast<char*>(workspace);
+  void* oa = ws + sp.off_a;
+  float* ga = reinterpret_cast<float*>(ws + sp.off_ga);
+  s2 = forward_one(&sp.head, q, k, v, oa, ga, ws, sp.sub_fwd, hip_stream);
+  if (s2) return s2;
+  const size_t esz = desc->dtype == FASTMAX_BF16 ? 2 : 4;
+  const char* kt = static_cast<const char*>(k) + size_t(sp.off) * desc->sk.n * esz;
+  const char* vt = static_cast<const char*>(v) + size_t(sp.off) * desc->sv.n * esz;
+  s2 = forward_one(&sp.tail, q, kt, vt, o, g, ws, sp.sub_fwd, hip_stream);
+  if (s2) return s2;
+  fm_stream_t stream = static_cast<fm_stream_t>(hip_stream);
+  if (desc->dtype == FASTMAX_BF16)
+    return desc->d == 64 ? merge_parts<fm_bf16, 64>(desc, sp, oa, ga, o, g, stream) : merge_parts<fm_bf16, 32>(desc, sp, oa, ga, o, g, stream);
+  return desc->d == 64 ? merge_parts<float, 64>(desc, sp, oa, ga, o, g, stream) : merge_parts<float, 32>(desc, sp, oa, ga, o, g, stream);
+}
+
+static int backward_one(const FastmaxDesc* desc, const void* q, const void* k, const void* v, const void* o,
+                        const float* g, const void* d_o, void* dq, void* dk, void* dv, const void* fwd_ws,
+                        size_t fwd_ws_bytes, void* workspace, size_t workspace_bytes, void* hip_stream) {
   Plan p;
   int st = make_plan(desc, p);
   if (st) return st;
@@ -387,6 +493,41 @@ static int backward_impl(const FastmaxDesc* desc, const void* q, const void* k, 
   }
   if (desc->d == 64) return run_backward<float, float, 64, 1>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);
   return run_backward<float, float, 32, 1>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);
+}
+
+static int backward_impl(const FastmaxDesc* desc, const void* q, const void* k, const void* v, const void* o,
+                         const float* g, const void* d_o, void* dq, void* dk, void* dv, const void* fwd_ws,
+                         size_t fwd_ws_bytes, void* workspace, size_t workspace_bytes, void* hip_stream) {
+  const int st = validate(desc);
+  if (st) return st;
+  if (!is_split(desc))
+    return backward_one(desc, q, k, v, o, g, d_o, dq, dk, dv, fwd_ws, fwd_ws_bytes, workspace, workspace_bytes, hip_stream);
+  // causal with nk > nq: both parts take the final o and g; dk and dv of the two parts are
+  // disjoint key ranges, dq is their sum.  The forward keeps nothing for this case.
+  if (fwd_ws) return FASTMAX_ERR_UNSUPPORTED;
+  SplitPlan sp;
+  int s2 = make_split(desc, sp);
+  if (s2) return s2;
+  if (!q || !k || !v || !o || !g || !d_o || !dq || !dk || !dv) return FASTMAX_ERR_NULL;
+  if (!strides_ok(desc->sk, desc->bh, desc->nk, desc->d) || !strides_ok(desc->sv, desc->bh, desc->nk, desc->d) ||
+      !strides_ok(desc->sdk, desc->bh, desc->nk, desc->d) || !strides_ok(desc->sdv, desc->bh, desc->nk, desc->d))
+    return FASTMAX_ERR_SHAPE;
+  if (!workspace || workspace_bytes < sp.bwd_bytes || reinterpret_cast<uintptr_t>(workspace) % 256)
+    return FASTMAX_ERR_WORKSPACE;
+  char* ws = static_cast<char*>(workspace);
+  void* dqa = ws + sp.off_b;
+  const size_t esz = desc->dtype == FASTMAX_BF16 ? 2 : 4;
+  s2 = backward_one(&sp.head_b, q, k, v, o, g, d_o, dqa, dk, dv, nullptr, 0, ws, sp.sub_bwd, hip_stream);
+  if (s2) return s2;
+  const size_t ko = size_t(sp.off) * desc->sk.n * esz, vo = size_t(sp.off) * desc->sv.n * esz;
+  const size_t dko = size_t(sp.off) * desc->sdk.n * esz, dvo = size_t(sp.off) * desc->sdv.n * esz;
+  s2 = backward_one(&sp.tail, q, static_cast<const char*>(k) + ko, static_cast<const char*>(v) + vo, o, g, d_o, dq,
+                    static_cast<char*>(dk) + dko, static_cast<char*>(dv) + dvo, nullptr, 0, ws, sp.sub_bwd, hip_stream);
+  if (s2) return s2;
+  fm_stream_t stream = static_cast<fm_stream_t>(hip_stream);
+  if (desc->dtype == FASTMAX_BF16)
+    return desc->d == 64 ? add_rows<fm_bf16, 64>(desc, sp, dqa, dq, stream) : add_rows<fm_bf16, 32>(desc, sp, dqa, dq, stream);
+  return desc->d == 64 ? add_rows<float, 64>(desc, sp, dqa, dq, stream) : add_rows<float, 32>(desc, sp, dqa, dq, stream);
 }
 
 int fastmax_backward(const FastmaxDesc* desc, const void* q, const void* k, const void* v, const void* o,

@@ -268,7 +268,8 @@ std::vector<torch::Tensor> backward_any(torch::Tensor q_, torch::Tensor k_, torc
   size_t fwd = 0, bwd = 0;
   check_status(fastmax_workspace_bytes(&d, &fwd, &bwd), "fastmax_workspace_bytes");
   torch::Tensor ws = workspace(bwd, q.t);
-  if (saved) {
+  // causal with more keys than queries keeps nothing from its forward: the plain backward runs
+  if (saved && !(mask && k.n > q.n)) {
     TORCH_CHECK(saved->is_cuda() && saved->scalar_type() == torch::kUInt8 && saved->is_contiguous(),
                 "saved workspace must be the uint8 tensor returned by forward_save");
     check_status(fastmax_backward_saved(&d, q.t.data_ptr(), k.t.data_ptr(), v.t.data_ptr(), o.t.data_ptr(),

@@ -61,7 +61,9 @@ def test_workspace_sizes_and_status_codes(lib):
     assert st == 0 and f >= 256 and b >= f
     assert ws(lib, base_desc(d=48))[0] == 3          # unsupported head size
     assert ws(lib, base_desc(p=3))[0] == 3           # unsupported order
-    assert ws(lib, base_desc(nk=256))[0] == 3        # masked needs nq == nk
+    assert ws(lib, base_desc(nq=256))[0] == 3        # masked needs nq <= nk
+    st2, f2, b2 = ws(lib, base_desc(nk=256))         # masked, more keys than queries: two parts and a merge
+    assert st2 == 0 and f2 > f and b2 > b
     assert ws(lib, base_desc(nk=256, mask=0))[0] == 0
     assert ws(lib, base_desc(dtype=7))[0] == 6
     assert ws(lib, base_desc(bh=0))[0] == 2

@@ -210,3 +210,25 @@ def test_normalize_backward_on_projection_layout(ext):
     _normalize_ref(xd, 2, 1.0).backward(dy.cpu().double())
     assert rel_err(dx, xd.grad) < 1e-5
 
+
+@pytest.mark.parametrize("nq", [1, 200])
+def test_autograd_wrapper_with_cached_keys(sf, nq):
+    """Causal call with fewer queries than keys (the queries are the last tokens, the other keys a
+    cache: fastmax_cuda_forward.cu:161-172), through the autograd wrapper, gradients included."""
+    b, h, nk, d, t = 2, 2, 450, 64, 9.0
+    q = rnd(b, h, nq, d, seed=60)
+    k, v = rnd(b, h, nk, d, seed=61), rnd(b, h, nk, d, seed=62)
+    go = rnd(b, h, nq, d, seed=63)
+    qd, kd, vd = (x.to(DEV).requires_grad_(True) for x in (q, k, v))
+    o = sf.FASTMultiHeadAttention_Function.apply(qd, kd, vd, None, None, True, 0.0, False, t, 1.0, 1.0, 0.5, 1.0, 2)
+    o.backward(go.to(DEV))
+    ref = O.closed_form_forward_backward(q, k, v, go, mask=True, tau=t, p=2)
+    assert rel_err(o, ref[0]) < 1e-5
+    for got, want in ((qd.grad, ref[2]), (kd.grad, ref[3]), (vd.grad, ref[4])):
+        assert rel_err(got, want) < 1e-5
+    # the last rows of the full square problem are the same thing
+    qf = torch.cat([rnd(b, h, nk - nq, d, seed=64), q], dim=2).to(DEV)
+    of = sf.FASTMultiHeadAttention_Function.apply(qf, kd.detach(), vd.detach(), None, None, True, 0.0, False, t,
+                                                  1.0, 1.0, 0.5, 1.0, 2)
+    assert rel_err(o, of[:, :, nk - nq:]) < 1e-5
+

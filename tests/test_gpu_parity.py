@@ -149,3 +149,15 @@ def test_batch_and_head_strides(lib, dtype, mask, chunk):
     print(f"case two-level strides dtype={dtype} mask={mask} chunk={chunk}", flush=True)
     check_batch_head_strides(lib, 3, 4, 700, 64, dtype, DEV, mask=mask, p=2, chunk=chunk, seed=30)
     check_batch_head_strides(lib, 2, 8, 130, 32, dtype, DEV, mask=mask, p=1, chunk=chunk, seed=31)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("p", [1, 2])
+@pytest.mark.parametrize("nq,nk", [(1, 700), (300, 301), (513, 2100), (2048, 6000)])
+def test_causal_more_keys_than_queries(lib, dtype, p, nq, nk):
+    """Causal with nk > nq, queries aligned to the last keys (fastmax_cuda_forward.cu:161-172):
+    prompt keys every query sees plus the square causal part (nq = 1: one decoding step)."""
+    print(f"case causal nk>nq dtype={dtype} p={p} nq={nq} nk={nk}", flush=True)
+    d = 64 if nq != 300 else 32
+    check_forward_backward(lib, 3, nq, d, dtype, DEV, mask=True, p=p, nk=nk, seed=50)
+

@@ -99,3 +99,9 @@ def test_normalize_backward(sim):
         dx = sim.normalize_backward(x, dy, centre=centre, max_norm=True, scale=1.5)
         assert O.rel_l2(dx, xd.grad) < 1e-5
 
+
+def test_causal_with_more_keys_than_queries(sim):
+    # query i sees keys 0 .. nk - nq + i (fastmax_cuda_forward.cu:161-172): head + square tail, merged
+    check_forward_backward(sim, 1, 40, 32, torch.float32, "cpu", mask=True, p=2, nk=75, seed=13)
+    check_forward_backward(sim, 2, 33, 32, torch.bfloat16, "cpu", mask=True, p=1, nk=34, seed=14)
+
