@@ -208,8 +208,14 @@ int launch_build(const BuildArgs<E>& args, int bh, fm_stream_t stream) {
     // MI355X than two values per wavefront at one workgroup per CU (0.092 vs 0.115 ms at
     // B*H = 32, N = 4096, D = 64).
     constexpr int G = DH / 4;
-    a.seg_parallel = 0;
-    return launch_build_cfg<E, DH, 1, 64, (NSMALL + G - 1) / G, true>(a, G, bh, nsteps, stream);
+#ifndef FM_TUNE_QSP
+#define FM_TUNE_QSP 256
+#endif
+#ifndef FM_TUNE_BUILD_TT
+#define FM_TUNE_BUILD_TT 64
+#endif
+    a.seg_parallel = nsteps > 1 && bh * G < FM_TUNE_QSP;
+    return launch_build_cfg<E, DH, 1, FM_TUNE_BUILD_TT, (NSMALL + G - 1) / G, true>(a, G, bh, nsteps, stream);
   }
   // Order 1: the sums are a few 32x32 tiles per segment, far too little work per token tile for
   // a staged walk.  One workgroup per (segment, batch*head) sums its segment from fragments loaded
