@@ -295,20 +295,23 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
     const int nst = (G.send - G.sbeg + KT - 1) / KT;
     const int s_first = OWN == FM_OWN_Q ? G.sbeg : G.sbeg + KT * (nst - 1);
     const int s_step = OWN == FM_OWN_Q ? KT : -KT;
+    // Two stage buffers.  The tiles of stage i+1 travel global memory -> registers during stage i-1
+    // and registers -> LDS in the middle of stage i (between the two groups of matrix products),
+    // so the only thing left at the top of a stage is the barrier.
+    auto more = [&](int sx) { return OWN == FM_OWN_Q ? (sx < G.send) : (sx >= G.sbeg); };
     rx.load(xb + int64_t(s_first) * DH, DH, tid);
     rz.load(zb + s_first, A.npad_str, tid);
+    rx.store(Own, PQ, tid);
+    rz.store(Own + KT * PQ, PV, tid);
+    if (more(s_first + s_step)) {
+      rx.load(xb + int64_t(s_first + s_step) * DH, DH, tid);
+      rz.load(zb + s_first + s_step, A.npad_str, tid);
+    }
     int buf = 0;
-    for (int s0 = s_first; OWN == FM_OWN_Q ? (s0 < G.send) : (s0 >= G.sbeg); s0 += s_step) {
+    for (int s0 = s_first; more(s0); s0 += s_step) {
       E* Xs = Own + buf * STAGE;                        // the own rows and the slabs are spent
       E* Zt = Xs + KT * PQ;
-      rx.store(Xs, PQ, tid);
-      rz.store(Zt, PV, tid);
       FM_SYNC();
-      const int sn = s0 + s_step;
-      if (OWN == FM_OWN_Q ? (sn < G.send) : (sn >= G.sbeg)) {
-        rx.load(xb + int64_t(sn) * DH, DH, tid);
-        rz.load(zb + sn, A.npad_str, tid);
-      }
       // One code path for every tile: the products always run, and a tile that touches the mask
       // or the end of the sequence (a wavefront-uniform test) zeroes the entries outside its row
       // window before they are used; a tile wholly outside the mask has an empty window.
@@ -329,6 +332,20 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
 #pragma unroll
           for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
             zf[ct][ss] = M::load_perm(Zt + (32 * ct + lr) * PV + 32 * st, ss, lh);
+        if (st == KT / 32 - 1) {
+          // next stage: registers -> the other buffer (its readers finished before this stage's
+          // barrier), then the stage after it: global memory -> registers
+          const int sn = s0 + s_step;
+          if (more(sn)) {
+            E* Xn = Own + (buf ^ 1) * STAGE;
+            rx.store(Xn, PQ, tid);
+            rz.store(Xn + KT * PQ, PV, tid);
+            if (more(sn + s_step)) {
+              rx.load(xb + int64_t(sn + s_step) * DH, DH, tid);
+              rz.load(zb + sn + s_step, A.npad_str, tid);
+            }
+          }
+        }
 #pragma unroll
         for (int j = 0; j < QT; ++j) {
           const int ss0 = s0 + 32 * st, lo = t0 + tw[j] * 32;
@@ -490,27 +507,34 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
     TileRegs<E, KT, DH> rx, ry;
     TileRegs<E, DH, KT> rz, rz2;
     E creg = E(0.f);
-    rx.load(xb + int64_t(s_first) * DH, DH, tid);
-    ry.load(yb + int64_t(s_first) * DH, DH, tid);
-    rz.load(zb + s_first, A.npad_str, tid);
-    if (DV) rz2.load(z2b + s_first, A.npad_str, tid);
-    if (OWN == FM_OWN_K && tid < KT) creg = cvb[s_first + tid];
+    auto more = [&](int sx) { return OWN == FM_OWN_Q ? (sx < G.send) : (sx >= G.sbeg); };
+    auto fetch = [&](int sx) {                          // global memory -> registers
+      rx.load(xb + int64_t(sx) * DH, DH, tid);
+      ry.load(yb + int64_t(sx) * DH, DH, tid);
+      rz.load(zb + sx, A.npad_str, tid);
+      if (DV) rz2.load(z2b + sx, A.npad_str, tid);
+      if (OWN == FM_OWN_K && tid < KT) creg = cvb[sx + tid];
+    };
+    auto put = [&](int b) {                             // registers -> stage buffer b
+      E* Xn = Own + b * STAGE; E* Yn = Xn + KT * PQ; E* Zn = Yn + KT * PQ; E* cn = Zn + DH * PV;
+      rx.store(Xn, PQ, tid); ry.store(Yn, PQ, tid); rz.store(Zn, PV, tid);
+      if (DV) rz2.store(cn + KT, PV, tid);
+      if (OWN == FM_OWN_K && tid < KT) cn[tid] = creg;
+    };
+    // Two buffers: the tiles of stage i+1 travel global memory -> registers during stage i-1 and
+    // registers -> LDS in the middle of stage i (see k_pv).  One buffer (fp32): both at the top.
+    fetch(s_first);
+    if (NBUF == 2) {
+      put(0);
+      if (more(s_first + s_step)) fetch(s_first + s_step);
+    }
     int buf = 0;
-    for (int s0 = s_first; OWN == FM_OWN_Q ? (s0 < G.send) : (s0 >= G.sbeg); s0 += s_step) {
+    for (int s0 = s_first; more(s0); s0 += s_step) {
       E* Xs = Own + buf * STAGE; E* Ys = Xs + KT * PQ; E* Zt = Ys + KT * PQ; E* cs = Zt + DH * PV;
       E* Zt2 = cs + KT;
-      rx.store(Xs, PQ, tid); ry.store(Ys, PQ, tid); rz.store(Zt, PV, tid);
-      if (DV) rz2.store(Zt2, PV, tid);
-      if (OWN == FM_OWN_K && tid < KT) cs[tid] = creg;
+      if (NBUF == 1) put(0);
       FM_SYNC();
-      const int sn = s0 + s_step;
-      if (OWN == FM_OWN_Q ? (sn < G.send) : (sn >= G.sbeg)) {
-        rx.load(xb + int64_t(sn) * DH, DH, tid);
-        ry.load(yb + int64_t(sn) * DH, DH, tid);
-        rz.load(zb + sn, A.npad_str, tid);
-        if (DV) rz2.load(z2b + sn, A.npad_str, tid);
-        if (OWN == FM_OWN_K && tid < KT) creg = cvb[sn + tid];
-      }
+      if (NBUF == 1 && more(s0 + s_step)) fetch(s0 + s_step);
       // One code path for every tile (see k_pv).  The score fragments and the transposed fragments
       // serve all own tiles of the wavefront; gh.v is formed per own tile.
 #pragma unroll
@@ -530,6 +554,13 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
           if (OWN == FM_OWN_K) crow[ss] = M::load_perm(cs + 32 * st, ss, lh);
 #pragma unroll
           for (int mt = 0; mt < NT; ++mt) zf[mt][ss] = M::load_perm(Zt + (32 * mt + lr) * PV + 32 * st, ss, lh);
+        }
+        if (NBUF == 2 && st == KT / 32 - 1) {
+          const int sn = s0 + s_step;
+          if (more(sn)) {
+            put(buf ^ 1);
+            if (more(sn + s_step)) fetch(sn + s_step);
+          }
         }
 #pragma unroll
         for (int j = 0; j < QT; ++j) {
