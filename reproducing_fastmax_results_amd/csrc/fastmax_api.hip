@@ -229,20 +229,19 @@ int launch_build(const BuildArgs<E>& args, int bh, fm_stream_t stream) {
   return launch_scan<E, DH>(a, bh, nsteps, stream);
 }
 
-// Dynamic LDS of k_pv and k_ds (one size for both): va, vb | own rows | region, where the
-// dense stages of k_ds and the output staging lie over the own rows and the region.
-template <typename E, int DH, int QT> size_t tok_lds_bytes() {
+// Dynamic LDS of a token kernel (kind 0: k_pv, 1: k_ds, 2: k_ds with dV): va, vb | own rows |
+// region, where the dense stages and the output staging lie over the own rows and the region.
+template <typename E, int DH, int QT> size_t tok_lds_bytes(int kind) {
   typedef TokCfg<E, DH, QT> C;
   size_t region = size_t(2) * C::SLAB * sizeof(E);
   const size_t zs = size_t(C::NZ) * DH * C::PS * sizeof(E);
   if (zs > region) region = zs;
   size_t body = size_t(C::QW) * C::PQ * sizeof(E) + region;
   const size_t outst = size_t(C::QW) * (DH + 1) * 4;
-  const size_t pv = size_t(2) * C::PV_STAGE * sizeof(E);
-  const size_t ds = size_t(C::DS_NBUF) * C::DS_STAGE2 * sizeof(E);
+  const size_t stage = kind == 0 ? size_t(2) * C::PV_STAGE * sizeof(E)
+                                 : size_t(C::DS_NBUF) * (kind == 2 ? C::DV_STAGE : C::DS_STAGE) * sizeof(E);
   if (outst > body) body = outst;
-  if (pv > body) body = pv;
-  if (ds > body) body = ds;
+  if (stage > body) body = stage;
   return size_t(2 * DH) * 4 + body;
 }
 
@@ -258,7 +257,7 @@ template <typename TIO, typename E> void tok_common(TokArgs<TIO, E>& a, const Fa
 template <typename TIO, typename E, int DH, int QT, int OWN>
 int launch_pv(const TokArgs<TIO, E>& a, int bh, int kernel_id, fm_stream_t stream) {
   typedef TokCfg<E, DH, QT> C;
-  const size_t lds = tok_lds_bytes<E, DH, QT>();
+  const size_t lds = tok_lds_bytes<E, DH, QT>(0);
   fm_allow_lds(reinterpret_cast<const void*>(&k_pv<TIO, E, DH, QT, OWN>), lds);
   ProfScope prof(kernel_id, stream);
   FM_KERNEL_LAUNCH((k_pv<TIO, E, DH, QT, OWN>), fm_dim3((a.n_own + C::QW - 1) / C::QW, bh), fm_dim3(FM_THREADS), lds,
@@ -269,7 +268,7 @@ int launch_pv(const TokArgs<TIO, E>& a, int bh, int kernel_id, fm_stream_t strea
 template <typename TIO, typename E, int DH, int QT, int OWN, int DV = 0>
 int launch_ds(const TokArgs<TIO, E>& a, int bh, int kernel_id, fm_stream_t stream) {
   typedef TokCfg<E, DH, QT> C;
-  const size_t lds = tok_lds_bytes<E, DH, QT>();
+  const size_t lds = tok_lds_bytes<E, DH, QT>(DV ? 2 : 1);
   fm_allow_lds(reinterpret_cast<const void*>(&k_ds<TIO, E, DH, QT, OWN, DV>), lds);
   ProfScope prof(kernel_id, stream);
   FM_KERNEL_LAUNCH((k_ds<TIO, E, DH, QT, OWN, DV>), fm_dim3((a.n_own + C::QW - 1) / C::QW, bh), fm_dim3(FM_THREADS), lds,

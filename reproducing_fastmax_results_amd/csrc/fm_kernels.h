@@ -697,12 +697,15 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_state_scan(E* FM_RESTRICT big, E* FM_REST
 // LDS sizes (in elements of E) used by k_pv / k_ds; the host computes the dynamic LDS
 // bytes from the same struct.
 // Stream tokens per stage of the dense loops of the _Float16 token kernels (64-token stages
-// measured slower on MI355X: the larger tile movers cost registers).
+// measured slower on MI355X for k_pv and the plain k_ds, which lose a workgroup per CU to them).
 #ifndef FM_TUNE_KT_PV
 #define FM_TUNE_KT_PV 32
 #endif
 #ifndef FM_TUNE_KT_DS
 #define FM_TUNE_KT_DS 32
+#endif
+#ifndef FM_TUNE_KT_DV
+#define FM_TUNE_KT_DV 64
 #endif
 template <typename E, int DH, int QT>
 struct TokCfg {
@@ -724,13 +727,17 @@ struct TokCfg {
   static constexpr int SA = sizeof(E) == 2 ? QT : 2;                      // values of a per state slab
   static constexpr int KT_PV = sizeof(E) == 2 ? FM_TUNE_KT_PV : 64;   // stream tokens per stage of the dense loop, k_pv
   static constexpr int KT_DS = sizeof(E) == 2 ? FM_TUNE_KT_DS : 64;   //                                           k_ds
+  // the dK + dV pass runs two workgroups per CU whatever its stages are, and 64-token stages
+  // halve its barriers (0.163 vs 0.173 ms at the shape above)
+  static constexpr int KT_DV = sizeof(E) == 2 ? FM_TUNE_KT_DV : 64;   //                                           k_ds with dV
   static constexpr int PV_PV = KT_PV + M::PAD;      // pitch of the transposed token tiles
   static constexpr int PV_DS = KT_DS + M::PAD;
+  static constexpr int PV_DV = KT_DV + M::PAD;
   static constexpr int NZ = sizeof(E) == 2 ? 2 : 1; // hi/lo split of fp32 denominators
   static constexpr int SLAB = SA * DH * PS;         // elements per slab buffer
   static constexpr int PV_STAGE = KT_PV * PQ + DH * PV_PV;                // k_pv: stream rows, stream transposed
   static constexpr int DS_STAGE = 2 * KT_DS * PQ + DH * PV_DS + KT_DS;    // k_ds: two row tiles, transposed tile, c values
-  static constexpr int DS_STAGE2 = DS_STAGE + DH * PV_DS;                 // k_ds with dV: + gh transposed
+  static constexpr int DV_STAGE = 2 * KT_DV * PQ + 2 * DH * PV_DV + KT_DV; // k_ds with dV: + gh transposed
   static constexpr int DS_NBUF = sizeof(E) == 2 ? 2 : 1;
 };
 

@@ -420,9 +420,10 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
   typedef Mma<E> M;
   typedef TileMath<E> TM;
   typedef typename M::frag frag;
-  constexpr int NT = C::NT, NKS = C::NKS, QW = C::QW, PQ = C::PQ, KT = C::KT_DS, PV = C::PV_DS;
+  constexpr int NT = C::NT, NKS = C::NKS, QW = C::QW, PQ = C::PQ;
+  constexpr int KT = DV ? C::KT_DV : C::KT_DS, PV = DV ? C::PV_DV : C::PV_DS;
   constexpr int NBUF = C::DS_NBUF;
-  constexpr int STAGE = DV ? C::DS_STAGE2 : C::DS_STAGE;
+  constexpr int STAGE = DV ? C::DV_STAGE : C::DS_STAGE;
   FM_DYN_SMEM(smem);
   float* vecs = reinterpret_cast<float*>(smem);
   E* Own = reinterpret_cast<E*>(vecs + 2 * DH);       // [QW][PQ]
