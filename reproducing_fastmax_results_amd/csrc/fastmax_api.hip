@@ -157,13 +157,14 @@ template <typename T> TRef<const T> cref(const void* ptr, const FastmaxStrides& 
 }
 template <typename T> TRef<T> mref(void* ptr, const FastmaxStrides& s) { return fm_ref<T>(static_cast<T*>(ptr), s); }
 
+// k and v (same length) in one launch
 template <typename TIO, typename E, int DH>
-int launch_transpose(const void* x, const FastmaxStrides& s, int bh, int n, int npad, E* xt, E* xr, float scale,
-                     fm_stream_t stream) {
-  TRef<const TIO> r = cref<TIO>(x, s);
+int launch_transpose2(const void* x0, const FastmaxStrides& s0, E* xt0, E* xr0, float scale0, const void* x1,
+                      const FastmaxStrides& s1, E* xt1, E* xr1, float scale1, int bh, int n, int npad,
+                      fm_stream_t stream) {
+  const TransposeJob<TIO, E> j0{cref<TIO>(x0, s0), xt0, xr0, scale0}, j1{cref<TIO>(x1, s1), xt1, xr1, scale1};
   ProfScope prof(FM_K_TRANSPOSE, stream);
-  FM_KERNEL_LAUNCH((k_transpose<TIO, E, DH>), fm_dim3(npad / 64, bh), fm_dim3(FM_THREADS), 0, stream, r, n, npad, xt,
-                   xr, scale);
+  FM_KERNEL_LAUNCH((k_transpose<TIO, E, DH>), fm_dim3(npad / 64, bh, 2), fm_dim3(FM_THREADS), 0, stream, j0, j1, n, npad);
   return fm_after_launch();
 }
 
@@ -285,9 +286,7 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   float* small = reinterpret_cast<float*>(ws + p.small);
   E* kr = reinterpret_cast<E*>(ws + p.kr);
   E* vr = p.save ? reinterpret_cast<E*>(ws + p.vr) : nullptr;
-  int st = launch_transpose<TIO, E, DH>(v, d->sv, d->bh, d->nk, p.npad_k, vt, vr, 1.0f, stream);
-  if (st) return st;
-  st = launch_transpose<TIO, E, DH>(k, d->sk, d->bh, d->nk, p.npad_k, kt, kr, p.sc, stream);
+  int st = launch_transpose2<TIO, E, DH>(v, d->sv, vt, vr, 1.0f, k, d->sk, kt, kr, p.sc, d->bh, d->nk, p.npad_k, stream);
   if (st) return st;
   if (p.use_state) {
     BuildArgs<E> b;

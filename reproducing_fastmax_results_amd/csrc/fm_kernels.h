@@ -142,15 +142,23 @@ template <typename T> inline TRef<T> fm_ref(T* ptr, const FastmaxStrides& s) {
 // k_transpose: x (bh, n, DH) strided, interface type  ->  compute type, multiplied by
 // `scale`, zero for tokens >= n:  xt [bh][DH][npad] (transposed) and, when xr is not
 // null, xr [bh][npad][DH] (row-major).  The token-side kernels stage their tiles from
-// these copies with plain 16-byte moves.  grid (npad/64, bh).
+// these copies with plain 16-byte moves.  Two tensors of the same length (k and v) go in one
+// launch: grid (npad/64, bh, 2), the second set of arguments serves z = 1.
 // ------------------------------------------------------------------------------
+template <typename TIO, typename E> struct TransposeJob { TRef<const TIO> x; E* xt; E* xr; float scale; };
+
 template <typename TIO, typename E, int DH>
 FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS)
-k_transpose(TRef<const TIO> x, int n, int npad, E* FM_RESTRICT xt, E* FM_RESTRICT xr, float scale) {
+k_transpose(TransposeJob<TIO, E> j0, TransposeJob<TIO, E> j1, int n, int npad) {
   constexpr int PT = 64 + Mma<E>::PAD;
   constexpr int VEC = Mma<E>::VEC;
   FM_SHARED E tile[DH * PT];
   const int tid = FM_TID_X, t0 = FM_BID_X * 64, bh = FM_BID_Y;
+  const bool second = FM_BID_Z != 0;
+  const TRef<const TIO> x = second ? j1.x : j0.x;
+  E* FM_RESTRICT xt = second ? j1.xt : j0.xt;
+  E* FM_RESTRICT xr = second ? j1.xr : j0.xr;
+  const float scale = second ? j1.scale : j0.scale;
   const TIO* xb = x.base(bh);
   const int64_t s_n = x.s_n;
   const int vec = x.vec;
