@@ -110,6 +110,17 @@ def test_long_sequence_default_segments(lib, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("d", [32, 64])
+def test_order1_default_segments(lib, dtype, d):
+    # order 1 beyond 1536 tokens: 256-token segments summed apart, then scanned (16 and 28 segments, the
+    # second with a ragged end); unmasked with many keys: one total over all keys by a single walk step
+    print(f"case order1 segments dtype={dtype} d={d}", flush=True)
+    check_forward_backward(lib, 3, 4096, d, dtype, DEV, mask=True, p=1, seed=22, saved=True)
+    check_forward_backward(lib, 2, 7000, d, dtype, DEV, mask=True, p=1, seed=23)
+    check_forward_backward(lib, 2, 300, d, dtype, DEV, mask=False, p=1, nk=5000, seed=24)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_backward_ragged_and_cross(lib, dtype):
     print(f"case bwd ragged dtype={dtype}", flush=True)
     check_forward_backward(lib, 2, 1, 64, dtype, DEV, mask=True, p=2, seed=10)
