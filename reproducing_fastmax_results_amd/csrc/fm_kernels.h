@@ -333,20 +333,19 @@ FM_DEVICE void fm_put_small(const BuildArgs<E>& A, E* big, E* big2, float* ds, i
   }
 }
 
-// k_build: one workgroup per (group of 4*NA values of a, batch*head) walks the tokens
+// k_build (order 2): one workgroup per (group of 4*NA values of a, batch*head) walks the tokens
 // once, keeping its slice of the order-2 state in accumulators and writing a snapshot at
 // every segment boundary, so the prefix (or suffix) scan over segments is implicit.
 // The order-1 state, the denominator matrix Z and the two vector sums are 2*NT*NT + 2*NT
-// further 32x32 tiles; they are dealt round-robin to the workgroups of a batch*head, and
+// further 32x32 tiles; they are dealt round-robin to the workgroups of a batch*head (SPW each), and
 // inside a workgroup each wavefront adds its quarter of the k-steps, so every workgroup
-// does the same amount of work and the grid is exactly (DH / (4*NA)) x bh.  Order 1 has only the
-// lower-order tiles: QUAD = false drops the order-2 code and the grid shrinks to
-// ceil(tiles / SPW) workgroups per batch*head, each taking SPW tiles, so that the token tiles are
-// staged by four workgroups instead of sixteen.
+// does the same amount of work and the grid is exactly (DH / (4*NA)) x bh.  With seg_parallel
+// the grid gets a third axis, one walk step per workgroup, and k_state_scan follows (used when
+// batch*heads is too small to fill the chip otherwise).  Order 1 has its own kernel, k_build1.
 // Replaces the running sums of fastmax_cuda_forward.cu:165-276 (one thread per feature,
 // serial over tokens) and the cumsum of materialised outer products of
 // fastattention_einops.py:237-248.
-template <typename E, int DH, int NA, int TT, int SPW, bool QUAD>
+template <typename E, int DH, int NA, int TT, int SPW>
 FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <= 4 ? 2 : 1)) k_build(BuildArgs<E> A) {
   typedef Mma<E> M;
   typedef typename M::frag frag;
@@ -372,7 +371,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <
   E* big2 = A.big2 ? A.big2 + int64_t(bh) * A.nslots * StateDims<DH>::BIG : nullptr;
   float* sml = A.small + int64_t(bh) * A.nslots * StateDims<DH>::SMALL;
   const bool has_z = A.zt != nullptr;
-  const bool quad = QUAD && A.quad != 0;
+  const bool quad = A.quad != 0;
 
   // small tiles of this workgroup: offsets (elements from s0) of the operand rows in LDS for
   // the A side and the B side (-1: a column of ones)
