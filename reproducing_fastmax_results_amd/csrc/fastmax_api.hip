@@ -309,6 +309,10 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   a.out = mref<TIO>(o, d->so);
   a.g = mref<float>(g, d->sg);
   a.n_own = d->nq; a.n_str = d->nk;
+  // order-2 states: two tiles per wavefront halve the state bytes a token reads (forward 1.38 -> 0.94 ms
+  // at B*H = 16, N = 65536 on MI355X); without states one tile per wavefront and more workgroups per CU win
+  if (sizeof(E) == 2 && p.use_state && p.quad)
+    return launch_pv<TIO, E, DH, (sizeof(E) == 2 ? 2 : QT), FM_OWN_Q>(a, d->bh, FM_K_FWD, stream);
   return launch_pv<TIO, E, DH, QT, FM_OWN_Q>(a, d->bh, FM_K_FWD, stream);
 }
 
