@@ -179,7 +179,7 @@ int launch_scan(const BuildArgs<E>& a, int bh, int nsteps, fm_stream_t stream) {
   return fm_after_launch();
 }
 
-template <typename E, int DH, int NA, int TT, int SPW>
+template <typename E, int DH, int NA, int TT, int SPW, int KB>
 int launch_build_cfg(const BuildArgs<E>& a, int groups, int bh, int nsteps, fm_stream_t stream) {
   constexpr int PT = TT + Mma<E>::PAD;
   constexpr int AW = 4 * NA;
@@ -188,8 +188,8 @@ int launch_build_cfg(const BuildArgs<E>& a, int groups, int bh, int nsteps, fm_s
   const size_t snap = size_t(AW) * DH * (DH + Mma<E>::PAD) * sizeof(E);      // snapshot staging
   if (lds < red) lds = red;
   if (lds < snap) lds = snap;
-  fm_allow_lds(reinterpret_cast<const void*>(&k_build<E, DH, NA, TT, SPW>), lds);
-  FM_KERNEL_LAUNCH((k_build<E, DH, NA, TT, SPW>), fm_dim3(groups, bh, a.seg_parallel ? nsteps : 1),
+  fm_allow_lds(reinterpret_cast<const void*>(&k_build<E, DH, NA, TT, SPW, KB>), lds);
+  FM_KERNEL_LAUNCH((k_build<E, DH, NA, TT, SPW, KB>), fm_dim3(groups, bh, a.seg_parallel ? nsteps : 1),
                    fm_dim3(FM_THREADS), lds, stream, a);
   int st = fm_after_launch();
   if (st || !a.seg_parallel || nsteps < 2) return st;
@@ -216,7 +216,16 @@ int launch_build(const BuildArgs<E>& args, int bh, fm_stream_t stream) {
 #define FM_TUNE_BUILD_TT 64
 #endif
     a.seg_parallel = nsteps > 1 && bh * G < FM_TUNE_QSP;
-    return launch_build_cfg<E, DH, 1, FM_TUNE_BUILD_TT, (NSMALL + G - 1) / G>(a, G, bh, nsteps, stream);
+#ifndef FM_TUNE_KB_SMALL
+#define FM_TUNE_KB_SMALL 4
+#endif
+#ifndef FM_TUNE_KB_LARGE
+#define FM_TUNE_KB_LARGE 2
+#endif
+    // at most one workgroup per CU: all the registers are its own, every fragment of a tile is in flight at once
+    if (bh * G * (a.seg_parallel ? nsteps : 1) <= 256)
+      return launch_build_cfg<E, DH, 1, FM_TUNE_BUILD_TT, (NSMALL + G - 1) / G, FM_TUNE_KB_SMALL>(a, G, bh, nsteps, stream);
+    return launch_build_cfg<E, DH, 1, FM_TUNE_BUILD_TT, (NSMALL + G - 1) / G, FM_TUNE_KB_LARGE>(a, G, bh, nsteps, stream);
   }
   // Order 1: the sums are a few 32x32 tiles per segment, far too little work per token tile for
   // a staged walk.  One workgroup per (segment, batch*head) sums its segment from fragments loaded

@@ -345,8 +345,8 @@ FM_DEVICE void fm_put_small(const BuildArgs<E>& A, E* big, E* big2, float* ds, i
 // Replaces the running sums of fastmax_cuda_forward.cu:165-276 (one thread per feature,
 // serial over tokens) and the cumsum of materialised outer products of
 // fastattention_einops.py:237-248.
-template <typename E, int DH, int NA, int TT, int SPW>
-FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <= 4 ? 2 : 1)) k_build(BuildArgs<E> A) {
+template <typename E, int DH, int NA, int TT, int SPW, int KB>
+FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <= 4 && KB < 4 ? 2 : 1)) k_build(BuildArgs<E> A) {
   typedef Mma<E> M;
   typedef typename M::frag frag;
   constexpr int AW = 4 * NA;
@@ -439,36 +439,68 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <
       if (has_z) rz.load(A.zt + tb_off + nt, A.npad, tid);
     }
     if (quad) {
-      // fragments of k-step ks+1 are fetched while the products of k-step ks are issued
       const E* pb_ = s0 + lr * PT + lh * M::KPL;
       const E* rb_ = s1 + lr * PT + lh * M::KPL;
       const E* xb_ = s2 + (wave * NA) * PT + lh * M::KPL;
-      frag fb[NT], fp[NT], fx[NA];
+      if (NSTEP <= 4) {
+        // Few k-steps per tile (_Float16): the fragments of KB k-steps are requested from LDS
+        // before their first product, so the wavefront waits for LDS NSTEP / KB times per tile
+        // (with one k-step of lookahead the walk ran at the LDS latency, not at the MFMA rate).
+        // KB = NSTEP needs more than 256 registers: one workgroup per CU.
 #pragma unroll
-      for (int j = 0; j < NT; ++j) { fb[j] = M::load(rb_ + 32 * j * PT); fp[j] = M::load(pb_ + 32 * j * PT); }
+        for (int k0 = 0; k0 < NSTEP; k0 += KB) {
+          frag fb[KB][NT], fp[KB][NT], fx[KB][NA];
 #pragma unroll
-      for (int i = 0; i < NA; ++i) fx[i] = M::load(xb_ + i * PT);
-#pragma unroll 2
-      for (int ks = 0; ks < NSTEP; ++ks) {
-        const int kn = (ks + 1 < NSTEP ? ks + 1 : ks) * M::KSTEP;
-        frag nb[NT], np[NT], nx[NA];
+          for (int u = 0; u < KB; ++u) {
 #pragma unroll
-        for (int j = 0; j < NT; ++j) { nb[j] = M::load(rb_ + 32 * j * PT + kn); np[j] = M::load(pb_ + 32 * j * PT + kn); }
+            for (int j = 0; j < NT; ++j) {
+              fb[u][j] = M::load(rb_ + 32 * j * PT + (k0 + u) * M::KSTEP);
+              fp[u][j] = M::load(pb_ + 32 * j * PT + (k0 + u) * M::KSTEP);
+            }
 #pragma unroll
-        for (int i = 0; i < NA; ++i) nx[i] = M::load(xb_ + i * PT + kn);
-#pragma unroll
-        for (int i = 0; i < NA; ++i) {
-#pragma unroll
-          for (int j = 0; j < NT; ++j) {
-            const frag fa = fp[j] * fx[i];
-#pragma unroll
-            for (int k = 0; k < NT; ++k) acc[i][j][k] = M::mma(fa, fb[k], acc[i][j][k]);
+            for (int i = 0; i < NA; ++i) fx[u][i] = M::load(xb_ + i * PT + (k0 + u) * M::KSTEP);
           }
+#pragma unroll
+          for (int u = 0; u < KB; ++u)
+#pragma unroll
+            for (int i = 0; i < NA; ++i)
+#pragma unroll
+              for (int j = 0; j < NT; ++j) {
+                const frag fa = fp[u][j] * fx[u][i];
+#pragma unroll
+                for (int k = 0; k < NT; ++k) acc[i][j][k] = M::mma(fa, fb[u][k], acc[i][j][k]);
+              }
         }
+      } else {
+        // many k-steps per tile (fp32): fragments of k-step ks+1 are fetched while the products of
+        // k-step ks are issued
+        frag fb[NT], fp[NT], fx[NA];
 #pragma unroll
-        for (int j = 0; j < NT; ++j) { fb[j] = nb[j]; fp[j] = np[j]; }
+        for (int j = 0; j < NT; ++j) { fb[j] = M::load(rb_ + 32 * j * PT); fp[j] = M::load(pb_ + 32 * j * PT); }
 #pragma unroll
-        for (int i = 0; i < NA; ++i) fx[i] = nx[i];
+        for (int i = 0; i < NA; ++i) fx[i] = M::load(xb_ + i * PT);
+#pragma unroll 2
+        for (int ks = 0; ks < NSTEP; ++ks) {
+          const int kn = (ks + 1 < NSTEP ? ks + 1 : ks) * M::KSTEP;
+          frag nb[NT], np[NT], nx[NA];
+#pragma unroll
+          for (int j = 0; j < NT; ++j) { nb[j] = M::load(rb_ + 32 * j * PT + kn); np[j] = M::load(pb_ + 32 * j * PT + kn); }
+#pragma unroll
+          for (int i = 0; i < NA; ++i) nx[i] = M::load(xb_ + i * PT + kn);
+#pragma unroll
+          for (int i = 0; i < NA; ++i) {
+#pragma unroll
+            for (int j = 0; j < NT; ++j) {
+              const frag fa = fp[j] * fx[i];
+#pragma unroll
+              for (int k = 0; k < NT; ++k) acc[i][j][k] = M::mma(fa, fb[k], acc[i][j][k]);
+            }
+          }
+#pragma unroll
+          for (int j = 0; j < NT; ++j) { fb[j] = nb[j]; fp[j] = np[j]; }
+#pragma unroll
+          for (int i = 0; i < NA; ++i) fx[i] = nx[i];
+        }
       }
     }
     // the lower-order tiles: this wavefront takes the k-steps ks = wave (mod 4)

@@ -121,6 +121,15 @@ def test_order1_default_segments(lib, dtype, d):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_order2_states_mid_sized_batch(lib, dtype):
+    # 16 <= batch*heads < 32 at D = 64: the state walk is serial over segments with one workgroup per CU
+    print(f"case order2 mid batch dtype={dtype}", flush=True)
+    check_forward_backward(lib, 16, 1100, 64, dtype, DEV, mask=True, p=2, chunk=256, seed=25)
+    check_forward_backward(lib, 20, 1100, 64, dtype, DEV, mask=True, p=2, chunk=256, seed=26, saved=True)
+    check_forward_backward(lib, 17, 300, 64, dtype, DEV, mask=False, p=2, nk=700, seed=27, flags=FLAG_FORCE_MOMENTS)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_backward_ragged_and_cross(lib, dtype):
     print(f"case bwd ragged dtype={dtype}", flush=True)
     check_forward_backward(lib, 2, 1, 64, dtype, DEV, mask=True, p=2, seed=10)
