@@ -49,11 +49,22 @@ class Attention(nn.Module):
         self.linear = nn.Linear(h * d_head, d_model)
         self.dropout = nn.Dropout(dropout_rate)
 
-    def forward(self, x):
+    def forward(self, x, cache=None):
+        """``cache``: None, or a dict holding the key and value projections of the tokens seen so far
+        (``"k"``, ``"v"``: ``(b, n_past, h*d)``); x then holds only the new tokens, attends to past and
+        new keys (causal, queries aligned to the last keys) and the dict is updated in place."""
         b, n, _ = x.shape
         q = self.query_transform(x).view(b, n, self.h, self.d_head).transpose(1, 2)   # (b, h, n, d) views
-        k = self.key_transform(x).view(b, n, self.h, self.d_head).transpose(1, 2)
-        v = self.value_transform(x).view(b, n, self.h, self.d_head).transpose(1, 2)
+        kp, vp = self.key_transform(x), self.value_transform(x)
+        if cache is not None:
+            if self.normalize:
+                raise ValueError("cached keys need normalize=False: the max-norm scaling looks at every token")
+            if "k" in cache:
+                kp, vp = torch.cat((cache["k"], kp), dim=1), torch.cat((cache["v"], vp), dim=1)
+            cache["k"], cache["v"] = kp, vp
+        nk = kp.shape[1]
+        k = kp.view(b, nk, self.h, self.d_head).transpose(1, 2)
+        v = vp.view(b, nk, self.h, self.d_head).transpose(1, 2)
         a0, a1, a2 = self.coefficients
         o = self.attention_fn(q, k, v, mask=self.use_masking, normalize=self.normalize, lim=self.lim,
                               temperature=self.temperature, a0=a0, a1=a1, a2=a2, p=self.p)
@@ -72,8 +83,8 @@ class TransformerBlock(nn.Module):
         self.mlp_subblock = nn.Sequential(nn.Linear(d_model, d_mlp), nn.GELU(), nn.Linear(d_mlp, d_model),
                                           nn.Dropout(dropout_rate))
 
-    def forward(self, x):
-        a = self.attention_subblock(self.layer_norm1(x)) + x
+    def forward(self, x, cache=None):
+        a = self.attention_subblock(self.layer_norm1(x), cache) + x
         # the reference adds the block input, not the attention output, to the MLP branch (model.py:366)
         return self.mlp_subblock(self.layer_norm2(a)) + x
 
@@ -136,14 +147,35 @@ class Transformer(nn.Module):
             if prm.dim() > 1:
                 nn.init.xavier_uniform_(prm)
 
-    def forward(self, tokens):
+    def forward(self, tokens, caches=None):
+        """``caches``: None, or one dict per block (see ``Attention.forward``); ``tokens`` then holds
+        only the tokens that follow the cached ones."""
         x = self.token_embedding(tokens)
         if self.classifier.kind == "cls_token":
             x = torch.cat((self.class_token.expand(x.shape[0], 1, -1), x), dim=1)
-        x = x + self.pos_embedding(torch.arange(x.shape[1], device=x.device))
-        for block in self.blocks:
-            x = block(x)
+        past = caches[0]["k"].shape[1] if caches and "k" in caches[0] else 0
+        x = x + self.pos_embedding(torch.arange(past, past + x.shape[1], device=x.device))
+        for i, block in enumerate(self.blocks):
+            x = block(x, caches[i] if caches is not None else None)
         return self.classifier(x)
+
+    @torch.no_grad()
+    def generate(self, tokens, max_new_tokens, sample=False, use_cache=True):
+        """Next-token generation (reference ``transformer/eval.py:8-32``): ``tokens`` ``(b, n)`` grows
+        by ``max_new_tokens``.  The reference runs the whole context through the model for every
+        new token.  With ``use_cache`` the key and value projections of every block are kept and a
+        step runs the new token only; its attention is one causal call with one query and all the
+        keys so far.  That is exact for ``normalize=False`` models (the max-norm scaling of the
+        others depends on every token, so they take the reference's route).  Contexts longer than
+        the position table are not handled (the reference crops to the last ``max_tokens``)."""
+        cached = use_cache and not any(b.attention_subblock.normalize for b in self.blocks)
+        caches = [dict() for _ in self.blocks] if cached else None
+        logits = self(tokens, caches)[:, -1, :]
+        for _ in range(max_new_tokens):
+            nxt = torch.multinomial(torch.softmax(logits, -1), 1) if sample else logits.argmax(-1, keepdim=True)
+            tokens = torch.cat((tokens, nxt), dim=1)
+            logits = (self(nxt, caches) if cached else self(tokens))[:, -1, :]
+        return tokens
 
 
 def vit_for_c4(**overrides):

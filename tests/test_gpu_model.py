@@ -89,3 +89,33 @@ def test_attention_layout_needs_no_copies():
     att.attention_fn = spy
     y = att(torch.randn(2, 70, 128, device=DEV))
     assert y.shape == (2, 70, 128) and seen["q_view"] and seen["o_merge_is_view"]
+
+
+def test_cached_generation_matches_full_recompute():
+    """Greedy next-token generation with cached keys and values (one causal call with one query and
+    all keys so far per block and step) against the reference's loop that runs the whole context for
+    every token (transformer/eval.py:8-32), and the step logits against the oracle inside the model."""
+    from reproducing_fastmax_results_amd.transformer.model import gpt_for_c5
+    torch.manual_seed(5)
+    cfg = dict(out_dim=97, vocab_size=97, max_tokens=96, d_model=128, d_mlp=256, heads_per_block=4, num_blocks=2,
+               normalize=False, temperature=8.0 * 32 ** 0.5)
+    hip = gpt_for_c5(**cfg).to(DEV).eval()
+    prompt = torch.randint(0, 97, (3, 40), generator=torch.Generator().manual_seed(6)).to(DEV)
+    fast = hip.generate(prompt, 24, use_cache=True)
+    slow = hip.generate(prompt, 24, use_cache=False)
+    assert fast.shape == (3, 64) and torch.equal(fast[:, :40], prompt)
+    assert torch.equal(fast, slow)
+    # logits of one cached step against the oracle's full forward over the same tokens
+    ref = copy.deepcopy(hip)
+    for blk in ref.blocks:
+        blk.attention_subblock.attention_fn = oracle_attention
+    with torch.no_grad():
+        caches = [dict() for _ in hip.blocks]
+        hip(fast[:, :50], caches)
+        step = hip(fast[:, 50:51], caches)[:, -1, :]
+        want = ref(fast[:, :51])[:, -1, :]
+    assert float((step - want).norm() / want.norm()) < 1e-4
+    # models that normalise q and k cannot cache (the scaling sees every token): same route as the reference
+    norm_model = gpt_for_c5(**dict(cfg, normalize=True, temperature=1.0)).to(DEV).eval()
+    assert norm_model.generate(prompt, 3).shape == (3, 43)
+
