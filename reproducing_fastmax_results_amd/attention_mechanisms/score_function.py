@@ -35,6 +35,23 @@ __all__ = [
 CENTRE_NONE, CENTRE_FEATURE, CENTRE_TOKEN = 0, 1, 2
 
 
+_HEAD_SIZES = (32, 64)      # what the kernels are built for
+
+
+def _pad_features(x):
+    """x itself, or a copy zero-padded along the feature axis to the next head size the kernels
+    are built for.  Zero features change neither q.k nor any norm, padded value columns come out
+    as zero output columns, and the padded columns of every gradient are zero as well, so callers
+    pad on the way in and slice on the way out."""
+    d = x.shape[-1]
+    for size in _HEAD_SIZES:
+        if d == size:
+            return x
+        if d < size:
+            return torch.nn.functional.pad(x, (0, size - d))
+    raise RuntimeError(f"fastmax: unsupported head size {d} (the kernels cover up to {_HEAD_SIZES[-1]})")
+
+
 class FastmaxNormalize(torch.autograd.Function):
     """``y = scale * (x - centre) / max_n ||x_n - centre||_2`` per (b, h), forward and
     backward on the HIP passes.  The reference's extension drops this gradient; its
@@ -43,14 +60,19 @@ class FastmaxNormalize(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, centre: int = CENTRE_NONE, scale: float = 1.0):
+        d = x.shape[-1]
+        if centre != CENTRE_FEATURE:            # the feature mean is the one thing padding would change
+            x = _pad_features(x)
         ctx.save_for_backward(x)
-        ctx.centre, ctx.scale = centre, scale
-        return _ext.normalize(x, centre, True, scale)
+        ctx.centre, ctx.scale, ctx.d = centre, scale, d
+        return _ext.normalize(x, centre, True, scale)[..., :d]
 
     @staticmethod
     def backward(ctx, grad_y):
         (x,) = ctx.saved_tensors
-        return _ext.normalize_backward(x, grad_y, ctx.centre, True, ctx.scale), None, None
+        if x.shape[-1] != ctx.d:
+            grad_y = _pad_features(grad_y)
+        return _ext.normalize_backward(x, grad_y, ctx.centre, True, ctx.scale)[..., :ctx.d], None, None
 
 
 class FASTMultiHeadAttention_Function(torch.autograd.Function):
@@ -59,7 +81,8 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
     as in the reference extension (``fastmax_cuda_forward.cu:289, 443``).  With
     ``normalize`` the tensors are first mapped to ``lim * x / max_n ||x_n||`` (the
     semantics spelled out in ``transformer/model.py:97-102``) and, like the reference,
-    the returned gradients are those with respect to the normalised q and k.
+    the returned gradients are those with respect to the normalised q and k.  Head sizes other
+    than 32 and 64 (up to 64) run zero-padded to the next of the two.
     """
 
     @staticmethod
@@ -68,6 +91,8 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
         if q.dim() not in (3, 4):
             raise ValueError("q, k, and v should be either 3 or 4 dimensional tensors. "
                              "If 3D: (b*h,n,d), if 4D: (b,h,n,d).")
+        d = q.shape[-1]
+        q, k, v = _pad_features(q), _pad_features(k), _pad_features(v)
         if normalize:
             q = _ext.normalize(q, CENTRE_NONE, True, float(lim))
             k = _ext.normalize(k, CENTRE_NONE, True, float(lim))
@@ -79,15 +104,17 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
             ctx.save_for_backward(q, k, v, o, g, saved)
         else:
             o, g = _ext.forward_ex(q, k, v, bool(mask), inv_tau, float(a0), float(a1), float(a2), int(p), 0, 0)
-        ctx.cfg = (bool(mask), inv_tau, float(a0), float(a1), float(a2), int(p))
-        return o
+        ctx.cfg = (bool(mask), inv_tau, float(a0), float(a1), float(a2), int(p), d)
+        return o[..., :d]
 
     @staticmethod
     def backward(ctx, grad_output):
         q, k, v, o, g, saved = ctx.saved_tensors
-        mask, inv_tau, a0, a1, a2, p = ctx.cfg
+        mask, inv_tau, a0, a1, a2, p, d = ctx.cfg
+        if q.shape[-1] != d:
+            grad_output = _pad_features(grad_output)
         gq, gk, gv = _ext.backward_saved(q, k, v, o, g, grad_output, saved, mask, inv_tau, a0, a1, a2, p, 0, 0)
-        return (gq, gk, gv) + (None,) * 11
+        return (gq[..., :d], gk[..., :d], gv[..., :d]) + (None,) * 11
 
 
 def fastmax_function(q, k, v, mask=0, dropout_rate=0.0, normalize=0, temperature=1, a0=1, a1=1, a2=0.5, lim=1, p=2):

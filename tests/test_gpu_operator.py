@@ -232,3 +232,36 @@ def test_autograd_wrapper_with_cached_keys(sf, nq):
                                                   1.0, 1.0, 0.5, 1.0, 2)
     assert rel_err(o, of[:, :, nk - nq:]) < 1e-5
 
+
+@pytest.mark.parametrize("d", [20, 48])
+@pytest.mark.parametrize("normalize", [False, True])
+def test_other_head_sizes_run_padded(sf, d, normalize):
+    """Head sizes between the two the kernels are built for: zero-padded inside the autograd
+    function, results and gradients of the caller's shape, against the oracle at the true size."""
+    b, h, n, t = 2, 3, 333, 5.0
+    q, k, v, go = (rnd(b, h, n, d, seed=s) for s in (70, 71, 72, 73))
+    qd, kd, vd = (x.to(DEV).requires_grad_(True) for x in (q, k, v))
+    o = sf.FASTMultiHeadAttention_Function.apply(qd, kd, vd, None, None, True, 0.0, normalize, t, 1.0, 1.0, 0.5, 1.5, 2)
+    assert o.shape == (b, h, n, d)
+    o.backward(go.to(DEV))
+    qr, kr, vr = (x.double().requires_grad_(True) for x in (q, k, v))
+    qn, kn = (O.normalize_lim(qr, 1.5), O.normalize_lim(kr, 1.5)) if normalize else (qr, kr)
+    qn.retain_grad(); kn.retain_grad()
+    oref, _ = O.closed_form_forward(qn, kn, vr, mask=True, tau=t, p=2)
+    oref.backward(go.double())
+    assert rel_err(o, oref) < 1e-5
+    # like the reference, the function returns the gradients with respect to the normalised q and k
+    for got, want in ((qd.grad, qn.grad), (kd.grad, kn.grad), (vd.grad, vr.grad)):
+        assert got.shape == want.shape and rel_err(got, want) < 1e-5
+    # the differentiable normalisation on its own, token-mean centring
+    x = rnd(b, h, n, d, seed=74)
+    xd = x.to(DEV).requires_grad_(True)
+    y = sf.FastmaxNormalize.apply(xd, sf.CENTRE_TOKEN, 2.0)
+    y.backward(go.to(DEV))
+    xr = x.double().requires_grad_(True)
+    yr = O.normalize_token_mean(xr, xr)[0] * 2.0
+    yr.backward(go.double())
+    assert rel_err(y, yr) < 1e-5 and rel_err(xd.grad, xr.grad) < 1e-5
+    with pytest.raises(RuntimeError, match="unsupported head size"):
+        sf.FASTMultiHeadAttention_Function.apply(*(rnd(1, 1, 8, 80).to(DEV) for _ in range(3)))
+
