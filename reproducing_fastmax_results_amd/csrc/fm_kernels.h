@@ -775,8 +775,10 @@ struct TokCfg {
   static constexpr int NZ = sizeof(E) == 2 ? 2 : 1; // hi/lo split of fp32 denominators
   static constexpr int SLAB = SA * DH * PS;         // elements per slab buffer
   static constexpr int PV_STAGE = KT_PV * PQ + DH * PV_PV;                // k_pv: stream rows, stream transposed
-  static constexpr int DS_STAGE = 2 * KT_DS * PQ + DH * PV_DS + KT_DS;    // k_ds: two row tiles, transposed tile, c values
-  static constexpr int DV_STAGE = 2 * KT_DV * PQ + 2 * DH * PV_DV + KT_DV; // k_ds with dV: + gh transposed
+  static constexpr int DS_STAGE = 2 * KT_DS * PQ + (M::HAS_TR ? 0 : DH * PV_DS) + KT_DS;   // k_ds: two row tiles, (transposed tile,) c values
+  // k_ds with dV: two row tiles and the c values; the transposed fragments come from the row tiles
+  // through transposing LDS reads where the type has them, from two more (transposed) tiles otherwise
+  static constexpr int DV_STAGE = 2 * KT_DV * PQ + (M::HAS_TR ? 0 : 2 * DH * PV_DV) + KT_DV;
   static constexpr int DS_NBUF = sizeof(E) == 2 ? 2 : 1;
 };
 

@@ -40,6 +40,18 @@ template <> struct Mma<fm_half> {
     for (int i = 0; i < 8; ++i) r[i] = fm_half(c[8 * s + i]);
     return r;
   }
+  // The fragment load_perm would read from a transposed tile, taken from the ROW-MAJOR tile
+  // instead (tokens x features, `pitch` elements per token) with two transposing reads: lane
+  // (lr, lh) gets feature col0 + lr of the tokens tok0 + 4 lh + {0..3} and tok0 + 8 + 4 lh + {0..3},
+  // the rows its accumulator k-step holds.  HAS_TR: the interface type for which this exists.
+  static constexpr bool HAS_TR = true;
+  static FM_DEVICE frag load_tr(const fm_half* tile, int pitch, int tok0, int col0, int lane) {
+    const int lh = lane >> 5, half16 = (lane >> 4) & 1, s = (lane & 15) >> 2, q = lane & 3;
+    const fm_half* p = tile + (tok0 + 4 * lh + s) * pitch + col0 + 16 * half16 + 4 * q;
+    const fm_half4 lo = fm_lds_tr4(p), hi = fm_lds_tr4(p + 8 * pitch);
+    frag r = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return r;
+  }
 };
 
 template <> struct Mma<float> {
@@ -54,6 +66,8 @@ template <> struct Mma<float> {
   static FM_DEVICE frag splat(float x) { return x; }
   static FM_DEVICE int tperm(int t) { return t; }
   static FM_DEVICE frag load_perm(const float* row, int s, int lh) { return row[8 * (s / 4) + 4 * lh + (s % 4)]; }
+  static constexpr bool HAS_TR = false;
+  static FM_DEVICE frag load_tr(const float*, int, int, int, int) { return 0.f; }   // never called
   static FM_DEVICE frag from_acc(const fm_f32x16& c, int s) { return c[s]; }
 };
 

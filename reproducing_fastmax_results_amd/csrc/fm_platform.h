@@ -63,6 +63,20 @@ FM_DEVICE fm_f32x16 fm_mfma_f32(float a, float b, fm_f32x16 c) {
 FM_DEVICE float fm_shfl_xor(float v, int m) { return hostsim::shfl(v, hostsim::g_t.lane ^ m); }
 FM_DEVICE int fm_shfl_xor_i(int v, int m) { return hostsim::shfl(v, hostsim::g_t.lane ^ m); }
 FM_DEVICE float fm_dot2(fm_half2 a, fm_half2 b, float c) { return float(a[0]) * float(b[0]) + float(a[1]) * float(b[1]) + c; }
+// Transposing LDS read (ds_read_b64_tr_b16): every lane names four consecutive halves; inside each
+// group of 16 lanes, lane i receives element i % 4 of the words named by lanes i/4, 4 + i/4,
+// 8 + i/4 and 12 + i/4 (layout read off the instruction on an MI355X by a probe kernel).
+FM_DEVICE fm_half4 fm_lds_tr4(const fm_half* p) {
+  fm_half4 w;
+  __builtin_memcpy(&w, p, 8);
+  const int lane = hostsim::g_t.lane, g = lane & ~15, i = lane & 15;
+  fm_half4 r;
+  for (int t = 0; t < 4; ++t) {
+    const fm_half4 o = hostsim::shfl(w, g + 4 * t + i / 4);
+    r[t] = o[i % 4];
+  }
+  return r;
+}
 FM_DEVICE float fm_fmaxf(float a, float b) { return a > b ? a : b; }
 FM_DEVICE float fm_clampf(float x, float lim) { return x > lim ? lim : (x < -lim ? -lim : x); }
 FM_DEVICE float fm_rsqrtf(float a) { return 1.0f / std::sqrt(a); }
@@ -110,6 +124,16 @@ FM_DEVICE fm_f32x16 fm_mfma_f32(float a, float b, fm_f32x16 c) {
 FM_DEVICE float fm_shfl_xor(float v, int m) { return __shfl_xor(v, m, 64); }
 FM_DEVICE int fm_shfl_xor_i(int v, int m) { return __shfl_xor(v, m, 64); }
 FM_DEVICE float fm_dot2(fm_half2 a, fm_half2 b, float c) { return __builtin_amdgcn_fdot2(a, b, c, false); }
+// Transposing LDS read (ds_read_b64_tr_b16): every lane names four consecutive halves; inside each
+// group of 16 lanes, lane i receives element i % 4 of the words named by lanes i/4, 4 + i/4,
+// 8 + i/4 and 12 + i/4 (layout read off the instruction on an MI355X by a probe kernel).
+FM_DEVICE fm_half4 fm_lds_tr4(const fm_half* p) {
+  typedef short fm_s16x4 __attribute__((ext_vector_type(4)));
+  const fm_s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) fm_s16x4*)(p));
+  fm_half4 r;
+  __builtin_memcpy(&r, &v, 8);
+  return r;
+}
 FM_DEVICE float fm_fmaxf(float a, float b) { return fmaxf(a, b); }
 // clamp to [-lim, lim] in one instruction (v_med3_f32)
 FM_DEVICE float fm_clampf(float x, float lim) { return __builtin_amdgcn_fmed3f(x, -lim, lim); }
