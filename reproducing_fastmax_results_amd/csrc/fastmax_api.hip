@@ -137,7 +137,7 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   p.big = take(size_t(d->bh) * p.nslots * bigsz);
   p.small = take(size_t(d->bh) * p.nslots * smallsz);
   p.save = (d->flags & FASTMAX_FLAG_SAVE_FOR_BACKWARD) != 0;
-  p.vr = take(p.save ? tk : 0);
+  p.vr = take(p.save || p.half ? tk : 0);      // _Float16: the forward stages v rows (transposing LDS reads)
   p.big2 = take(p.save ? size_t(d->bh) * p.nslots * bigsz : 0);
   p.fwd_bytes = off ? off : 256;
   off = 0;
@@ -294,7 +294,10 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   E* big = reinterpret_cast<E*>(ws + p.big);
   float* small = reinterpret_cast<float*>(ws + p.small);
   E* kr = reinterpret_cast<E*>(ws + p.kr);
-  E* vr = p.save ? reinterpret_cast<E*>(ws + p.vr) : nullptr;
+  E* vr = (p.save || p.half) ? reinterpret_cast<E*>(ws + p.vr) : nullptr;
+  // the transposed copies feed the state walk and the fp32 kernels; the _Float16 token kernels read
+  // transposed fragments out of row tiles
+  if (sizeof(E) == 2 && !p.use_state) { kt = nullptr; vt = nullptr; }
   int st = launch_transpose2<TIO, E, DH>(v, d->sv, vt, vr, 1.0f, k, d->sk, kt, kr, p.sc, d->bh, d->nk, p.npad_k, stream);
   if (st) return st;
   if (p.use_state) {
@@ -313,7 +316,7 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   TokArgs<TIO, E> a;
   tok_common(a, d, p);
   a.own_io = cref<TIO>(q, d->sq);
-  a.xr = kr; a.zt = vt; a.npad_own = p.npad_q; a.npad_str = p.npad_k;
+  a.xr = kr; a.yr = vr; a.zt = vt; a.npad_own = p.npad_q; a.npad_str = p.npad_k;
   a.big = big; a.small = small;
   a.out = mref<TIO>(o, d->so);
   a.g = mref<float>(g, d->sg);

@@ -141,7 +141,8 @@ template <typename T> inline TRef<T> fm_ref(T* ptr, const FastmaxStrides& s) {
 // ------------------------------------------------------------------------------
 // k_transpose: x (bh, n, DH) strided, interface type  ->  compute type, multiplied by
 // `scale`, zero for tokens >= n:  xt [bh][DH][npad] (transposed) and, when xr is not
-// null, xr [bh][npad][DH] (row-major).  The token-side kernels stage their tiles from
+// null, xr [bh][npad][DH] (row-major); xt may be null as well (the _Float16 token kernels read
+// transposed fragments out of row tiles; only the state walk needs xt).  The token-side kernels stage their tiles from
 // these copies with plain 16-byte moves.  Two tensors of the same length (k and v) go in one
 // launch: grid (npad/64, bh, 2), the second set of arguments serves z = 1.
 // ------------------------------------------------------------------------------
@@ -174,9 +175,12 @@ k_transpose(TransposeJob<TIO, E> j0, TransposeJob<TIO, E> j1, int n, int npad) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) v[j] *= scale;
     if (xr) CE<E>::st8(xr + (int64_t(bh) * npad + t0 + tok) * DH + d0, v);
+    if (xt) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) tile[(d0 + j) * PT + Mma<E>::tperm(tok)] = CE<E>::from(v[j]);
+      for (int j = 0; j < 8; ++j) tile[(d0 + j) * PT + Mma<E>::tperm(tok)] = CE<E>::from(v[j]);
+    }
   }
+  if (!xt) return;                                     // only the row-major copy was asked for
   FM_SYNC();
   E* ob = xt + int64_t(bh) * DH * npad + t0;
   for (int c = tid; c < DH * (64 / VEC); c += FM_THREADS) {
@@ -241,6 +245,7 @@ k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, TRef<const
   E* qrrow = qr + (int64_t(bh) * npad + row) * DH + d0;
 #pragma unroll
   for (int j = 0; j < EPT; j += 8) { CE<E>::st8(ghrow + j, &vg[j]); CE<E>::st8(qrrow + j, &vq[j]); }
+  if (!qt) return;                                     // ght, qt, qct: only the state walk and the fp32 kernels read them
 #pragma unroll
   for (int j = 0; j < EPT; ++j) {
     tg[(d0 + j) * PT + Mma<E>::tperm(tok)] = CE<E>::from(vg[j]);
@@ -774,7 +779,7 @@ struct TokCfg {
   static constexpr int PV_DV = KT_DV + M::PAD;
   static constexpr int NZ = sizeof(E) == 2 ? 2 : 1; // hi/lo split of fp32 denominators
   static constexpr int SLAB = SA * DH * PS;         // elements per slab buffer
-  static constexpr int PV_STAGE = KT_PV * PQ + DH * PV_PV;                // k_pv: stream rows, stream transposed
+  static constexpr int PV_STAGE = M::HAS_TR ? 2 * KT_PV * PQ : KT_PV * PQ + DH * PV_PV;   // k_pv: two row tiles, or stream rows + stream transposed
   static constexpr int DS_STAGE = 2 * KT_DS * PQ + (M::HAS_TR ? 0 : DH * PV_DS) + KT_DS;   // k_ds: two row tiles, (transposed tile,) c values
   // k_ds with dV: two row tiles and the c values; the transposed fragments come from the row tiles
   // through transposing LDS reads where the type has them, from two more (transposed) tiles otherwise

@@ -285,10 +285,23 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
   // ---- dense tiles over the stream tokens of this segment ----
   if (G.send > G.sbeg) {
     const typename TM::Coef coef = TM::coef(A.a0, A.a1, A.a2);
-    TileRegs<E, KT, DH> rx;
+    // _Float16: the second stream tile is staged row-major too (yr: v rows for the forward, gh rows
+    // for dV) and its transposed fragments come from transposing LDS reads; zt is not read then
+    constexpr bool TR = M::HAS_TR;
+    TileRegs<E, KT, DH> rx, ry;
     TileRegs<E, DH, KT> rz;
     const E* xb = A.xr + int64_t(bh) * A.npad_str * DH;
-    const E* zb = A.zt + int64_t(bh) * DH * A.npad_str;
+    const E* yb = TR ? A.yr + int64_t(bh) * A.npad_str * DH : nullptr;
+    const E* zb = TR ? nullptr : A.zt + int64_t(bh) * DH * A.npad_str;
+    auto fetch = [&](int sx) {                          // global memory -> registers
+      rx.load(xb + int64_t(sx) * DH, DH, tid);
+      if (TR) ry.load(yb + int64_t(sx) * DH, DH, tid); else rz.load(zb + sx, A.npad_str, tid);
+    };
+    auto put = [&](int b) {                             // registers -> stage buffer b
+      E* Xn = Own + b * STAGE;
+      rx.store(Xn, PQ, tid);
+      if (TR) ry.store(Xn + KT * PQ, PQ, tid); else rz.store(Xn + KT * PQ, PV, tid);
+    };
     // Stages are walked so that all blocks of a batch*head start at the same end of the stream
     // (queries start at the first key of the segment, keys at its last query): blocks that run at
     // the same time then read the same tiles at about the same time and share them in the L2.
@@ -299,14 +312,9 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
     // and registers -> LDS in the middle of stage i (between the two groups of matrix products),
     // so the only thing left at the top of a stage is the barrier.
     auto more = [&](int sx) { return OWN == FM_OWN_Q ? (sx < G.send) : (sx >= G.sbeg); };
-    rx.load(xb + int64_t(s_first) * DH, DH, tid);
-    rz.load(zb + s_first, A.npad_str, tid);
-    rx.store(Own, PQ, tid);
-    rz.store(Own + KT * PQ, PV, tid);
-    if (more(s_first + s_step)) {
-      rx.load(xb + int64_t(s_first + s_step) * DH, DH, tid);
-      rz.load(zb + s_first + s_step, A.npad_str, tid);
-    }
+    fetch(s_first);
+    put(0);
+    if (more(s_first + s_step)) fetch(s_first + s_step);
     int buf = 0;
     for (int s0 = s_first; more(s0); s0 += s_step) {
       E* Xs = Own + buf * STAGE;                        // the own rows and the slabs are spent
@@ -331,19 +339,15 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
         for (int ct = 0; ct < NT; ++ct)
 #pragma unroll
           for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
-            zf[ct][ss] = M::load_perm(Zt + (32 * ct + lr) * PV + 32 * st, ss, lh);
+            zf[ct][ss] = TR ? M::load_tr(Zt, PQ, 32 * st + 16 * ss, 32 * ct, lane)
+                            : M::load_perm(Zt + (32 * ct + lr) * PV + 32 * st, ss, lh);
         if (st == KT / 32 - 1) {
           // next stage: registers -> the other buffer (its readers finished before this stage's
           // barrier), then the stage after it: global memory -> registers
           const int sn = s0 + s_step;
           if (more(sn)) {
-            E* Xn = Own + (buf ^ 1) * STAGE;
-            rx.store(Xn, PQ, tid);
-            rz.store(Xn + KT * PQ, PV, tid);
-            if (more(sn + s_step)) {
-              rx.load(xb + int64_t(sn + s_step) * DH, DH, tid);
-              rz.load(zb + sn + s_step, A.npad_str, tid);
-            }
+            put(buf ^ 1);
+            if (more(sn + s_step)) fetch(sn + s_step);
           }
         }
 #pragma unroll
