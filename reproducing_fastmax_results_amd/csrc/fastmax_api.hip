@@ -239,8 +239,9 @@ int launch_build(const BuildArgs<E>& args, int bh, fm_stream_t stream) {
   return launch_scan<E, DH>(a, bh, nsteps, stream);
 }
 
-// Dynamic LDS of a token kernel (kind 0: k_pv, 1: k_ds, 2: k_ds with dV): va, vb | own rows |
-// region, where the dense stages and the output staging lie over the own rows and the region.
+// Dynamic LDS of a token kernel (kind 0: k_pv, 1: k_ds, 2: k_ds with dV, 3: k_ds with the fused
+// preparation): va, vb | own rows | region, where the dense stages and the output staging lie over
+// the own rows and the region.
 template <typename E, int DH, int QT> size_t tok_lds_bytes(int kind) {
   typedef TokCfg<E, DH, QT> C;
   size_t region = size_t(2) * C::SLAB * sizeof(E);
@@ -250,8 +251,10 @@ template <typename E, int DH, int QT> size_t tok_lds_bytes(int kind) {
   const size_t outst = size_t(C::QW) * (DH + 1) * 4;
   const size_t stage = kind == 0 ? size_t(2) * C::PV_STAGE * sizeof(E)
                                  : size_t(C::DS_NBUF) * (kind == 2 ? C::DV_STAGE : C::DS_STAGE) * sizeof(E);
+  const size_t prep = size_t(2) * C::QW * C::PQ * sizeof(E) + size_t(C::QW) * 4;   // own q' rows, gh rows, c
   if (outst > body) body = outst;
   if (stage > body) body = stage;
+  if (kind == 3 && prep > body) body = prep;
   return size_t(2 * DH) * 4 + body;
 }
 
@@ -262,6 +265,8 @@ template <typename TIO, typename E> void tok_common(TokArgs<TIO, E>& a, const Fa
   a.g = TRef<float>{nullptr, 0, 0, 0, 0, 0};
   a.nslots = p.nslots; a.L = p.L; a.nseg = p.nseg; a.causal = d->mask != 0; a.use_state = p.use_state;
   a.quad = p.quad; a.a0 = p.a0; a.a1 = p.a1; a.a2 = p.a2; a.sc = p.sc; a.out_scale = 1.0f; a.zscale = 1.0f;
+  a.own_o = TRef<const TIO>{nullptr, 0, 0, 0, 0, 0}; a.own_do = a.own_o;
+  a.w_gh = nullptr; a.w_qr = nullptr; a.w_cv = nullptr; a.gscale = p.gscale;
 }
 
 template <typename TIO, typename E, int DH, int QT, int OWN>
@@ -275,13 +280,13 @@ int launch_pv(const TokArgs<TIO, E>& a, int bh, int kernel_id, fm_stream_t strea
   return fm_after_launch();
 }
 
-template <typename TIO, typename E, int DH, int QT, int OWN, int DV = 0>
+template <typename TIO, typename E, int DH, int QT, int OWN, int DV = 0, int PREP = 0>
 int launch_ds(const TokArgs<TIO, E>& a, int bh, int kernel_id, fm_stream_t stream) {
   typedef TokCfg<E, DH, QT> C;
-  const size_t lds = tok_lds_bytes<E, DH, QT>(DV ? 2 : 1);
-  fm_allow_lds(reinterpret_cast<const void*>(&k_ds<TIO, E, DH, QT, OWN, DV>), lds);
+  const size_t lds = tok_lds_bytes<E, DH, QT>(PREP ? 3 : (DV ? 2 : 1));
+  fm_allow_lds(reinterpret_cast<const void*>(&k_ds<TIO, E, DH, QT, OWN, DV, PREP>), lds);
   ProfScope prof(kernel_id, stream);
-  FM_KERNEL_LAUNCH((k_ds<TIO, E, DH, QT, OWN, DV>), fm_dim3((a.n_own + C::QW - 1) / C::QW, bh), fm_dim3(FM_THREADS), lds,
+  FM_KERNEL_LAUNCH((k_ds<TIO, E, DH, QT, OWN, DV, PREP>), fm_dim3((a.n_own + C::QW - 1) / C::QW, bh), fm_dim3(FM_THREADS), lds,
                    stream, a);
   return fm_after_launch();
 }

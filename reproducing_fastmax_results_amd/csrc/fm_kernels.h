@@ -740,13 +740,15 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_state_scan(E* FM_RESTRICT big, E* FM_REST
 // ------------------------------------------------------------------------------
 // LDS sizes (in elements of E) used by k_pv / k_ds; the host computes the dynamic LDS
 // bytes from the same struct.
-// Stream tokens per stage of the dense loops of the _Float16 token kernels (64-token stages
-// measured slower on MI355X for k_pv and the plain k_ds, which lose a workgroup per CU to them).
+// Stream tokens per stage of the dense loops of the _Float16 token kernels.  k_ds stages two row
+// tiles only (its transposed fragments come from transposing LDS reads), so 64-token stages cost it
+// no occupancy and halve its barriers (dQ 0.117 -> 0.114 ms at B*H = 32, N = 4096 on MI355X); k_pv
+// measured slower with them (0.092 vs 0.087 ms).
 #ifndef FM_TUNE_KT_PV
 #define FM_TUNE_KT_PV 32
 #endif
 #ifndef FM_TUNE_KT_DS
-#define FM_TUNE_KT_DS 32
+#define FM_TUNE_KT_DS 64
 #endif
 #ifndef FM_TUNE_KT_DV
 #define FM_TUNE_KT_DV 64

@@ -44,6 +44,12 @@ template <typename TIO, typename E> struct TokArgs {
   float out_scale;                      // factor on the stored gradient
   float out2_scale;                     // k_ds with dV: factor on dV
   float zscale;                         // factor on the Z of the state (k_ds)
+  // k_ds with PREP (own = queries): the kernel makes gh = gscale * dO / g, c = gh . o and q' = sc * q of
+  // its own queries itself, from the caller's tensors, and leaves them in w_gh, w_qr (row-major
+  // [bh][npad_own][DH]) and w_cv ([bh][npad_own], tile order) for the key-side pass that follows
+  TRef<const TIO> own_o, own_do;
+  E* w_gh; E* w_qr; E* w_cv;
+  float gscale;
 };
 
 // Z (fp32, [DH][DH]) -> LDS in the compute type (hi/lo split for _Float16), va/vb -> vecs.
@@ -418,7 +424,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
 // score tiles it already has, P = f(S), dV^T += gh^T P, which saves the four score
 // products per tile that a separate k_pv launch would repeat.
 // ------------------------------------------------------------------------------
-template <typename TIO, typename E, int DH, int QT, int OWN, int DV>
+template <typename TIO, typename E, int DH, int QT, int OWN, int DV, int PREP>
 FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS)) k_ds(TokArgs<TIO, E> A) {
   typedef TokCfg<E, DH, QT> C;
   typedef Mma<E> M;
@@ -443,7 +449,63 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
   const int bh = G.bh, t0 = G.t0;
   const bool causal = A.causal != 0;
 
-  {
+  if (PREP) {
+    // own queries straight from the caller's q, o, dO and g (four threads per token, 64 tokens per
+    // pass): q' rows -> Own, gh rows -> R, c behind them; the same values go to the workspace copies
+    // the key-side pass streams.  Rows past the end are zeros.  Replaces div_grad_output
+    // (fastmax_cuda_backward.cu:494-501) and the "grad * o" row sums of fastattention_einops.py:405-407.
+    constexpr int EPT = DH / 4;
+    static_assert(!PREP || (OWN == FM_OWN_Q && QT == 1), "the fused preparation is for one query tile per wavefront");
+    float* cl = reinterpret_cast<float*>(R + QW * PQ);   // c per own query, behind the gh rows
+    const int part = tid & 3, d0 = part * EPT;
+    constexpr int NH = QW / 64;
+    float ra[NH][EPT], rb[NH][EPT], rc[NH][EPT], gi[NH];
+    // every load of the block is issued before the first result is used
+#pragma unroll
+    for (int h = 0; h < NH; ++h) {
+      const int row = t0 + 64 * h + (tid >> 2);
+      if (row < A.n_own) {
+        gi[h] = A.g.base(bh)[int64_t(row) * A.g.s_n];
+#pragma unroll
+        for (int j = 0; j < EPT; j += 8) {
+          IO<TIO>::ld8(A.own_do.base(bh) + int64_t(row) * A.own_do.s_n + d0 + j, A.own_do.vec != 0, &ra[h][j]);
+          IO<TIO>::ld8(A.own_o.base(bh) + int64_t(row) * A.own_o.s_n + d0 + j, A.own_o.vec != 0, &rb[h][j]);
+          IO<TIO>::ld8(A.own_io.base(bh) + int64_t(row) * A.own_io.s_n + d0 + j, A.own_io.vec != 0, &rc[h][j]);
+        }
+      } else {
+        gi[h] = 1.0f;
+#pragma unroll
+        for (int j = 0; j < EPT; ++j) { ra[h][j] = 0.f; rb[h][j] = 0.f; rc[h][j] = 0.f; }
+      }
+    }
+#pragma unroll
+    for (int h = 0; h < NH; ++h) {
+      const int tok = 64 * h + (tid >> 2), row = t0 + tok;
+      const float ginv = A.gscale / gi[h];
+      float vg[EPT], vq[EPT];
+      float csum = 0.f;
+#pragma unroll
+      for (int j = 0; j < EPT; ++j) {
+        vg[j] = ra[h][j] * ginv;
+        csum += vg[j] * rb[h][j];
+        vq[j] = rc[h][j] * A.sc;
+      }
+      csum += fm_shfl_xor(csum, 1);
+      csum += fm_shfl_xor(csum, 2);
+      const E ch = CE<E>::from(csum);
+      if (part == 0) {
+        A.w_cv[int64_t(bh) * A.npad_own + t0 + 64 * h + M::tperm(tid >> 2)] = ch;
+        cl[tok] = float(ch);
+      }
+      E* ghrow = A.w_gh + (int64_t(bh) * A.npad_own + row) * DH + d0;
+      E* qrrow = A.w_qr + (int64_t(bh) * A.npad_own + row) * DH + d0;
+#pragma unroll
+      for (int j = 0; j < EPT; j += 8) {
+        CE<E>::st8(ghrow + j, &vg[j]); CE<E>::st8(qrrow + j, &vq[j]);
+        CE<E>::st8(R + tok * PQ + d0 + j, &vg[j]); CE<E>::st8(Own + tok * PQ + d0 + j, &vq[j]);
+      }
+    }
+  } else {
     TileRegs<E, QW, DH> ro;
     ro.load(A.own_r + (int64_t(bh) * A.npad_own + t0) * DH, DH, tid);
     ro.store(Own, PQ, tid);
@@ -462,13 +524,15 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
   for (int j = 0; j < QT; ++j) {
     tw[j] = (j == 0) ? wave : (4 * QT - 1 - wave);
     xrow[j] = tw[j] * 32 + lr;
-    ci[j] = (OWN == FM_OWN_Q) ? float(A.cv[int64_t(bh) * A.npad_own + t0 + M::tperm(xrow[j])]) : 1.0f;
+    ci[j] = (OWN == FM_OWN_Q) ? (PREP ? reinterpret_cast<const float*>(R + QW * PQ)[xrow[j]]
+                                      : float(A.cv[int64_t(bh) * A.npad_own + t0 + M::tperm(xrow[j])])) : 1.0f;
     cs_own[j] = TM::splat_c(ci[j]);
   }
   frag of[QT][NKS], of2[QT][NKS];
 #pragma unroll
   for (int j = 0; j < QT; ++j) {
-    const E* o2 = A.own2_r + (int64_t(bh) * A.npad_own + t0 + xrow[j]) * DH + lh * M::KPL;
+    const E* o2 = PREP ? R + xrow[j] * PQ + lh * M::KPL
+                       : A.own2_r + (int64_t(bh) * A.npad_own + t0 + xrow[j]) * DH + lh * M::KPL;
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
       of[j][ks] = M::load(Own + xrow[j] * PQ + ks * M::KSTEP + lh * M::KPL);
