@@ -35,7 +35,7 @@ PEAK_HBM_GBS = 8000.0
 
 # HBM bytes per launch of the dominant kernel at the workload below, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this file scaled by a copy of known size; keyed by (dtype, --chunk, kernel).
-TRAFFIC_BYTES = {("bf16", 0, "dkv"): 115728 * 1024}
+TRAFFIC_BYTES = {("bf16", 0, "dkv"): 115648 * 1024}
 
 WORKLOAD = dict(name="configs[1]: causal order-2 fwd+bwd", B=4, H=8, N=4096, D=64, p=2, mask=True)
 
