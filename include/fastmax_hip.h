@@ -160,6 +160,12 @@ int fastmax_profile_end(int* kernel_ids, float* milliseconds, int capacity);
  * registers, the value found (out_f16 and out_f32: 1024 floats each, device memory). */
 int fastmax_probe_mfma(float* out_f16, float* out_f32, void* hip_stream);
 
+/* Self-check of the transposing LDS read (ds_read_b64_tr_b16) the _Float16 kernels use for transposed
+ * fragments: one wavefront reads a 16 x 64 tile holding 64 * row + col; lane l addresses the four
+ * values at (row l % 16, columns 4 * (l / 16) ..).  out: 256 floats (device memory), four per lane.
+ * Expected: lane l, value t = 64 * (4 t + (l % 16) / 4) + 4 * (l / 16) + l % 4. */
+int fastmax_probe_lds_transpose(float* out, void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -52,7 +52,7 @@ class NormDesc(C.Structure):
 EXPORTS = (
     "fastmax_workspace_bytes", "fastmax_forward", "fastmax_backward", "fastmax_backward_saved", "fastmax_normalize",
     "fastmax_normalize_backward", "fastmax_normalize_backward_stats_bytes",
-    "fastmax_status_string", "fastmax_version", "fastmax_probe_mfma",
+    "fastmax_status_string", "fastmax_version", "fastmax_probe_mfma", "fastmax_probe_lds_transpose",
     "fastmax_profile_begin", "fastmax_profile_end",
 )
 
@@ -127,6 +127,8 @@ class FastmaxLib:
         L.fastmax_version.restype = C.c_int
         L.fastmax_probe_mfma.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
         L.fastmax_probe_mfma.restype = C.c_int
+        L.fastmax_probe_lds_transpose.argtypes = [C.c_void_p, C.c_void_p]
+        L.fastmax_probe_lds_transpose.restype = C.c_int
         L.fastmax_profile_begin.restype = C.c_int
         L.fastmax_profile_end.argtypes = [C.POINTER(C.c_int), C.POINTER(C.c_float), C.c_int]
         L.fastmax_profile_end.restype = C.c_int
@@ -269,6 +271,12 @@ class FastmaxLib:
         ms = (C.c_float * capacity)()
         n = min(self.lib.fastmax_profile_end(ids, ms, capacity), capacity)
         return [(self.KERNEL_NAMES[ids[i]], float(ms[i])) for i in range(n)]
+
+    def probe_lds_transpose(self, device):
+        """(64 lanes, 4) values the transposing LDS read returns for the header's test pattern."""
+        out = torch.zeros(256, dtype=torch.float32, device=device)
+        self.check(self.lib.fastmax_probe_lds_transpose(out.data_ptr(), 0), "fastmax_probe_lds_transpose")
+        return out.view(64, 4)
 
     def probe_mfma(self, device):
         a = torch.zeros(1024, dtype=torch.float32, device=device)

@@ -404,7 +404,7 @@ int add_rows(const FastmaxDesc* d, const SplitPlan& sp, const void* dqa, void* d
 
 extern "C" {
 
-int fastmax_version(void) { return 102; }
+int fastmax_version(void) { return 103; }
 
 const char* fastmax_status_string(int status) {
   switch (status) {
@@ -617,6 +617,12 @@ int fastmax_profile_end(int* kernel_ids, float* milliseconds, int capacity) {
 int fastmax_probe_mfma(float* out_f16, float* out_f32, void* hip_stream) {
   if (!out_f16 || !out_f32) return FASTMAX_ERR_NULL;
   FM_KERNEL_LAUNCH(k_probe_mfma, fm_dim3(1), fm_dim3(64), 0, static_cast<fm_stream_t>(hip_stream), out_f16, out_f32);
+  return fm_after_launch();
+}
+
+int fastmax_probe_lds_transpose(float* out, void* hip_stream) {
+  if (!out) return FASTMAX_ERR_NULL;
+  FM_KERNEL_LAUNCH(k_probe_lds_tr, fm_dim3(1), fm_dim3(64), 0, static_cast<fm_stream_t>(hip_stream), out);
   return fm_after_launch();
 }
 

@@ -768,7 +768,10 @@ struct TokCfg {
   // _Float16, QT = 2: two tiles per wavefront share every state fragment read from LDS and halve
   // the state bytes staged per token; used by k_ds when there are states to read (dQ + dK
   // 0.20 vs 0.23 ms at the same shape with 1024-token segments).
-  static constexpr int OCC_PV = sizeof(E) == 2 ? (QT == 1 ? 4 : 2) : 1;   // workgroups per CU the kernels are sized for
+#ifndef FM_TUNE_OCC_PV
+#define FM_TUNE_OCC_PV 4
+#endif
+  static constexpr int OCC_PV = sizeof(E) == 2 ? (QT == 1 ? FM_TUNE_OCC_PV : 2) : 1;   // workgroups per CU the kernels are sized for
   static constexpr int OCC_DS = sizeof(E) == 2 ? (QT == 1 ? 3 : 2) : 1;
   static constexpr int SA = sizeof(E) == 2 ? QT : 2;                      // values of a per state slab
   static constexpr int KT_PV = sizeof(E) == 2 ? FM_TUNE_KT_PV : 64;   // stream tokens per stage of the dense loop, k_pv
@@ -870,3 +873,18 @@ FM_GLOBAL void k_probe_mfma(float* out_f16, float* out_f32) {
 #pragma unroll
   for (int e = 0; e < 16; ++e) out_f32[lane * 16 + e] = c2[e];
 }
+
+// ------------------------------------------------------------------------------
+// k_probe_lds_tr: one wavefront; a 16 x 64 _Float16 tile holding 64 * row + col (all exact); lane l
+// reads through fm_lds_tr4 at (row l % 16, column 4 * (l / 16)) and writes its four values.
+// ------------------------------------------------------------------------------
+FM_GLOBAL void k_probe_lds_tr(float* out) {
+  FM_SHARED fm_half tile[16 * 64];
+  const int l = FM_TID_X & 63;
+  for (int i = l; i < 16 * 64; i += 64) tile[i] = fm_half(float(i));
+  FM_SYNC();
+  const fm_half4 v = fm_lds_tr4(tile + (l % 16) * 64 + 4 * (l / 16));
+#pragma unroll
+  for (int t = 0; t < 4; ++t) out[l * 4 + t] = float(v[t]);
+}
+

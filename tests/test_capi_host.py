@@ -112,6 +112,7 @@ def test_forward_backward_reject_bad_arguments_before_launching(lib):
     nd.sx = nd.sy = _capi.Strides(640, 64)
     assert lib.lib.fastmax_normalize(C.byref(nd), one, one, None, None) == 4   # max_norm needs stats scratch
     assert lib.lib.fastmax_probe_mfma(None, None, None) == 1
+    assert lib.lib.fastmax_probe_lds_transpose(None, None) == 1
     assert lib.lib.fastmax_version() >= 101
 
 

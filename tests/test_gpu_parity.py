@@ -32,6 +32,17 @@ def test_mfma_lane_layout(lib):
     assert torch.equal(a32.cpu(), want)
 
 
+def test_lds_transpose_read_layout(lib):
+    """The kernels (and the host simulator) assume: inside each group of 16 lanes, lane i receives
+    element i % 4 of the four-value words addressed by lanes i/4, 4 + i/4, 8 + i/4, 12 + i/4."""
+    got = lib.probe_lds_transpose(DEV)
+    torch.cuda.synchronize()
+    lane = torch.arange(64).view(64, 1)
+    t = torch.arange(4).view(1, 4)
+    want = (64 * (4 * t + (lane % 16) // 4) + 4 * (lane // 16) + lane % 4).float()
+    assert torch.equal(got.cpu(), want)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("mask", [False, True])
 @pytest.mark.parametrize("p", [1, 2])

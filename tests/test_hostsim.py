@@ -42,6 +42,13 @@ def test_probe_matches_assumed_layout(sim):
     assert torch.equal(a16, want) and torch.equal(a32, want)
 
 
+def test_lds_transpose_read_matches_assumed_layout(sim):
+    got = sim.probe_lds_transpose("cpu")
+    lane = torch.arange(64).view(64, 1)
+    t = torch.arange(4).view(1, 4)
+    assert torch.equal(got, (64 * (4 * t + (lane % 16) // 4) + 4 * (lane // 16) + lane % 4).float())
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_dense_forward_backward(sim, dtype):
     check_forward_backward(sim, 1, 70, 32, dtype, "cpu", mask=True, p=2, flags=_capi.FLAG_FORCE_DENSE, seed=1)
