@@ -143,8 +143,8 @@ def main() -> int:
     ap.add_argument("--cpu-max-n", type=int, default=2048, help="longest slice the CPU baseline materialises")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build measures one GPU only (every (b,h) slice is independent; "
-              "see DESIGN.md for how the path would shard); run with --gpus 1", file=sys.stderr)
+        print("bench.py: this build measures one GPU only (every (b,h) slice is independent, so the path "
+              "would shard over batch*heads without communication); run with --gpus 1", file=sys.stderr)
         return 2
 
     import torch

@@ -179,9 +179,9 @@ class Transformer(nn.Module):
 
 
 def vit_for_c4(**overrides):
-    """The image-classification configuration of the reference's lightning script scaled as the
-    survey's C4: 28x28 one-channel images, 4x4 patches (49 tokens + class token), d_model 128,
-    4 layers, 4 heads of 32, 10 classes."""
+    """The image-classification configuration of the reference's lightning script at MNIST scale:
+    28x28 one-channel images, 4x4 patches (49 tokens + class token), d_model 128, 4 layers,
+    4 heads of 32, 10 classes."""
     cfg = dict(out_dim=10, max_tokens=49, d_model=128, d_mlp=512, heads_per_block=4, num_blocks=4, use_masking=False,
                embedding="patch_conv", classifier="cls_token", patch_shape=(4, 4), patch_channels=1, normalize=True, p=2)
     cfg.update(overrides)
@@ -189,8 +189,8 @@ def vit_for_c4(**overrides):
 
 
 def gpt_for_c5(**overrides):
-    """Decoder-only language model of the survey's C5: 6 layers, d_model 512, 8 heads of 64,
-    context 1024, GPT-2 vocabulary size."""
+    """Decoder-only language model: 6 layers, d_model 512, 8 heads of 64, context 1024, GPT-2
+    vocabulary size."""
     cfg = dict(out_dim=50257, max_tokens=1024, d_model=512, d_mlp=2048, heads_per_block=8, num_blocks=6,
                use_masking=True, embedding="discrete_set", classifier="per_token", vocab_size=50257, normalize=True, p=2)
     cfg.update(overrides)
