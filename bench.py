@@ -246,6 +246,29 @@ def main() -> int:
                    "chunk": args.chunk or "auto", "launch": "hip graph replay" if args.graph else "eager"},
         "roofline": roofline,
     }
+    # the bandwidth-bound helpers of the path on the same tensors: event-timed passes against the HBM peak
+    esz = 2 if args.dtype == "bf16" else 4
+    tensor = bh * N * D * esz
+    helpers = {}
+    for name, fn, nbytes in (
+            # forward: one statistics read, one apply read, one write; backward: x and dy twice, dx once
+            ("normalize", lambda: lib.normalize(q, centre=0, max_norm=True, scale=1.0), 3 * tensor),
+            ("normalize_backward", lambda: lib.normalize_backward(q, go, centre=0, max_norm=True, scale=1.0), 5 * tensor)):
+        fn()
+        torch.cuda.synchronize()
+        lib.profile_begin()
+        for _ in range(5):
+            fn()
+        ms = sum(t for nme, t in lib.profile_end() if nme == "normalize") / 5
+        helpers[name] = {"ms": ms, "bytes": nbytes, "achieved_GBps": nbytes / (ms * 1e-3) / 1e9,
+                         "frac_of_8TBps": nbytes / (ms * 1e-3) / 8e12}
+    if "transpose" in roofline["kernels_ms_per_step"]:
+        t_ms = roofline["kernels_ms_per_step"]["transpose"]
+        ncopies = 2 if (args.dtype == "bf16" and "build" not in per_kernel) else 4    # row-major (+ transposed) copies of k and v
+        nbytes = 2 * tensor + ncopies * bh * N * D * esz
+        helpers["transpose"] = {"ms": t_ms, "bytes": nbytes, "achieved_GBps": nbytes / (t_ms * 1e-3) / 1e9,
+                                "frac_of_8TBps": nbytes / (t_ms * 1e-3) / 8e12}
+    out["hbm_bound_helpers"] = helpers
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
