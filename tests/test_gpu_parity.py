@@ -228,3 +228,31 @@ def test_step_replays_as_a_hip_graph(lib):
         for a, b in zip(got, want):
             assert torch.equal(a, b), f"replay {rep} differs from the eager call"
 
+
+def _random_cases(count, seed):
+    import random
+    rng = random.Random(seed)
+    cases = []
+    for _ in range(count):
+        d = rng.choice((32, 64))
+        mask = rng.random() < 0.6
+        nq = rng.choice((1, 2, 31, 33, 64, 127, 129, 255, 257, 300, 511, 640, 777, 1025, 1500))
+        if mask:
+            nk = nq if rng.random() < 0.7 else nq + rng.choice((1, 17, 128, 300))
+        else:
+            nk = rng.choice((5, 64, 130, 257, 900))     # one key makes dq = dk = 0 exactly: nothing to compare rounding noise with
+        cases.append(dict(bh=rng.choice((1, 2, 3, 5)), nq=nq, nk=nk, d=d, mask=mask, p=rng.choice((1, 2)),
+                          chunk=rng.choice((0, 0, 256)), dtype=rng.choice((torch.float32, torch.bfloat16)),
+                          saved=mask and nk == nq and rng.random() < 0.5, seed=rng.randrange(1 << 20)))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_cases(48, 2024), ids=lambda c: "-".join(
+    f"{k}{v}" for k, v in c.items() if k not in ("seed", "dtype")) + ("-bf16" if c["dtype"] == torch.bfloat16 else "-f32"))
+def test_seeded_random_shapes(lib, case):
+    """Forward and backward against the oracle on a fixed list of odd shapes (ragged lengths around
+    the 32 / 64 / 128 / 256 tile sizes, cross attention, cached keys, both orders, segments)."""
+    print(f"case random {case}", flush=True)
+    check_forward_backward(lib, case["bh"], case["nq"], case["d"], case["dtype"], DEV, mask=case["mask"], p=case["p"],
+                           nk=case["nk"], chunk=case["chunk"], seed=case["seed"], saved=case["saved"])
+
