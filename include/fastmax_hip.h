@@ -113,7 +113,10 @@ int fastmax_backward_saved(const FastmaxDesc* desc, const void* q, const void* k
  * centre: 0 none; 1 mean over the feature axis (fastattention_einops.py:327-334);
  *         2 mean over the token axis (score_function.py:42-47).
  * x and y may be the same buffer with the same strides.
- * stats: device pointer to bh*(d+2) floats of scratch, or null when max_norm == 0 and centre != 2. */
+ * stats: device scratch of fastmax_normalize_stats_bytes(desc) bytes (8-byte aligned), or null
+ * when max_norm == 0 and centre != 2.  Every workgroup leaves its partial maximum / column sums
+ * there and the next kernel joins them in a fixed order: no atomics, no clearing beforehand, the
+ * same bits on every run. */
 typedef struct FastmaxNormDesc {
   int32_t bh, n, d;
   int32_t dtype;
@@ -122,6 +125,7 @@ typedef struct FastmaxNormDesc {
   float scale;
   FastmaxStrides sx, sy;
 } FastmaxNormDesc;
+size_t fastmax_normalize_stats_bytes(const FastmaxNormDesc* desc);
 int fastmax_normalize(const FastmaxNormDesc* desc, const void* x, void* y, float* stats,
                       void* hip_stream);
 

@@ -51,7 +51,7 @@ class NormDesc(C.Structure):
 
 EXPORTS = (
     "fastmax_workspace_bytes", "fastmax_forward", "fastmax_backward", "fastmax_backward_saved", "fastmax_normalize",
-    "fastmax_normalize_backward", "fastmax_normalize_backward_stats_bytes",
+    "fastmax_normalize_stats_bytes", "fastmax_normalize_backward", "fastmax_normalize_backward_stats_bytes",
     "fastmax_status_string", "fastmax_version", "fastmax_probe_mfma", "fastmax_probe_lds_transpose",
     "fastmax_profile_begin", "fastmax_profile_end",
 )
@@ -117,6 +117,8 @@ class FastmaxLib:
         L.fastmax_backward_saved.restype = C.c_int
         L.fastmax_normalize.argtypes = [C.POINTER(NormDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         L.fastmax_normalize.restype = C.c_int
+        L.fastmax_normalize_stats_bytes.argtypes = [C.POINTER(NormDesc)]
+        L.fastmax_normalize_stats_bytes.restype = C.c_size_t
         L.fastmax_normalize_backward.argtypes = [C.POINTER(NormDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                                  C.c_void_p]
         L.fastmax_normalize_backward.restype = C.c_int
@@ -239,7 +241,8 @@ class FastmaxLib:
         if out is None:
             out = torch.empty(tuple(x.shape), dtype=x.dtype, device=x.device)
         nd.sx, nd.sy = _strides(x), _strides(out)
-        stats = torch.empty(nd.bh * (nd.d + 2), dtype=torch.float32, device=x.device)
+        nbytes = self.lib.fastmax_normalize_stats_bytes(C.byref(nd))
+        stats = torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device=x.device)
         st = self.lib.fastmax_normalize(C.byref(nd), x.data_ptr(), out.data_ptr(), stats.data_ptr(), self._stream(x))
         self.check(st, "fastmax_normalize")
         return out

@@ -404,7 +404,7 @@ int add_rows(const FastmaxDesc* d, const SplitPlan& sp, const void* dqa, void* d
 
 extern "C" {
 
-int fastmax_version(void) { return 103; }
+int fastmax_version(void) { return 104; }
 
 const char* fastmax_status_string(int status) {
   switch (status) {
@@ -570,6 +570,11 @@ int fastmax_backward_saved(const FastmaxDesc* desc, const void* q, const void* k
                        workspace_bytes, hip_stream);
 }
 
+size_t fastmax_normalize_stats_bytes(const FastmaxNormDesc* desc) {
+  if (!desc || desc->bh <= 0 || desc->n <= 0 || desc->d <= 0) return 0;
+  return size_t(desc->bh) * size_t(fm_norm_stride(desc->d, desc->n, desc->centre)) * sizeof(float);
+}
+
 int fastmax_normalize(const FastmaxNormDesc* desc, const void* x, void* y, float* stats, void* hip_stream) {
   ProfScope prof(FM_K_NORM, static_cast<fm_stream_t>(hip_stream));   // the whole pass (its kernels together)
   return fm_normalize_dispatch(desc, x, y, stats, static_cast<fm_stream_t>(hip_stream));
@@ -577,7 +582,7 @@ int fastmax_normalize(const FastmaxNormDesc* desc, const void* x, void* y, float
 
 size_t fastmax_normalize_backward_stats_bytes(const FastmaxNormDesc* desc) {
   if (!desc || desc->bh <= 0 || desc->n <= 0 || desc->d <= 0) return 0;
-  return size_t(desc->bh) * size_t(fm_normb_stride(desc->d, desc->n)) * sizeof(float);
+  return size_t(desc->bh) * size_t(fm_normb_stride(desc->d, desc->n, desc->centre)) * sizeof(float);
 }
 
 int fastmax_normalize_backward(const FastmaxNormDesc* desc, const void* x, const void* dy, void* dx, float* stats,

@@ -49,7 +49,8 @@ void scale_or_normalize(torch::Tensor& x, int64_t bh, int64_t n, int64_t d, bool
   nd.bh = static_cast<int32_t>(bh); nd.n = static_cast<int32_t>(n); nd.d = static_cast<int32_t>(d);
   nd.dtype = dtype_code(x); nd.centre = 0; nd.max_norm = max_norm ? 1 : 0; nd.scale = scale;
   nd.sx = legacy_strides(bh, d); nd.sy = nd.sx;
-  torch::Tensor stats = torch::empty({bh * (d + 2)}, x.options().dtype(torch::kFloat32));
+  torch::Tensor stats = torch::empty({int64_t(fastmax_normalize_stats_bytes(&nd) / sizeof(float))},
+                                     x.options().dtype(torch::kFloat32));
   check_status(fastmax_normalize(&nd, x.data_ptr(), x.data_ptr(), stats.data_ptr<float>(), stream_of(x)),
                "fastmax_normalize");
 }
@@ -311,7 +312,8 @@ torch::Tensor normalize(torch::Tensor x_, int64_t centre, bool max_norm, double 
   nd.scale = float(scale);
   torch::Tensor y = empty_like_layout(x.t, x.n, x.t.scalar_type());
   nd.sx = x.s; nd.sy = view_of(y, "y").s;
-  torch::Tensor stats = torch::empty({int64_t(nd.bh) * (nd.d + 2)}, x.t.options().dtype(torch::kFloat32));
+  torch::Tensor stats = torch::empty({int64_t(fastmax_normalize_stats_bytes(&nd) / sizeof(float))},
+                                     x.t.options().dtype(torch::kFloat32));
   check_status(fastmax_normalize(&nd, x.t.data_ptr(), y.data_ptr(), stats.data_ptr<float>(), stream_of(x.t)),
                "fastmax_normalize");
   return y;

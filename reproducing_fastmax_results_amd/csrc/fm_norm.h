@@ -4,61 +4,25 @@
 // centre: 0 none (transformer/model.py:97-102), 1 feature mean
 // (fastattention_einops.py:327-334), 2 token mean (score_function.py:42-47).
 // Replaces apply_rpe_and_temp / calc_norms / find_max / apply_norm
-// (fastmax_cuda_forward.cu:282-338).  Reductions use no floating-point atomics:
-// the maximum is taken with an integer atomicMax on the bit pattern of a
-// non-negative float, which is order independent.
+// (fastmax_cuda_forward.cu:282-338).  Reductions use no atomics at all: every workgroup leaves
+// its partial result (largest squared norm, column sums) in the scratch buffer and the consumers add
+// or compare the partials in a fixed order, so the result is the same bit pattern on every run.
 #pragma once
 #include "fastmax_hip.h"
 #include "fm_kernels.h"
 
-// stats layout per batch*head: [0] max squared norm (as float bits), [1] unused, [2..2+d) token mean
-template <int DH> struct NormStats { static constexpr int N = DH + 2; };
+// Token blocks of 64 (four threads per token) per workgroup in the kernels below: the loads of all
+// its blocks are issued before the first is used, so a thread has NP * DH / 32 16-byte loads in flight.
+static constexpr int FM_NORM_NP = 4;     // forward kernels and the backward's second pass
+static constexpr int FM_NORMB_NP = 2;    // backward statistics (two tensors per token)
 
-template <int DH>
-FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_clear(float* stats) {
-  const int i = FM_BID_X * 256 + FM_TID_X;
-  if (FM_TID_X < NormStats<DH>::N) stats[FM_BID_X * NormStats<DH>::N + FM_TID_X] = 0.f;
-  (void)i;
-}
-
-// token mean per feature: one workgroup per (8 features, batch*head), 16-byte loads, a fixed
-// reduction tree (the same sum order on every run).  grid (DH / 8, bh).
-template <typename TIO, int DH>
-FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_colmean(TRef<const TIO> x, int n, float* FM_RESTRICT out, int64_t out_stride) {
-  FM_SHARED float part[8 * 256];
-  const int tid = FM_TID_X, d0 = FM_BID_X * 8, bh = FM_BID_Y;
-  float s[8];
-#pragma unroll
-  for (int j = 0; j < 8; ++j) s[j] = 0.f;
-  // eight rows in flight per thread (one row per trip left the kernel waiting on memory latency)
-  for (int t = tid; t < n; t += 256 * 8) {
-    float v[8][8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int tt = t + 256 * u;
-      if (tt < n) {
-        IO<TIO>::ld8(x.base(bh) + int64_t(tt) * x.s_n + d0, x.vec != 0, v[u]);
-      } else {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) v[u][j] = 0.f;
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < 8; ++u)
-#pragma unroll
-      for (int j = 0; j < 8; ++j) s[j] += v[u][j];
-  }
-#pragma unroll
-  for (int j = 0; j < 8; ++j) part[j * 256 + tid] = s[j];
-  FM_SYNC();
-  for (int stride = 128; stride > 0; stride >>= 1) {
-    if (tid < stride) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) part[j * 256 + tid] += part[j * 256 + tid + stride];
-    }
-    FM_SYNC();
-  }
-  if (tid < 8) out[bh * out_stride + d0 + tid] = part[tid * 256] / float(n);   // out: DH means per batch*head
+// forward scratch per batch*head (floats): [0], [1] unused; [2 .. 2+d) token mean; then one largest
+// squared norm per workgroup of k_norm_maxnorm; then, with the token-mean centring, d column sums per
+// workgroup of k_norm_colsum
+inline int fm_norm_blocks(int n) { return (n + 64 * FM_NORM_NP - 1) / (64 * FM_NORM_NP); }
+inline int64_t fm_norm_stride(int dh, int n, int centre) {
+  const int64_t nb = fm_norm_blocks(n);
+  return (2 + int64_t(dh) + nb + (centre == 2 ? nb * dh : 0) + 1) / 2 * 2;
 }
 
 // A thread's quarter of one token row, and the centring of it (the feature mean needs the four
@@ -91,18 +55,76 @@ FM_DEVICE void fm_norm_load_centred(const TIO* row, bool vec, int d0, int centre
   fm_norm_centre<DH>(v, d0, centre, mean);
 }
 
-// Token blocks of 64 (four threads per token) per workgroup in the kernels below: the loads of all
-// its blocks are issued before the first is used, so a thread has NP * DH / 32 16-byte loads in flight.
-static constexpr int FM_NORM_NP = 4;     // forward kernels and the backward's second pass
-static constexpr int FM_NORMB_NP = 2;    // backward statistics (two tensors per token)
+// Column sums over the workgroup's 64 * FM_NORM_NP tokens -> out[bh][block][DH]; k_norm_colfinal adds the
+// blocks in a fixed order and divides.  grid (blocks, bh, tensors) and (bh, tensors).
+template <typename TIO, int DH>
+FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_colsum(TRef<const TIO> x0, TRef<const TIO> x1, int n, float* FM_RESTRICT out,
+                                                   int64_t out_stride) {
+  constexpr int EPT = DH / 4, NP = FM_NORM_NP;
+  FM_SHARED float part[64 * (DH + 1)];
+  const int tid = FM_TID_X, bh = FM_BID_Y;
+  const TRef<const TIO> x = FM_BID_Z ? x1 : x0;     // grid z: which tensor
+  out += int64_t(FM_BID_Z) * FM_GDIM_X * DH;
+  const int tok0 = FM_BID_X * 64 * NP + (tid >> 2), d0 = (tid & 3) * EPT;
+  float v[NP][EPT];
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    const int tok = tok0 + 64 * p;
+    if (tok < n) {
+      fm_norm_load<TIO, DH>(x.base(bh) + int64_t(tok) * x.s_n, x.vec != 0, d0, v[p]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < EPT; ++j) v[p][j] = 0.f;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) {
+    float a = 0.f;
+#pragma unroll
+    for (int p = 0; p < NP; ++p) a += v[p][j];
+    part[(tid >> 2) * (DH + 1) + d0 + j] = a;
+  }
+  FM_SYNC();
+  if (tid < DH) {
+    float a = 0.f;
+    for (int r = 0; r < 64; ++r) a += part[r * (DH + 1) + tid];
+    out[bh * out_stride + int64_t(FM_BID_X) * DH + tid] = a;
+  }
+}
+template <int DH>
+FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_colfinal(const float* FM_RESTRICT sums, int64_t sums_stride, int nblk, int n,
+                                                     float* FM_RESTRICT mean, int64_t mean_stride) {
+  constexpr int G = 256 / DH;                 // groups of DH threads, each takes every G-th block
+  FM_SHARED float part[256];
+  const int tid = FM_TID_X, bh = FM_BID_X, which = FM_BID_Y;     // which: tensor (sums and means of several lie side by side)
+  const int g = tid / DH, f = tid % DH;
+  sums += bh * sums_stride + int64_t(which) * nblk * DH;
+  float a = 0.f;
+  int b = g;
+  for (; b + 3 * G < nblk; b += 4 * G) {      // four loads in flight
+    const float v0 = sums[int64_t(b) * DH + f], v1 = sums[int64_t(b + G) * DH + f];
+    const float v2 = sums[int64_t(b + 2 * G) * DH + f], v3 = sums[int64_t(b + 3 * G) * DH + f];
+    a += v0; a += v1; a += v2; a += v3;
+  }
+  for (; b < nblk; b += G) a += sums[int64_t(b) * DH + f];
+  part[tid] = a;
+  FM_SYNC();
+  if (tid < DH) {
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < G; ++i) t += part[i * DH + tid];
+    mean[bh * mean_stride + which * DH + tid] = t / float(n);
+  }
+}
 
 // grid (ceil(n / (64 * FM_NORM_NP)), bh); four threads per token
 template <typename TIO, int DH>
-FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_maxnorm(TRef<const TIO> x, int n, int centre, float* FM_RESTRICT stats) {
+FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_maxnorm(TRef<const TIO> x, int n, int centre, float* FM_RESTRICT stats, int64_t stride) {
   constexpr int EPT = DH / 4, NP = FM_NORM_NP;
+  FM_SHARED float wmax[4];
   const int tid = FM_TID_X, bh = FM_BID_Y;
   const int tok0 = FM_BID_X * 64 * NP + (tid >> 2), d0 = (tid & 3) * EPT;
-  float* st = stats + bh * NormStats<DH>::N;
+  float* st = stats + bh * stride;
   float v[NP][EPT];
   // every lane takes part in the shuffles; rows past the end re-read the last row and count as zero
 #pragma unroll
@@ -123,25 +145,18 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_maxnorm(TRef<const TIO> x, int n, in
   }
 #pragma unroll
   for (int m = 4; m < 64; m <<= 1) mx = fm_fmaxf(mx, fm_shfl_xor(mx, m));
-  if ((tid & 63) == 0) {
-    uint32_t bits;
-    __builtin_memcpy(&bits, &mx, 4);
-#if defined(FM_HOSTSIM)
-    uint32_t* p = reinterpret_cast<uint32_t*>(st);
-    if (bits > *p) *p = bits;            // workgroups run one after another in the simulator
-#else
-    atomicMax(reinterpret_cast<unsigned int*>(st), bits);
-#endif
-  }
+  if ((tid & 63) == 0) wmax[tid >> 6] = mx;
+  FM_SYNC();
+  if (tid == 0) st[2 + DH + FM_BID_X] = fm_fmaxf(fm_fmaxf(wmax[0], wmax[1]), fm_fmaxf(wmax[2], wmax[3]));
 }
 
 template <typename TIO, int DH>
 FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_apply(TRef<const TIO> x, TRef<TIO> y, int n, int centre, int max_norm, float scale,
-                                                  const float* FM_RESTRICT stats) {
+                                                  const float* FM_RESTRICT stats, int64_t stride) {
   constexpr int EPT = DH / 4, NP = FM_NORM_NP;
   const int tid = FM_TID_X, bh = FM_BID_Y;
   const int tok0 = FM_BID_X * 64 * NP + (tid >> 2), d0 = (tid & 3) * EPT;
-  const float* st = stats ? stats + bh * NormStats<DH>::N : nullptr;
+  const float* st = stats ? stats + bh * stride : nullptr;
   float v[NP][EPT];
 #pragma unroll
   for (int p = 0; p < NP; ++p) {
@@ -149,7 +164,15 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_apply(TRef<const TIO> x, TRef<TIO> y
     fm_norm_load<TIO, DH>(x.base(bh) + int64_t(tk) * x.s_n, x.vec != 0, d0, v[p]);
   }
   float f = scale;
-  if (max_norm) f = scale / fm_sqrtf(st[0]);
+  if (max_norm) {
+    // the largest of the workgroups' maxima: every lane takes a share, a butterfly joins them
+    const int nblk = int(FM_GDIM_X);
+    float m2 = 0.f;
+    for (int b = tid & 63; b < nblk; b += 64) m2 = fm_fmaxf(m2, st[2 + DH + b]);
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) m2 = fm_fmaxf(m2, fm_shfl_xor(m2, m));
+    f = scale / fm_sqrtf(m2);
+  }
 #pragma unroll
   for (int p = 0; p < NP; ++p) {
     const int tok = tok0 + 64 * p;
@@ -168,16 +191,17 @@ int fm_normalize_run(const FastmaxNormDesc* d, const void* x, void* y, float* st
   const TRef<const TIO> xr = fm_ref<const TIO>(static_cast<const TIO*>(x), d->sx);
   const TRef<TIO> yr = fm_ref<TIO>(static_cast<TIO*>(y), d->sy);
   const fm_dim3 grid((d->n + 64 * FM_NORM_NP - 1) / (64 * FM_NORM_NP), d->bh);
-  if (d->max_norm || d->centre == 2) {
-    FM_KERNEL_LAUNCH((k_norm_clear<DH>), fm_dim3(d->bh), fm_dim3(256), 0, stream, stats);
-    if (d->centre == 2)
-      FM_KERNEL_LAUNCH((k_norm_colmean<TIO, DH>), fm_dim3(DH / 8, d->bh), fm_dim3(256), 0, stream, xr, d->n, stats + 2,
-                       int64_t(NormStats<DH>::N));
-    if (d->max_norm)
-      FM_KERNEL_LAUNCH((k_norm_maxnorm<TIO, DH>), grid, fm_dim3(256), 0, stream, xr, d->n, d->centre, stats);
+  const int64_t stride = fm_norm_stride(DH, d->n, d->centre);
+  if (d->centre == 2) {
+    float* sums = stats + 2 + DH + grid.x;
+    FM_KERNEL_LAUNCH((k_norm_colsum<TIO, DH>), grid, fm_dim3(256), 0, stream, xr, xr, d->n, sums, stride);
+    FM_KERNEL_LAUNCH((k_norm_colfinal<DH>), fm_dim3(d->bh), fm_dim3(256), 0, stream, sums, stride, int(grid.x), d->n, stats + 2,
+                     stride);
   }
+  if (d->max_norm)
+    FM_KERNEL_LAUNCH((k_norm_maxnorm<TIO, DH>), grid, fm_dim3(256), 0, stream, xr, d->n, d->centre, stats, stride);
   FM_KERNEL_LAUNCH((k_norm_apply<TIO, DH>), grid, fm_dim3(256), 0, stream, xr, yr, d->n, d->centre, d->max_norm,
-                   d->scale, stats);
+                   d->scale, stats, stride);
 #if defined(FM_HOSTSIM)
   return FASTMAX_OK;
 #else
@@ -207,16 +231,20 @@ inline int fm_normalize_dispatch(const FastmaxNormDesc* d, const void* x, void* 
 // (fastmax_cuda_backward.cu returns the gradients with respect to the normalised tensors); its
 // Python variants carry it through autograd (score_function.py:40-55, fastattention_einops.py:327-334).
 //
-// stats per batch*head, fm_normb_stride(d, n) floats: [0..1] one 64-bit word, the bit pattern of the
-// largest squared norm in the high half and ~token in the low half (an integer atomicMax finds
-// the largest norm and, among equal ones, the first token); [2], [3] unused; [4 .. 4+d) token mean
-// of x; [4+d .. 4+2d) token mean of dy; then one partial sum of dy * c per 64-token block, added
-// in a fixed order by every workgroup of the second kernel (no floating-point atomics).
+// stats per batch*head, fm_normb_stride(d, n, centre) floats: [0 .. 4) unused; [4 .. 4+d) token mean of x;
+// [4+d .. 4+2d) token mean of dy; one partial sum of dy * c per 64-token block; one 64-bit key per
+// workgroup of the statistics kernel (the bit pattern of its largest squared norm in the high half and
+// ~token in the low half, so that an integer maximum finds the largest norm and, among equal ones, the
+// first token); with the token-mean centring, the column sums of x and of dy per workgroup of
+// k_norm_colsum.  Every workgroup of the second kernel joins the partials in the same fixed order:
+// no atomics, nothing to clear, the same bits on every run.
 // ------------------------------------------------------------------------------
-inline int64_t fm_normb_stride(int dh, int n) { return 4 + 2 * int64_t(dh) + ((n + 63) / 64 + 1) / 2 * 2; }
-
-FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_normb_clear(float* stats, int64_t stride) {
-  if (FM_TID_X < 4) stats[FM_BID_X * stride + FM_TID_X] = 0.f;
+FM_HOST_DEVICE inline int fm_normb_blocks(int n) { return (n + 64 * FM_NORMB_NP - 1) / (64 * FM_NORMB_NP); }
+FM_HOST_DEVICE inline int64_t fm_normb_keys(int dh, int n) { return 4 + 2 * int64_t(dh) + ((n + 63) / 64 + 1) / 2 * 2; }
+inline int64_t fm_normb_base(int dh, int n) { return fm_normb_keys(dh, n) + 2 * int64_t(fm_normb_blocks(n)); }
+// with the token-mean centring the column sums of x and of dy per workgroup of k_norm_colsum follow
+inline int64_t fm_normb_stride(int dh, int n, int centre) {
+  return fm_normb_base(dh, n) + (centre == 2 ? 2 * int64_t(fm_norm_blocks(n)) * dh : 0);
 }
 
 // grid (ceil(n / (64 * FM_NORMB_NP)), bh); four threads per token
@@ -225,6 +253,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_normb_stats(TRef<const TIO> x, TRef<const
                                                    float* FM_RESTRICT stats, int64_t stride) {
   constexpr int EPT = DH / 4, NP = FM_NORMB_NP;
   FM_SHARED float wsum[NP][4];
+  FM_SHARED unsigned long long wkey[4];
   const int tid = FM_TID_X, bh = FM_BID_Y;
   const int tok0 = FM_BID_X * 64 * NP + (tid >> 2), d0 = (tid & 3) * EPT;
   float* st = stats + bh * stride;
@@ -259,20 +288,22 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_normb_stats(TRef<const TIO> x, TRef<const
   int wc = (mx == wmx && mx >= 0.f) ? cand : 0x7fffffff;
 #pragma unroll
   for (int m = 4; m < 64; m <<= 1) { const int o = fm_shfl_xor_i(wc, m); wc = o < wc ? o : wc; }
-  if ((tid & 63) == 0 && max_norm && wc != 0x7fffffff) {
-    uint32_t bits;
-    __builtin_memcpy(&bits, &wmx, 4);
-    const unsigned long long key = (static_cast<unsigned long long>(bits) << 32) | uint32_t(~uint32_t(wc));
-    unsigned long long* p = reinterpret_cast<unsigned long long*>(st);
-#if defined(FM_HOSTSIM)
-    if (key > *p) *p = key;              // workgroups run one after another in the simulator
-#else
-    atomicMax(p, key);
-#endif
+  if ((tid & 63) == 0) {
+    unsigned long long key = 0;          // no token of this wavefront has a norm that compares (all NaN)
+    if (wc != 0x7fffffff) {
+      uint32_t bits;
+      __builtin_memcpy(&bits, &wmx, 4);
+      key = (static_cast<unsigned long long>(bits) << 32) | uint32_t(~uint32_t(wc));
+    }
+    wkey[tid >> 6] = key;
   }
   FM_SYNC();
   if (tid < NP && (FM_BID_X * NP + tid) * 64 < n)
     st[4 + 2 * DH + FM_BID_X * NP + tid] = (wsum[tid][0] + wsum[tid][1]) + (wsum[tid][2] + wsum[tid][3]);
+  if (tid == 64) {
+    const unsigned long long a = wkey[0] > wkey[1] ? wkey[0] : wkey[1], b = wkey[2] > wkey[3] ? wkey[2] : wkey[3];
+    reinterpret_cast<unsigned long long*>(st + fm_normb_keys(DH, n))[FM_BID_X] = a > b ? a : b;
+  }
 }
 
 // grid (ceil(n / (64 * FM_NORM_NP)), bh); four threads per token
@@ -281,6 +312,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_normb_apply(TRef<const TIO> x, TRef<const
                                                    int max_norm, float scale, const float* FM_RESTRICT stats, int64_t stride) {
   constexpr int EPT = DH / 4, NP = FM_NORM_NP;
   FM_SHARED float red[256];
+  FM_SHARED unsigned long long redk[256];
   const int tid = FM_TID_X, bh = FM_BID_Y;
   const int tok0 = FM_BID_X * 64 * NP + (tid >> 2), d0 = (tid & 3) * EPT;
   const float* st = stats ? stats + bh * stride : nullptr;
@@ -298,12 +330,21 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_normb_apply(TRef<const TIO> x, TRef<const
     float s = 0.f;
     for (int i = tid; i < nblk; i += 256) s += st[4 + 2 * DH + i];
     red[tid] = s;
+    // the largest key of the statistics kernel's workgroups: largest norm, first token among equal ones
+    const unsigned long long* keys = reinterpret_cast<const unsigned long long*>(st + fm_normb_keys(DH, n));
+    const int nkeys = fm_normb_blocks(n);
+    unsigned long long kmax = 0;
+    for (int i = tid; i < nkeys; i += 256) { const unsigned long long k = keys[i]; kmax = k > kmax ? k : kmax; }
+    redk[tid] = kmax;
     FM_SYNC();
     for (int w = 128; w > 0; w >>= 1) {
-      if (tid < w) red[tid] += red[tid + w];
+      if (tid < w) {
+        red[tid] += red[tid + w];
+        redk[tid] = redk[tid + w] > redk[tid] ? redk[tid + w] : redk[tid];
+      }
       FM_SYNC();
     }
-    const unsigned long long key = *reinterpret_cast<const unsigned long long*>(st);
+    const unsigned long long key = redk[0];
     const uint32_t bits = uint32_t(key >> 32);
     float m2;
     __builtin_memcpy(&m2, &bits, 4);
@@ -339,13 +380,14 @@ int fm_normalize_bwd_run(const FastmaxNormDesc* d, const void* x, const void* dy
   const TRef<TIO> dxr = fm_ref<TIO>(static_cast<TIO*>(dx), d->sx);
   const fm_dim3 grid_stats((d->n + 64 * FM_NORMB_NP - 1) / (64 * FM_NORMB_NP), d->bh);
   const fm_dim3 grid((d->n + 64 * FM_NORM_NP - 1) / (64 * FM_NORM_NP), d->bh);
-  const int64_t stride = fm_normb_stride(DH, d->n);
+  const int64_t stride = fm_normb_stride(DH, d->n, d->centre);
   if (d->max_norm || d->centre == 2) {
-    FM_KERNEL_LAUNCH(k_normb_clear, fm_dim3(d->bh), fm_dim3(64), 0, stream, stats, stride);
     if (d->centre == 2) {
-      FM_KERNEL_LAUNCH((k_norm_colmean<TIO, DH>), fm_dim3(DH / 8, d->bh), fm_dim3(256), 0, stream, xr, d->n, stats + 4, stride);
-      FM_KERNEL_LAUNCH((k_norm_colmean<TIO, DH>), fm_dim3(DH / 8, d->bh), fm_dim3(256), 0, stream, gr, d->n, stats + 4 + DH,
-                       stride);
+      // the means of x and of dy lie side by side: one launch of the last step covers both
+      float* sums = stats + fm_normb_base(DH, d->n);
+      FM_KERNEL_LAUNCH((k_norm_colsum<TIO, DH>), fm_dim3(grid.x, grid.y, 2), fm_dim3(256), 0, stream, xr, gr, d->n, sums, stride);
+      FM_KERNEL_LAUNCH((k_norm_colfinal<DH>), fm_dim3(d->bh, 2), fm_dim3(256), 0, stream, sums, stride, int(grid.x), d->n,
+                       stats + 4, stride);
     }
     if (d->max_norm)
       FM_KERNEL_LAUNCH((k_normb_stats<TIO, DH>), grid_stats, fm_dim3(256), 0, stream, xr, gr, d->n, d->centre, d->max_norm, stats,

@@ -113,15 +113,24 @@ def test_forward_backward_reject_bad_arguments_before_launching(lib):
     assert lib.lib.fastmax_normalize(C.byref(nd), one, one, None, None) == 4   # max_norm needs stats scratch
     assert lib.lib.fastmax_probe_mfma(None, None, None) == 1
     assert lib.lib.fastmax_probe_lds_transpose(None, None) == 1
-    assert lib.lib.fastmax_version() >= 101
+    assert lib.lib.fastmax_version() >= 104
 
 
 def test_normalize_backward_arguments(lib):
     nd = _capi.NormDesc()
     nd.bh, nd.n, nd.d, nd.dtype, nd.centre, nd.max_norm, nd.scale = 4, 130, 64, _capi.F32, 2, 1, 1.0
     nd.sx = nd.sy = _capi.Strides(130 * 64, 64)
-    # per batch*head: 4 header floats, the token means of x and dy, one partial sum per 64 tokens (even count)
-    assert lib.lib.fastmax_normalize_backward_stats_bytes(C.byref(nd)) == 4 * 4 * (4 + 2 * 64 + 4)
+    # per batch*head: 4 header floats, the token means of x and dy, one partial sum per 64 tokens (even count),
+    # one 8-byte key per 128 tokens, and with the token-mean centring the column sums of x and dy per 256 tokens
+    assert lib.lib.fastmax_normalize_backward_stats_bytes(C.byref(nd)) == 4 * 4 * (4 + 2 * 64 + 4 + 2 * 2 + 2 * 64)
+    nd.centre = 0
+    assert lib.lib.fastmax_normalize_backward_stats_bytes(C.byref(nd)) == 4 * 4 * (4 + 2 * 64 + 4 + 2 * 2)
+    # forward: 2 header floats, the token mean, one maximum per 256 tokens (+ column sums per 256 tokens), even count
+    assert lib.lib.fastmax_normalize_stats_bytes(C.byref(nd)) == 4 * 4 * (2 + 64 + 1 + 1)
+    nd.centre, nd.n = 2, 600
+    assert lib.lib.fastmax_normalize_stats_bytes(C.byref(nd)) == 4 * 4 * (2 + 64 + 3 + 3 * 64 + 1)
+    assert lib.lib.fastmax_normalize_stats_bytes(None) == 0
+    nd.n = 130
     assert lib.lib.fastmax_normalize_backward_stats_bytes(None) == 0
     one = C.c_void_p(256)     # never dereferenced: validation fails first
     assert lib.lib.fastmax_normalize_backward(C.byref(nd), None, one, one, one, None) == 1

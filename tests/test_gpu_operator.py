@@ -199,6 +199,25 @@ def test_normalize_backward_kernel(ext, centre, dtype, shape):
     assert rel_err(dx0, want) < (1e-5 if dtype == torch.float32 else 1e-2)
 
 
+def test_normalize_backward_equal_norms_and_repeat(ext):
+    """Two tokens share the largest norm, in different workgroups: the gradient's one-token term goes
+    to the first of them (the rule the header states), and two runs give the same bits."""
+    n, d = 1000, 64
+    x, dy = rnd(2, n, d, seed=44), rnd(2, n, d, seed=45)
+    x[:, 700] = 50.0 * x[:, 700] / x[:, 700].norm(dim=-1, keepdim=True)
+    x[:, 130] = x[:, 700]
+    dx = ext.normalize_backward(x.to(DEV), dy.to(DEV), 0, True, 1.0)
+    again = ext.normalize_backward(x.to(DEV), dy.to(DEV), 0, True, 1.0)
+    assert torch.equal(dx, again)
+    xd, dyd = x.double(), dy.double()
+    m = xd.norm(dim=-1).amax(-1)                                    # (bh,)
+    plain = dyd / m[:, None, None]                                  # every token but the first largest one
+    assert rel_err(dx[:, 700], plain[:, 700]) < 1e-5
+    spike = (dx.cpu().double() - plain)[:, 130]
+    want = -((dyd * xd).sum((-1, -2)) / m ** 3)[:, None] * xd[:, 130]
+    assert rel_err(spike, want) < 1e-4
+
+
 def test_normalize_backward_on_projection_layout(ext):
     """x and dy as the (b, h, n, d) views of (b, n, h*d) projections: no copies, dx in x's layout."""
     b, h, n, d = 2, 4, 130, 64

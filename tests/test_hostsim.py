@@ -92,6 +92,12 @@ def test_normalize(sim):
         assert O.rel_l2(y, ref) < 1e-6
     y = sim.normalize(x, centre=0, max_norm=False, scale=0.25)
     assert torch.allclose(y, 0.25 * x)
+    # several workgroups per batch*head: their partial maxima and column sums are joined by the last kernel
+    x = torch.randn(3, 600, 64, generator=torch.Generator().manual_seed(7))
+    x[1, 555] *= 3.0
+    for centre, ref in ((0, O.normalize_lim(x.double(), 0.5)), (2, 0.5 * O.normalize_token_mean(x.double(), x.double())[0])):
+        assert O.rel_l2(sim.normalize(x, centre=centre, max_norm=True, scale=0.5), ref) < 1e-6
+    assert O.rel_l2(sim.normalize(x, centre=2, max_norm=False, scale=2.0), 2.0 * (x - x.mean(1, keepdim=True)).double()) < 1e-6
 
 
 def test_normalize_backward(sim):
@@ -105,6 +111,10 @@ def test_normalize_backward(sim):
         fn(xd).backward(dy.double())
         dx = sim.normalize_backward(x, dy, centre=centre, max_norm=True, scale=1.5)
         assert O.rel_l2(dx, xd.grad) < 1e-5
+    x, dy = torch.randn(2, 600, 64, generator=g), torch.randn(2, 600, 64, generator=g)
+    xd = x.double().requires_grad_(True)
+    (1.5 * O.normalize_token_mean(xd, xd)[0]).backward(dy.double())
+    assert O.rel_l2(sim.normalize_backward(x, dy, centre=2, max_norm=True, scale=1.5), xd.grad) < 1e-5
 
 
 def test_causal_with_more_keys_than_queries(sim):
