@@ -399,14 +399,35 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <
     sm_b[s] = pb >= 0 ? pb + lr * PT + lh * M::KPL : -1;
   }
 
-  // the steps of the walk this workgroup takes: all of them in turn, or the one its grid z names
+  // the steps of the walk this workgroup takes: all of them in turn, or the one its grid z names.
+  // Two cursors run along the walk: `cur` names the token tile being summed, `pf` the tile whose
+  // loads are issued next, two tiles ahead (with one tile of lookahead the walk ran at the latency
+  // of the memory system: a tile's products take a fraction of a microsecond).
   const int w_end = A.seg_parallel ? FM_BID_Z + 1 : nsteps;
-  int w = A.seg_parallel ? FM_BID_Z : 0, tb, te, slot;
-  fm_walk_step(A.mode, A.nseg, A.L, A.npad, w, tb, te, slot);
-  int t = tb;
+  struct Cursor { int t, w, tb, te, slot; bool valid; };
+  auto advance = [&](Cursor& c) {
+    c.t += TT;
+    if (c.t >= c.te) {
+      c.w += 1;
+      if (c.w < w_end) { fm_walk_step(A.mode, A.nseg, A.L, A.npad, c.w, c.tb, c.te, c.slot); c.t = c.tb; }
+      else c.valid = false;
+    }
+  };
+  Cursor cur;
+  cur.w = A.seg_parallel ? FM_BID_Z : 0;
+  cur.valid = true;
+  fm_walk_step(A.mode, A.nseg, A.L, A.npad, cur.w, cur.tb, cur.te, cur.slot);
+  cur.t = cur.tb;
+  Cursor pf = cur;
   const int a0 = grp * AW;
-  TileRegs<E, DH, TT> rp, rr, rz;
-  TileRegs<E, AW, TT> rx;
+  struct Regs { TileRegs<E, DH, TT> p, r, z; TileRegs<E, AW, TT> x; };
+  Regs R0, R1;
+  auto fetch = [&](Regs& R, const Cursor& c) {
+    R.p.load(A.pt + tb_off + c.t, A.npad, tid);
+    R.r.load(A.rt + tb_off + c.t, A.npad, tid);
+    if (quad) R.x.load(A.xt + tb_off + int64_t(a0) * A.npad + c.t, A.npad, tid);
+    if (has_z) R.z.load(A.zt + tb_off + c.t, A.npad, tid);
+  };
   fm_f32x16 acc[NA][NT][NT];
   fm_f32x16 sacc[SPW];
 #pragma unroll
@@ -417,37 +438,23 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <
       for (int k = 0; k < NT; ++k) acc[i][j][k] = fm_zero16();
 #pragma unroll
   for (int s = 0; s < SPW; ++s) sacc[s] = fm_zero16();
-  rp.load(A.pt + tb_off + t, A.npad, tid);
-  rr.load(A.rt + tb_off + t, A.npad, tid);
-  if (quad) rx.load(A.xt + tb_off + int64_t(a0) * A.npad + t, A.npad, tid);
-  if (has_z) rz.load(A.zt + tb_off + t, A.npad, tid);
-  bool have = true;
-  while (have) {
+  fetch(R0, pf);
+  advance(pf);
+  if (pf.valid) { fetch(R1, pf); advance(pf); }
+  auto stage = [&](Regs& R) FM_ALWAYS_INLINE {
     FM_SYNC();
-    rp.store(s0, PT, tid); rr.store(s1, PT, tid);
-    if (quad) rx.store(s2, PT, tid);
-    if (has_z) rz.store(s3, PT, tid);
+    R.p.store(s0, PT, tid); R.r.store(s1, PT, tid);
+    if (quad) R.x.store(s2, PT, tid);
+    if (has_z) R.z.store(s3, PT, tid);
     FM_SYNC();
-
-    int nt = t + TT, nw = w, ntb = tb, nte = te, nslot = slot;
-    const bool last = (nt >= te);
-    bool has_next = true;
-    if (last) {
-      nw = w + 1;
-      if (nw < w_end) { fm_walk_step(A.mode, A.nseg, A.L, A.npad, nw, ntb, nte, nslot); nt = ntb; }
-      else has_next = false;
-    }
-    if (has_next) {
-      rp.load(A.pt + tb_off + nt, A.npad, tid);
-      rr.load(A.rt + tb_off + nt, A.npad, tid);
-      if (quad) rx.load(A.xt + tb_off + int64_t(a0) * A.npad + nt, A.npad, tid);
-      if (has_z) rz.load(A.zt + tb_off + nt, A.npad, tid);
-    }
+    if (pf.valid) { fetch(R, pf); advance(pf); }
+    const bool last = cur.t + TT >= cur.te;
+    const int slot = cur.slot;
     if (quad) {
       const E* pb_ = s0 + lr * PT + lh * M::KPL;
       const E* rb_ = s1 + lr * PT + lh * M::KPL;
       const E* xb_ = s2 + (wave * NA) * PT + lh * M::KPL;
-      if (NSTEP <= 4) {
+      if (sizeof(E) == 2) {
         // Few k-steps per tile (_Float16): the fragments of KB k-steps are requested from LDS
         // before their first product, so the wavefront waits for LDS NSTEP / KB times per tile
         // (with one k-step of lookahead the walk ran at the LDS latency, not at the MFMA rate).
@@ -520,6 +527,17 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <
       }
     }
     if (last) {
+#if !defined(FM_HOSTSIM)
+      // The accumulators live in the accumulation registers while the products run; without this the
+      // compiler copies all of them to vector registers at the end of every tile, ahead of this branch.
+#pragma unroll
+      for (int i = 0; i < NA; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+          for (int k = 0; k < NT; ++k)
+            if (sizeof(E) == 2 && KB >= 4) asm volatile("" : "+a"(acc[i][j][k]));    // the one-workgroup-per-CU variant
+#endif
       if (quad) {
         // snapshot through LDS (the token tiles are spent): accumulators -> staged tiles ->
         // coalesced 16-byte stores; a second pass writes the transposed tiles
@@ -590,7 +608,13 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <
         }
       }
     }
-    t = nt; w = nw; tb = ntb; te = nte; slot = nslot; have = has_next;
+    advance(cur);
+  };
+  while (true) {
+    stage(R0);
+    if (!cur.valid) break;
+    stage(R1);
+    if (!cur.valid) break;
   }
 }
 

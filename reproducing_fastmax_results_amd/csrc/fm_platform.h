@@ -25,6 +25,7 @@ typedef uint16_t fm_bf16;  // raw storage of a bfloat16
 #include "hostsim.h"
 #define FM_GLOBAL
 #define FM_DEVICE inline
+#define FM_ALWAYS_INLINE __attribute__((always_inline))
 #define FM_HOST_DEVICE
 #define FM_LAUNCH_BOUNDS(n)
 #define FM_LAUNCH_BOUNDS2(n, m)
@@ -88,6 +89,7 @@ FM_DEVICE float fm_sqrtf(float a) { return std::sqrt(a); }
 #include <hip/hip_runtime.h>
 #define FM_GLOBAL __global__
 #define FM_DEVICE __device__ __forceinline__
+#define FM_ALWAYS_INLINE __attribute__((always_inline))
 #define FM_HOST_DEVICE __host__ __device__
 #define FM_LAUNCH_BOUNDS(n) __launch_bounds__(n)
 #define FM_LAUNCH_BOUNDS2(n, m) __launch_bounds__(n, m)
