@@ -321,8 +321,15 @@ FM_DEVICE void fm_put_small(const BuildArgs<E>& A, E* big, E* big2, float* ds, i
     for (int e = 0; e < 16; ++e) d1[(r0 + fm_acc_row(e, lh)) * DH + c] = CE<E>::from(A.coef1 * v[e]);
     if (big2) {
       E* d2 = big2 + int64_t(slot) * StateDims<DH>::BIG + int64_t(DH) * DH * DH;
+      // a lane owns four consecutive rows four times over: one 8-byte (16-byte for float) store each
+      struct alignas(4 * sizeof(E)) Four { E v[4]; };
 #pragma unroll
-      for (int e = 0; e < 16; ++e) d2[c * DH + r0 + fm_acc_row(e, lh)] = CE<E>::from(A.coef1b * v[e]);
+      for (int g = 0; g < 4; ++g) {
+        Four f;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) f.v[u] = CE<E>::from(A.coef1b * v[4 * g + u]);
+        *reinterpret_cast<Four*>(d2 + c * DH + r0 + fm_acc_row(4 * g, lh)) = f;
+      }
     }
   } else if (tl < 2 * NT * NT) {
     const int u = tl - NT * NT;
