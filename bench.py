@@ -15,7 +15,8 @@ Besides the contract fields the line carries
                 work (state build, readout, dQ, dK, dV each count one unit);
   cpu_baseline: the oracle's port of the reference's einops algorithm timed on
                 this box's host cores on a bounded sample (one (b, h) slice).
-Everything runs on one GPU; --gpus N > 1 is refused.
+Everything runs on one GPU; --gpus N > 1 is refused.  --workload long / --order 1 time the
+long-context parity configuration (B=1, H=16, N=65536) for profiling; the metric is the default.
 """
 from __future__ import annotations
 
@@ -37,7 +38,9 @@ PEAK_HBM_GBS = 8000.0
 # WRITE_SIZE runs of this file scaled by a copy of known size; keyed by (dtype, --chunk, kernel).
 TRAFFIC_BYTES = {("bf16", 0, "dkv"): 115648 * 1024}
 
-WORKLOAD = dict(name="configs[1]: causal order-2 fwd+bwd", B=4, H=8, N=4096, D=64, p=2, mask=True)
+WORKLOAD = dict(name="configs[1]: causal order-2 fwd+bwd", B=4, H=8, N=4096, D=64, p=2, mask=True, scale=1.0)
+# not a bench line of its own: the long-context parity configuration, selectable for profiling (--workload long)
+LONG_WORKLOAD = dict(name="configs[2]: causal long-context fwd+bwd", B=1, H=16, N=65536, D=64, p=2, mask=True, scale=0.5)
 
 # Units of algorithmic work (each 2*M_p*(Dv+1) flop per (b, h, token)) carried by one launch of
 # each kernel; 7 units per forward+backward in both cases (fwd 4, bwd 10 of the 14*M_p*(Dv+1)).
@@ -140,6 +143,10 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device copy, the yardstick for the HBM traffic counters")
+    ap.add_argument("--workload", choices=["headline", "long"], default="headline",
+                    help="headline: the configuration the metric is quoted on (default); long: B=1, H=16, N=65536 "
+                         "(inputs scaled by 0.5), for profiling the moment-state kernels")
+    ap.add_argument("--order", type=int, choices=[1, 2], default=2, help="order of the polynomial (the metric is order 2)")
     ap.add_argument("--graph", action="store_true", help="time replays of the step captured as one HIP graph")
     ap.add_argument("--cpu-max-n", type=int, default=2048, help="longest slice the CPU baseline materialises")
     args = ap.parse_args()
@@ -159,12 +166,13 @@ def main() -> int:
     if args.model_step:
         print(json.dumps(model_step(args, dev)))
         return 0
-    W = WORKLOAD
+    W = dict(WORKLOAD if args.workload == "headline" else LONG_WORKLOAD, p=args.order)
     B, H, N, D, p = W["B"], W["H"], W["N"], W["D"], W["p"]
     bh = B * H
     tdtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
     gen = torch.Generator(device="cpu").manual_seed(1)
-    q, k, v, go = (torch.randn(B, H, N, D, generator=gen).to(tdtype).to(dev).view(bh, N, D) for _ in range(4))
+    q, k, v = ((W["scale"] * torch.randn(B, H, N, D, generator=gen)).to(tdtype).to(dev).view(bh, N, D) for _ in range(3))
+    go = torch.randn(B, H, N, D, generator=gen).to(tdtype).to(dev).view(bh, N, D)
     tau = 8.0 * math.sqrt(D)
     kw = dict(mask=True, inv_tau=1.0 / tau, a0=1.0, a1=1.0, a2=0.5, p=p, chunk=args.chunk)
 
@@ -226,7 +234,20 @@ def main() -> int:
                 "whole_step": {"achieved": 7 * unit / (ms_per_step * 1e-3) / 1e12,
                                "frac": 7 * unit / (ms_per_step * 1e-3) / 1e12 / peak},
                 "kernels_ms_per_step": {nme: tot / nprof for nme, (tot, cnt) in sorted(per_kernel.items())}}
-    if "build" not in per_kernel and args.dtype == "bf16":
+    if p == 1:
+        # order 1 is bandwidth bound (M_1 = D features: 130 flop per byte of q, k, v, o): price it against HBM.
+        # Algorithmic bytes: the forward reads q, k, v and writes o; the backward reads q, k, v, o, dO and
+        # writes dq, dk, dv; per kernel, the tensors it must read and write once.
+        esz_io = 2 if args.dtype == "bf16" else 4
+        tensor_b = bh * N * D * esz_io
+        k_tensors = {"fwd": 4, "dq": 5, "dk": 5, "dv": 4, "dkv": 7, "build": 2}
+        dom_b = k_tensors.get(dominant, 4) * tensor_b
+        roofline = {"bound": "hbm", "kernel": dominant, "achieved": dom_b / (avg_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                    "unit": "GB/s", "frac": dom_b / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None, "avg_ms": avg_ms,
+                    "whole_step": {"achieved": 12 * tensor_b / (ms_per_step * 1e-3) / 1e9,
+                                   "frac": 12 * tensor_b / (ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBS},
+                    "kernels_ms_per_step": roofline["kernels_ms_per_step"]}
+    if "build" not in per_kernel and args.dtype == "bf16" and p == 2:
         # what the matrix cores actually execute when one segment covers the sequence: causal 32x32 tiles only
         nt = (N + 31) // 32
         tiles = bh * nt * (nt + 1) // 2
@@ -234,15 +255,15 @@ def main() -> int:
         roofline["executed_mfma"] = {"flop_per_step": executed,
                                      "achieved": executed / (ms_per_step * 1e-3) / 1e12,
                                      "frac": executed / (ms_per_step * 1e-3) / 1e12 / peak}
-    if TRAFFIC_BYTES.get((args.dtype, args.chunk, dominant)) is not None:
+    if args.workload == "headline" and p == 2 and TRAFFIC_BYTES.get((args.dtype, args.chunk, dominant)) is not None:
         roofline["traffic"] = TRAFFIC_BYTES[(args.dtype, args.chunk, dominant)]
 
     out = {
-        "metric": "Fastmax fwd+bwd tokens/s, causal order-2 N=4096 D=64",
+        "metric": f"Fastmax fwd+bwd tokens/s, causal order-{p} N={N} D={D}",
         "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic",
-        "config": {"workload": f"{W['name']} B={B} H={H} N={N} D=Dv={D} tau=8*sqrt(D) a=(1,1,0.5)",
+        "config": {"workload": f"{W['name'].replace('order-2', f'order-{p}')} B={B} H={H} N={N} D=Dv={D} tau=8*sqrt(D) a=(1,1,0.5)",
                    "chunk": args.chunk or "auto", "launch": "hip graph replay" if args.graph else "eager"},
         "roofline": roofline,
     }
@@ -274,7 +295,7 @@ def main() -> int:
         dst = torch.empty_like(src)
         dst.copy_(src)
         torch.cuda.synchronize()
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and args.workload == "headline" and p == 2:
         out["cpu_baseline"] = cpu_baseline(N, D, p, tokens, bh, args.cpu_max_n)
     print(json.dumps(out))
     return 0
