@@ -853,11 +853,18 @@ FM_DEVICE void fm_readout(const E* FM_RESTRICT state, bool quad, const E* xs, co
     frag fa[C::NT];
 #pragma unroll
     for (int ct = 0; ct < C::NT; ++ct) fa[ct] = M::load(sl + (32 * ct) * C::PS);
+    // the own tokens' x_a: the value for the next a is read from LDS while this one's products run
+    E xv[QT];
+#pragma unroll
+    for (int j = 0; j < QT; ++j) xv[j] = (as < DH) ? xs[xrow[j] * C::PQ + as] : E(1.0f);
     for (int al = 0; al < na; ++al) {
       const int a = as + al;
       frag xr[QT];
 #pragma unroll
-      for (int j = 0; j < QT; ++j) xr[j] = (a < DH) ? M::splat(xs[xrow[j] * C::PQ + a]) : M::splat(E(1.0f));
+      for (int j = 0; j < QT; ++j) xr[j] = M::splat(xv[j]);
+      const int an = (al + 1 < na) ? a + 1 : a;        // re-reads a valid element at the end of a slab
+#pragma unroll
+      for (int j = 0; j < QT; ++j) xv[j] = (an < DH) ? xs[xrow[j] * C::PQ + an] : E(1.0f);
 #pragma unroll
       for (int ks = 0; ks < C::NKS; ++ks) {
         // prefetch the fragments of the next (a, k-step); the last one of a slab re-reads a valid row
