@@ -1,0 +1,125 @@
+"""GPU parity at the full benchmark sizes, every (b, h) slice, through checks whose cost does
+not grow with the square of the sequence length:
+
+* the upstream gradient is zero outside a few query rows, so only those rows of the score
+  matrix enter any result and the fp64 closed form restricted to them
+  (``oracle.sampled_rows_forward_backward``) is an exact oracle for o and g at the rows, dq
+  everywhere (zero off the rows) and the whole of dk and dv;
+* ``a1 = a2 = 0`` turns causal Fastmax into the running mean of v (every row, fp64 cumsum);
+* keys and values after a token do not reach it: the outputs of the first tokens are the
+  bits of a run on the truncated sequence.
+
+Tolerances as everywhere: rel-L2 1e-5 (fp32), 2e-2 (bf16, oracle fed the rounded inputs)."""
+import math
+
+import pytest
+import torch
+
+from oracle import fastmax_oracle as O
+from tests.parity import TOL, rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from reproducing_fastmax_results_amd._capi import get_lib
+    return get_lib()
+
+
+def _inputs(bh, n, d, dtype, seed, scale):
+    gen = torch.Generator().manual_seed(seed)
+    return [(s * torch.randn(bh, n, d, generator=gen)).to(dtype) for s in (scale, scale, scale, 1.0)]
+
+
+def _rows(n, count, seed):
+    """first and last token, both sides of the 256-, 1024- and 2048-token segment boundaries
+    and of a 128-token block, and seeded random rows"""
+    fixed = [0, 1, 31, 32, 127, 128, 255, 256, 1023, 1024, 2047, 2048, n // 2 - 1, n // 2, n - 2, n - 1]
+    gen = torch.Generator().manual_seed(seed)
+    rnd = torch.randint(0, n, (count,), generator=gen).tolist()
+    return torch.tensor(sorted({r for r in fixed + rnd if 0 <= r < n}))
+
+
+def _check_sparse_rows(lib, bh, n, d, dtype, p, seed, scale, chunk=0, count=48):
+    q, k, v, go = _inputs(bh, n, d, dtype, seed, scale)
+    rows = _rows(n, count, seed + 1)
+    sparse = torch.zeros_like(go)
+    sparse[:, rows] = go[:, rows]
+    tau = 8.0 * math.sqrt(d)
+    kw = dict(mask=True, inv_tau=1.0 / tau, p=p, chunk=chunk)
+    qd, kd, vd, gd = (t.to(DEV) for t in (q, k, v, sparse))
+    o, g, ws = lib.forward(qd, kd, vd, save=True, **kw)
+    dq, dk, dv = lib.backward(qd, kd, vd, o, g, gd, saved=ws, **kw)
+    torch.cuda.synchronize()
+    ref = O.sampled_rows_forward_backward(q, k, v, rows, go[:, rows], tau=tau, p=p)
+    dq = dq.cpu()
+    off = torch.ones(n, dtype=torch.bool)
+    off[rows] = False
+    assert float(dq[:, off].float().abs().max()) == 0.0, "dq of a row without upstream gradient"
+    got = (o.cpu()[:, rows], g.cpu()[:, rows], dq[:, rows], dk.cpu(), dv.cpu())
+    errs = {name: rel_err(x, r) for name, x, r in zip(("o", "g", "dq", "dk", "dv"), got, ref)}
+    for name, e in errs.items():
+        assert e < TOL[dtype], f"{name} rel-L2 {e:.3e} (all: {errs})"
+    # per slice as well: one bad (b, h) must not hide among the others
+    for i in range(bh):
+        for name, x, r in zip(("o", "dk", "dv"), (got[0], got[3], got[4]), (ref[0], ref[3], ref[4])):
+            e = rel_err(x[i], r[i])
+            assert e < TOL[dtype], f"slice {i}: {name} rel-L2 {e:.3e}"
+    return errs
+
+
+def _check_running_mean(lib, bh, n, d, dtype, p, seed, chunk=0):
+    q, k, v, _ = _inputs(bh, n, d, dtype, seed, 1.0)
+    o, g = lib.forward(q.to(DEV), k.to(DEV), v.to(DEV), mask=True, inv_tau=1.0 / (8.0 * math.sqrt(d)),
+                       a0=1.0, a1=0.0, a2=0.0, p=p, chunk=chunk)
+    count = torch.arange(1, n + 1, dtype=torch.float64)
+    want = v.double().cumsum(1) / count.view(1, n, 1)
+    assert torch.equal(g.cpu().double(), count.expand(bh, n)), "g must be the number of visible keys"
+    e = rel_err(o, want)
+    assert e < TOL[dtype], f"o rel-L2 {e:.3e}"
+
+
+def _prefix_runs(lib, bh, n, cut, d, dtype, p, seed, scale, chunk):
+    """forward on the whole sequence and on its first ``cut`` tokens, same segment length (so the
+    same sums in the same order)"""
+    q, k, v, _ = _inputs(bh, n, d, dtype, seed, scale)
+    kw = dict(mask=True, inv_tau=1.0 / (8.0 * math.sqrt(d)), p=p, chunk=chunk)
+    qd, kd, vd = (t.to(DEV) for t in (q, k, v))
+    o, g = lib.forward(qd, kd, vd, **kw)
+    o2, g2 = lib.forward(qd[:, :cut].contiguous(), kd[:, :cut].contiguous(), vd[:, :cut].contiguous(), **kw)
+    torch.cuda.synchronize()
+    return o, g, o2, g2
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_config2_all_slices(lib, dtype):
+    # causal order 2, B*H = 32, N = 4096, D = 64: all 32 slices
+    print(f"case full config2 dtype={dtype}", flush=True)
+    _check_sparse_rows(lib, 32, 4096, 64, dtype, 2, seed=101, scale=1.0)
+    _check_running_mean(lib, 32, 4096, 64, dtype, 2, seed=102)
+
+
+@pytest.mark.parametrize("chunk", [1024, 2048])
+def test_config2_all_slices_through_states(lib, chunk):
+    # the same shape cut into segments, through their prefix / suffix states
+    print(f"case full config2 chunk={chunk}", flush=True)
+    _check_sparse_rows(lib, 32, 4096, 64, torch.bfloat16, 2, seed=103, scale=1.0, chunk=chunk)
+
+
+@pytest.mark.parametrize("p", [1, 2])
+def test_config3_all_slices(lib, p):
+    # causal long context, B*H = 16, N = 65536, D = 64, bf16, inputs scaled by 0.5
+    print(f"case full config3 p={p}", flush=True)
+    _check_sparse_rows(lib, 16, 65536, 64, torch.bfloat16, p, seed=110 + p, scale=0.5)
+    _check_running_mean(lib, 16, 65536, 64, torch.bfloat16, p, seed=120 + p)
+
+
+@pytest.mark.parametrize("p", [1, 2])
+def test_config3_prefix_is_independent_of_later_tokens(lib, p):
+    print(f"case config3 prefix p={p}", flush=True)
+    n, cut = 65536, 8192
+    seg = 256 if p == 1 else 1024
+    o, g, o2, g2 = _prefix_runs(lib, 16, n, cut, 64, torch.bfloat16, p, seed=130 + p, scale=0.5, chunk=seg)
+    assert torch.equal(o[:, :cut], o2) and torch.equal(g[:, :cut], g2)

@@ -125,6 +125,23 @@ def test_manual_blocked_backward_equals_autograd(mask, p):
         assert O.rel_l2(a, b_) < 1e-12
 
 
+@pytest.mark.parametrize("p", [1, 2])
+def test_sampled_rows_equal_autograd_with_sparse_upstream_gradient(p):
+    # dO zero outside a few query rows: autograd through the full closed form must give the
+    # same o, g and dq at those rows, zero dq elsewhere, and the same full dk, dv
+    bh, n, d = 3, 41, 5
+    q, k, v, go = (rnd(1, bh, n, d, seed=s)[0] for s in (31, 32, 33, 34))
+    rows = torch.tensor([0, 7, 8, 23, 40])
+    sparse = torch.zeros_like(go)
+    sparse[:, rows] = go[:, rows]
+    o, g, dq, dk, dv = O.closed_form_forward_backward(q, k, v, sparse, mask=True, tau=1.7, p=p, a0=0.9, a1=0.7, a2=0.6)
+    got = O.sampled_rows_forward_backward(q, k, v, rows, go[:, rows], tau=1.7, p=p, a0=0.9, a1=0.7, a2=0.6)
+    other = torch.ones(n, dtype=torch.bool); other[rows] = False
+    assert dq[:, other].abs().max() == 0
+    for a, b_ in zip(got, (o[:, rows], g[:, rows], dq[:, rows], dk, dv)):
+        assert O.rel_l2(a, b_) < 1e-12
+
+
 def test_causality_and_first_token():
     # reference: test_fastmax_iscausal (:257-274): a[i, j] == 0 for j > i
     q, k, v = rnd(1, 2, 6, 3, seed=19), rnd(1, 2, 6, 3, seed=20), rnd(1, 2, 6, 3, seed=21)
