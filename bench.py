@@ -212,6 +212,16 @@ def main() -> int:
     tokens = B * N
     value = tokens * args.steps / elapsed
 
+    # forward alone (the inference call: no workspace kept for a backward)
+    for _ in range(3):
+        lib.forward(q, k, v, **kw)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        lib.forward(q, k, v, **kw)
+    torch.cuda.synchronize()
+    fwd_ms = 1e3 * (time.perf_counter() - t0) / args.steps
+
     # per-kernel durations, HIP events on the launch stream
     nprof = max(3, min(10, args.steps))
     lib.profile_begin()
@@ -266,6 +276,9 @@ def main() -> int:
         "config": {"workload": f"{W['name'].replace('order-2', f'order-{p}')} B={B} H={H} N={N} D=Dv={D} tau=8*sqrt(D) a=(1,1,0.5)",
                    "chunk": args.chunk or "auto", "launch": "hip graph replay" if args.graph else "eager"},
         "roofline": roofline,
+        "forward_only": {"ms": fwd_ms, "tokens_per_s": tokens / (fwd_ms * 1e-3),
+                         "algorithmic_TFLOPs": 2 * unit / (fwd_ms * 1e-3) / 1e12,
+                         "frac_of_peak": 2 * unit / (fwd_ms * 1e-3) / 1e12 / peak},
     }
     # the bandwidth-bound helpers of the path on the same tensors: event-timed passes against the HBM peak
     esz = 2 if args.dtype == "bf16" else 4
@@ -290,6 +303,23 @@ def main() -> int:
         helpers["transpose"] = {"ms": t_ms, "bytes": nbytes, "achieved_GBps": nbytes / (t_ms * 1e-3) / 1e9,
                                 "frac_of_8TBps": nbytes / (t_ms * 1e-3) / 8e12}
     out["hbm_bound_helpers"] = helpers
+    # what this box sustains, beside the published peaks the fractions above are priced against: a
+    # register-only loop of 32x32x16 _Float16 matrix products, and a 1 GiB device-to-device copy
+    # (read + write counted)
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(5):
+        dst.copy_(src)
+    e1.record()
+    e1.synchronize()
+    out["measured_on_this_box"] = {"mfma_f16_loop_TFLOPs": lib.mfma_rate(dev),
+                                   "hbm_copy_GBps": 5 * 2 * float(1 << 30) / (e0.elapsed_time(e1) * 1e-3) / 1e9,
+                                   "published": {"mfma_bf16_TFLOPs": PEAK_TFLOPS["bf16"], "mfma_f32_TFLOPs": PEAK_TFLOPS["f32"],
+                                                 "hbm_GBps": PEAK_HBM_GBS}}
+    del src, dst
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)

@@ -164,6 +164,13 @@ int fastmax_profile_end(int* kernel_ids, float* milliseconds, int capacity);
  * registers, the value found (out_f16 and out_f32: 1024 floats each, device memory). */
 int fastmax_probe_mfma(float* out_f16, float* out_f32, void* hip_stream);
 
+/* Yardstick for benchmarks (no counterpart in the reference): `workgroups` workgroups of four
+ * wavefronts each issue `iters` rounds of eight independent 32x32x16 _Float16 matrix products on
+ * register operands, i.e. workgroups * 4 * iters * 8 * 32768 flop with no memory traffic; timed by
+ * the caller with events on `hip_stream`, it gives the matrix rate this device sustains.
+ * out: workgroups * 256 floats (device memory, checksums).  workgroups <= 65536, iters <= 2^20. */
+int fastmax_probe_mfma_rate(int workgroups, int iters, float* out, void* hip_stream);
+
 /* Self-check of the transposing LDS read (ds_read_b64_tr_b16) the _Float16 kernels use for transposed
  * fragments: one wavefront reads a 16 x 64 tile holding 64 * row + col; lane l addresses the four
  * values at (row l % 16, columns 4 * (l / 16) ..).  out: 256 floats (device memory), four per lane.

@@ -53,6 +53,7 @@ EXPORTS = (
     "fastmax_workspace_bytes", "fastmax_forward", "fastmax_backward", "fastmax_backward_saved", "fastmax_normalize",
     "fastmax_normalize_stats_bytes", "fastmax_normalize_backward", "fastmax_normalize_backward_stats_bytes",
     "fastmax_status_string", "fastmax_version", "fastmax_probe_mfma", "fastmax_probe_lds_transpose",
+    "fastmax_probe_mfma_rate",
     "fastmax_profile_begin", "fastmax_profile_end",
 )
 
@@ -131,6 +132,8 @@ class FastmaxLib:
         L.fastmax_probe_mfma.restype = C.c_int
         L.fastmax_probe_lds_transpose.argtypes = [C.c_void_p, C.c_void_p]
         L.fastmax_probe_lds_transpose.restype = C.c_int
+        L.fastmax_probe_mfma_rate.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+        L.fastmax_probe_mfma_rate.restype = C.c_int
         L.fastmax_profile_begin.restype = C.c_int
         L.fastmax_profile_end.argtypes = [C.POINTER(C.c_int), C.POINTER(C.c_float), C.c_int]
         L.fastmax_profile_end.restype = C.c_int
@@ -286,6 +289,19 @@ class FastmaxLib:
         b = torch.zeros(1024, dtype=torch.float32, device=device)
         self.check(self.lib.fastmax_probe_mfma(a.data_ptr(), b.data_ptr(), 0), "fastmax_probe_mfma")
         return a.view(64, 16), b.view(64, 16)
+
+    def mfma_rate(self, device, workgroups: int = 2048, iters: int = 4000) -> float:
+        """TFLOP/s of a register-only loop of 32x32x16 _Float16 matrix products on `device`
+        (event-timed on torch's current stream after one short warm-up launch)."""
+        out = torch.empty(workgroups * 256, dtype=torch.float32, device=device)
+        stream = torch.cuda.current_stream(out.device).cuda_stream
+        self.check(self.lib.fastmax_probe_mfma_rate(workgroups, 10, out.data_ptr(), stream), "fastmax_probe_mfma_rate")
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        self.check(self.lib.fastmax_probe_mfma_rate(workgroups, iters, out.data_ptr(), stream), "fastmax_probe_mfma_rate")
+        e1.record()
+        e1.synchronize()
+        return workgroups * 4 * iters * 8 * 32768.0 / (e0.elapsed_time(e1) * 1e-3) / 1e12
 
 
 _lock = threading.Lock()

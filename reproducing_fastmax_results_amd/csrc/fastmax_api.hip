@@ -410,7 +410,7 @@ int add_rows(const FastmaxDesc* d, const SplitPlan& sp, const void* dqa, void* d
 
 extern "C" {
 
-int fastmax_version(void) { return 104; }
+int fastmax_version(void) { return 105; }
 
 const char* fastmax_status_string(int status) {
   switch (status) {
@@ -628,6 +628,14 @@ int fastmax_profile_end(int* kernel_ids, float* milliseconds, int capacity) {
 int fastmax_probe_mfma(float* out_f16, float* out_f32, void* hip_stream) {
   if (!out_f16 || !out_f32) return FASTMAX_ERR_NULL;
   FM_KERNEL_LAUNCH(k_probe_mfma, fm_dim3(1), fm_dim3(64), 0, static_cast<fm_stream_t>(hip_stream), out_f16, out_f32);
+  return fm_after_launch();
+}
+
+int fastmax_probe_mfma_rate(int workgroups, int iters, float* out, void* hip_stream) {
+  if (!out) return FASTMAX_ERR_NULL;
+  if (workgroups <= 0 || workgroups > 65536 || iters <= 0 || iters > (1 << 20)) return FASTMAX_ERR_SHAPE;
+  FM_KERNEL_LAUNCH(k_probe_mfma_rate, fm_dim3(workgroups), fm_dim3(FM_THREADS), 0, static_cast<fm_stream_t>(hip_stream),
+                   out, iters);
   return fm_after_launch();
 }
 

@@ -913,6 +913,30 @@ FM_GLOBAL void k_probe_mfma(float* out_f16, float* out_f32) {
 }
 
 // ------------------------------------------------------------------------------
+// k_probe_mfma_rate: what the matrix cores sustain on this device with nothing in their way: every
+// wavefront issues `iters` rounds of eight independent 32x32x16 _Float16 products on register
+// operands (no memory, no LDS, no vector work).  2 * 32 * 32 * 16 flop per product.
+// ------------------------------------------------------------------------------
+FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 1) k_probe_mfma_rate(float* out, int iters) {
+  fm_half8 a, b;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) { a[i] = fm_half(float((FM_TID_X & 7) + i) * 0.125f); b[i] = fm_half(float(i) * 0.25f); }
+  fm_f32x16 acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = fm_zero16();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = fm_mfma_f16(a, b, acc[i]);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) s += acc[i][e];
+  out[FM_BID_X * FM_THREADS + FM_TID_X] = s;
+}
+
+// ------------------------------------------------------------------------------
 // k_probe_lds_tr: one wavefront; a 16 x 64 _Float16 tile holding 64 * row + col (all exact); lane l
 // reads through fm_lds_tr4 at (row l % 16, column 4 * (l / 16)) and writes its four values.
 // ------------------------------------------------------------------------------

@@ -113,7 +113,10 @@ def test_forward_backward_reject_bad_arguments_before_launching(lib):
     assert lib.lib.fastmax_normalize(C.byref(nd), one, one, None, None) == 4   # max_norm needs stats scratch
     assert lib.lib.fastmax_probe_mfma(None, None, None) == 1
     assert lib.lib.fastmax_probe_lds_transpose(None, None) == 1
-    assert lib.lib.fastmax_version() >= 104
+    assert lib.lib.fastmax_probe_mfma_rate(1, 1, None, None) == 1
+    assert lib.lib.fastmax_probe_mfma_rate(0, 1, one, None) == 2
+    assert lib.lib.fastmax_probe_mfma_rate(1, (1 << 20) + 1, one, None) == 2
+    assert lib.lib.fastmax_version() >= 105
 
 
 def test_normalize_backward_arguments(lib):
