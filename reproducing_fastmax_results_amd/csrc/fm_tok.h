@@ -126,32 +126,31 @@ FM_DEVICE int fm_snake_rank(int j, int total) {
   return base + cnt - 1 - pos;
 }
 
-// rank (0 = heaviest) -> block index, for a causal launch with bps blocks per segment
+// rank (0 = heaviest) -> block index, for a causal launch with bps blocks per segment.
+// Own = queries: the blocks that have a state (segments >= 1) come first, late positions w inside
+// the segment before early ones and, for one position, late segments before early ones; then the
+// blocks of segment 0, late positions first.  Own = keys: the blocks that have a state (all but the
+// last segment), early positions first and, for one position, early segments first; then the last
+// segment.  The last segment may be short (wl of bps blocks).  Closed form: a launch over a long
+// sequence has hundreds of blocks per batch*head and every wavefront needs its own.
 template <int OWN> FM_DEVICE int fm_block_of_rank(int rank, int nblk, int bps) {
   const int nseg = (nblk + bps - 1) / bps;
-  int n = 0;
+  const int wl = nblk - (nseg - 1) * bps;              // blocks of the last segment, 1 .. bps
   if (OWN == FM_OWN_Q) {
-    // with a state (segments >= 1): late positions first; then segment 0
-    for (int w = bps - 1; w >= 0; --w)
-      for (int sg = nseg - 1; sg >= 1; --sg) {
-        const int b = sg * bps + w;
-        if (b < nblk) { if (n == rank) return b; ++n; }
-      }
-    for (int w = bps - 1; w >= 0; --w)
-      if (w < nblk) { if (n == rank) return w; ++n; }
-  } else {
-    // with a state (all but the last segment): early positions first; then the last segment
-    for (int w = 0; w < bps; ++w)
-      for (int sg = 0; sg < nseg - 1; ++sg) {
-        const int b = sg * bps + w;
-        if (b < nblk) { if (n == rank) return b; ++n; }
-      }
-    for (int w = 0; w < bps; ++w) {
-      const int b = (nseg - 1) * bps + w;
-      if (b < nblk) { if (n == rank) return b; ++n; }
+    if (nseg > 1) {
+      const int per_hi = nseg - 2, n_hi = (bps - wl) * per_hi;   // positions the last segment lacks
+      if (rank < n_hi) return (nseg - 2 - rank % per_hi) * bps + (bps - 1 - rank / per_hi);
+      rank -= n_hi;
+      const int per_lo = nseg - 1, n_lo = wl * per_lo;
+      if (rank < n_lo) return (nseg - 1 - rank % per_lo) * bps + (wl - 1 - rank / per_lo);
+      rank -= n_lo;
     }
+    return (nblk < bps ? nblk : bps) - 1 - rank;
+  } else {
+    const int per = nseg - 1;
+    if (rank < bps * per) return (rank % per) * bps + rank / per;
+    return per * bps + (rank - bps * per);
   }
-  return rank;   // not reached
 }
 
 // Which part of the stream a block of own tokens starting at t0 sees densely, and which state slot.
