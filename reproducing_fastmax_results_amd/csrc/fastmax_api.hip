@@ -237,12 +237,18 @@ int launch_build(const BuildArgs<E>& args, int bh, fm_stream_t stream) {
   // a staged walk.  One workgroup per (segment, batch*head) sums its segment from fragments loaded
   // straight from the operands, and a scan over the segments follows.
   a.seg_parallel = 1;
+  if (nsteps > 1) {
+    // several segments: operand tiles staged through LDS, sum tiles dealt to the wavefronts (see k_build1_seg)
+    const size_t lds1 = Build1Cfg<E, DH>::lds_bytes(a.zt != nullptr && a.za_sel == FM_SRC_Z);
+    fm_allow_lds(reinterpret_cast<const void*>(&k_build1_seg<E, DH>), lds1);
+    FM_KERNEL_LAUNCH((k_build1_seg<E, DH>), fm_dim3(1, bh, nsteps), fm_dim3(FM_THREADS), lds1, stream, a);
+    const int st = fm_after_launch();
+    return st ? st : launch_scan<E, DH>(a, bh, nsteps, stream);
+  }
   const size_t lds = size_t(4) * 4 * 64 * 16 * 4;
   fm_allow_lds(reinterpret_cast<const void*>(&k_build1<E, DH>), lds);
   FM_KERNEL_LAUNCH((k_build1<E, DH>), fm_dim3(1, bh, nsteps), fm_dim3(FM_THREADS), lds, stream, a);
-  const int st = fm_after_launch();
-  if (st || nsteps < 2) return st;
-  return launch_scan<E, DH>(a, bh, nsteps, stream);
+  return fm_after_launch();
 }
 
 // Dynamic LDS of a token kernel (kind 0: k_pv, 1: k_ds, 2: k_ds with dV, 3: k_ds with the fused

@@ -708,6 +708,95 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_build1(BuildArgs<E> A) {
   }
 }
 
+// k_build1_seg: the same sums for a walk of several steps (one workgroup per segment and
+// batch*head, k_state_scan follows).  A lane's MFMA fragment is 16 bytes of one feature row of a
+// transposed operand, and the rows lie a power of two apart: loaded straight from memory, the 32
+// rows of one load instruction queue up behind one another (measured on MI355X: the loads alone
+// were 145 of the 170 us of a launch over 16 x 65536 tokens).  So the workgroup stages the operand
+// tiles of 128 tokens through LDS with whole 256-byte row pieces per 16 lanes (the next tile
+// travels global memory -> registers meanwhile), and the tiles of the sums, not the tokens, are
+// dealt to the wavefronts: wavefront w sums tiles w, w + 4, .. (for D = 64 one tile of the D x D
+// sum and one vector-sum tile) over all tokens, so no partial sums meet anywhere.
+// Needs (te - tb) to be a multiple of 128 tokens.
+template <typename E, int DH> struct Build1Cfg {
+  static constexpr int TT = 128, PT = TT + Mma<E>::VEC;
+  static constexpr size_t lds_bytes(bool has_z) { return size_t(has_z ? 3 : 2) * DH * PT * sizeof(E); }
+};
+
+template <typename E, int DH>
+FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_build1_seg(BuildArgs<E> A) {
+  typedef Mma<E> M;
+  typedef typename M::frag frag;
+  constexpr int NT = DH / 32, NTILE = NT * NT + 2 * NT, NS = (NTILE + 3) / 4;
+  constexpr int TT = Build1Cfg<E, DH>::TT, PT = Build1Cfg<E, DH>::PT;
+  FM_DYN_SMEM(smem);
+  E* Lp = reinterpret_cast<E*>(smem);                  // [DH][PT] each
+  E* Lr = Lp + DH * PT;
+  E* Lz = Lr + DH * PT;                                // only there (and only used) with a third operand
+  const int tid = FM_TID_X, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int wave = FM_UNIFORM(tid >> 6);
+  const int bh = FM_BID_Y;
+  int tb, te, slot;
+  fm_walk_step(A.mode, A.nseg, A.L, A.npad, FM_BID_Z, tb, te, slot);
+  E* big = A.big + int64_t(bh) * A.nslots * StateDims<DH>::BIG;
+  E* big2 = A.big2 ? A.big2 + int64_t(bh) * A.nslots * StateDims<DH>::BIG : nullptr;
+  float* ds = A.small + (int64_t(bh) * A.nslots + slot) * StateDims<DH>::SMALL;
+  const bool has_z = A.zt != nullptr && A.za_sel == FM_SRC_Z;
+  const int64_t base = int64_t(bh) * DH * A.npad;
+  const E* gp = A.pt + base;
+  const E* gr = A.rt + base;
+  const E* gz = has_z ? A.zt + base : gp;
+  const E* va_src = A.za_sel == FM_SRC_P ? Lp : (A.za_sel == FM_SRC_R ? Lr : Lz);
+  const E* vb_src = A.vb_from_r ? Lr : Lp;
+  const E* la[NS];
+  const E* lb[NS];                                      // null: a vector sum (the B operand is all ones)
+  int tl[NS];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) {
+    const int t = wave + 4 * s;
+    const int frag_off = lr * PT + lh * M::KPL;
+    tl[s] = t;
+    la[s] = Lp + frag_off; lb[s] = nullptr;
+    if (t < NT * NT) { la[s] = Lp + (t / NT) * 32 * PT + frag_off; lb[s] = Lr + (t % NT) * 32 * PT + frag_off; }
+    else if (t < NT * NT + NT) la[s] = va_src + (t - NT * NT) * 32 * PT + frag_off;
+    else if (t < NTILE) la[s] = vb_src + (t - NT * NT - NT) * 32 * PT + frag_off;
+  }
+  fm_f32x16 acc[NS];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) acc[s] = fm_zero16();
+  const frag ones = M::splat(E(1.0f));
+  TileRegs<E, DH, TT> rp, rr, rz;
+  auto fetch = [&](int t0) {                            // global memory -> registers
+    rp.load(gp + t0, A.npad, tid);
+    rr.load(gr + t0, A.npad, tid);
+    if (has_z) rz.load(gz + t0, A.npad, tid);
+  };
+  fetch(tb);
+  for (int t0 = tb; t0 < te; t0 += TT) {
+    if (t0 != tb) FM_SYNC();                            // the previous tile has been read
+    rp.store(Lp, PT, tid);
+    rr.store(Lr, PT, tid);
+    if (has_z) rz.store(Lz, PT, tid);
+    if (t0 + TT < te) fetch(t0 + TT);
+    FM_SYNC();
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+      if (tl[s] < NTILE) {
+#pragma unroll 8
+        for (int k = 0; k < TT; k += M::KSTEP)
+          acc[s] = M::mma(M::load(la[s] + k), lb[s] ? M::load(lb[s] + k) : ones, acc[s]);
+      }
+  }
+#pragma unroll
+  for (int s = 0; s < NS; ++s)
+    if (tl[s] < NTILE) {
+      float v[16];
+#pragma unroll
+      for (int e = 0; e < 16; ++e) v[e] = acc[s][e];
+      fm_put_small<E, DH>(A, big, big2, ds, slot, tl[s] < NT * NT ? tl[s] : tl[s] + NT * NT, v, lr, lh);
+    }
+}
+
 // ------------------------------------------------------------------------------
 // k_state_scan: turns per-segment sums (k_build with seg_parallel) into the states the readers
 // expect: slot s becomes the sum over the walk up to and including its own step.  Elementwise
@@ -715,10 +804,11 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_build1(BuildArgs<E> A) {
 // the vector sums (and Z when quad) of `small`; the running sum is kept in fp32.
 // ------------------------------------------------------------------------------
 // Running sums over the walk of the 16 bytes at p: `stride` elements lie between the slots of two
-// consecutive steps.  Eight steps are loaded before any is added and stored, so the chain of
-// dependent memory round trips is an eighth as long as the walk.
+// consecutive steps.  32 steps are loaded before any is added and stored, so the chain of
+// dependent memory round trips is a 32nd as long as the walk (the launch is a few dozen
+// workgroups, so the round trips, not the bytes, set its time).
 template <typename T> FM_DEVICE void fm_scan_run(T* p, int64_t stride, int nsteps) {
-  constexpr int UB = 8, VE = 16 / sizeof(T);
+  constexpr int UB = 32, VE = 16 / sizeof(T);
   float run[VE];
 #pragma unroll
   for (int i = 0; i < VE; ++i) run[i] = 0.f;
