@@ -174,8 +174,10 @@ int launch_scan(const BuildArgs<E>& a, int bh, int nsteps, fm_stream_t stream) {
   constexpr int VE = 16 / sizeof(E);                            // 16-byte items, as k_state_scan counts them
   const int64_t nbig = (a.quad ? int64_t(DH + 1) * DH * DH : int64_t(DH) * DH) / VE;
   const int64_t total = nbig * (a.big2 ? 2 : 1) + (StateDims<DH>::SMALL - (a.quad ? 0 : DH * DH)) / 4;
-  FM_KERNEL_LAUNCH((k_state_scan<E, DH>), fm_dim3(int((total + 255) / 256), bh), fm_dim3(256), 0, stream, a.big, a.big2,
-                   a.small, a.nslots, nsteps, a.mode, a.nseg, a.quad);
+  // one wavefront per workgroup: an order-1 scan is a thousand items per batch*head, and spread over
+  // four times as many CUs each of them moves a quarter of the bytes
+  FM_KERNEL_LAUNCH((k_state_scan<E, DH>), fm_dim3(int((total + FM_SCAN_THREADS - 1) / FM_SCAN_THREADS), bh),
+                   fm_dim3(FM_SCAN_THREADS), 0, stream, a.big, a.big2, a.small, a.nslots, nsteps, a.mode, a.nseg, a.quad);
   return fm_after_launch();
 }
 

@@ -831,9 +831,10 @@ template <typename T> FM_DEVICE void fm_scan_run(T* p, int64_t stride, int nstep
   }
 }
 
-// grid (ceil(items / 256), bh); an item is 16 bytes of one state array.
+// grid (ceil(items / FM_SCAN_THREADS), bh); an item is 16 bytes of one state array.
+#define FM_SCAN_THREADS 64
 template <typename E, int DH>
-FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_state_scan(E* FM_RESTRICT big, E* FM_RESTRICT big2, float* FM_RESTRICT small,
+FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_SCAN_THREADS) k_state_scan(E* FM_RESTRICT big, E* FM_RESTRICT big2, float* FM_RESTRICT small,
                                                   int nslots, int nsteps, int mode, int nseg, int quad) {
   constexpr int VE = 16 / sizeof(E);
   const int bh = FM_BID_Y;
@@ -842,7 +843,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_state_scan(E* FM_RESTRICT big, E* FM_REST
   const int64_t sfirst = quad ? 0 : int64_t(DH) * DH;           // order 1 has no Z: only the two vectors
   const int64_t nsmall = (StateDims<DH>::SMALL - sfirst) / 4;
   const int64_t nb2 = nbig * (big2 ? 2 : 1);
-  const int64_t i = int64_t(FM_BID_X) * 256 + FM_TID_X;
+  const int64_t i = int64_t(FM_BID_X) * FM_SCAN_THREADS + FM_TID_X;
   if (i >= nb2 + nsmall) return;
   // the slot k_build's step w writes is slot0 + w * dir
   const int slot0 = mode == FM_WALK_PREFIX ? 1 : nseg - 2;
