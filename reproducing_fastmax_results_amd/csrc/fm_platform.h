@@ -33,6 +33,7 @@ typedef uint16_t fm_bf16;  // raw storage of a bfloat16
 #define FM_UNIFORM(x) (x)
 #define FM_OPAQUE_ZERO() 0
 #define FM_SCHED_FENCE()
+#define FM_SCHED_MFMA_DS(n)
 #define FM_KEEP_BRANCH()
 typedef void* fm_stream_t;
 typedef hostsim::Dim3 fm_dim3;
@@ -103,6 +104,10 @@ static __device__ __forceinline__ int fm_opaque_zero() { int z = 0; asm volatile
 #define FM_OPAQUE_ZERO() fm_opaque_zero()
 // Nothing is scheduled across this point (keeps the live ranges of one phase out of the next).
 #define FM_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+// Asks the instruction scheduler to interleave the LDS reads of this block with its matrix
+// instructions (strategy 0: small products, 1: one wavefront's view); it changes the order of
+// instructions only.  On MI355X the dense stages run 1 to 2 % faster with it.
+#define FM_SCHED_MFMA_DS(n) __builtin_amdgcn_iglp_opt(n)
 // Inside a rarely taken wavefront-uniform branch: keeps it a branch (the optimiser would
 // otherwise run its body on every pass and select the result).
 #define FM_KEEP_BRANCH() asm volatile("")

@@ -330,6 +330,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
       // window before they are used; a tile wholly outside the mask has an empty window.
 #pragma unroll
       for (int st = 0; st < KT / 32; ++st) {
+        if (QT == 1) { FM_SCHED_MFMA_DS(0); }
         fm_f32x16 s[QT];
 #pragma unroll
         for (int j = 0; j < QT; ++j) s[j] = fm_zero16();
@@ -612,6 +613,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
       // serve all own tiles of the wavefront; gh.v is formed per own tile.
 #pragma unroll
       for (int st = 0; st < KT / 32; ++st) {
+        if (QT == 1) { FM_SCHED_MFMA_DS(DV ? 0 : 1); }   // two tiles per wavefront: measured slower with it
         fm_f32x16 s[QT];
 #pragma unroll
         for (int j = 0; j < QT; ++j) s[j] = fm_zero16();
