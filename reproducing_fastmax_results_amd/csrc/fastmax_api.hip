@@ -85,7 +85,12 @@ int validate(const FastmaxDesc* d) {
   return FASTMAX_OK;
 }
 
-template <int DH> size_t big_bytes(int esz) { return size_t(StateDims<DH>::BIG) * esz; }
+// bytes of one `big` state array: the slots of all segments of all batch*heads and, when a slot is the
+// order-1 slab alone, the padding that the readers' four-slab fetches may touch behind the last one
+template <int DH> size_t big_array_bytes(int esz, bool quad, size_t slots) {
+  if (!slots) return 0;
+  return (slots * size_t(StateDims<DH>::stride(quad)) + (quad ? 0 : size_t(StateDims<DH>::PAD_SLABS) * StateDims<DH>::SLAB)) * esz;
+}
 
 int make_plan(const FastmaxDesc* d, Plan& p) {
   int st = validate(d);
@@ -125,7 +130,8 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
     p.use_state = force_m || (!force_dense && int64_t(d->nk) > int64_t(d->d) * d->d + d->d);
     p.nslots = p.use_state ? 1 : 0;
   }
-  const size_t bigsz = d->d == 64 ? big_bytes<64>(p.esz) : big_bytes<32>(p.esz);
+  const size_t slots = size_t(d->bh) * p.nslots;
+  const size_t bigarr = d->d == 64 ? big_array_bytes<64>(p.esz, p.quad, slots) : big_array_bytes<32>(p.esz, p.quad, slots);
   const size_t smallsz = size_t(d->d == 64 ? StateDims<64>::SMALL : StateDims<32>::SMALL) * 4;
   const size_t tq = size_t(d->bh) * d->d * p.npad_q * p.esz;
   const size_t tk = size_t(d->bh) * d->d * p.npad_k * p.esz;
@@ -134,20 +140,20 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   p.kt = take(tk);
   p.vt = take(tk);
   p.kr = take(tk);
-  p.big = take(size_t(d->bh) * p.nslots * bigsz);
+  p.big = take(bigarr);
   p.small = take(size_t(d->bh) * p.nslots * smallsz);
   p.save = (d->flags & FASTMAX_FLAG_SAVE_FOR_BACKWARD) != 0;
   p.vr = take(p.save || p.half ? tk : 0);      // _Float16: the forward stages v rows (transposing LDS reads)
-  p.big2 = take(p.save ? size_t(d->bh) * p.nslots * bigsz : 0);
+  p.big2 = take(p.save ? bigarr : 0);
   p.fwd_bytes = off ? off : 256;
   off = 0;
   p.b_kt = take(tk); p.b_vt = take(tk); p.b_qt = take(tq); p.b_qct = take(tq);
   p.b_kr = take(tk); p.b_vr = take(tk); p.b_qr = take(tq);
   p.b_gh = take(tq); p.b_ght = take(tq);
   p.b_cv = take(size_t(d->bh) * p.npad_q * 4);
-  p.b_bigq = take(size_t(d->bh) * p.nslots * bigsz); p.b_smallq = take(size_t(d->bh) * p.nslots * smallsz);
-  p.b_bigk = take(size_t(d->bh) * p.nslots * bigsz); p.b_smallk = take(size_t(d->bh) * p.nslots * smallsz);
-  p.b_bigv = take(size_t(d->bh) * p.nslots * bigsz);
+  p.b_bigq = take(bigarr); p.b_smallq = take(size_t(d->bh) * p.nslots * smallsz);
+  p.b_bigk = take(bigarr); p.b_smallk = take(size_t(d->bh) * p.nslots * smallsz);
+  p.b_bigv = take(bigarr);
   p.bwd_bytes = off ? off : 256;
   return FASTMAX_OK;
 }

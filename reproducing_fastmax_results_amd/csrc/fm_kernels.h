@@ -278,6 +278,15 @@ k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, TRef<const
 template <int DH> struct StateDims {
   static constexpr int64_t BIG = int64_t(DH + 4) * DH * DH;
   static constexpr int64_t SMALL = int64_t(DH) * DH + 2 * DH;
+  static constexpr int64_t SLAB = int64_t(DH) * DH;
+  static constexpr int PAD_SLABS = 3;                  // readers fetch up to four slabs at a time
+  // Elements between the slots of two consecutive segments in a `big` array, and where the order-1
+  // slab lies inside a slot.  With order-2 states a slot is the D slabs T[a], the order-1 slab and
+  // the padding; without them it is the order-1 slab alone (the padding follows the last slot), so
+  // that the hundreds of small states of a long order-1 sequence lie side by side instead of half
+  // a megabyte apart.
+  static FM_HOST_DEVICE int64_t stride(bool quad) { return quad ? BIG : SLAB; }
+  static FM_HOST_DEVICE int64_t slab1(bool quad) { return quad ? DH * SLAB : 0; }
 };
 
 enum { FM_WALK_PREFIX = 0, FM_WALK_SUFFIX = 1, FM_WALK_TOTAL = 2 };
@@ -316,11 +325,11 @@ FM_DEVICE void fm_put_small(const BuildArgs<E>& A, E* big, E* big2, float* ds, i
   constexpr int NT = DH / 32;
   if (tl < NT * NT) {
     const int r0 = 32 * (tl / NT), c = 32 * (tl % NT) + lr;
-    E* d1 = big + int64_t(slot) * StateDims<DH>::BIG + int64_t(DH) * DH * DH;
+    E* d1 = big + int64_t(slot) * StateDims<DH>::stride(A.quad != 0) + StateDims<DH>::slab1(A.quad != 0);
 #pragma unroll
     for (int e = 0; e < 16; ++e) d1[(r0 + fm_acc_row(e, lh)) * DH + c] = CE<E>::from(A.coef1 * v[e]);
     if (big2) {
-      E* d2 = big2 + int64_t(slot) * StateDims<DH>::BIG + int64_t(DH) * DH * DH;
+      E* d2 = big2 + int64_t(slot) * StateDims<DH>::stride(A.quad != 0) + StateDims<DH>::slab1(A.quad != 0);
       // a lane owns four consecutive rows four times over: one 8-byte (16-byte for float) store each
       struct alignas(4 * sizeof(E)) Four { E v[4]; };
 #pragma unroll
@@ -379,8 +388,8 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <
   const int64_t tb_off = int64_t(bh) * DH * A.npad;
   const int nsteps = (A.mode == FM_WALK_TOTAL) ? 1 : A.nseg - 1;
   if (nsteps <= 0) return;
-  E* big = A.big + int64_t(bh) * A.nslots * StateDims<DH>::BIG;
-  E* big2 = A.big2 ? A.big2 + int64_t(bh) * A.nslots * StateDims<DH>::BIG : nullptr;
+  E* big = A.big + int64_t(bh) * A.nslots * StateDims<DH>::stride(A.quad != 0);
+  E* big2 = A.big2 ? A.big2 + int64_t(bh) * A.nslots * StateDims<DH>::stride(A.quad != 0) : nullptr;
   float* sml = A.small + int64_t(bh) * A.nslots * StateDims<DH>::SMALL;
   const bool has_z = A.zt != nullptr;
   const bool quad = A.quad != 0;
@@ -643,8 +652,8 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_build1(BuildArgs<E> A) {
   const int bh = FM_BID_Y;
   int tb, te, slot;
   fm_walk_step(A.mode, A.nseg, A.L, A.npad, FM_BID_Z, tb, te, slot);
-  E* big = A.big + int64_t(bh) * A.nslots * StateDims<DH>::BIG;
-  E* big2 = A.big2 ? A.big2 + int64_t(bh) * A.nslots * StateDims<DH>::BIG : nullptr;
+  E* big = A.big + int64_t(bh) * A.nslots * StateDims<DH>::stride(A.quad != 0);
+  E* big2 = A.big2 ? A.big2 + int64_t(bh) * A.nslots * StateDims<DH>::stride(A.quad != 0) : nullptr;
   float* ds = A.small + (int64_t(bh) * A.nslots + slot) * StateDims<DH>::SMALL;
   const int per_wave = (te - tb) / 4;                  // tokens of this wavefront
   const int64_t row = (int64_t(bh) * DH + lr) * A.npad + tb + wave * per_wave + lh * M::KPL;
@@ -738,8 +747,8 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_build1_seg(BuildArgs<E> A) {
   const int bh = FM_BID_Y;
   int tb, te, slot;
   fm_walk_step(A.mode, A.nseg, A.L, A.npad, FM_BID_Z, tb, te, slot);
-  E* big = A.big + int64_t(bh) * A.nslots * StateDims<DH>::BIG;
-  E* big2 = A.big2 ? A.big2 + int64_t(bh) * A.nslots * StateDims<DH>::BIG : nullptr;
+  E* big = A.big + int64_t(bh) * A.nslots * StateDims<DH>::stride(A.quad != 0);
+  E* big2 = A.big2 ? A.big2 + int64_t(bh) * A.nslots * StateDims<DH>::stride(A.quad != 0) : nullptr;
   float* ds = A.small + (int64_t(bh) * A.nslots + slot) * StateDims<DH>::SMALL;
   const bool has_z = A.zt != nullptr && A.za_sel == FM_SRC_Z;
   const int64_t base = int64_t(bh) * DH * A.npad;
@@ -839,7 +848,8 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_SCAN_THREADS) k_state_scan(E* FM_RESTRICT big
   constexpr int VE = 16 / sizeof(E);
   const int bh = FM_BID_Y;
   const int64_t nbig = (quad ? int64_t(DH + 1) * DH * DH : int64_t(DH) * DH) / VE;   // items of big
-  const int64_t first = quad ? 0 : int64_t(DH) * DH * DH;       // the order-1 slab is the last one
+  const int64_t first = 0;                                      // order 1: the slot is the order-1 slab alone
+  const int64_t sstride = StateDims<DH>::stride(quad != 0);
   const int64_t sfirst = quad ? 0 : int64_t(DH) * DH;           // order 1 has no Z: only the two vectors
   const int64_t nsmall = (StateDims<DH>::SMALL - sfirst) / 4;
   const int64_t nb2 = nbig * (big2 ? 2 : 1);
@@ -849,8 +859,8 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_SCAN_THREADS) k_state_scan(E* FM_RESTRICT big
   const int slot0 = mode == FM_WALK_PREFIX ? 1 : nseg - 2;
   const int dir = mode == FM_WALK_PREFIX ? 1 : -1;
   if (i < nb2) {
-    E* b = (i < nbig ? big : big2) + (int64_t(bh) * nslots + slot0) * StateDims<DH>::BIG + first + (i < nbig ? i : i - nbig) * VE;
-    fm_scan_run<E>(b, int64_t(dir) * StateDims<DH>::BIG, nsteps);
+    E* b = (i < nbig ? big : big2) + (int64_t(bh) * nslots + slot0) * sstride + first + (i < nbig ? i : i - nbig) * VE;
+    fm_scan_run<E>(b, int64_t(dir) * sstride, nsteps);
   } else {
     float* sp = small + (int64_t(bh) * nslots + slot0) * StateDims<DH>::SMALL + sfirst + (i - nb2) * 4;
     fm_scan_run<float>(sp, int64_t(dir) * StateDims<DH>::SMALL, nsteps);
@@ -931,14 +941,15 @@ FM_DEVICE void fm_readout(const E* FM_RESTRICT state, bool quad, const E* xs, co
   const int lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   const int a_begin = quad ? 0 : DH;
   TileRegs<E, C::SA * DH, DH> regs;
-  regs.load(state + int64_t(a_begin) * DH * DH, DH, tid);   // rows [a][c] are contiguous
+  // `state` points at the first slab to read (T[0] with order-2 states, else the order-1 slab)
+  regs.load(state, DH, tid);                                  // rows [a][c] are contiguous
   int buf = 0;
   const int lane_off = lr * C::PS + lh * M::KPL;
   for (int as = a_begin; as <= DH; as += C::SA) {
     E* sb = slab + buf * C::SLAB;
     regs.store(sb, C::PS, tid);
     FM_SYNC();
-    if (as + C::SA <= DH) regs.load(state + int64_t(as + C::SA) * DH * DH, DH, tid);
+    if (as + C::SA <= DH) regs.load(state + int64_t(as + C::SA - a_begin) * DH * DH, DH, tid);
     const int na = (as + C::SA <= DH) ? C::SA : (DH + 1 - as);
     const E* sl = sb + lane_off;
     frag fa[C::NT];

@@ -281,7 +281,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
         }
       FM_SYNC();                                       // Z is overwritten by the slabs
     }
-    const E* state = A.big + (int64_t(bh) * A.nslots + G.slot) * StateDims<DH>::BIG;
+    const E* state = A.big + (int64_t(bh) * A.nslots + G.slot) * StateDims<DH>::stride(A.quad != 0);
     fm_readout<E, DH, QT, NT>(state, A.quad != 0, Own, xrow, of, R, acc, tid);
   } else {
     FM_SYNC();                                         // own rows are overwritten by the dense stages
@@ -560,7 +560,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
         for (int e = 0; e < 16; ++e) acc[j][mt][e] = -ci[j] * (y[e] + vecs[32 * mt + fm_acc_row(e, lh)]);
       }
     FM_SYNC();                                         // Z is overwritten by the slabs
-    const E* state = A.big + (int64_t(bh) * A.nslots + G.slot) * StateDims<DH>::BIG;
+    const E* state = A.big + (int64_t(bh) * A.nslots + G.slot) * StateDims<DH>::stride(A.quad != 0);
     fm_readout<E, DH, QT, NT>(state, A.quad != 0, Own, xrow, of2, R, acc, tid);
   } else {
     FM_SYNC();                                         // own rows are overwritten by the dense stages
