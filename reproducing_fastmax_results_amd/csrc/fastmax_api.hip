@@ -50,6 +50,7 @@ struct Plan {
   int esz;              // sizeof compute element
   int L, nseg, nslots;
   bool use_state, quad;
+  bool rows_build;      // order-1 segment sums read the row-major copies: no transposed copy is written
   int npad_q, npad_k;
   float a0, a1, a2;     // polynomial on the score s = (q.k) / tau
   float sc;             // sqrt(1/tau), folded into q and k when they are converted
@@ -130,6 +131,7 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
     p.use_state = force_m || (!force_dense && int64_t(d->nk) > int64_t(d->d) * d->d + d->d);
     p.nslots = p.use_state ? 1 : 0;
   }
+  p.rows_build = p.half && p.use_state && !p.quad && d->mask;
   const size_t slots = size_t(d->bh) * p.nslots;
   const size_t bigarr = d->d == 64 ? big_array_bytes<64>(p.esz, p.quad, slots) : big_array_bytes<32>(p.esz, p.quad, slots);
   const size_t smallsz = size_t(d->d == 64 ? StateDims<64>::SMALL : StateDims<32>::SMALL) * 4;
@@ -245,6 +247,14 @@ int launch_build(const BuildArgs<E>& args, int bh, fm_stream_t stream) {
   // a staged walk.  One workgroup per (segment, batch*head) sums its segment from fragments loaded
   // straight from the operands, and a scan over the segments follows.
   a.seg_parallel = 1;
+  if (Mma<E>::HAS_TR && a.pr && a.mode != FM_WALK_TOTAL) {
+    // row-major operands, transposing LDS reads: nobody had to write transposed copies (see k_build1_rows)
+    const size_t ldsr = Build1RowsCfg<E, DH>::lds_bytes();
+    fm_allow_lds(reinterpret_cast<const void*>(&k_build1_rows<E, DH>), ldsr);
+    FM_KERNEL_LAUNCH((k_build1_rows<E, DH>), fm_dim3(1, bh, nsteps), fm_dim3(FM_THREADS), ldsr, stream, a);
+    const int st = fm_after_launch();
+    return (st || nsteps < 2) ? st : launch_scan<E, DH>(a, bh, nsteps, stream);
+  }
   if (nsteps > 1) {
     // several segments: operand tiles staged through LDS, sum tiles dealt to the wavefronts (see k_build1_seg)
     const size_t lds1 = Build1Cfg<E, DH>::lds_bytes(a.zt != nullptr && a.za_sel == FM_SRC_Z);
@@ -322,13 +332,14 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   E* vr = (p.save || p.half) ? reinterpret_cast<E*>(ws + p.vr) : nullptr;
   // the transposed copies feed the state walk and the fp32 kernels; the _Float16 token kernels read
   // transposed fragments out of row tiles
-  if (sizeof(E) == 2 && !p.use_state) { kt = nullptr; vt = nullptr; }
+  if (sizeof(E) == 2 && (!p.use_state || p.rows_build)) { kt = nullptr; vt = nullptr; }
   int st = launch_transpose2<TIO, E, DH>(v, d->sv, vt, vr, 1.0f, k, d->sk, kt, kr, p.sc, d->bh, d->nk, p.npad_k, stream);
   if (st) return st;
   if (p.use_state) {
     BuildArgs<E> b;
     b.seg_parallel = 0;
     b.xt = kt; b.pt = vt; b.rt = kt; b.zt = nullptr; b.za_sel = FM_SRC_R; b.zb_sel = FM_SRC_R;
+    b.pr = p.rows_build ? vr : nullptr; b.rr = p.rows_build ? kr : nullptr; b.cw = nullptr;
     b.npad = p.npad_k; b.nseg = p.nseg; b.L = p.L; b.mode = d->mask ? FM_WALK_PREFIX : FM_WALK_TOTAL;
     b.quad = p.quad; b.big = big; b.small = small; b.nslots = p.nslots;
     // saved for the backward: the transposed tiles are the (k, k, v) state that dQ reads

@@ -306,6 +306,10 @@ template <typename E> struct BuildArgs {
   float coef2b, coef1b;                    // coefficients of the transposed copy
   int seg_parallel;                        // grid z = walk step: every workgroup sums one segment only and
                                            // k_state_scan turns the per-segment sums into prefix / suffix states
+  // Order-1 sums from row-major operands (k_build1_rows; null: the transposed operands above are read):
+  const E* pr; const E* rr;                // [bh][npad][DH] rows of the p and r operands
+  const E* cw;                             // [bh][npad] per-token weights (stored in `tperm` order): the third
+                                           // operand is then cw_t * p_t, and zt is not read; or null
 };
 
 FM_DEVICE void fm_walk_step(int mode, int nseg, int L, int npad, int w, int& tb, int& te, int& slot) {
@@ -796,6 +800,102 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_build1_seg(BuildArgs<E> A) {
           acc[s] = M::mma(M::load(la[s] + k), lb[s] ? M::load(lb[s] + k) : ones, acc[s]);
       }
   }
+#pragma unroll
+  for (int s = 0; s < NS; ++s)
+    if (tl[s] < NTILE) {
+      float v[16];
+#pragma unroll
+      for (int e = 0; e < 16; ++e) v[e] = acc[s][e];
+      fm_put_small<E, DH>(A, big, big2, ds, slot, tl[s] < NT * NT ? tl[s] : tl[s] + NT * NT, v, lr, lh);
+    }
+}
+
+// k_build1_rows: k_build1_seg for element types with a transposing LDS read, from the ROW-major
+// operand copies the token kernels stream anyway ([token][feature], a segment's 128 tokens are one
+// contiguous 16 KB piece): the tiles are staged as they lie and every MFMA fragment (tokens along
+// the contraction axis) is a transposing read, so no transposed copy of any operand has to exist
+// for an order-1 problem.  The transposing read hands a lane the 16 tokens of a k-step in `tperm`
+// order, which is the order the per-token weights `cw` are stored in, so a weighted vector sum
+// (sum_t cw_t p_t: the third operand of the backward's walk) takes its B fragment straight from
+// the staged weights.  Tiles are dealt to the wavefronts as in k_build1_seg.
+template <typename E, int DH> struct Build1RowsCfg {
+  static constexpr int TT = 128, PQ = DH + Mma<E>::PAD;
+  static constexpr size_t lds_bytes() { return (size_t(2) * TT * PQ + TT) * sizeof(E); }
+};
+
+template <typename E, int DH>
+FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_build1_rows(BuildArgs<E> A) {
+  typedef Mma<E> M;
+  typedef typename M::frag frag;
+  constexpr int NT = DH / 32, NTILE = NT * NT + 2 * NT, NS = (NTILE + 3) / 4;
+  constexpr int TT = Build1RowsCfg<E, DH>::TT, PQ = Build1RowsCfg<E, DH>::PQ;
+  FM_DYN_SMEM(smem);
+  E* Lp = reinterpret_cast<E*>(smem);                  // [TT][PQ] each
+  E* Lr = Lp + TT * PQ;
+  E* Lc = Lr + TT * PQ;                                // [TT] weights
+  const int tid = FM_TID_X, lane = tid & 63, lh = lane >> 5;
+  const int wave = FM_UNIFORM(tid >> 6);
+  const int bh = FM_BID_Y;
+  int tb, te, slot;
+  fm_walk_step(A.mode, A.nseg, A.L, A.npad, FM_BID_Z, tb, te, slot);
+  E* big = A.big + int64_t(bh) * A.nslots * StateDims<DH>::stride(A.quad != 0);
+  E* big2 = A.big2 ? A.big2 + int64_t(bh) * A.nslots * StateDims<DH>::stride(A.quad != 0) : nullptr;
+  float* ds = A.small + (int64_t(bh) * A.nslots + slot) * StateDims<DH>::SMALL;
+  const bool has_w = A.cw != nullptr;
+  const E* gp = A.pr + int64_t(bh) * A.npad * DH;
+  const E* gr = A.rr + int64_t(bh) * A.npad * DH;
+  const E* gc = has_w ? A.cw + int64_t(bh) * A.npad : nullptr;
+  // the tiles of this wavefront: A operand (tile, feature offset), B operand (tile or null = weights / ones)
+  const E* ta[NS]; const E* tbt[NS];
+  int fa_off[NS], fb_off[NS], tl[NS];
+  bool wsum[NS];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) {
+    const int t = wave + 4 * s;
+    tl[s] = t;
+    ta[s] = Lp; tbt[s] = nullptr; fa_off[s] = 0; fb_off[s] = 0; wsum[s] = false;
+    if (t < NT * NT) { fa_off[s] = 32 * (t / NT); tbt[s] = Lr; fb_off[s] = 32 * (t % NT); }
+    else if (t < NT * NT + NT) {
+      fa_off[s] = 32 * (t - NT * NT);
+      if (A.za_sel == FM_SRC_R) ta[s] = Lr;
+      wsum[s] = A.za_sel == FM_SRC_Z;                   // sum_t cw_t p_t
+    } else if (t < NTILE) {
+      fa_off[s] = 32 * (t - NT * NT - NT);
+      if (A.vb_from_r) ta[s] = Lr;
+    }
+  }
+  fm_f32x16 acc[NS];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) acc[s] = fm_zero16();
+  const frag ones = M::splat(E(1.0f));
+  TileRegs<E, TT, DH> rp, rr;
+  E creg = E(0.f);
+  auto fetch = [&](int t0) {                            // global memory -> registers
+    rp.load(gp + int64_t(t0) * DH, DH, tid);
+    rr.load(gr + int64_t(t0) * DH, DH, tid);
+    if (has_w && tid < TT) creg = gc[t0 + tid];
+  };
+  fetch(tb);
+  for (int t0 = tb; t0 < te; t0 += TT) {
+    if (t0 != tb) FM_SYNC();                            // the previous tile has been read
+    rp.store(Lp, PQ, tid);
+    rr.store(Lr, PQ, tid);
+    if (has_w && tid < TT) Lc[tid] = creg;
+    if (t0 + TT < te) fetch(t0 + TT);
+    FM_SYNC();
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+      if (tl[s] < NTILE) {
+#pragma unroll 4
+        for (int k = 0; k < TT; k += M::KSTEP) {
+          const frag fa = M::load_tr(ta[s], PQ, k, fa_off[s], lane);
+          const frag fb = tbt[s] ? M::load_tr(tbt[s], PQ, k, fb_off[s], lane)
+                                 : (wsum[s] ? M::load_perm(Lc + k, 0, lh) : ones);
+          acc[s] = M::mma(fa, fb, acc[s]);
+        }
+      }
+  }
+  const int lr = lane & 31;
 #pragma unroll
   for (int s = 0; s < NS; ++s)
     if (tl[s] < NTILE) {
