@@ -25,6 +25,7 @@ template <> struct Mma<fm_half> {
   static FM_DEVICE fm_f32x16 mma(frag a, frag b, fm_f32x16 c) { return fm_mfma_f16(a, b, c); }
   static FM_DEVICE frag load(const fm_half* p) { return *reinterpret_cast<const fm_half8*>(p); }
   static FM_DEVICE frag splat(fm_half x) { frag r = {x, x, x, x, x, x, x, x}; return r; }
+  static FM_DEVICE float elem(const frag& f, int i) { return float(f[i]); }   // operand element i of a lane's fragment
   // Transposed token tiles are stored with the 16 tokens of every group in the order
   // 0-3, 8-11, 4-7, 12-15 (`tperm`), so that the eight accumulator rows a lane needs for
   // accumulator k-step s (16s + 4lh + {0..3}, 16s + 8 + 4lh + {0..3}) are one 16-byte read.
@@ -64,6 +65,7 @@ template <> struct Mma<float> {
   static FM_DEVICE fm_f32x16 mma(frag a, frag b, fm_f32x16 c) { return fm_mfma_f32(a, b, c); }
   static FM_DEVICE frag load(const float* p) { return *p; }
   static FM_DEVICE frag splat(float x) { return x; }
+  static FM_DEVICE float elem(const frag& f, int) { return f; }
   static FM_DEVICE int tperm(int t) { return t; }
   static FM_DEVICE frag load_perm(const float* row, int s, int lh) { return row[8 * (s / 4) + 4 * lh + (s % 4)]; }
   static constexpr bool HAS_TR = false;

@@ -266,13 +266,13 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
   for (int j = 0; j < QT; ++j) gsum[j] = 0.f;
 
   if (G.use_state) {
-    if (OWN == FM_OWN_Q) {
+    if (OWN == FM_OWN_Q && A.quad) {
       // denominator: g_i += sum_m q_im (va[m] + sum_l Z[m][l] q_il)
 #pragma unroll
       for (int j = 0; j < QT; ++j)
 #pragma unroll
         for (int mt = 0; mt < NT; ++mt) {
-          const fm_f32x16 y = A.quad ? fm_zy<E, DH, QT>(R, of[j], mt, lr, lh) : fm_zero16();
+          const fm_f32x16 y = fm_zy<E, DH, QT>(R, of[j], mt, lr, lh);
 #pragma unroll
           for (int e = 0; e < 16; ++e) {
             const int m = 32 * mt + fm_acc_row(e, lh);
@@ -280,6 +280,16 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
           }
         }
       FM_SYNC();                                       // Z is overwritten by the slabs
+    } else if (OWN == FM_OWN_Q) {
+      // order 1: g_i += q_i . va, from the half of its row that the lane holds as B fragments (the
+      // other half is the other 32 lanes'; the two meet in the epilogue).  No Z was staged, so
+      // nothing has to be waited for before the state readout.
+#pragma unroll
+      for (int j = 0; j < QT; ++j)
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks)
+#pragma unroll
+          for (int i = 0; i < M::KPL; ++i) gsum[j] += vecs[ks * M::KSTEP + lh * M::KPL + i] * M::elem(of[j][ks], i);
     }
     const E* state = A.big + (int64_t(bh) * A.nslots + G.slot) * StateDims<DH>::stride(A.quad != 0);
     fm_readout<E, DH, QT, NT>(state, A.quad != 0, Own, xrow, of, R, acc, tid);
