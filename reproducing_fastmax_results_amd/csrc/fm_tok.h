@@ -369,6 +369,8 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
 #pragma unroll
         for (int j = 0; j < QT; ++j) {
           const int ss0 = s0 + 32 * st, lo = t0 + tw[j] * 32;
+          // two tiles per wavefront: skip the second half of tile pairs wholly outside the mask (see k_ds)
+          if (QT == 2 && causal && (OWN == FM_OWN_Q ? (ss0 > lo + 31) : (ss0 + 31 < lo))) continue;
           const bool edge = fm_tile_edge<OWN>(causal, ss0, lo, A.n_str);
           int wlo, whi;
           fm_tile_window<OWN>(causal, ss0, lo, lr, A.n_str, wlo, whi);
