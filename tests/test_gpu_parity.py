@@ -32,6 +32,18 @@ def test_mfma_lane_layout(lib):
     assert torch.equal(a32.cpu(), want)
 
 
+def test_matrix_rate_probe_runs(lib):
+    """The bench's yardstick: a register-only loop of matrix products; here only that it runs, writes
+    every checksum and reports a rate (16 workgroups, 64 rounds)."""
+    import ctypes as C
+    out = torch.full((16 * 256,), float("nan"), device=DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    assert lib.lib.fastmax_probe_mfma_rate(16, 64, C.c_void_p(out.data_ptr()), C.c_void_p(stream)) == 0
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all())
+    assert lib.mfma_rate(DEV, workgroups=256, iters=200) > 0.0
+
+
 def test_lds_transpose_read_layout(lib):
     """The kernels (and the host simulator) assume: inside each group of 16 lanes, lane i receives
     element i % 4 of the four-value words addressed by lanes i/4, 4 + i/4, 8 + i/4, 12 + i/4."""
