@@ -115,9 +115,10 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
     // Segment length.  Dense tiles cost grows with L, the moment states cost the same per token
     // whatever L is (readout) plus the walk that builds them.  Measured on MI355X (D = 64, bf16):
     // order 2: one segment (no states at all) wins up to about 6000 tokens, 1024-token segments
-    // beyond; order 1 (one D x D state per segment): one segment up to about 1500 tokens,
+    // beyond; order 1 (one D x D state per segment): one segment up to 1024 tokens (0.150 against 0.159 ms
+    // per step at B*H = 128; at 1536 tokens, B*H = 96: 0.209 against 0.190),
     // 256-token segments beyond.
-    const int auto_L = p.quad ? (d->nq > 6144 ? 1024 : p.npad_q) : (d->nq > 1536 ? 256 : p.npad_q);
+    const int auto_L = p.quad ? (d->nq > 6144 ? 1024 : p.npad_q) : (d->nq > 1024 ? 256 : p.npad_q);
     int L = d->chunk > 0 ? int(round_up(d->chunk, 256)) : auto_L;
     if (force_dense || L > p.npad_q) L = p.npad_q;
     p.L = L;

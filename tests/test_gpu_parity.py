@@ -135,7 +135,7 @@ def test_long_sequence_default_segments(lib, dtype):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("d", [32, 64])
 def test_order1_default_segments(lib, dtype, d):
-    # order 1 beyond 1536 tokens: 256-token segments summed apart, then scanned (16 and 28 segments, the
+    # order 1 beyond 1024 tokens: 256-token segments summed apart, then scanned (16 and 28 segments, the
     # second with a ragged end); unmasked with many keys: one total over all keys by a single walk step
     print(f"case order1 segments dtype={dtype} d={d}", flush=True)
     check_forward_backward(lib, 3, 4096, d, dtype, DEV, mask=True, p=1, seed=22, saved=True)
