@@ -140,8 +140,11 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   const size_t tk = size_t(d->bh) * d->d * p.npad_k * p.esz;
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off = align256(off + bytes); return o; };
-  p.kt = take(tk);
-  p.vt = take(tk);
+  // transposed copies: only the order-2 state walk, the one-total order-1 walk and the fp32 kernels read them
+  const bool need_t = !(p.half && (!p.use_state || p.rows_build));
+  const size_t tkt = need_t ? tk : 0, tqt = need_t ? tq : 0;
+  p.kt = take(tkt);
+  p.vt = take(tkt);
   p.kr = take(tk);
   p.big = take(bigarr);
   p.small = take(size_t(d->bh) * p.nslots * smallsz);
@@ -150,9 +153,9 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   p.big2 = take(p.save ? bigarr : 0);
   p.fwd_bytes = off ? off : 256;
   off = 0;
-  p.b_kt = take(tk); p.b_vt = take(tk); p.b_qt = take(tq); p.b_qct = take(tq);
+  p.b_kt = take(tkt); p.b_vt = take(tkt); p.b_qt = take(tqt); p.b_qct = take(tqt);
   p.b_kr = take(tk); p.b_vr = take(tk); p.b_qr = take(tq);
-  p.b_gh = take(tq); p.b_ght = take(tq);
+  p.b_gh = take(tq); p.b_ght = take(tqt);
   p.b_cv = take(size_t(d->bh) * p.npad_q * 4);
   p.b_bigq = take(bigarr); p.b_smallq = take(size_t(d->bh) * p.nslots * smallsz);
   p.b_bigk = take(bigarr); p.b_smallk = take(size_t(d->bh) * p.nslots * smallsz);
