@@ -37,6 +37,9 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel at the workload below, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this file scaled by a copy of known size; keyed by (dtype, --chunk, kernel).
 TRAFFIC_BYTES = {("bf16", 0, "dkv"): 115648 * 1024}
+# the same for --workload long --order 1 (read + written bytes per launch), keyed by kernel
+TRAFFIC_BYTES_LONG_ORDER1 = {"fwd": (593327 + 135168) * 1024, "dq": (562733 + 131072) * 1024,
+                             "dk": (601611 + 176955) * 1024, "dv": (593267 + 131072) * 1024}
 
 WORKLOAD = dict(name="configs[1]: causal order-2 fwd+bwd", B=4, H=8, N=4096, D=64, p=2, mask=True, scale=1.0)
 # not a bench line of its own: the long-context parity configuration, selectable for profiling (--workload long)
@@ -267,6 +270,8 @@ def main() -> int:
                                      "frac": executed / (ms_per_step * 1e-3) / 1e12 / peak}
     if args.workload == "headline" and p == 2 and TRAFFIC_BYTES.get((args.dtype, args.chunk, dominant)) is not None:
         roofline["traffic"] = TRAFFIC_BYTES[(args.dtype, args.chunk, dominant)]
+    if args.workload == "long" and p == 1 and args.dtype == "bf16" and args.chunk == 0:
+        roofline["traffic"] = TRAFFIC_BYTES_LONG_ORDER1.get(dominant)
 
     out = {
         "metric": f"Fastmax fwd+bwd tokens/s, causal order-{p} N={N} D={D}",
