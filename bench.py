@@ -39,7 +39,7 @@ PEAK_HBM_GBS = 8000.0
 TRAFFIC_BYTES = {("bf16", 0, "dkv"): 115648 * 1024}
 # the same for --workload long --order 1 (read + written bytes per launch), keyed by kernel
 TRAFFIC_BYTES_LONG_ORDER1 = {"fwd": (593327 + 135168) * 1024, "dq": (562733 + 131072) * 1024,
-                             "dk": (601611 + 176955) * 1024, "dv": (593267 + 131072) * 1024}
+                             "dk": (601611 + 176955) * 1024, "dv": (428990 + 131072) * 1024}
 
 WORKLOAD = dict(name="configs[1]: causal order-2 fwd+bwd", B=4, H=8, N=4096, D=64, p=2, mask=True, scale=1.0)
 # not a bench line of its own: the long-context parity configuration, selectable for profiling (--workload long)
