@@ -35,10 +35,24 @@ enum { FASTMAX_F32 = 0, FASTMAX_BF16 = 1 };
 enum {
   FASTMAX_FLAG_FORCE_MOMENTS = 1,   /* unmasked: always use the moment (linear-time) path */
   FASTMAX_FLAG_FORCE_DENSE = 2,     /* never build moment states (quadratic-time path) */
-  FASTMAX_FLAG_SAVE_FOR_BACKWARD = 4 /* forward: also leave in its workspace what the backward of the same
+  FASTMAX_FLAG_SAVE_FOR_BACKWARD = 4, /* forward: also leave in its workspace what the backward of the same
                                         problem can reuse (converted k, v and the key-side moment states);
                                         forward_bytes grows accordingly */
+  FASTMAX_FLAG_F32_COMPUTE = 8       /* bf16 tensors: do all arithmetic in fp32 (matrix products included)
+                                        instead of _Float16; for inputs outside the range stated below.
+                                        Many times slower; workspace sizes grow.  Ignored for fp32 tensors. */
 };
+
+/* Numeric range of the bf16 interface.  bf16 tensors are computed in _Float16 with fp32 accumulation
+ * (the order-2 operands k_a * k_b have to be formed on the fly, and gfx950 has packed half
+ * multiplies but no packed bf16 arithmetic).  _Float16 has 11 significand bits (bf16: 8) but a
+ * narrow exponent: values beyond 65504 become infinities and values below 6e-5 lose precision.
+ * Supported: |s_ij| = |q_i . k_j| * inv_tau <= 250 for every pair (so that a2 * s^2 <= 65504 / 2 for
+ * a2 = 1/2; in general |a1 s| + |a2| s^2 < 6e4), |q|, |k| * sqrt(inv_tau) <= 6e4, and v, dO of
+ * ordinary magnitude (about 1e-3 .. 1e4).  The reference model's normalised q and k (|q_i|, |k_j| <=
+ * lim, transformer/model.py:97-102) satisfy this by construction.  Nothing saturates: an input
+ * beyond the range turns into infinities that reach the outputs as inf / NaN rather than as finite
+ * wrong numbers.  FASTMAX_FLAG_F32_COMPUTE lifts the limits at fp32 speed. */
 
 /* Where slice i of the batch*head axis, token t, feature f of a tensor lives:
  *   heads <= 1:  i * bh + t * n + f

@@ -18,7 +18,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_NAME = "libfastmax_hip.so"
 
 F32, BF16 = 0, 1
-FLAG_FORCE_MOMENTS, FLAG_FORCE_DENSE, FLAG_SAVE_FOR_BACKWARD = 1, 2, 4
+FLAG_FORCE_MOMENTS, FLAG_FORCE_DENSE, FLAG_SAVE_FOR_BACKWARD, FLAG_F32_COMPUTE = 1, 2, 4, 8
 STATUS_OK = 0
 
 
@@ -79,6 +79,10 @@ def _strides(t: torch.Tensor) -> Strides:
         raise FastmaxError("fastmax: the feature axis must be contiguous")
     if t.dim() == 3:
         return Strides(t.stride(0), t.stride(1))
+    if t.shape[1] == 1:
+        # one head per batch: the batch stride is the stride of the whole axis (stride(1) of such a view is
+        # arbitrary: d for the transposed (b, n, 1, d) projection layout)
+        return Strides(t.stride(0), t.stride(2))
     return Strides(t.stride(1), t.stride(2), t.stride(0), t.shape[1])
 
 
@@ -91,6 +95,8 @@ def _dims(t: torch.Tensor):
 
 def _gstrides(g: torch.Tensor) -> Strides:
     """Strides of the denominators: (bh, n) or (b, h, n)."""
+    if g.dim() == 3 and g.shape[1] == 1:
+        return Strides(g.stride(0), g.stride(2))
     if g.dim() == 3:
         return Strides(g.stride(1), g.stride(2), g.stride(0), g.shape[1])
     return Strides(g.stride(0), g.stride(1))

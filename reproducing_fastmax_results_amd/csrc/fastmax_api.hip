@@ -5,19 +5,33 @@
 #include "fm_tok.h"
 #include "fm_norm.h"
 #include "fm_split.h"
+#include <atomic>
 #include <cmath>
+#include <mutex>
+#include <unordered_map>
 #include <vector>
 
 namespace {
 
+inline int fm_launch_status() { return fm_after_launch() ? FASTMAX_ERR_LAUNCH : FASTMAX_OK; }
 #if defined(FM_HOSTSIM)
-inline int fm_after_launch() { return FASTMAX_OK; }
 inline void fm_allow_lds(const void*, size_t) {}
 #else
-inline int fm_after_launch() { return hipGetLastError() == hipSuccess ? FASTMAX_OK : FASTMAX_ERR_LAUNCH; }
+// Dynamic LDS above the 64 KiB default has to be allowed once per kernel function (and device); the
+// attribute call costs microseconds of host time, so it is made the first time a kernel asks for more
+// than it has been granted so far and skipped afterwards.
 inline void fm_allow_lds(const void* fn, size_t bytes) {
-  // needed above the 64 KiB default; harmless below it
-  (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, int(bytes));
+  if (bytes <= 64 * 1024) return;
+  struct Key { const void* fn; int dev; bool operator==(const Key& o) const { return fn == o.fn && dev == o.dev; } };
+  struct Hash { size_t operator()(const Key& k) const { return std::hash<const void*>()(k.fn) ^ (size_t(k.dev) * 0x9e3779b97f4a7c15ull); } };
+  static std::mutex mu;
+  static std::unordered_map<Key, size_t, Hash> granted;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+  std::lock_guard<std::mutex> lock(mu);
+  size_t& have = granted[Key{fn, dev}];
+  if (bytes <= have) return;
+  if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, int(bytes)) == hipSuccess) have = bytes;
 }
 #endif
 
@@ -27,11 +41,11 @@ enum { FM_K_TRANSPOSE = 0, FM_K_PREP_BWD = 1, FM_K_BUILD = 2, FM_K_FWD = 3, FM_K
 struct ProfScope { ProfScope(int, fm_stream_t) {} };
 #else
 struct ProfRec { int id; hipEvent_t a, b; };
-bool g_prof_on = false;
+std::atomic<bool> g_prof_on{false};   // read by every launch: atomic, so that a launch on another thread sees a whole value
 std::vector<ProfRec> g_prof;
 struct ProfScope {
   bool on; fm_stream_t s; size_t idx;
-  ProfScope(int id, fm_stream_t stream) : on(g_prof_on), s(stream), idx(0) {
+  ProfScope(int id, fm_stream_t stream) : on(g_prof_on.load(std::memory_order_relaxed)), s(stream), idx(0) {
     if (!on) return;
     ProfRec r; r.id = id;
     hipEventCreate(&r.a); hipEventCreate(&r.b);
@@ -78,6 +92,9 @@ int validate(const FastmaxDesc* d) {
   if (d->dtype != FASTMAX_F32 && d->dtype != FASTMAX_BF16) return FASTMAX_ERR_DTYPE;
   if (d->bh <= 0 || d->nq <= 0 || d->nk <= 0 || d->d <= 0) return FASTMAX_ERR_SHAPE;
   if (d->bh > 65535) return FASTMAX_ERR_SHAPE;
+  // padded lengths, segment lengths and their byte counts are formed in 32- and 64-bit arithmetic that
+  // assumes token counts and the segment length stay below 2^30
+  if (d->nq > (1 << 30) || d->nk > (1 << 30) || d->chunk > (1 << 30)) return FASTMAX_ERR_SHAPE;
   if (d->p != 1 && d->p != 2) return FASTMAX_ERR_UNSUPPORTED;
   if (d->d != 32 && d->d != 64) return FASTMAX_ERR_UNSUPPORTED;
   if (d->mask && d->nq > d->nk) return FASTMAX_ERR_UNSUPPORTED;   // nk > nq: see SplitPlan
@@ -96,7 +113,7 @@ template <int DH> size_t big_array_bytes(int esz, bool quad, size_t slots) {
 int make_plan(const FastmaxDesc* d, Plan& p) {
   int st = validate(d);
   if (st != FASTMAX_OK) return st;
-  p.half = d->dtype == FASTMAX_BF16;
+  p.half = d->dtype == FASTMAX_BF16 && !(d->flags & FASTMAX_FLAG_F32_COMPUTE);
   p.esz = p.half ? 2 : 4;
   p.npad_q = int(round_up(d->nq, 256));
   p.npad_k = int(round_up(d->nk, 256));
@@ -119,7 +136,7 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
     // per step at B*H = 128; at 1536 tokens, B*H = 96: 0.209 against 0.190),
     // 256-token segments beyond.
     const int auto_L = p.quad ? (d->nq > 6144 ? 1024 : p.npad_q) : (d->nq > 1024 ? 256 : p.npad_q);
-    int L = d->chunk > 0 ? int(round_up(d->chunk, 256)) : auto_L;
+    int L = d->chunk > 0 ? (d->chunk >= d->nq ? p.npad_q : int(round_up(d->chunk, 256))) : auto_L;
     if (force_dense || L > p.npad_q) L = p.npad_q;
     p.L = L;
     p.nseg = (d->nq + L - 1) / L;
@@ -177,7 +194,7 @@ int launch_transpose2(const void* x0, const FastmaxStrides& s0, E* xt0, E* xr0, 
   const TransposeJob<TIO, E> j0{cref<TIO>(x0, s0), xt0, xr0, scale0}, j1{cref<TIO>(x1, s1), xt1, xr1, scale1};
   ProfScope prof(FM_K_TRANSPOSE, stream);
   FM_KERNEL_LAUNCH((k_transpose<TIO, E, DH>), fm_dim3(npad / 64, bh, 2), fm_dim3(FM_THREADS), 0, stream, j0, j1, n, npad);
-  return fm_after_launch();
+  return fm_launch_status();
 }
 
 // per-segment sums -> prefix / suffix states (after a build whose workgroups took one step each)
@@ -190,7 +207,7 @@ int launch_scan(const BuildArgs<E>& a, int bh, int nsteps, fm_stream_t stream) {
   // four times as many CUs each of them moves a quarter of the bytes
   FM_KERNEL_LAUNCH((k_state_scan<E, DH>), fm_dim3(int((total + FM_SCAN_THREADS - 1) / FM_SCAN_THREADS), bh),
                    fm_dim3(FM_SCAN_THREADS), 0, stream, a.big, a.big2, a.small, a.nslots, nsteps, a.mode, a.nseg, a.quad);
-  return fm_after_launch();
+  return fm_launch_status();
 }
 
 template <typename E, int DH, int NA, int TT, int SPW, int KB>
@@ -205,7 +222,7 @@ int launch_build_cfg(const BuildArgs<E>& a, int groups, int bh, int nsteps, fm_s
   fm_allow_lds(reinterpret_cast<const void*>(&k_build<E, DH, NA, TT, SPW, KB>), lds);
   FM_KERNEL_LAUNCH((k_build<E, DH, NA, TT, SPW, KB>), fm_dim3(groups, bh, a.seg_parallel ? nsteps : 1),
                    fm_dim3(FM_THREADS), lds, stream, a);
-  int st = fm_after_launch();
+  int st = fm_launch_status();
   if (st || !a.seg_parallel || nsteps < 2) return st;
   return launch_scan<E, DH>(a, bh, nsteps, stream);
 }
@@ -256,7 +273,7 @@ int launch_build(const BuildArgs<E>& args, int bh, fm_stream_t stream) {
     const size_t ldsr = Build1RowsCfg<E, DH>::lds_bytes();
     fm_allow_lds(reinterpret_cast<const void*>(&k_build1_rows<E, DH>), ldsr);
     FM_KERNEL_LAUNCH((k_build1_rows<E, DH>), fm_dim3(1, bh, nsteps), fm_dim3(FM_THREADS), ldsr, stream, a);
-    const int st = fm_after_launch();
+    const int st = fm_launch_status();
     return (st || nsteps < 2) ? st : launch_scan<E, DH>(a, bh, nsteps, stream);
   }
   if (nsteps > 1) {
@@ -264,13 +281,13 @@ int launch_build(const BuildArgs<E>& args, int bh, fm_stream_t stream) {
     const size_t lds1 = Build1Cfg<E, DH>::lds_bytes(a.zt != nullptr && a.za_sel == FM_SRC_Z);
     fm_allow_lds(reinterpret_cast<const void*>(&k_build1_seg<E, DH>), lds1);
     FM_KERNEL_LAUNCH((k_build1_seg<E, DH>), fm_dim3(1, bh, nsteps), fm_dim3(FM_THREADS), lds1, stream, a);
-    const int st = fm_after_launch();
+    const int st = fm_launch_status();
     return st ? st : launch_scan<E, DH>(a, bh, nsteps, stream);
   }
   const size_t lds = size_t(4) * 4 * 64 * 16 * 4;
   fm_allow_lds(reinterpret_cast<const void*>(&k_build1<E, DH>), lds);
   FM_KERNEL_LAUNCH((k_build1<E, DH>), fm_dim3(1, bh, nsteps), fm_dim3(FM_THREADS), lds, stream, a);
-  return fm_after_launch();
+  return fm_launch_status();
 }
 
 // Dynamic LDS of a token kernel (kind 0: k_pv, 1: k_ds, 2: k_ds with dV, 3: k_ds with the fused
@@ -311,7 +328,7 @@ int launch_pv(const TokArgs<TIO, E>& a, int bh, int kernel_id, fm_stream_t strea
   ProfScope prof(kernel_id, stream);
   FM_KERNEL_LAUNCH((k_pv<TIO, E, DH, QT, OWN>), fm_dim3((a.n_own + C::QW - 1) / C::QW, bh), fm_dim3(FM_THREADS), lds,
                    stream, a);
-  return fm_after_launch();
+  return fm_launch_status();
 }
 
 template <typename TIO, typename E, int DH, int QT, int OWN, int DV = 0, int PREP = 0>
@@ -322,7 +339,7 @@ int launch_ds(const TokArgs<TIO, E>& a, int bh, int kernel_id, fm_stream_t strea
   ProfScope prof(kernel_id, stream);
   FM_KERNEL_LAUNCH((k_ds<TIO, E, DH, QT, OWN, DV, PREP>), fm_dim3((a.n_own + C::QW - 1) / C::QW, bh), fm_dim3(FM_THREADS), lds,
                    stream, a);
-  return fm_after_launch();
+  return fm_launch_status();
 }
 
 template <typename TIO, typename E, int DH, int QT>
@@ -422,7 +439,7 @@ int merge_parts(const FastmaxDesc* d, const SplitPlan& sp, const void* oa, const
   FM_KERNEL_LAUNCH((k_merge_parts<TIO, DH>), fm_dim3(int((items + 255) / 256), d->bh), fm_dim3(256), 0, stream, oar, gar,
                    mref<TIO>(o, d->so), gr, d->nq);
   FM_KERNEL_LAUNCH(k_merge_denominators, fm_dim3((d->nq + 255) / 256, d->bh), fm_dim3(256), 0, stream, gar, gr, d->nq);
-  return fm_after_launch();
+  return fm_launch_status();
 }
 
 template <typename TIO, int DH>
@@ -430,7 +447,7 @@ int add_rows(const FastmaxDesc* d, const SplitPlan& sp, const void* dqa, void* d
   const int64_t items = int64_t(d->nq) * (DH / 8);
   FM_KERNEL_LAUNCH((k_add_rows<TIO, DH>), fm_dim3(int((items + 255) / 256), d->bh), fm_dim3(256), 0, stream,
                    cref<TIO>(dqa, sp.head_b.sdq), mref<TIO>(dq, d->sdq), d->nq);
-  return fm_after_launch();
+  return fm_launch_status();
 }
 
 }  // namespace
@@ -491,6 +508,10 @@ static int forward_one(const FastmaxDesc* desc, const void* q, const void* k, co
     if (desc->d == 64) return run_forward<fm_bf16, fm_half, 64, 1>(desc, p, q, k, v, o, g, ws, stream);
     return run_forward<fm_bf16, fm_half, 32, 1>(desc, p, q, k, v, o, g, ws, stream);
   }
+  if (desc->dtype == FASTMAX_BF16) {               // bf16 tensors, fp32 arithmetic (FASTMAX_FLAG_F32_COMPUTE)
+    if (desc->d == 64) return run_forward<fm_bf16, float, 64, 1>(desc, p, q, k, v, o, g, ws, stream);
+    return run_forward<fm_bf16, float, 32, 1>(desc, p, q, k, v, o, g, ws, stream);
+  }
   if (desc->d == 64) return run_forward<float, float, 64, 1>(desc, p, q, k, v, o, g, ws, stream);
   return run_forward<float, float, 32, 1>(desc, p, q, k, v, o, g, ws, stream);
 }
@@ -550,6 +571,10 @@ static int backward_one(const FastmaxDesc* desc, const void* q, const void* k, c
   if (p.half) {
     if (desc->d == 64) return run_backward<fm_bf16, fm_half, 64, 1>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);
     return run_backward<fm_bf16, fm_half, 32, 1>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);
+  }
+  if (desc->dtype == FASTMAX_BF16) {
+    if (desc->d == 64) return run_backward<fm_bf16, float, 64, 1>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);
+    return run_backward<fm_bf16, float, 32, 1>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);
   }
   if (desc->d == 64) return run_backward<float, float, 64, 1>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);
   return run_backward<float, float, 32, 1>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);
@@ -657,7 +682,7 @@ int fastmax_profile_end(int* kernel_ids, float* milliseconds, int capacity) {
 int fastmax_probe_mfma(float* out_f16, float* out_f32, void* hip_stream) {
   if (!out_f16 || !out_f32) return FASTMAX_ERR_NULL;
   FM_KERNEL_LAUNCH(k_probe_mfma, fm_dim3(1), fm_dim3(64), 0, static_cast<fm_stream_t>(hip_stream), out_f16, out_f32);
-  return fm_after_launch();
+  return fm_launch_status();
 }
 
 int fastmax_probe_mfma_rate(int workgroups, int iters, float* out, void* hip_stream) {
@@ -665,13 +690,13 @@ int fastmax_probe_mfma_rate(int workgroups, int iters, float* out, void* hip_str
   if (workgroups <= 0 || workgroups > 65536 || iters <= 0 || iters > (1 << 20)) return FASTMAX_ERR_SHAPE;
   FM_KERNEL_LAUNCH(k_probe_mfma_rate, fm_dim3(workgroups), fm_dim3(FM_THREADS), 0, static_cast<fm_stream_t>(hip_stream),
                    out, iters);
-  return fm_after_launch();
+  return fm_launch_status();
 }
 
 int fastmax_probe_lds_transpose(float* out, void* hip_stream) {
   if (!out) return FASTMAX_ERR_NULL;
   FM_KERNEL_LAUNCH(k_probe_lds_tr, fm_dim3(1), fm_dim3(64), 0, static_cast<fm_stream_t>(hip_stream), out);
-  return fm_after_launch();
+  return fm_launch_status();
 }
 
 }  // extern "C"

@@ -174,7 +174,10 @@ View view_of(const torch::Tensor& t_, const char* name) {
     w.s = FastmaxStrides{x.stride(0), x.stride(1), 0, 0, 0};
     w.bh = x.size(0); w.n = x.size(1); w.d = x.size(2);
   } else {
-    w.s = FastmaxStrides{x.stride(1), x.stride(2), x.stride(0), static_cast<int32_t>(x.size(1)), 0};
+    // one head per batch: the batch stride is the stride of the whole batch*head axis (stride(1) of such
+    // a view says nothing: for the projection layout (b, n, 1, d) transposed it is d)
+    if (x.size(1) == 1) w.s = FastmaxStrides{x.stride(0), x.stride(2), 0, 0, 0};
+    else w.s = FastmaxStrides{x.stride(1), x.stride(2), x.stride(0), static_cast<int32_t>(x.size(1)), 0};
     w.bh = x.size(0) * x.size(1); w.n = x.size(2); w.d = x.size(3);
   }
   return w;
@@ -192,6 +195,7 @@ torch::Tensor empty_like_layout(const torch::Tensor& like, int64_t n, torch::Sca
 }
 
 FastmaxStrides gstrides_of(const torch::Tensor& g) {
+  if (g.dim() == 3 && g.size(1) == 1) return FastmaxStrides{g.stride(0), g.stride(2), 0, 0, 0};
   if (g.dim() == 3) return FastmaxStrides{g.stride(1), g.stride(2), g.stride(0), static_cast<int32_t>(g.size(1)), 0};
   return FastmaxStrides{g.stride(0), g.stride(1), 0, 0, 0};
 }
@@ -203,6 +207,9 @@ FastmaxDesc ex_desc(const View& q, const View& k, const View& v, bool mask, doub
               "q, k, v must be (bh, nq, d), (bh, nk, d), (bh, nk, d)");
   TORCH_CHECK(k.t.scalar_type() == q.t.scalar_type() && v.t.scalar_type() == q.t.scalar_type(),
               "q, k, v must share one dtype");
+  TORCH_CHECK(chunk >= 0 && chunk <= (int64_t(1) << 30), "chunk must be between 0 and 2^30, got ", chunk);
+  TORCH_CHECK(flags >= 0 && flags <= 15, "unknown flags ", flags);
+  TORCH_CHECK(q.bh <= 65535 && q.n <= (int64_t(1) << 30) && k.n <= (int64_t(1) << 30), "problem too large for 32-bit sizes");
   FastmaxDesc d{};
   d.bh = static_cast<int32_t>(q.bh); d.nq = static_cast<int32_t>(q.n); d.nk = static_cast<int32_t>(k.n);
   d.d = static_cast<int32_t>(q.d); d.dtype = dtype_code(q.t);

@@ -143,17 +143,18 @@ template <> struct IO<fm_bf16> {
 };
 
 // ---- compute element types ----------------------------------------------------
-// Conversion to _Float16 saturates at the largest finite half so that an
-// out-of-range input degrades instead of producing infinities.
+// Conversion to _Float16 rounds to nearest and does NOT saturate: a value beyond the largest finite
+// half (65504) becomes an infinity, which every kernel carries through to a non-finite output.  An input
+// outside the supported range therefore shows as inf / NaN in the results, never as a finite wrong number.
 template <typename E> struct CE;
 template <> struct CE<fm_half> {
-  static FM_DEVICE fm_half from(float x) { return fm_half(fm_clampf(x, 65504.f)); }
+  static FM_DEVICE fm_half from(float x) { return fm_half(x); }
   // eight consecutive elements to LDS / workspace (16-byte aligned)
   static FM_DEVICE void st8(fm_half* p, const float in[8]) {
     fm_half8 h;
 #pragma unroll
     for (int i = 0; i < 8; i += 2) {
-      fm_f32x2 v = {fm_clampf(in[i], 65504.f), fm_clampf(in[i + 1], 65504.f)};
+      fm_f32x2 v = {in[i], in[i + 1]};
       const fm_half2 c = __builtin_convertvector(v, fm_half2);
       h[i] = c[0]; h[i + 1] = c[1];
     }

@@ -15,6 +15,10 @@
 // its blocks are issued before the first is used, so a thread has NP * DH / 32 16-byte loads in flight.
 static constexpr int FM_NORM_NP = 4;     // forward kernels and the backward's second pass
 static constexpr int FM_NORMB_NP = 2;    // backward statistics (two tensors per token)
+// A slice whose largest squared norm is not above this value (all zeros: padding) comes out as zeros, with
+// zero gradient, instead of 0 / 0.  (The reference's CUDA kernel floors at 0.1, fastmax_cuda_forward.cu:333;
+// its Python variants do not floor at all; anything that is not an all-zero slice is far above this value.)
+static constexpr float FM_NORM_FLOOR = 1e-30f;
 
 // forward scratch per batch*head (floats): [0], [1] unused; [2 .. 2+d) token mean; then one largest
 // squared norm per workgroup of k_norm_maxnorm; then, with the token-mean centring, d column sums per
@@ -171,7 +175,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_norm_apply(TRef<const TIO> x, TRef<TIO> y
     for (int b = tid & 63; b < nblk; b += 64) m2 = fm_fmaxf(m2, st[2 + DH + b]);
 #pragma unroll
     for (int m = 1; m < 64; m <<= 1) m2 = fm_fmaxf(m2, fm_shfl_xor(m2, m));
-    f = scale / fm_sqrtf(m2);
+    f = m2 > FM_NORM_FLOOR ? scale / fm_sqrtf(m2) : 0.0f;
   }
 #pragma unroll
   for (int p = 0; p < NP; ++p) {
@@ -202,11 +206,7 @@ int fm_normalize_run(const FastmaxNormDesc* d, const void* x, void* y, float* st
     FM_KERNEL_LAUNCH((k_norm_maxnorm<TIO, DH>), grid, fm_dim3(256), 0, stream, xr, d->n, d->centre, stats, stride);
   FM_KERNEL_LAUNCH((k_norm_apply<TIO, DH>), grid, fm_dim3(256), 0, stream, xr, yr, d->n, d->centre, d->max_norm,
                    d->scale, stats, stride);
-#if defined(FM_HOSTSIM)
-  return FASTMAX_OK;
-#else
-  return hipGetLastError() == hipSuccess ? FASTMAX_OK : FASTMAX_ERR_LAUNCH;
-#endif
+  return fm_after_launch() ? FASTMAX_ERR_LAUNCH : FASTMAX_OK;
 }
 
 inline int fm_normalize_dispatch(const FastmaxNormDesc* d, const void* x, void* y, float* stats, fm_stream_t stream) {
@@ -350,8 +350,9 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_normb_apply(TRef<const TIO> x, TRef<const
     __builtin_memcpy(&m2, &bits, 4);
     nstar = int(~uint32_t(key));
     if (nstar < 0 || nstar >= n) nstar = 0;            // no token won (every norm is a NaN)
-    f = scale / fm_sqrtf(m2);
-    kf = red[0] / m2;
+    const bool some = m2 > FM_NORM_FLOOR;
+    f = some ? scale / fm_sqrtf(m2) : 0.0f;
+    kf = some ? red[0] / m2 : 0.0f;
     // every lane takes part in the shuffles of the centring
     fm_norm_load_centred<TIO, DH>(x.base(bh) + int64_t(nstar) * x.s_n, x.vec != 0, d0, centre, st + 4, cs);
   }
@@ -395,11 +396,7 @@ int fm_normalize_bwd_run(const FastmaxNormDesc* d, const void* x, const void* dy
   }
   FM_KERNEL_LAUNCH((k_normb_apply<TIO, DH>), grid, fm_dim3(256), 0, stream, xr, gr, dxr, d->n, d->centre, d->max_norm,
                    d->scale, stats, stride);
-#if defined(FM_HOSTSIM)
-  return FASTMAX_OK;
-#else
-  return hipGetLastError() == hipSuccess ? FASTMAX_OK : FASTMAX_ERR_LAUNCH;
-#endif
+  return fm_after_launch() ? FASTMAX_ERR_LAUNCH : FASTMAX_OK;
 }
 
 inline int fm_normalize_bwd_dispatch(const FastmaxNormDesc* d, const void* x, const void* dy, void* dx, float* stats,

@@ -47,6 +47,7 @@ typedef hostsim::Dim3 fm_dim3;
 #define FM_DYN_SMEM(name) unsigned char* name = hostsim::g_t.blk->dyn_smem
 #define FM_KERNEL_LAUNCH(kern, grid, block, smem, stream, ...) \
   hostsim::launch((grid), (block), (smem), [=]() { kern(__VA_ARGS__); })
+inline int fm_after_launch() { return 0; }
 
 FM_DEVICE fm_f32x16 fm_mfma_f16(fm_half8 a, fm_half8 b, fm_f32x16 c) {
   fm_half av[8], bv[8]; float cv[16];
@@ -121,8 +122,19 @@ typedef dim3 fm_dim3;
 #define FM_GDIM_Y (int(gridDim.y))
 #define FM_SYNC() __syncthreads()
 #define FM_DYN_SMEM(name) extern __shared__ __align__(16) unsigned char name[]
-#define FM_KERNEL_LAUNCH(kern, grid, block, smem, stream, ...) \
-  hipLaunchKernelGGL(kern, (grid), (block), (smem), (stream), __VA_ARGS__)
+// A launch the runtime refuses leaves its error as the calling thread's last error.  Only an error that
+// appears across the launch is this library's: it is taken (cleared) and remembered until
+// fm_after_launch() asks; an error some other library left pending before the launch stays where its
+// owner will look for it and is not blamed on the launch.
+inline thread_local int fm_launch_refused = 0;
+#define FM_KERNEL_LAUNCH(kern, grid, block, smem, stream, ...)                                      \
+  do {                                                                                              \
+    const bool fm_clean_ = hipPeekAtLastError() == hipSuccess;                                      \
+    hipLaunchKernelGGL(kern, (grid), (block), (smem), (stream), __VA_ARGS__);                       \
+    if (fm_clean_ && hipPeekAtLastError() != hipSuccess) { (void)hipGetLastError(); fm_launch_refused = 1; } \
+  } while (0)
+// 0, or non-zero when a launch since the last call was refused
+inline int fm_after_launch() { const int r = fm_launch_refused; fm_launch_refused = 0; return r; }
 
 FM_DEVICE fm_f32x16 fm_mfma_f16(fm_half8 a, fm_half8 b, fm_f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);

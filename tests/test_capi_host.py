@@ -119,6 +119,14 @@ def test_forward_backward_reject_bad_arguments_before_launching(lib):
     assert lib.lib.fastmax_version() >= 105
 
 
+def test_segment_length_and_size_limits(lib):
+    # segment lengths beyond 2^30 and token counts beyond 2^30 are refused (32-bit padding arithmetic)
+    assert ws(lib, base_desc(chunk=2 ** 31 - 1))[0] == 2
+    assert ws(lib, base_desc(chunk=1 << 30))[0] == 0
+    assert ws(lib, base_desc(nq=(1 << 30) + 1, nk=(1 << 30) + 1))[0] == 2
+    assert ws(lib, base_desc(chunk=1 << 20))[1] == ws(lib, base_desc())[1]      # "no chunking" sentinel: one segment
+
+
 def test_normalize_backward_arguments(lib):
     nd = _capi.NormDesc()
     nd.bh, nd.n, nd.d, nd.dtype, nd.centre, nd.max_norm, nd.scale = 4, 130, 64, _capi.F32, 2, 1, 1.0

@@ -100,6 +100,27 @@ def test_autograd_wrapper(sf, dtype, four_d):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_one_head_per_batch_projection_layout(sf, ext, dtype):
+    """(b, n, 1*d) projections viewed as (b, 1, n, d): stride(1) of that view is d, not the distance between
+    the batches; the binding must address batch i at i * n * d (heads_per_block = 1 in the model)."""
+    b, n, d, t = 3, 200, 64, 9.0
+    q, k, v, go = (rnd(b, n, d, seed=s).to(dtype).to(DEV).view(b, n, 1, d).transpose(1, 2) for s in (40, 41, 42, 43))
+    assert q.shape == (b, 1, n, d) and q.stride(1) == d
+    qd, kd, vd = (x.detach().clone().requires_grad_(True) for x in (q, k, v))   # clone keeps the strides
+    assert qd.stride() == q.stride()
+    noise, rpe = torch.zeros_like(qd), sf.rpe_matrix_creator(n, d, DEV, torch.float32)
+    o = sf.FASTMultiHeadAttention_Function.apply(qd, kd, vd, noise, rpe, True, 0.0, False, t, 1.0, 1.0, 0.5, 1.0, 2)
+    o.backward(go)
+    ref = O.manual_backward_blocked(*(x.double().cpu().contiguous() for x in (q, k, v, go)), mask=True, tau=t, p=2)
+    assert rel_err(o, ref[0]) < TOL[dtype]
+    for got, want in ((qd.grad, ref[2]), (kd.grad, ref[3]), (vd.grad, ref[4])):
+        assert rel_err(got, want) < TOL[dtype]
+    o1, g1 = ext.forward_ex(q, k, v, True, 1.0 / t, 1.0, 1.0, 0.5, 2, 0, 0)
+    o2, g2 = ext.forward_ex(q.contiguous(), k.contiguous(), v.contiguous(), True, 1.0 / t, 1.0, 1.0, 0.5, 2, 0, 0)
+    assert torch.equal(o1, o2) and torch.equal(g1, g2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_transposed_projection_layout(sf, ext, dtype):
     """(b, n, h*d) projections viewed as (b, h, n, d) - the layout Attention.forward produces
     (transformer/model.py:283-285) - are consumed through batch and head strides, without a copy,

@@ -193,6 +193,7 @@ def test_batch_and_head_strides(lib, dtype, mask, chunk):
     check_batch_head_strides(lib, 3, 4, 700, 64, dtype, DEV, mask=mask, p=2, chunk=chunk, seed=30)
     check_batch_head_strides(lib, 2, 8, 130, 32, dtype, DEV, mask=mask, p=1, chunk=chunk, seed=31)
     check_batch_head_strides(lib, 2, 4, 1300, 64, dtype, DEV, mask=mask, p=1, chunk=chunk, seed=32)   # order-1 segments
+    check_batch_head_strides(lib, 5, 1, 300, 64, dtype, DEV, mask=mask, p=2, chunk=chunk, seed=33)    # one head per batch
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

@@ -15,7 +15,8 @@ import pytest
 import torch
 
 from reproducing_fastmax_results_amd import _capi
-from tests.parity import check_batch_head_strides, check_forward, check_forward_backward
+from tests.parity import (TOL, check_batch_head_strides, check_forward, check_forward_backward, make_inputs, oracle_all,
+                          rel_err)
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CLANG = shutil.which("clang++", path="/opt/rocm/llvm/bin:" + os.environ.get("PATH", ""))
@@ -76,6 +77,9 @@ def test_batch_and_head_strides(sim):
     # (b, n, h*d) projections viewed as (b, h, n, d): FastmaxStrides with heads > 1
     check_batch_head_strides(sim, 2, 2, 70, 32, torch.bfloat16, "cpu", mask=True, p=2, seed=7)
     check_batch_head_strides(sim, 2, 2, 40, 32, torch.float32, "cpu", mask=False, p=1, seed=8)
+    # one head per batch: stride(1) of the transposed (b, n, 1, d) view is d, the slices lie n*d apart
+    check_batch_head_strides(sim, 3, 1, 40, 32, torch.bfloat16, "cpu", mask=True, p=2, seed=9)
+    check_batch_head_strides(sim, 3, 1, 33, 32, torch.float32, "cpu", mask=False, p=2, seed=10)
 
 
 def test_moment_path_forward_fp32_d64(sim):
@@ -122,3 +126,67 @@ def test_causal_with_more_keys_than_queries(sim):
     check_forward_backward(sim, 1, 40, 32, torch.float32, "cpu", mask=True, p=2, nk=75, seed=13)
     check_forward_backward(sim, 2, 33, 32, torch.bfloat16, "cpu", mask=True, p=1, nk=34, seed=14)
 
+
+
+def test_segment_length_sentinels(sim):
+    # a segment length at or beyond the sequence means "one segment", whatever its size; beyond 2^30 it is rejected
+    import ctypes as C
+    q, k, v, go = make_inputs(1, 300, 300, 32, torch.float32, "cpu", seed=15)
+    kw = dict(mask=True, inv_tau=0.1, p=2)
+    o0, g0 = sim.forward(q, k, v, chunk=0, **kw)
+    for chunk in (300, 301, 1 << 20, 1 << 30):
+        o1, g1 = sim.forward(q, k, v, chunk=chunk, **kw)
+        assert torch.equal(o0, o1) and torch.equal(g0, g1)
+    for chunk in ((1 << 30) + 1, 2 ** 31 - 1):
+        d = sim.make_desc(q, k, v, mask=True, inv_tau=0.1, a0=1.0, a1=1.0, a2=0.5, p=2, chunk=chunk)
+        assert sim.lib.fastmax_workspace_bytes(C.byref(d), None, None) == 2
+    d = sim.make_desc(q, k, v, mask=True, inv_tau=0.1, a0=1.0, a1=1.0, a2=0.5, p=2)
+    d.nq = d.nk = (1 << 30) + 1
+    assert sim.lib.fastmax_workspace_bytes(C.byref(d), None, None) == 2
+
+
+def _domain_case(sim, scale, flags, a=(1.0, 1.0, 0.5)):
+    bh, n, d = 1, 70, 32
+    q, k, v, go = make_inputs(bh, n, n, d, torch.bfloat16, "cpu", seed=16, scale=scale)
+    kw = dict(mask=True, inv_tau=1.0, a0=a[0], a1=a[1], a2=a[2], p=2, flags=flags)
+    o, g = sim.forward(q, k, v, **kw)
+    grads = sim.backward(q, k, v, o, g, go, **kw)
+    ref = oracle_all(q, k, v, go, mask=True, tau=1.0, p=2, a=a)
+    smax = float((q.double() @ k.double().transpose(1, 2)).abs().max())
+    return smax, [(x, r) for x, r in zip((o, g) + tuple(grads), ref)]
+
+
+def test_bf16_range_is_loud_not_wrong(sim):
+    """bf16 tensors are computed in _Float16.  Inside the documented range (|s| <= 250) the results meet
+    the bf16 bar; beyond it every result is either still within the bar or not finite - never a finite
+    wrong number; and with FASTMAX_FLAG_F32_COMPUTE the same inputs meet the bar."""
+    smax, pairs = _domain_case(sim, 2.2, 0)                         # |s| up to about 200
+    assert 100.0 < smax <= 250.0
+    for x, r in pairs:
+        assert bool(torch.isfinite(x).all()) and rel_err(x, r) < TOL[torch.bfloat16]
+    for scale in (8.0, 30.0, 300.0):                               # |s| ~ 2e3, 3e4, 3e6
+        smax, pairs = _domain_case(sim, scale, 0)
+        assert smax > 362.0
+        for x, r in pairs:
+            assert (not bool(torch.isfinite(x).all())) or rel_err(x, r) < TOL[torch.bfloat16]
+        _, pairs = _domain_case(sim, scale, _capi.FLAG_F32_COMPUTE)
+        for x, r in pairs:
+            assert bool(torch.isfinite(x).all()) and rel_err(x, r) < TOL[torch.bfloat16]
+    # a0 = 0: denominators no longer grow with the token index (g_0 = s + s^2 / 2 can be tiny)
+    _, pairs = _domain_case(sim, 1.0, _capi.FLAG_F32_COMPUTE, a=(0.0, 1.0, 0.5))
+    for x, r in pairs:
+        assert bool(torch.isfinite(x).all()) and rel_err(x, r) < TOL[torch.bfloat16]
+    _, pairs = _domain_case(sim, 1.0, 0, a=(0.0, 1.0, 0.5))
+    for x, r in pairs:
+        assert (not bool(torch.isfinite(x).all())) or rel_err(x, r) < TOL[torch.bfloat16]
+
+
+def test_normalize_zero_slice(sim):
+    # an all-zero (b, h) slice (padding) comes out as zeros with zero gradient, not 0 / 0
+    g = torch.Generator().manual_seed(17)
+    x, dy = torch.randn(3, 70, 32, generator=g), torch.randn(3, 70, 32, generator=g)
+    x[1] = 0.0
+    y = sim.normalize(x, centre=0, max_norm=True, scale=1.5)
+    assert bool(torch.isfinite(y).all()) and float(y[1].abs().max()) == 0.0
+    dx = sim.normalize_backward(x, dy, centre=0, max_norm=True, scale=1.5)
+    assert bool(torch.isfinite(dx).all()) and float(dx[1].abs().max()) == 0.0
