@@ -26,7 +26,8 @@ enum {
   FASTMAX_ERR_UNSUPPORTED = 3,   /* valid, but not implemented (head size, order, masked nq > nk) */
   FASTMAX_ERR_WORKSPACE = 4,     /* workspace missing, too small or misaligned */
   FASTMAX_ERR_LAUNCH = 5,        /* the HIP runtime refused a launch */
-  FASTMAX_ERR_DTYPE = 6          /* unknown element type */
+  FASTMAX_ERR_DTYPE = 6,         /* unknown element type */
+  FASTMAX_ERR_TOO_LARGE = 7      /* fastmax_forward_static: the problem needs more scratch than the static buffer */
 };
 
 enum { FASTMAX_F32 = 0, FASTMAX_BF16 = 1 };
@@ -99,6 +100,23 @@ int fastmax_workspace_bytes(const FastmaxDesc* desc, size_t* forward_bytes, size
  * with strides (d+1, bh*(d+1)).  workspace: >= forward_bytes, 256-byte aligned device memory. */
 int fastmax_forward(const FastmaxDesc* desc, const void* q, const void* k, const void* v,
                     void* o, float* g, void* workspace, size_t workspace_bytes, void* hip_stream);
+
+/* fastmax_forward for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose forward_cuda
+ * allocates its output and four scratch tensors on every call (fastmax_cuda_forward.cu:404-414).
+ * Same arguments, results and kernels as fastmax_forward, but the workspace is a buffer of
+ * FASTMAX_STATIC_SCRATCH_BYTES that is part of the loaded library (one copy per GPU, held until the
+ * process ends); the call allocates and frees nothing.  A problem whose forward_bytes
+ * (fastmax_workspace_bytes) exceed that size is refused with FASTMAX_ERR_TOO_LARGE before anything is
+ * launched.  All calls on one GPU share that GPU's buffer: calls that overlap in time on one GPU (two
+ * streams, two threads) race and give wrong results; calls on one stream are ordered and safe.  The
+ * buffer keeps the last call's contents; nothing in it needs clearing between calls.
+ * FASTMAX_FLAG_SAVE_FOR_BACKWARD is honoured (the saved data then lives in the static buffer, until the
+ * next call).  The first call on a device looks the buffer's address up and must not be made while a
+ * stream capture is in progress; later calls may be captured. */
+#define FASTMAX_STATIC_SCRATCH_BYTES (64u << 20)
+int fastmax_forward_static(const FastmaxDesc* desc, const void* q, const void* k, const void* v,
+                           void* o, float* g, void* hip_stream);
 
 /* Replaces backward_cuda (reference fastmax_cuda.cpp:26-32 -> fastmax_cuda_backward.cu:518-613):
  * gradients of sum(o * dO) with respect to q, k and v, where s_ij = (q_i . k_j) * inv_tau.

@@ -54,8 +54,9 @@ EXPORTS = (
     "fastmax_normalize_stats_bytes", "fastmax_normalize_backward", "fastmax_normalize_backward_stats_bytes",
     "fastmax_status_string", "fastmax_version", "fastmax_probe_mfma", "fastmax_probe_lds_transpose",
     "fastmax_probe_mfma_rate",
-    "fastmax_profile_begin", "fastmax_profile_end",
+    "fastmax_profile_begin", "fastmax_profile_end", "fastmax_forward_static",
 )
+STATIC_SCRATCH_BYTES = 64 << 20     # FASTMAX_STATIC_SCRATCH_BYTES
 
 
 class FastmaxError(RuntimeError):
@@ -118,6 +119,8 @@ class FastmaxLib:
         L.fastmax_workspace_bytes.restype = C.c_int
         L.fastmax_forward.argtypes = [C.POINTER(Desc)] + [C.c_void_p] * 6 + [C.c_size_t, C.c_void_p]
         L.fastmax_forward.restype = C.c_int
+        L.fastmax_forward_static.argtypes = [C.POINTER(Desc)] + [C.c_void_p] * 6
+        L.fastmax_forward_static.restype = C.c_int
         L.fastmax_backward.argtypes = [C.POINTER(Desc)] + [C.c_void_p] * 10 + [C.c_size_t, C.c_void_p]
         L.fastmax_backward.restype = C.c_int
         L.fastmax_backward_saved.argtypes = [C.POINTER(Desc)] + [C.c_void_p] * 10 + [C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p]
@@ -209,6 +212,17 @@ class FastmaxLib:
         self.check(st, "fastmax_forward")
         if save:
             return out, g, ws
+        return out, g
+
+    def forward_static(self, q, k, v, out, g, *, mask, inv_tau, a0=1.0, a1=1.0, a2=0.5, p=2, chunk=0, flags=0):
+        """fastmax_forward_static: the forward on the library's own static scratch buffer.  The caller owns
+        ``out`` (shaped like q) and ``g``; nothing is allocated here or in the library."""
+        desc = self.make_desc(q, k, v, mask=mask, inv_tau=inv_tau, a0=a0, a1=a1, a2=a2, p=p, chunk=chunk, flags=flags)
+        desc.so = _strides(out)
+        desc.sg = _gstrides(g)
+        st = self.lib.fastmax_forward_static(C.byref(desc), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                             g.data_ptr(), self._stream(q))
+        self.check(st, "fastmax_forward_static")
         return out, g
 
     def backward(self, q, k, v, o, g, d_o, *, mask, inv_tau, a0=1.0, a1=1.0, a2=0.5, p=2, chunk=0, flags=0,

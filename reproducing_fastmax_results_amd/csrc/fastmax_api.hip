@@ -11,6 +11,34 @@
 #include <unordered_map>
 #include <vector>
 
+// ---- static scratch of fastmax_forward_static ------------------------------------------------
+// Device memory that belongs to the loaded library: every GPU the library runs on holds its own copy
+// of this array, at its own address, until the process ends.
+#if defined(FM_HOSTSIM)
+static alignas(256) unsigned char scratch[FASTMAX_STATIC_SCRATCH_BYTES];
+static inline int fm_static_scratch(void** out) { *out = scratch; return FASTMAX_OK; }
+#else
+static __device__ __align__(256) unsigned char scratch[FASTMAX_STATIC_SCRATCH_BYTES];
+// In host code the array's name is only a handle for the runtime, not a device address.  The address
+// on the current device is asked for once per device (with that device current) and kept; kernels and
+// copies are only ever given that address.
+static inline int fm_static_scratch(void** out) {
+  enum { MAX_DEVICES = 64 };
+  static std::mutex mu;
+  static void* addr[MAX_DEVICES] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return FASTMAX_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!addr[dev]) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return FASTMAX_ERR_LAUNCH;
+    addr[dev] = ptr;
+  }
+  *out = addr[dev];
+  return FASTMAX_OK;
+}
+#endif
+
 namespace {
 
 inline int fm_launch_status() { return fm_after_launch() ? FASTMAX_ERR_LAUNCH : FASTMAX_OK; }
@@ -467,6 +495,7 @@ const char* fastmax_status_string(int status) {
     case FASTMAX_ERR_WORKSPACE: return "workspace missing, too small or not 256-byte aligned";
     case FASTMAX_ERR_LAUNCH: return "HIP launch failed";
     case FASTMAX_ERR_DTYPE: return "unknown dtype";
+    case FASTMAX_ERR_TOO_LARGE: return "problem needs more scratch than the library's static buffer holds";
     default: return "unknown status";
   }
 }
@@ -544,6 +573,19 @@ int fastmax_forward(const FastmaxDesc* desc, const void* q, const void* k, const
   if (desc->dtype == FASTMAX_BF16)
     return desc->d == 64 ? merge_parts<fm_bf16, 64>(desc, sp, oa, ga, o, g, stream) : merge_parts<fm_bf16, 32>(desc, sp, oa, ga, o, g, stream);
   return desc->d == 64 ? merge_parts<float, 64>(desc, sp, oa, ga, o, g, stream) : merge_parts<float, 32>(desc, sp, oa, ga, o, g, stream);
+}
+
+int fastmax_forward_static(const FastmaxDesc* desc, const void* q, const void* k, const void* v, void* o, float* g,
+                           void* hip_stream) {
+  size_t need = 0;
+  const int st = fastmax_workspace_bytes(desc, &need, nullptr);
+  if (st) return st;
+  if (need > size_t(FASTMAX_STATIC_SCRATCH_BYTES)) return FASTMAX_ERR_TOO_LARGE;
+  void* ws = nullptr;
+  const int sa = fm_static_scratch(&ws);
+  if (sa) return sa;
+  // nothing in the scratch has to start at zero: every kernel of the forward writes what a later one reads
+  return fastmax_forward(desc, q, k, v, o, g, ws, size_t(FASTMAX_STATIC_SCRATCH_BYTES), hip_stream);
 }
 
 static int backward_one(const FastmaxDesc* desc, const void* q, const void* k, const void* v, const void* o,

@@ -119,6 +119,24 @@ def test_forward_backward_reject_bad_arguments_before_launching(lib):
     assert lib.lib.fastmax_version() >= 105
 
 
+def test_static_scratch_entry_rejects_before_touching_the_device(lib):
+    # fastmax_forward_static: argument and size checks come before the first HIP call
+    one = C.c_void_p(256)
+    assert lib.lib.fastmax_forward_static(None, one, one, one, one, one, None) == 1
+    assert lib.lib.fastmax_forward_static(C.byref(base_desc(d=48)), one, one, one, one, one, None) == 3
+    big = base_desc(bh=16, nq=65536, nk=65536)
+    for name in ("sq", "sk", "sv", "so"):
+        setattr(big, name, _capi.Strides(65536 * 64, 64))
+    big.sg = _capi.Strides(65536, 1)
+    st, f, _ = ws(lib, big)
+    assert st == 0 and f > _capi.STATIC_SCRATCH_BYTES
+    assert lib.lib.fastmax_forward_static(C.byref(big), one, one, one, one, one, None) == 7
+    assert "static buffer" in lib.status_string(7)
+    # the headline forward (B*H = 32, N = 4096, D = 64, bf16) fits
+    c2 = base_desc(bh=32, nq=4096, nk=4096)
+    assert ws(lib, c2)[1] <= _capi.STATIC_SCRATCH_BYTES
+
+
 def test_segment_length_and_size_limits(lib):
     # segment lengths beyond 2^30 and token counts beyond 2^30 are refused (32-bit padding arithmetic)
     assert ws(lib, base_desc(chunk=2 ** 31 - 1))[0] == 2
