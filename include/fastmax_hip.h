@@ -53,7 +53,10 @@ enum {
  * ordinary magnitude (about 1e-3 .. 1e4).  The reference model's normalised q and k (|q_i|, |k_j| <=
  * lim, transformer/model.py:97-102) satisfy this by construction.  Nothing saturates: an input
  * beyond the range turns into infinities that reach the outputs as inf / NaN rather than as finite
- * wrong numbers.  FASTMAX_FLAG_F32_COMPUTE lifts the limits at fp32 speed. */
+ * wrong numbers.  FASTMAX_FLAG_F32_COMPUTE lifts the limits at fp32 speed.  The size of dO is free (the
+ * backward rescales dO / g per batch*head to the _Float16 range and back).  The 2e-2 accuracy of this
+ * path also rests on weights f(s) that add up without cancelling, as the Taylor weights do (f > 0):
+ * with a0 <= 0 the library computes bf16 tensors in fp32 on its own, as if the flag were set. */
 
 /* Where slice i of the batch*head axis, token t, feature f of a tensor lives:
  *   heads <= 1:  i * bh + t * n + f

@@ -15,7 +15,7 @@
 // Device memory that belongs to the loaded library: every GPU the library runs on holds its own copy
 // of this array, at its own address, until the process ends.
 #if defined(FM_HOSTSIM)
-static alignas(256) unsigned char scratch[FASTMAX_STATIC_SCRATCH_BYTES];
+alignas(256) static unsigned char scratch[FASTMAX_STATIC_SCRATCH_BYTES];
 static inline int fm_static_scratch(void** out) { *out = scratch; return FASTMAX_OK; }
 #else
 static __device__ __align__(256) unsigned char scratch[FASTMAX_STATIC_SCRATCH_BYTES];
@@ -96,11 +96,10 @@ struct Plan {
   int npad_q, npad_k;
   float a0, a1, a2;     // polynomial on the score s = (q.k) / tau
   float sc;             // sqrt(1/tau), folded into q and k when they are converted
-  float gscale;         // power of two folded into dO / g in the backward
   // workspace offsets (bytes)
   size_t kt, vt, kr, vr, big, big2, small, fwd_bytes;
   bool save;
-  size_t b_kr, b_vr, b_qr, b_kt, b_vt, b_qt, b_qct, b_gh, b_ght, b_cv, b_bigq, b_smallq, b_bigk, b_smallk, b_bigv, bwd_bytes;
+  size_t b_kr, b_vr, b_qr, b_kt, b_vt, b_qt, b_qct, b_gh, b_ght, b_cv, b_bigq, b_smallq, b_bigk, b_smallk, b_bigv, b_gpart, bwd_bytes;
 };
 
 bool strides_ok(const FastmaxStrides& s, int bh, int n, int d) {
@@ -141,7 +140,10 @@ template <int DH> size_t big_array_bytes(int esz, bool quad, size_t slots) {
 int make_plan(const FastmaxDesc* d, Plan& p) {
   int st = validate(d);
   if (st != FASTMAX_OK) return st;
-  p.half = d->dtype == FASTMAX_BF16 && !(d->flags & FASTMAX_FLAG_F32_COMPUTE);
+  // _Float16 arithmetic serves weights that are positive sums: with a0 <= 0 the weights f(s) change sign
+  // around s = 0, numerator and denominator cancel, and 11 bits per weight no longer bound the error of
+  // their ratio; such problems are computed in fp32 like the ones that ask for it
+  p.half = d->dtype == FASTMAX_BF16 && !(d->flags & FASTMAX_FLAG_F32_COMPUTE) && d->a0 > 0.0f;
   p.esz = p.half ? 2 : 4;
   p.npad_q = int(round_up(d->nq, 256));
   p.npad_k = int(round_up(d->nk, 256));
@@ -150,11 +152,6 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   p.a1 = d->a1;
   p.a2 = p.quad ? d->a2 : 0.0f;
   p.sc = std::sqrt(std::fabs(d->inv_tau));
-  {
-    int e = 0;
-    while ((int64_t(1) << e) < d->nq) ++e;
-    p.gscale = e > 6 ? float(int64_t(1) << (e - 6)) : 1.0f;
-  }
   const bool force_dense = (d->flags & FASTMAX_FLAG_FORCE_DENSE) != 0;
   if (d->mask) {
     // Segment length.  Dense tiles cost grows with L, the moment states cost the same per token
@@ -205,6 +202,7 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   p.b_bigq = take(bigarr); p.b_smallq = take(size_t(d->bh) * p.nslots * smallsz);
   p.b_bigk = take(bigarr); p.b_smallk = take(size_t(d->bh) * p.nslots * smallsz);
   p.b_bigv = take(bigarr);
+  p.b_gpart = take(p.half ? size_t(d->bh) * fm_grad_scale_blocks(d->nq) * 4 : 0);   // see k_grad_scale
   p.bwd_bytes = off ? off : 256;
   return FASTMAX_OK;
 }
@@ -345,7 +343,7 @@ template <typename TIO, typename E> void tok_common(TokArgs<TIO, E>& a, const Fa
   a.nslots = p.nslots; a.L = p.L; a.nseg = p.nseg; a.causal = d->mask != 0; a.use_state = p.use_state;
   a.quad = p.quad; a.a0 = p.a0; a.a1 = p.a1; a.a2 = p.a2; a.sc = p.sc; a.out_scale = 1.0f; a.zscale = 1.0f;
   a.own_o = TRef<const TIO>{nullptr, 0, 0, 0, 0, 0}; a.own_do = a.own_o;
-  a.w_gh = nullptr; a.w_qr = nullptr; a.w_cv = nullptr; a.gscale = p.gscale;
+  a.w_gh = nullptr; a.w_qr = nullptr; a.w_cv = nullptr; a.gpart = nullptr; a.gnblk = 0;
 }
 
 template <typename TIO, typename E, int DH, int QT, int OWN>

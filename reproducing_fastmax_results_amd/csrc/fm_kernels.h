@@ -191,15 +191,83 @@ k_transpose(TransposeJob<TIO, E> j0, TransposeJob<TIO, E> j1, int n, int npad) {
 }
 
 // ------------------------------------------------------------------------------
+// Scale of the upstream gradient.  Every gradient is linear in gh_i = dO_i / g_i, and the size of dO is the
+// caller's: a loss averaged over tens of thousands of tokens hands over dO of 1e-6 and less, and g grows with
+// the token index, so gh can lie anywhere - far below what _Float16 holds included.  k_grad_scale finds, per
+// workgroup of 64 tokens, the largest |dO_if| / |g_i|; every later kernel joins the partial maxima of its
+// batch*head (fm_grad_scale: the same few values in the same order everywhere, so all kernels agree on the
+// bits) into the power of two that brings the largest |gh| element of the batch*head to [32, 64), multiplies
+// gh by it when it is formed and divides the gradients by it when they are stored.  Inside a batch*head gh
+// varies by about the sequence length (g_i ~ i), which leaves the smallest rows of a 65536-token sequence near
+// 1e-3, well inside the normal _Float16 range, and the dot products gh.v and gh.o (64 terms) below 65504.
+// grid (ceil(n / 64), bh); part [bh][nblk].
+// ------------------------------------------------------------------------------
+static constexpr int FM_GS_TOKENS = 64;
+inline int fm_grad_scale_blocks(int n) { return (n + FM_GS_TOKENS - 1) / FM_GS_TOKENS; }
+
+template <typename TIO, int DH>
+FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_grad_scale(TRef<const TIO> d_o, TRef<const float> g, int n, float* FM_RESTRICT part) {
+  constexpr int EPT = DH / 4, NP = FM_GS_TOKENS / 64;
+  FM_SHARED float wmax[4];
+  const int tid = FM_TID_X, bh = FM_BID_Y;
+  const int tok0 = FM_BID_X * FM_GS_TOKENS + (tid >> 2), d0 = (tid & 3) * EPT;
+  float v[NP][EPT], gi[NP];
+  // all loads first; rows past the end re-read the last row (every lane takes part in the shuffles)
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    const int tok = tok0 + 64 * p, tk = tok < n ? tok : n - 1;
+    gi[p] = g.base(bh)[int64_t(tk) * g.s_n];
+#pragma unroll
+    for (int j = 0; j < EPT; j += 8) IO<TIO>::ld8(d_o.base(bh) + int64_t(tk) * d_o.s_n + d0 + j, d_o.vec != 0, &v[p][j]);
+  }
+  float mx = 0.f;
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    float m = 0.f;
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) m = fm_fmaxf(m, v[p][j] < 0.f ? -v[p][j] : v[p][j]);
+    const float ga = gi[p] < 0.f ? -gi[p] : gi[p];
+    mx = fm_fmaxf(mx, m / ga);                       // fmax drops a NaN (0 / 0); an infinity (g = 0) is kept and ignored by the consumers
+  }
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) mx = fm_fmaxf(mx, fm_shfl_xor(mx, m));
+  if ((tid & 63) == 0) wmax[tid >> 6] = mx;
+  FM_SYNC();
+  if (tid == 0) part[int64_t(bh) * FM_GDIM_X + FM_BID_X] = fm_fmaxf(fm_fmaxf(wmax[0], wmax[1]), fm_fmaxf(wmax[2], wmax[3]));
+}
+
+// The power of two described above, from the nblk partial maxima of one batch*head; 1 when there are none
+// (part == null: the fp32 kernels need no scaling) or when the maximum is zero or not finite.  Every lane of the
+// wavefront must call it; every lane gets the same value.
+FM_DEVICE float fm_grad_scale(const float* part, int nblk, int lane) {
+  if (!part) return 1.0f;
+  float m = 0.f;
+  for (int i = lane; i < nblk; i += 64) { const float x = part[i]; if (x < 3.0e38f) m = fm_fmaxf(m, x); }
+#pragma unroll
+  for (int w = 1; w < 64; w <<= 1) m = fm_fmaxf(m, fm_shfl_xor(m, w));
+  if (!(m > 0.f)) return 1.0f;
+  uint32_t bits;
+  __builtin_memcpy(&bits, &m, 4);
+  int eb = int((bits >> 23) & 0xffu);                 // m = 1.x * 2^(eb - 127)  (eb = 0: subnormal, treated as 2^-126)
+  if (eb < 1) eb = 1;
+  int sb = 259 - eb;                                  // 2^(5 - (eb - 127))
+  if (sb > 254) sb = 254;
+  if (sb < 1) sb = 1;
+  const uint32_t out = uint32_t(sb) << 23;
+  float r;
+  __builtin_memcpy(&r, &out, 4);
+  return r;
+}
+
+// ------------------------------------------------------------------------------
 // k_prep_bwd: per token  gh = gscale * dO / g,  c = gh . o,  q' = qscale * q ; writes
 //   gh  [bh][npad][DH]  (row-major, compute type)      ght [bh][DH][npad]
 //   qt  [bh][DH][npad]  (q' transposed)                 qct [bh][DH][npad]  (c_i q'_i; skipped when null:
 //                                                        only the state walk reads it)
 //   qr  [bh][npad][DH]  (q' row-major)
 //   cv  [bh][npad]      (c, compute type)
-// gscale is a power of two that keeps gh inside the _Float16 range for long sequences
-// (g grows like the token index); every gradient is linear in (gh, c) and is divided
-// by gscale again when it is stored.
+// gscale is the power of two of fm_grad_scale (see k_grad_scale): it keeps gh inside the _Float16
+// range; every gradient is linear in (gh, c) and is divided by gscale again when it is stored.
 // Tokens >= n are written as zeros.  grid (npad/64, bh).
 // Reference: div_grad_output, fastmax_cuda_backward.cu:494-501, and the
 // "grad * o" row sums of fastattention_einops.py:405-407.
@@ -207,7 +275,8 @@ k_transpose(TransposeJob<TIO, E> j0, TransposeJob<TIO, E> j1, int n, int npad) {
 template <typename TIO, typename E, int DH>
 FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS)
 k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, TRef<const float> g, int n, int npad, E* FM_RESTRICT gh, E* FM_RESTRICT ght,
-           E* FM_RESTRICT qt, E* FM_RESTRICT qct, E* FM_RESTRICT qr, E* FM_RESTRICT cv, float qscale, float gscale) {
+           E* FM_RESTRICT qt, E* FM_RESTRICT qct, E* FM_RESTRICT qr, E* FM_RESTRICT cv, float qscale,
+           const float* FM_RESTRICT gpart, int gnblk) {
   constexpr int PT = 64 + Mma<E>::PAD;
   constexpr int VEC = Mma<E>::VEC;
   constexpr int EPT = DH / 4;                      // elements per thread (4 threads per token)
@@ -217,6 +286,7 @@ k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, TRef<const
   const int tid = FM_TID_X, t0 = FM_BID_X * 64, bh = FM_BID_Y;
   const int tok = tid >> 2, part = tid & 3, d0 = part * EPT;
   const int row = t0 + tok;
+  const float gscale = fm_grad_scale(gpart ? gpart + int64_t(bh) * gnblk : nullptr, gnblk, tid & 63);
   float vg[EPT], vq[EPT];
   float csum = 0.f;
   if (row < n) {

@@ -81,7 +81,7 @@ FM_DEVICE fm_half4 fm_lds_tr4(const fm_half* p) {
   }
   return r;
 }
-FM_DEVICE float fm_fmaxf(float a, float b) { return a > b ? a : b; }
+FM_DEVICE float fm_fmaxf(float a, float b) { return a != a ? b : (b != b ? a : (a > b ? a : b)); }   // drops a NaN, like fmaxf
 FM_DEVICE float fm_clampf(float x, float lim) { return x > lim ? lim : (x < -lim ? -lim : x); }
 FM_DEVICE float fm_rsqrtf(float a) { return 1.0f / std::sqrt(a); }
 FM_DEVICE float fm_sqrtf(float a) { return std::sqrt(a); }

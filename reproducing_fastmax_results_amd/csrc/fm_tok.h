@@ -49,7 +49,9 @@ template <typename TIO, typename E> struct TokArgs {
   // [bh][npad_own][DH]) and w_cv ([bh][npad_own], tile order) for the key-side pass that follows
   TRef<const TIO> own_o, own_do;
   E* w_gh; E* w_qr; E* w_cv;
-  float gscale;
+  // partial maxima of |dO| / |g| ([bh][gnblk], see k_grad_scale) or null: the kernels that form gh multiply it by
+  // fm_grad_scale of them, the kernels that store a gradient divide by it
+  const float* gpart; int gnblk;
 };
 
 // Z (fp32, [DH][DH]) -> LDS in the compute type (hi/lo split for _Float16), va/vb -> vecs.
@@ -422,7 +424,8 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
     }
   } else {
     // dV = (sums + vb) * out_scale; keys past n_own are discarded by the bounds check
-    fm_store_tokens<TIO, E, DH, QT>(acc, xrow, G.use_state ? vecs + DH : nullptr, A.out_scale, Os, A.out, bh, t0,
+    const float gsc = fm_grad_scale(A.gpart ? A.gpart + int64_t(bh) * A.gnblk : nullptr, A.gnblk, lane);
+    fm_store_tokens<TIO, E, DH, QT>(acc, xrow, G.use_state ? vecs + DH : nullptr, A.out_scale / gsc, Os, A.out, bh, t0,
                                     A.n_own, tid);
   }
 }
@@ -460,6 +463,8 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
   G.init(A);
   const int bh = G.bh, t0 = G.t0;
   const bool causal = A.causal != 0;
+  const float gsc = fm_grad_scale(A.gpart ? A.gpart + int64_t(bh) * A.gnblk : nullptr, A.gnblk, lane);
+  const float ginv_sc = 1.0f / gsc;
 
   if (PREP) {
     // own queries straight from the caller's q, o, dO and g (four threads per token, 64 tokens per
@@ -493,7 +498,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
 #pragma unroll
     for (int h = 0; h < NH; ++h) {
       const int tok = 64 * h + (tid >> 2), row = t0 + tok;
-      const float ginv = A.gscale / gi[h];
+      const float ginv = gsc / gi[h];
       float vg[EPT], vq[EPT];
       float csum = 0.f;
 #pragma unroll
@@ -683,9 +688,9 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
     }
     if (NBUF == 2) FM_SYNC();
   }
-  fm_store_tokens<TIO, E, DH, QT>(acc, xrow, nullptr, A.out_scale, reinterpret_cast<float*>(Own), A.out, bh, t0,
+  fm_store_tokens<TIO, E, DH, QT>(acc, xrow, nullptr, A.out_scale * ginv_sc, reinterpret_cast<float*>(Own), A.out, bh, t0,
                                   A.n_own, tid);
   if (DV)
-    fm_store_tokens<TIO, E, DH, QT>(av, xrow, nullptr, A.out2_scale, reinterpret_cast<float*>(Own), A.out2, bh, t0,
+    fm_store_tokens<TIO, E, DH, QT>(av, xrow, nullptr, A.out2_scale * ginv_sc, reinterpret_cast<float*>(Own), A.out2, bh, t0,
                                     A.n_own, tid);
 }

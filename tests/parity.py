@@ -8,12 +8,12 @@ from oracle import fastmax_oracle as O
 TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}   # rel-L2 bars: fp32 1e-5, bf16 2e-2
 
 
-def make_inputs(bh, nq, nk, d, dtype, device, seed=0, scale=1.0):
+def make_inputs(bh, nq, nk, d, dtype, device, seed=0, scale=1.0, go_scale=1.0):
     gen = torch.Generator().manual_seed(seed)
     q = (scale * torch.randn(bh, nq, d, generator=gen)).to(dtype)
     k = (scale * torch.randn(bh, nk, d, generator=gen)).to(dtype)
     v = (scale * torch.randn(bh, nk, d, generator=gen)).to(dtype)
-    go = torch.randn(bh, nq, d, generator=gen).to(dtype)
+    go = (go_scale * torch.randn(bh, nq, d, generator=gen)).to(dtype)
     return tuple(t.to(device) for t in (q, k, v, go))
 
 
@@ -48,11 +48,11 @@ def check_forward(lib, bh, nq, d, dtype, device, *, mask, p, nk=None, chunk=0, f
 
 
 def check_forward_backward(lib, bh, nq, d, dtype, device, *, mask, p, nk=None, chunk=0, flags=0, tau_mult=8.0,
-                           a=(1.0, 1.0, 0.5), seed=0, scale=1.0, saved=False):
+                           a=(1.0, 1.0, 0.5), seed=0, scale=1.0, saved=False, go_scale=1.0):
     """saved: run the backward on the workspace the forward leaves behind
-    (FASTMAX_FLAG_SAVE_FOR_BACKWARD / fastmax_backward_saved)."""
+    (FASTMAX_FLAG_SAVE_FOR_BACKWARD / fastmax_backward_saved).  go_scale: size of the upstream gradient."""
     nk = nk or nq
-    q, k, v, go = make_inputs(bh, nq, nk, d, dtype, device, seed, scale)
+    q, k, v, go = make_inputs(bh, nq, nk, d, dtype, device, seed, scale, go_scale)
     tau = tau_mult * math.sqrt(d)
     kw = dict(mask=mask, inv_tau=1.0 / tau, a0=a[0], a1=a[1], a2=a[2], p=p, chunk=chunk, flags=flags)
     if saved:

@@ -33,21 +33,29 @@ def _inputs(bh, n, d, dtype, seed, scale):
     return [(s * torch.randn(bh, n, d, generator=gen)).to(dtype) for s in (scale, scale, scale, 1.0)]
 
 
-def _rows(n, count, seed):
+def _rows(n, count, seed, seg):
     """first and last token, both sides of the 256-, 1024- and 2048-token segment boundaries
-    and of a 128-token block, and seeded random rows"""
+    and of a 128-token block, seeded random rows, and one seeded random row inside EVERY stretch of
+    ``seg`` tokens: with ``seg`` the segment length of the moment scan every segment holds a query with
+    an upstream gradient, so every segment's prefix state (o, dq) and suffix state (dk, dv of all earlier
+    keys) enters the compared results"""
     fixed = [0, 1, 31, 32, 127, 128, 255, 256, 1023, 1024, 2047, 2048, n // 2 - 1, n // 2, n - 2, n - 1]
     gen = torch.Generator().manual_seed(seed)
     rnd = torch.randint(0, n, (count,), generator=gen).tolist()
-    return torch.tensor(sorted({r for r in fixed + rnd if 0 <= r < n}))
+    nseg = (n + seg - 1) // seg
+    inside = torch.randint(0, seg, (nseg,), generator=gen)
+    per_seg = [min(i * seg + int(inside[i]), n - 1) for i in range(nseg)]
+    rows = torch.tensor(sorted({r for r in fixed + rnd + per_seg if 0 <= r < n}))
+    assert len(set((rows // seg).tolist())) == nseg
+    return rows
 
 
-def _check_sparse_rows(lib, bh, n, d, dtype, p, seed, scale, chunk=0, count=48):
+def _check_sparse_rows(lib, bh, n, d, dtype, p, seed, scale, chunk=0, count=48, seg=256, tau_mult=8.0):
     q, k, v, go = _inputs(bh, n, d, dtype, seed, scale)
-    rows = _rows(n, count, seed + 1)
+    rows = _rows(n, count, seed + 1, seg)
     sparse = torch.zeros_like(go)
     sparse[:, rows] = go[:, rows]
-    tau = 8.0 * math.sqrt(d)
+    tau = tau_mult * math.sqrt(d)
     kw = dict(mask=True, inv_tau=1.0 / tau, p=p, chunk=chunk)
     qd, kd, vd, gd = (t.to(DEV) for t in (q, k, v, sparse))
     o, g, ws = lib.forward(qd, kd, vd, save=True, **kw)
@@ -112,8 +120,25 @@ def test_config2_all_slices_through_states(lib, chunk):
 def test_config3_all_slices(lib, p):
     # causal long context, B*H = 16, N = 65536, D = 64, bf16, inputs scaled by 0.5
     print(f"case full config3 p={p}", flush=True)
-    _check_sparse_rows(lib, 16, 65536, 64, torch.bfloat16, p, seed=110 + p, scale=0.5)
+    # the library's segments at this length: 256 tokens (order 1), 1024 tokens (order 2); a row with an
+    # upstream gradient in every 256 tokens covers every segment of either (256 + rows per slice)
+    _check_sparse_rows(lib, 16, 65536, 64, torch.bfloat16, p, seed=110 + p, scale=0.5, seg=256)
     _check_running_mean(lib, 16, 65536, 64, torch.bfloat16, p, seed=120 + p)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_config2_all_slices_sharp_temperature(lib, dtype):
+    # temperature = sqrt(D) (what the reference's own tests use, test/test_einops_fastmax.py:77-225): scores of
+    # order one, so the quadratic term carries real weight
+    print(f"case full config2 tau=sqrt(D) dtype={dtype}", flush=True)
+    _check_sparse_rows(lib, 32, 4096, 64, dtype, 2, seed=140, scale=1.0, tau_mult=1.0)
+    _check_sparse_rows(lib, 32, 4096, 64, dtype, 2, seed=141, scale=1.0, tau_mult=1.0, chunk=1024)
+
+
+@pytest.mark.parametrize("p", [1, 2])
+def test_config3_all_slices_sharp_temperature(lib, p):
+    print(f"case full config3 tau=sqrt(D) p={p}", flush=True)
+    _check_sparse_rows(lib, 16, 65536, 64, torch.bfloat16, p, seed=150 + p, scale=0.5, seg=256, tau_mult=1.0)
 
 
 @pytest.mark.parametrize("p", [1, 2])

@@ -207,6 +207,61 @@ def test_causal_more_keys_than_queries(lib, dtype, p, nq, nk):
     check_forward_backward(lib, 3, nq, d, dtype, DEV, mask=True, p=p, nk=nk, seed=50)
 
 
+@pytest.mark.parametrize("go_scale", [1e-7, 1e-4, 3e4])
+def test_upstream_gradient_of_any_size(lib, go_scale):
+    """Gradients are linear in dO, whose size is the caller's: a loss averaged over 16 x 1024 tokens hands over
+    dO near 1e-6.  The bf16 path brings dO / g of every batch*head into the _Float16 range and back."""
+    print(f"case upstream gradient size {go_scale}", flush=True)
+    for p, chunk in ((2, 0), (2, 256), (1, 0), (1, 256)):
+        check_forward_backward(lib, 4, 1024, 64, torch.bfloat16, DEV, mask=True, p=p, chunk=chunk, seed=61,
+                               go_scale=go_scale, saved=True)
+    check_forward_backward(lib, 2, 300, 32, torch.bfloat16, DEV, mask=False, p=2, nk=700, seed=62, go_scale=go_scale)
+    check_forward_backward(lib, 2, 513, 64, torch.bfloat16, DEV, mask=True, p=2, nk=2100, seed=63, go_scale=go_scale)
+
+
+def test_bf16_range_is_loud_not_wrong(lib):
+    """bf16 tensors are computed in _Float16.  Inside the documented range (|s| <= 250) the results meet
+    the bf16 bar; beyond it a result is either still within the bar or not finite, never a finite wrong
+    number; FASTMAX_FLAG_F32_COMPUTE meets the bar on the same inputs.  Also a0 = 0 (denominators that do
+    not grow with the token index)."""
+    import math
+    from oracle import fastmax_oracle as O
+    from reproducing_fastmax_results_amd._capi import FLAG_F32_COMPUTE
+    from tests.parity import TOL, make_inputs, oracle_all, rel_err
+    bh, n, d = 2, 700, 64
+    tol = TOL[torch.bfloat16]
+
+    def run(scale, flags, a, tau):
+        q, k, v, go = make_inputs(bh, n, n, d, torch.bfloat16, DEV, seed=60, scale=scale)
+        kw = dict(mask=True, inv_tau=1.0 / tau, a0=a[0], a1=a[1], a2=a[2], p=2, flags=flags)
+        o, g = lib.forward(q, k, v, **kw)
+        grads = lib.backward(q, k, v, o, g, go, **kw)
+        ref = oracle_all(q, k, v, go, mask=True, tau=tau, p=2, a=a)
+        smax = float((q.double() @ k.double().transpose(1, 2)).abs().max()) / tau
+        return smax, list(zip((o, g) + tuple(grads), ref))
+
+    taylor, tau = (1.0, 1.0, 0.5), 8.0 * math.sqrt(d)
+    smax, pairs = run(15.0, 0, taylor, tau)                        # the edge of the documented range
+    print(f"case bf16 range smax={smax:.0f}", flush=True)
+    assert 120.0 < smax <= 250.0
+    for x, r in pairs:
+        assert bool(torch.isfinite(x).all()) and rel_err(x, r) < tol
+    for scale in (30.0, 300.0):
+        smax, pairs = run(scale, 0, taylor, tau)
+        print(f"case bf16 range scale={scale} smax={smax:.0f}", flush=True)
+        for x, r in pairs:
+            assert (not bool(torch.isfinite(x).all())) or rel_err(x, r) < tol, f"finite but wrong at scale {scale}"
+        _, pairs = run(scale, FLAG_F32_COMPUTE, taylor, tau)
+        for x, r in pairs:
+            assert bool(torch.isfinite(x).all()) and rel_err(x, r) < tol
+    # a0 = 0: the weights change sign around s = 0 and the sums cancel (some |g_i| are a thousandth of the sum
+    # of |f|); the library computes such problems in fp32 by itself
+    for tau in (math.sqrt(d), 8.0 * math.sqrt(d)):
+        _, pairs = run(1.0, 0, (0.0, 1.0, 0.5), tau)
+        for x, r in pairs:
+            assert bool(torch.isfinite(x).all()) and rel_err(x, r) < tol
+
+
 def test_step_replays_as_a_hip_graph(lib):
     """The entry points allocate nothing and never synchronise, so a caller can capture forward and
     backward into one HIP graph.  Every replay (with eager work and synchronisations in between, and
