@@ -14,7 +14,11 @@ Besides the contract fields the line carries
                 flop count 2*(D + D^2)*(Dv + 1) per (b, h, token) and unit of
                 work (state build, readout, dQ, dK, dV each count one unit);
   cpu_baseline: the oracle's port of the reference's einops algorithm timed on
-                this box's host cores on a bounded sample (one (b, h) slice).
+                this box's host cores on a bounded sample (a few (b, h) slices), and the
+                reference's unfactorised closed form (compute_attn) beside it;
+  step_ms:      median / p10 / p90 of the step, from HIP events on the launch stream;
+  extra:        the other configurations of the path, a few steps each: fp32 on the same
+                workload, and the long-context configuration (B=1, H=16, N=65536) in both orders.
 Everything runs on one GPU; --gpus N > 1 is refused.  --workload long / --order 1 time the
 long-context parity configuration (B=1, H=16, N=65536) for profiling; the metric is the default.
 """
@@ -34,12 +38,17 @@ if ROOT not in sys.path:
 PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}      # MI355X dense matrix peaks (published)
 PEAK_HBM_GBS = 8000.0
 
-# HBM bytes per launch of the dominant kernel at the workload below, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE runs of this file scaled by a copy of known size; keyed by (dtype, --chunk, kernel).
-TRAFFIC_BYTES = {("bf16", 0, "dkv"): 115648 * 1024}
-# the same for --workload long --order 1 (read + written bytes per launch), keyed by kernel
-TRAFFIC_BYTES_LONG_ORDER1 = {"fwd": (593327 + 135168) * 1024, "dq": (562733 + 131072) * 1024,
-                             "dk": (601611 + 176955) * 1024, "dv": (428990 + 131072) * 1024}
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this file
+# scaled by a copy of known size (the summaries under profiles/ give the commands); keyed by
+# (N, order, dtype, --chunk, kernel).  A constant, not a live measurement: it belongs to the kernels as they
+# were when the named summary was made.
+TRAFFIC = {
+    (4096, 2, "bf16", 0, "dkv"): {"bytes": 115648 * 1024, "source": "profiles/bench_c2_bf16_hbm_traffic.md"},
+    (65536, 1, "bf16", 0, "fwd"): {"bytes": (593327 + 135168) * 1024, "source": "profiles/bench_long_order1_bf16_hbm_traffic.md"},
+    (65536, 1, "bf16", 0, "dq"): {"bytes": (562733 + 131072) * 1024, "source": "profiles/bench_long_order1_bf16_hbm_traffic.md"},
+    (65536, 1, "bf16", 0, "dk"): {"bytes": (601611 + 176955) * 1024, "source": "profiles/bench_long_order1_bf16_hbm_traffic.md"},
+    (65536, 1, "bf16", 0, "dv"): {"bytes": (428990 + 131072) * 1024, "source": "profiles/bench_long_order1_bf16_hbm_traffic.md"},
+}
 
 WORKLOAD = dict(name="configs[1]: causal order-2 fwd+bwd", B=4, H=8, N=4096, D=64, p=2, mask=True, scale=1.0)
 # not a bench line of its own: the long-context parity configuration, selectable for profiling (--workload long)
@@ -59,6 +68,37 @@ MFMA_PER_TILE = {"fwd": 8, "dv": 8, "dq": 12, "dk": 12, "dkv": 16}
 def alg_flops_unit(bh: int, n: int, d: int, p: int) -> float:
     m = d + (d * d if p == 2 else 0)
     return 2.0 * m * (d + 1) * bh * n
+
+
+def cpu_model_name() -> str:
+    try:
+        with open("/proc/cpuinfo") as fh:
+            for line in fh:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_closed_form(n: int, d: int, p: int, tokens_per_step: int, heads_total: int, slices: int = 2):
+    """The reference's unfactorised form (compute_attn, fastattention_einops.py:337-381: the N x N weights of one
+    (b, h) slice at a time) with torch autograd for the gradients, fp32, on the host cores."""
+    import torch
+    from oracle import fastmax_oracle as O
+    gen = torch.Generator().manual_seed(2)
+    tau = 8.0 * math.sqrt(d)
+    slices = max(1, min(slices, heads_total))
+    dt = 0.0
+    for _ in range(slices):
+        q, k, v, go = (torch.randn(1, n, d, generator=gen) for _ in range(4))
+        t0 = time.perf_counter()
+        O.closed_form_forward_backward(q, k, v, go, mask=True, tau=tau, p=p, dtype=torch.float32)
+        dt += time.perf_counter() - t0
+    t_step = dt * heads_total / slices
+    return {"value": tokens_per_step / t_step, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"closed form (N x N weights) + autograd, {slices} of {heads_total} (b,h) slices at N={n}, fp32, "
+                      f"scaled x{heads_total / slices:g}; {dt:.1f} s measured"}
 
 
 def cpu_baseline(n: int, d: int, p: int, tokens_per_step: int, heads_total: int, max_n: int, slices: int = 4):
@@ -83,7 +123,8 @@ def cpu_baseline(n: int, d: int, p: int, tokens_per_step: int, heads_total: int,
     sample = f"{slices} of {heads_total} (b,h) slices, N={n_run}" + \
              ("" if n_run == n else f" (scaled linearly to N={n})") + \
              f", fp32, fwd+bwd, scaled x{heads_total / slices:g}; {dt:.1f} s measured"
-    return {"value": tokens_per_step / t_step, "unit": "tokens/s", "cores": threads, "kind": "port", "sample": sample}
+    return {"value": tokens_per_step / t_step, "unit": "tokens/s", "cores": threads, "kind": "port", "sample": sample,
+            "cpu_model": cpu_model_name()}
 
 
 def model_step(args, dev):
@@ -144,6 +185,7 @@ def main() -> int:
                     help="instead of the operator benchmark, time one training step (forward, backward, AdamW) of "
                          "the minimal ViT (fp32, 256 images of 28x28) or decoder-only LM (bf16, 16 x 1024 tokens)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="skip the short runs of the other configurations")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device copy, the yardstick for the HBM traffic counters")
     ap.add_argument("--workload", choices=["headline", "long"], default="headline",
@@ -170,28 +212,67 @@ def main() -> int:
         print(json.dumps(model_step(args, dev)))
         return 0
     W = dict(WORKLOAD if args.workload == "headline" else LONG_WORKLOAD, p=args.order)
+    out = operator_line(lib, dev, W, args.dtype, args, args.steps, args.warmup, full=True)
+    if args.workload == "headline" and args.order == 2 and args.dtype == "bf16" and not args.no_extra:
+        # the other configurations of the path, a few steps each (same measurement, shorter)
+        extra = {}
+        for key, w, dt in (("c2_fp32", dict(WORKLOAD), "f32"),
+                           ("c3_order1_bf16", dict(LONG_WORKLOAD, p=1), "bf16"),
+                           ("c3_order2_bf16", dict(LONG_WORKLOAD, p=2), "bf16")):
+            plain = argparse.Namespace(**dict(vars(args), chunk=0, graph=False, independent_backward=False))
+            r = operator_line(lib, dev, w, dt, plain, steps=10, warmup=3, full=False)
+            extra[key] = {"workload": r["config"]["workload"], "dtype": dt, "ms_per_step": r["ms_per_step"],
+                          "step_ms": r["step_ms"], "tokens_per_s": r["value"], "forward_only_ms": r["forward_only"]["ms"],
+                          "roofline": r["roofline"], "hbm_bound_helpers": r["hbm_bound_helpers"]}
+        out["extra"] = extra
+    print(json.dumps(out))
+    return 0
+
+
+def percentiles(xs):
+    xs = sorted(xs)
+
+    def at(f):
+        return xs[min(len(xs) - 1, max(0, int(round(f * (len(xs) - 1)))))]
+    return {"median": at(0.5), "p10": at(0.1), "p90": at(0.9), "n": len(xs)}
+
+
+def operator_line(lib, dev, W, dtype, args, steps, warmup, full):
+    """Times one workload: K steps by the wall clock between synchronisations (the contract's figure), the same
+    K steps again between HIP events on the launch stream (median / p10 / p90), the forward alone, and every
+    kernel by events inside the library.  Every buffer (outputs, workspaces) is allocated once, before."""
+    import torch
     B, H, N, D, p = W["B"], W["H"], W["N"], W["D"], W["p"]
     bh = B * H
-    tdtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    tdtype = torch.bfloat16 if dtype == "bf16" else torch.float32
     gen = torch.Generator(device="cpu").manual_seed(1)
     q, k, v = ((W["scale"] * torch.randn(B, H, N, D, generator=gen)).to(tdtype).to(dev).view(bh, N, D) for _ in range(3))
     go = torch.randn(B, H, N, D, generator=gen).to(tdtype).to(dev).view(bh, N, D)
     tau = 8.0 * math.sqrt(D)
     kw = dict(mask=True, inv_tau=1.0 / tau, a0=1.0, a1=1.0, a2=0.5, p=p, chunk=args.chunk)
+    from reproducing_fastmax_results_amd._capi import FLAG_SAVE_FOR_BACKWARD
+    indep = args.independent_backward
+    desc = lib.make_desc(q, k, v, flags=0 if indep else FLAG_SAVE_FOR_BACKWARD, **kw)
+    fwd_b, bwd_b = lib.workspace_bytes(desc)
+    fwd_plain_b, _ = lib.workspace_bytes(lib.make_desc(q, k, v, **kw))
+    o, g = torch.empty_like(q), torch.empty(bh, N, dtype=torch.float32, device=dev)
+    grads = tuple(torch.empty_like(q) for _ in range(3))
+    ws_f, ws_b = (torch.empty(nb, dtype=torch.uint8, device=dev) for nb in (fwd_b, bwd_b))
+    ws_p = torch.empty(fwd_plain_b, dtype=torch.uint8, device=dev)
 
     def step():
         # the training step of the autograd wrapper: the forward keeps its workspace
         # (key-side copies, prefix states) and the backward of the same step reads it
-        if args.independent_backward:
-            o, g = lib.forward(q, k, v, **kw)
-            return lib.backward(q, k, v, o, g, go, **kw)
-        o, g, saved = lib.forward(q, k, v, save=True, **kw)
-        return lib.backward(q, k, v, o, g, go, saved=saved, **kw)
+        if indep:
+            lib.forward(q, k, v, out=o, g=g, ws=ws_f, **kw)
+            return lib.backward(q, k, v, o, g, go, out=grads, ws=ws_b, **kw)
+        lib.forward(q, k, v, save=True, out=o, g=g, ws=ws_f, **kw)
+        return lib.backward(q, k, v, o, g, go, saved=ws_f, out=grads, ws=ws_b, **kw)
 
     run = step
     if args.graph:
         # the whole step as one HIP graph: the library allocates nothing and never synchronises, so
-        # a caller can capture it; replays skip the host side of the four launches
+        # a caller can capture it; replays skip the host side of the launches
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -203,30 +284,40 @@ def main() -> int:
         with torch.cuda.graph(graph):
             step()
         run = graph.replay
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         run()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         run()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    ms_per_step = 1e3 * elapsed / args.steps
+    ms_per_step = 1e3 * elapsed / steps
     tokens = B * N
-    value = tokens * args.steps / elapsed
+    value = tokens * steps / elapsed
+
+    # the same steps between HIP events on the launch stream (torch's current stream is the stream the library
+    # launches on): the distribution of one step
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    evs[0].record()
+    for i in range(steps):
+        run()
+        evs[i + 1].record()
+    torch.cuda.synchronize()
+    step_ms = percentiles([evs[i].elapsed_time(evs[i + 1]) for i in range(steps)])
 
     # forward alone (the inference call: no workspace kept for a backward)
     for _ in range(3):
-        lib.forward(q, k, v, **kw)
+        lib.forward(q, k, v, out=o, g=g, ws=ws_p, **kw)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        lib.forward(q, k, v, **kw)
+    for _ in range(steps):
+        lib.forward(q, k, v, out=o, g=g, ws=ws_p, **kw)
     torch.cuda.synchronize()
-    fwd_ms = 1e3 * (time.perf_counter() - t0) / args.steps
+    fwd_ms = 1e3 * (time.perf_counter() - t0) / steps
 
     # per-kernel durations, HIP events on the launch stream
-    nprof = max(3, min(10, args.steps))
+    nprof = max(3, min(10, steps))
     lib.profile_begin()
     for _ in range(nprof):
         step()
@@ -241,9 +332,13 @@ def main() -> int:
     avg_ms = per_kernel[dominant][0] / per_kernel[dominant][1]
     unit = alg_flops_unit(bh, N, D, p)
     achieved = units[dominant] * unit / (avg_ms * 1e-3) / 1e12
-    peak = PEAK_TFLOPS[args.dtype]
+    peak = PEAK_TFLOPS[dtype]
+    # `achieved` / `frac`: ALGORITHMIC flop of the moment formulation per launch of the dominant kernel (the
+    # definition the metric fixes, whatever form the kernel computes in); `executed`: what its matrix
+    # instructions actually execute (set below when the kernel runs dense causal tiles only)
     roofline = {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
                 "frac": achieved / peak, "traffic": None, "avg_ms": avg_ms,
+                "algorithmic_flop_per_launch": units[dominant] * unit,
                 "whole_step": {"achieved": 7 * unit / (ms_per_step * 1e-3) / 1e12,
                                "frac": 7 * unit / (ms_per_step * 1e-3) / 1e12 / peak},
                 "kernels_ms_per_step": {nme: tot / nprof for nme, (tot, cnt) in sorted(per_kernel.items())}}
@@ -251,7 +346,7 @@ def main() -> int:
         # order 1 is bandwidth bound (M_1 = D features: 130 flop per byte of q, k, v, o): price it against HBM.
         # Algorithmic bytes: the forward reads q, k, v and writes o; the backward reads q, k, v, o, dO and
         # writes dq, dk, dv; per kernel, the tensors it must read and write once.
-        esz_io = 2 if args.dtype == "bf16" else 4
+        esz_io = 2 if dtype == "bf16" else 4
         tensor_b = bh * N * D * esz_io
         k_tensors = {"fwd": 4, "dq": 5, "dk": 5, "dv": 4, "dkv": 7, "build": 2}
         dom_b = k_tensors.get(dominant, 4) * tensor_b
@@ -260,39 +355,47 @@ def main() -> int:
                     "whole_step": {"achieved": 12 * tensor_b / (ms_per_step * 1e-3) / 1e9,
                                    "frac": 12 * tensor_b / (ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBS},
                     "kernels_ms_per_step": roofline["kernels_ms_per_step"]}
-    if "build" not in per_kernel and args.dtype == "bf16" and p == 2:
+    if "build" not in per_kernel and dtype == "bf16" and p == 2:
         # what the matrix cores actually execute when one segment covers the sequence: causal 32x32 tiles only
         nt = (N + 31) // 32
         tiles = bh * nt * (nt + 1) // 2
-        executed = sum(MFMA_PER_TILE[nme] for nme in per_kernel if nme in MFMA_PER_TILE) * tiles * 2.0 * 32 * 32 * 16
+        per_tile = 2.0 * 32 * 32 * 16
+        executed = sum(MFMA_PER_TILE[nme] for nme in per_kernel if nme in MFMA_PER_TILE) * tiles * per_tile
+        dom_exec = MFMA_PER_TILE[dominant] * tiles * per_tile
+        roofline["executed"] = {"flop_per_launch": dom_exec, "achieved": dom_exec / (avg_ms * 1e-3) / 1e12,
+                                "frac": dom_exec / (avg_ms * 1e-3) / 1e12 / peak}
         roofline["executed_mfma"] = {"flop_per_step": executed,
                                      "achieved": executed / (ms_per_step * 1e-3) / 1e12,
                                      "frac": executed / (ms_per_step * 1e-3) / 1e12 / peak}
-    if args.workload == "headline" and p == 2 and TRAFFIC_BYTES.get((args.dtype, args.chunk, dominant)) is not None:
-        roofline["traffic"] = TRAFFIC_BYTES[(args.dtype, args.chunk, dominant)]
-    if args.workload == "long" and p == 1 and args.dtype == "bf16" and args.chunk == 0:
-        roofline["traffic"] = TRAFFIC_BYTES_LONG_ORDER1.get(dominant)
+    tkey = (W["N"], p, dtype, args.chunk, dominant)
+    if tkey in TRAFFIC:
+        roofline["traffic"] = TRAFFIC[tkey]["bytes"]
+        roofline["traffic_source"] = TRAFFIC[tkey]["source"]
 
     out = {
         "metric": f"Fastmax fwd+bwd tokens/s, causal order-{p} N={N} D={D}",
-        "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": args.dtype, "data": "synthetic",
+        "dtype": dtype, "data": "synthetic",
         "config": {"workload": f"{W['name'].replace('order-2', f'order-{p}')} B={B} H={H} N={N} D=Dv={D} tau=8*sqrt(D) a=(1,1,0.5)",
                    "chunk": args.chunk or "auto", "launch": "hip graph replay" if args.graph else "eager"},
+        "step_ms": step_ms,
         "roofline": roofline,
         "forward_only": {"ms": fwd_ms, "tokens_per_s": tokens / (fwd_ms * 1e-3),
                          "algorithmic_TFLOPs": 2 * unit / (fwd_ms * 1e-3) / 1e12,
                          "frac_of_peak": 2 * unit / (fwd_ms * 1e-3) / 1e12 / peak},
     }
     # the bandwidth-bound helpers of the path on the same tensors: event-timed passes against the HBM peak
-    esz = 2 if args.dtype == "bf16" else 4
+    esz = 2 if dtype == "bf16" else 4
     tensor = bh * N * D * esz
     helpers = {}
     for name, fn, nbytes in (
-            # forward: one statistics read, one apply read, one write; backward: x and dy twice, dx once
-            ("normalize", lambda: lib.normalize(q, centre=0, max_norm=True, scale=1.0), 3 * tensor),
-            ("normalize_backward", lambda: lib.normalize_backward(q, go, centre=0, max_norm=True, scale=1.0), 5 * tensor)):
+            # the statistics pass of the folded max-norm normalisation: q and k read once (the kernels scale as they load)
+            ("normalize", lambda: lib.maxnorm_stats(q, k), 2 * tensor),) + (() if not full else (
+            # the stand-alone passes (token-mean centring and other callers): forward one statistics read, one apply
+            # read, one write; backward: x and dy twice, dx once
+            ("normalize_pass", lambda: lib.normalize(q, centre=0, max_norm=True, scale=1.0), 3 * tensor),
+            ("normalize_backward", lambda: lib.normalize_backward(q, go, centre=0, max_norm=True, scale=1.0), 5 * tensor))):
         fn()
         torch.cuda.synchronize()
         lib.profile_begin()
@@ -303,11 +406,35 @@ def main() -> int:
                          "frac_of_8TBps": nbytes / (ms * 1e-3) / 8e12}
     if "transpose" in roofline["kernels_ms_per_step"]:
         t_ms = roofline["kernels_ms_per_step"]["transpose"]
-        ncopies = 2 if (args.dtype == "bf16" and "build" not in per_kernel) else 4    # row-major (+ transposed) copies of k and v
+        ncopies = 2 if (dtype == "bf16" and "build" not in per_kernel) else 4    # row-major (+ transposed) copies of k and v
         nbytes = 2 * tensor + ncopies * bh * N * D * esz
         helpers["transpose"] = {"ms": t_ms, "bytes": nbytes, "achieved_GBps": nbytes / (t_ms * 1e-3) / 1e9,
                                 "frac_of_8TBps": nbytes / (t_ms * 1e-3) / 8e12}
     out["hbm_bound_helpers"] = helpers
+    if not full:
+        return out
+    # the same step with q and k max-norm normalised on load and the gradients taken through the normalisation
+    # (what the reference model's attention does, transformer/model.py:292-300), against the plain step
+    qk, kk = lib.maxnorm_stats(q, k)
+    nkw = dict(kw, norm=(qk, kk, 1.0, True), inv_tau=1.0)
+    nf, nb = lib.workspace_bytes(lib.make_desc(q, k, v, flags=FLAG_SAVE_FOR_BACKWARD, **nkw))
+    ws_nf, ws_nb = (torch.empty(x, dtype=torch.uint8, device=dev) for x in (nf, nb))
+
+    def norm_step():
+        lib.maxnorm_stats(q, k)
+        lib.forward(q, k, v, save=True, out=o, g=g, ws=ws_nf, **nkw)
+        return lib.backward(q, k, v, o, g, go, saved=ws_nf, out=grads, ws=ws_nb, **nkw)
+
+    for _ in range(3):
+        norm_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        norm_step()
+    torch.cuda.synchronize()
+    norm_ms = 1e3 * (time.perf_counter() - t0) / steps
+    out["normalized_step"] = {"ms_per_step": norm_ms, "over_plain_step": norm_ms / ms_per_step,
+                              "what": "max-norm normalisation of q and k folded into the loads, its Jacobian in the backward"}
     # what this box sustains, beside the published peaks the fractions above are priced against: a
     # register-only loop of 32x32x16 _Float16 matrix products, and a 1 GiB device-to-device copy
     # (read + write counted)
@@ -332,8 +459,8 @@ def main() -> int:
         torch.cuda.synchronize()
     if not args.no_cpu_baseline and args.workload == "headline" and p == 2:
         out["cpu_baseline"] = cpu_baseline(N, D, p, tokens, bh, args.cpu_max_n)
-    print(json.dumps(out))
-    return 0
+        out["cpu_baseline_closed_form"] = cpu_closed_form(N, D, p, tokens, bh)
+    return out
 
 
 if __name__ == "__main__":

@@ -72,6 +72,22 @@ typedef struct FastmaxStrides {
   int32_t reserved;
 } FastmaxStrides;
 
+/* Optional: the max-norm normalisation of q and k (x_hat = lim * x / max_n ||x_n||_2 per batch*head,
+ * reference transformer/model.py:97-102, the `normalize` flag of forwardpass) folded into the kernels'
+ * loads instead of a pass that rewrites the tensors (reference apply_norm, fastmax_cuda_forward.cu:326-338).
+ * q_keys / k_keys: device buffers written by fastmax_maxnorm_stats for the same q / k (null: that tensor is
+ * used as it is).  grad (backward only): zero -> dq and dk are the gradients with respect to the normalised
+ * tensors, which is what the reference's extension returns (its backward has no counterpart of apply_norm);
+ * non-zero -> with respect to the raw q and k, the normalisation's own Jacobian included (what the
+ * reference's Python variants get from autograd, score_function.py:40-55).  Not available for masked
+ * problems with nk > nq. */
+typedef struct FastmaxNormFold {
+  const void* q_keys;
+  const void* k_keys;
+  float lim;
+  int32_t grad;
+} FastmaxNormFold;
+
 /* Problem description shared by forward and backward.
  * Score s_ij = (q_i . k_j) * inv_tau;  weight f(s) = a0 + a1 s + a2 s^2 (a2 ignored when p == 1);
  * mask != 0: causal with nq <= nk, query i sees keys 0 .. nk - nq + i (the queries are aligned to
@@ -90,6 +106,7 @@ typedef struct FastmaxDesc {
   int32_t chunk;     /* segment length of the causal moment scan; 0 = automatic */
   int32_t flags;
   FastmaxStrides sq, sk, sv, so, sg, sdo, sdq, sdk, sdv;   /* sg: strides of the fp32 denominator g (bh, n) */
+  FastmaxNormFold norm;                                    /* all zero: off */
 } FastmaxDesc;
 
 /* Replaces the tensor allocations inside forward_cuda / backward_cuda
@@ -163,6 +180,14 @@ typedef struct FastmaxNormDesc {
 size_t fastmax_normalize_stats_bytes(const FastmaxNormDesc* desc);
 int fastmax_normalize(const FastmaxNormDesc* desc, const void* x, void* y, float* stats,
                       void* hip_stream);
+
+/* Statistics for FastmaxNormFold: one read of x (desc->bh, n, d, dtype, sx are used), leaving
+ * fastmax_maxnorm_stats_bytes(bh, n) bytes in `keys` (8-byte aligned device memory): per 256 tokens the
+ * largest squared token norm and its token.  A second tensor of the same batch*heads, head size and type
+ * (k beside q) can go in the same launch: desc1 / x1 / keys1, or null. */
+size_t fastmax_maxnorm_stats_bytes(int32_t bh, int32_t n);
+int fastmax_maxnorm_stats(const FastmaxNormDesc* desc0, const void* x0, void* keys0,
+                          const FastmaxNormDesc* desc1, const void* x1, void* keys1, void* hip_stream);
 
 /* Gradient of fastmax_normalize with respect to x, given dy (the gradient with respect to y).
  * The reference's extension has no counterpart: fastmax_cuda_backward.cu:518-613 returns the

@@ -30,6 +30,11 @@ class Strides(C.Structure):
         super().__init__(bh, n, b, heads, 0)
 
 
+class NormFold(C.Structure):
+    """FastmaxNormFold: max-norm normalisation of q and k folded into the kernels' loads."""
+    _fields_ = [("q_keys", C.c_void_p), ("k_keys", C.c_void_p), ("lim", C.c_float), ("grad", C.c_int32)]
+
+
 class Desc(C.Structure):
     _fields_ = [
         ("bh", C.c_int32), ("nq", C.c_int32), ("nk", C.c_int32), ("d", C.c_int32),
@@ -38,6 +43,7 @@ class Desc(C.Structure):
         ("chunk", C.c_int32), ("flags", C.c_int32),
         ("sq", Strides), ("sk", Strides), ("sv", Strides), ("so", Strides), ("sg", Strides),
         ("sdo", Strides), ("sdq", Strides), ("sdk", Strides), ("sdv", Strides),
+        ("norm", NormFold),
     ]
 
 
@@ -55,6 +61,7 @@ EXPORTS = (
     "fastmax_status_string", "fastmax_version", "fastmax_probe_mfma", "fastmax_probe_lds_transpose",
     "fastmax_probe_mfma_rate",
     "fastmax_profile_begin", "fastmax_profile_end", "fastmax_forward_static",
+    "fastmax_maxnorm_stats", "fastmax_maxnorm_stats_bytes",
 )
 STATIC_SCRATCH_BYTES = 64 << 20     # FASTMAX_STATIC_SCRATCH_BYTES
 
@@ -134,6 +141,11 @@ class FastmaxLib:
         L.fastmax_normalize_backward.restype = C.c_int
         L.fastmax_normalize_backward_stats_bytes.argtypes = [C.POINTER(NormDesc)]
         L.fastmax_normalize_backward_stats_bytes.restype = C.c_size_t
+        L.fastmax_maxnorm_stats_bytes.argtypes = [C.c_int32, C.c_int32]
+        L.fastmax_maxnorm_stats_bytes.restype = C.c_size_t
+        L.fastmax_maxnorm_stats.argtypes = [C.POINTER(NormDesc), C.c_void_p, C.c_void_p, C.POINTER(NormDesc), C.c_void_p,
+                                            C.c_void_p, C.c_void_p]
+        L.fastmax_maxnorm_stats.restype = C.c_int
         L.fastmax_status_string.argtypes = [C.c_int]
         L.fastmax_status_string.restype = C.c_char_p
         L.fastmax_version.restype = C.c_int
@@ -161,7 +173,29 @@ class FastmaxLib:
             return torch.cuda.current_stream(t.device).cuda_stream
         return 0
 
-    def make_desc(self, q, k, v, *, mask, inv_tau, a0, a1, a2, p, chunk=0, flags=0) -> Desc:
+    def maxnorm_stats(self, q, k=None):
+        """Statistics of the folded max-norm normalisation (fastmax_maxnorm_stats): one int64 tensor
+        (bh, blocks of 256 tokens) per given tensor, q and k in one launch."""
+        descs, keys = [], []
+        for t in (q, k):
+            if t is None:
+                continue
+            nd = NormDesc()
+            nd.bh, nd.n, nd.d = _dims(t)
+            nd.dtype, nd.sx = _dtype_code(t), _strides(t)
+            descs.append(nd)
+            nbytes = self.lib.fastmax_maxnorm_stats_bytes(nd.bh, nd.n)
+            keys.append(torch.empty(nd.bh, nbytes // 8 // nd.bh, dtype=torch.int64, device=t.device))
+        if k is None:
+            st = self.lib.fastmax_maxnorm_stats(C.byref(descs[0]), q.data_ptr(), keys[0].data_ptr(), None, None, None,
+                                                self._stream(q))
+        else:
+            st = self.lib.fastmax_maxnorm_stats(C.byref(descs[0]), q.data_ptr(), keys[0].data_ptr(), C.byref(descs[1]),
+                                                k.data_ptr(), keys[1].data_ptr(), self._stream(q))
+        self.check(st, "fastmax_maxnorm_stats")
+        return keys[0] if k is None else tuple(keys)
+
+    def make_desc(self, q, k, v, *, mask, inv_tau, a0, a1, a2, p, chunk=0, flags=0, norm=None) -> Desc:
         d = Desc()
         d.bh, d.nq, d.d = _dims(q)
         kb, d.nk, kd = _dims(k)
@@ -174,6 +208,12 @@ class FastmaxLib:
         d.a0, d.a1, d.a2, d.inv_tau = float(a0), float(a1), float(a2), float(inv_tau)
         d.chunk, d.flags = int(chunk), int(flags)
         d.sq, d.sk, d.sv = _strides(q), _strides(k), _strides(v)
+        if norm is not None:
+            # (q_keys, k_keys, lim, grad): tensors from maxnorm_stats (or None), see FastmaxNormFold
+            qk, kk, lim, grad = norm
+            d.norm.q_keys = qk.data_ptr() if qk is not None else None
+            d.norm.k_keys = kk.data_ptr() if kk is not None else None
+            d.norm.lim, d.norm.grad = float(lim), int(bool(grad))
         return d
 
     def workspace_bytes(self, desc: Desc) -> Tuple[int, int]:
@@ -191,13 +231,17 @@ class FastmaxLib:
 
     # -- entry points ------------------------------------------------------------
     def forward(self, q, k, v, *, mask, inv_tau, a0=1.0, a1=1.0, a2=0.5, p=2, chunk=0, flags=0,
-                out: Optional[torch.Tensor] = None, g: Optional[torch.Tensor] = None, save: bool = False):
+                out: Optional[torch.Tensor] = None, g: Optional[torch.Tensor] = None, save: bool = False,
+                ws: Optional[torch.Tensor] = None, norm=None):
         """q (bh, nq, d), k, v (bh, nk, d) views with contiguous features, or (b, h, n, d) views.
         Returns (o, g): o shaped like q, g (bh, nq) or (b, h, nq) float32; with ``save`` also the
-        workspace tensor that ``backward(..., saved=...)`` can reuse."""
+        workspace tensor that ``backward(..., saved=...)`` can reuse.  ``out``, ``g`` and ``ws`` (a uint8
+        tensor of at least ``workspace_bytes(desc)[0]`` bytes, 256-byte aligned) may be the caller's: a
+        call that is given all three allocates nothing and asks the library nothing beforehand."""
         if save:
             flags |= FLAG_SAVE_FOR_BACKWARD
-        desc = self.make_desc(q, k, v, mask=mask, inv_tau=inv_tau, a0=a0, a1=a1, a2=a2, p=p, chunk=chunk, flags=flags)
+        desc = self.make_desc(q, k, v, mask=mask, inv_tau=inv_tau, a0=a0, a1=a1, a2=a2, p=p, chunk=chunk, flags=flags,
+                              norm=norm)
         lead = tuple(q.shape[:-2])
         if out is None:
             out = torch.empty(lead + (desc.nq, desc.d), dtype=q.dtype, device=q.device)
@@ -205,10 +249,11 @@ class FastmaxLib:
             g = torch.empty(lead + (desc.nq,), dtype=torch.float32, device=q.device)
         desc.so = _strides(out)
         desc.sg = _gstrides(g)
-        fwd, _ = self.workspace_bytes(desc)
-        ws = self._workspace(fwd, q.device)
+        if ws is None:
+            fwd, _ = self.workspace_bytes(desc)
+            ws = self._workspace(fwd, q.device)
         st = self.lib.fastmax_forward(C.byref(desc), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
-                                      g.data_ptr(), ws.data_ptr(), fwd, self._stream(q))
+                                      g.data_ptr(), ws.data_ptr(), ws.numel(), self._stream(q))
         self.check(st, "fastmax_forward")
         if save:
             return out, g, ws
@@ -226,23 +271,30 @@ class FastmaxLib:
         return out, g
 
     def backward(self, q, k, v, o, g, d_o, *, mask, inv_tau, a0=1.0, a1=1.0, a2=0.5, p=2, chunk=0, flags=0,
-                 saved: Optional[torch.Tensor] = None):
+                 saved: Optional[torch.Tensor] = None, out=None, ws: Optional[torch.Tensor] = None, norm=None):
         """Gradients (dq, dk, dv) of sum(o * d_o); all tensors are (bh, n, d) views.
-        ``saved``: the workspace returned by ``forward(..., save=True)`` for the same problem."""
+        ``saved``: the workspace returned by ``forward(..., save=True)`` for the same problem.
+        ``out``: caller-owned (dq, dk, dv); ``ws``: caller-owned workspace (see ``forward``)."""
         if saved is not None:
             flags |= FLAG_SAVE_FOR_BACKWARD
-        desc = self.make_desc(q, k, v, mask=mask, inv_tau=inv_tau, a0=a0, a1=a1, a2=a2, p=p, chunk=chunk, flags=flags)
+        desc = self.make_desc(q, k, v, mask=mask, inv_tau=inv_tau, a0=a0, a1=a1, a2=a2, p=p, chunk=chunk, flags=flags,
+                              norm=norm)
         if o.dtype != q.dtype or d_o.dtype != q.dtype or g.dtype != torch.float32:
             raise FastmaxError("fastmax: o and d_o must have q's dtype and g must be float32")
         lead = tuple(q.shape[:-2])
-        dq = torch.empty(lead + (desc.nq, desc.d), dtype=q.dtype, device=q.device)
-        dk = torch.empty(lead + (desc.nk, desc.d), dtype=q.dtype, device=q.device)
-        dv = torch.empty(lead + (desc.nk, desc.d), dtype=q.dtype, device=q.device)
+        if out is not None:
+            dq, dk, dv = out
+        else:
+            dq = torch.empty(lead + (desc.nq, desc.d), dtype=q.dtype, device=q.device)
+            dk = torch.empty(lead + (desc.nk, desc.d), dtype=q.dtype, device=q.device)
+            dv = torch.empty(lead + (desc.nk, desc.d), dtype=q.dtype, device=q.device)
         desc.so, desc.sdo = _strides(o), _strides(d_o)
         desc.sg = _gstrides(g)
         desc.sdq, desc.sdk, desc.sdv = _strides(dq), _strides(dk), _strides(dv)
-        _, bwd = self.workspace_bytes(desc)
-        ws = self._workspace(bwd, q.device)
+        if ws is None:
+            _, bwd = self.workspace_bytes(desc)
+            ws = self._workspace(bwd, q.device)
+        bwd = ws.numel()
         if saved is not None:
             st = self.lib.fastmax_backward_saved(C.byref(desc), q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
                                                  g.data_ptr(), d_o.data_ptr(), dq.data_ptr(), dk.data_ptr(),

@@ -29,7 +29,7 @@ from .. import fastmax_cuda as _ext   # the torch binding built by __graft_entry
 
 __all__ = [
     "FASTMultiHeadAttention_Function", "FASTMultiHeadAttention", "rpe_matrix_creator", "fastmax_custom",
-    "fastmax", "fastmax_einops", "FastmaxNormalize",
+    "fastmax", "fastmax_einops", "FastmaxNormalize", "FastmaxNormAttention",
 ]
 
 CENTRE_NONE, CENTRE_FEATURE, CENTRE_TOKEN = 0, 1, 2
@@ -75,6 +75,43 @@ class FastmaxNormalize(torch.autograd.Function):
         return _ext.normalize_backward(x, grad_y, ctx.centre, True, ctx.scale)[..., :ctx.d], None, None
 
 
+def _fold_possible(q, k, mask):
+    """The folded normalisation covers everything but causal attention with more keys than queries
+    (two sub-problems would share one Jacobian); that case takes the separate normalisation pass."""
+    return not (mask and k.shape[-2] > q.shape[-2])
+
+
+class FastmaxNormAttention(torch.autograd.Function):
+    """Fastmax attention on ``lim * x / max_n ||x_n||_2`` of q and k (per batch and head), the
+    normalisation folded into the kernels: one statistics pass reads q and k once, the attention
+    kernels scale the rows as they load them, and the backward returns the gradients with respect to
+    the RAW q and k, the normalisation's own Jacobian included (the dQ / dK kernels scale what they
+    store and one small kernel adds the rank-one term of the row with the largest norm).  Replaces the
+    reference's ``apply_norm`` pass (``fastmax_cuda_forward.cu:326-338``) and the autograd graph of its
+    Python variants (``score_function.py:40-55``); semantics of ``transformer/model.py:97-102``."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, mask=False, lim=1.0, temperature=1.0, a0=1.0, a1=1.0, a2=0.5, p=2):
+        d = q.shape[-1]
+        q, k, v = _pad_features(q), _pad_features(k), _pad_features(v)
+        qk, kk = _ext.maxnorm_stats(q, k)
+        cfg = (bool(mask), 1.0 / float(temperature), float(a0), float(a1), float(a2), int(p))
+        o, g, saved = _ext.forward_norm(q, k, v, qk, kk, float(lim), *cfg, 0, 0)
+        if any(ctx.needs_input_grad[:3]):
+            ctx.save_for_backward(q, k, v, o, g, saved, qk, kk)
+        ctx.cfg, ctx.lim, ctx.d = cfg, float(lim), d
+        return o[..., :d]
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        q, k, v, o, g, saved, qk, kk = ctx.saved_tensors
+        if q.shape[-1] != ctx.d:
+            grad_output = _pad_features(grad_output)
+        gq, gk, gv = _ext.backward_norm(q, k, v, o, g, grad_output, saved, qk, kk, ctx.lim, True, *ctx.cfg, 0, 0)
+        d = ctx.d
+        return (gq[..., :d], gk[..., :d], gv[..., :d]) + (None,) * 7
+
+
 class FASTMultiHeadAttention_Function(torch.autograd.Function):
     """Same call as reference ``transformer/model.py:16``.  q, k, v: ``(b, h, n, d)`` or
     ``(b*h, n, d)``.  ``drop_noise``, ``rpe_matrix`` and ``dropout`` are accepted and unused,
@@ -93,10 +130,22 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
                              "If 3D: (b*h,n,d), if 4D: (b,h,n,d).")
         d = q.shape[-1]
         q, k, v = _pad_features(q), _pad_features(k), _pad_features(v)
+        inv_tau = 1.0 / float(temperature)
+        ctx.fold = None
+        if normalize and _fold_possible(q, k, mask):
+            # normalised on load; like the reference, the backward returns the gradients with respect to the
+            # normalised q and k (its extension has no backward of apply_norm)
+            qk, kk = _ext.maxnorm_stats(q, k)
+            o, g, saved = _ext.forward_norm(q, k, v, qk, kk, float(lim), bool(mask), inv_tau, float(a0), float(a1),
+                                            float(a2), int(p), 0, 0)
+            if any(ctx.needs_input_grad[:3]):
+                ctx.save_for_backward(q, k, v, o, g, saved, qk, kk)
+            ctx.fold = float(lim)
+            ctx.cfg = (bool(mask), inv_tau, float(a0), float(a1), float(a2), int(p), d)
+            return o[..., :d]
         if normalize:
             q = _ext.normalize(q, CENTRE_NONE, True, float(lim))
             k = _ext.normalize(k, CENTRE_NONE, True, float(lim))
-        inv_tau = 1.0 / float(temperature)
         needs_grad = any(ctx.needs_input_grad[:3])
         if needs_grad:
             # keep the key-side copies and prefix states the forward built: the backward reuses them
@@ -109,8 +158,15 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_output):
-        q, k, v, o, g, saved = ctx.saved_tensors
         mask, inv_tau, a0, a1, a2, p, d = ctx.cfg
+        if ctx.fold is not None:
+            q, k, v, o, g, saved, qk, kk = ctx.saved_tensors
+            if q.shape[-1] != d:
+                grad_output = _pad_features(grad_output)
+            gq, gk, gv = _ext.backward_norm(q, k, v, o, g, grad_output, saved, qk, kk, ctx.fold, False, mask, inv_tau,
+                                            a0, a1, a2, p, 0, 0)
+            return (gq[..., :d], gk[..., :d], gv[..., :d]) + (None,) * 11
+        q, k, v, o, g, saved = ctx.saved_tensors
         if q.shape[-1] != d:
             grad_output = _pad_features(grad_output)
         gq, gk, gv = _ext.backward_saved(q, k, v, o, g, grad_output, saved, mask, inv_tau, a0, a1, a2, p, 0, 0)

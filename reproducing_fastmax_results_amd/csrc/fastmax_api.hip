@@ -93,13 +93,14 @@ struct Plan {
   int L, nseg, nslots;
   bool use_state, quad;
   bool rows_build;      // order-1 segment sums read the row-major copies: no transposed copy is written
+  bool qf;              // dense _Float16 kernels evaluate the order-2 weights in completed-square form (see TileMath)
   int npad_q, npad_k;
   float a0, a1, a2;     // polynomial on the score s = (q.k) / tau
   float sc;             // sqrt(1/tau), folded into q and k when they are converted
   // workspace offsets (bytes)
   size_t kt, vt, kr, vr, big, big2, small, fwd_bytes;
   bool save;
-  size_t b_kr, b_vr, b_qr, b_kt, b_vt, b_qt, b_qct, b_gh, b_ght, b_cv, b_bigq, b_smallq, b_bigk, b_smallk, b_bigv, b_gpart, bwd_bytes;
+  size_t b_kr, b_vr, b_qr, b_kt, b_vt, b_qt, b_qct, b_gh, b_ght, b_cv, b_bigq, b_smallq, b_bigk, b_smallk, b_bigv, b_gpart, b_bq, b_bk, bwd_bytes;
 };
 
 bool strides_ok(const FastmaxStrides& s, int bh, int n, int d) {
@@ -127,6 +128,11 @@ int validate(const FastmaxDesc* d) {
   if (d->mask && d->nq > d->nk) return FASTMAX_ERR_UNSUPPORTED;   // nk > nq: see SplitPlan
   if (d->chunk < 0) return FASTMAX_ERR_SHAPE;
   if (!(d->inv_tau > 0.0f) || !(d->inv_tau < 3.0e38f)) return FASTMAX_ERR_SHAPE;   // also rejects NaN
+  if (d->norm.q_keys || d->norm.k_keys) {
+    if (d->mask && d->nk > d->nq) return FASTMAX_ERR_UNSUPPORTED;                    // two parts would share one Jacobian
+    if (!(d->norm.lim > 0.0f) || !(d->norm.lim < 3.0e38f)) return FASTMAX_ERR_SHAPE;
+    if ((reinterpret_cast<uintptr_t>(d->norm.q_keys) | reinterpret_cast<uintptr_t>(d->norm.k_keys)) % 8) return FASTMAX_ERR_SHAPE;
+  }
   return FASTMAX_OK;
 }
 
@@ -175,6 +181,12 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
     p.nslots = p.use_state ? 1 : 0;
   }
   p.rows_build = p.half && p.use_state && !p.quad && d->mask;
+  {
+    // f = (h^2 + kc) / (4 a2) with h = 2 a2 s + a1: worth it, and safe in _Float16, when a2 and kc are of ordinary size
+    const float kc = 4.0f * p.a0 * p.a2 - p.a1 * p.a1;
+    p.qf = p.half && p.quad && !p.use_state && std::fabs(p.a2) >= 0.0625f && std::fabs(p.a2) <= 4.0f &&
+           std::fabs(kc) <= 1024.0f && std::fabs(p.a1) <= 64.0f;
+  }
   const size_t slots = size_t(d->bh) * p.nslots;
   const size_t bigarr = d->d == 64 ? big_array_bytes<64>(p.esz, p.quad, slots) : big_array_bytes<32>(p.esz, p.quad, slots);
   const size_t smallsz = size_t(d->d == 64 ? StateDims<64>::SMALL : StateDims<32>::SMALL) * 4;
@@ -203,6 +215,10 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   p.b_bigk = take(bigarr); p.b_smallk = take(size_t(d->bh) * p.nslots * smallsz);
   p.b_bigv = take(bigarr);
   p.b_gpart = take(p.half ? size_t(d->bh) * fm_grad_scale_blocks(d->nq) * 4 : 0);   // see k_grad_scale
+  // parts of B = sum dy . y per workgroup of the dQ and dK kernels (128 own tokens at least), see k_norm_fix
+  const bool jac = d->norm.grad != 0;
+  p.b_bq = take(jac && d->norm.q_keys ? size_t(d->bh) * ((d->nq + 127) / 128) * 4 : 0);
+  p.b_bk = take(jac && d->norm.k_keys ? size_t(d->bh) * ((d->nk + 127) / 128) * 4 : 0);
   p.bwd_bytes = off ? off : 256;
   return FASTMAX_OK;
 }
@@ -214,10 +230,10 @@ template <typename T> TRef<T> mref(void* ptr, const FastmaxStrides& s) { return 
 
 // k and v (same length) in one launch
 template <typename TIO, typename E, int DH>
-int launch_transpose2(const void* x0, const FastmaxStrides& s0, E* xt0, E* xr0, float scale0, const void* x1,
-                      const FastmaxStrides& s1, E* xt1, E* xr1, float scale1, int bh, int n, int npad,
-                      fm_stream_t stream) {
-  const TransposeJob<TIO, E> j0{cref<TIO>(x0, s0), xt0, xr0, scale0}, j1{cref<TIO>(x1, s1), xt1, xr1, scale1};
+int launch_transpose2(const void* x0, const FastmaxStrides& s0, E* xt0, E* xr0, float scale0, const NormFold& f0,
+                      const void* x1, const FastmaxStrides& s1, E* xt1, E* xr1, float scale1, const NormFold& f1, int bh,
+                      int n, int npad, fm_stream_t stream) {
+  const TransposeJob<TIO, E> j0{cref<TIO>(x0, s0), xt0, xr0, scale0, f0}, j1{cref<TIO>(x1, s1), xt1, xr1, scale1, f1};
   ProfScope prof(FM_K_TRANSPOSE, stream);
   FM_KERNEL_LAUNCH((k_transpose<TIO, E, DH>), fm_dim3(npad / 64, bh, 2), fm_dim3(FM_THREADS), 0, stream, j0, j1, n, npad);
   return fm_launch_status();
@@ -335,7 +351,15 @@ template <typename E, int DH, int QT> size_t tok_lds_bytes(int kind) {
   return size_t(2 * DH) * 4 + body;
 }
 
+inline NormFold fold_of(const void* keys, int n, float lim) {
+  return NormFold{static_cast<const unsigned long long*>(keys), fm_maxnorm_blocks(n), lim};
+}
+inline NormFold q_fold(const FastmaxDesc* d) { return fold_of(d->norm.q_keys, d->nq, d->norm.lim); }
+inline NormFold k_fold(const FastmaxDesc* d) { return fold_of(d->norm.k_keys, d->nk, d->norm.lim); }
+const NormFold no_fold{nullptr, 0, 1.0f};
+
 template <typename TIO, typename E> void tok_common(TokArgs<TIO, E>& a, const FastmaxDesc* d, const Plan& p) {
+  a.own_fold = no_fold; a.out_fold = no_fold; a.brows = nullptr; a.bpart = nullptr;
   a.own_io = TRef<const TIO>{nullptr, 0, 0, 0, 0, 0};
   a.own_r = nullptr; a.own2_r = nullptr; a.cv = nullptr; a.xr = nullptr; a.yr = nullptr; a.zt = nullptr; a.zt2 = nullptr;
   a.out2 = TRef<TIO>{nullptr, 0, 0, 0, 0, 0}; a.out2_scale = 1.0f;
@@ -346,24 +370,24 @@ template <typename TIO, typename E> void tok_common(TokArgs<TIO, E>& a, const Fa
   a.w_gh = nullptr; a.w_qr = nullptr; a.w_cv = nullptr; a.gpart = nullptr; a.gnblk = 0;
 }
 
-template <typename TIO, typename E, int DH, int QT, int OWN>
+template <typename TIO, typename E, int DH, int QT, int OWN, int QF = 0>
 int launch_pv(const TokArgs<TIO, E>& a, int bh, int kernel_id, fm_stream_t stream) {
   typedef TokCfg<E, DH, QT> C;
   const size_t lds = tok_lds_bytes<E, DH, QT>(0);
-  fm_allow_lds(reinterpret_cast<const void*>(&k_pv<TIO, E, DH, QT, OWN>), lds);
+  fm_allow_lds(reinterpret_cast<const void*>(&k_pv<TIO, E, DH, QT, OWN, QF>), lds);
   ProfScope prof(kernel_id, stream);
-  FM_KERNEL_LAUNCH((k_pv<TIO, E, DH, QT, OWN>), fm_dim3((a.n_own + C::QW - 1) / C::QW, bh), fm_dim3(FM_THREADS), lds,
+  FM_KERNEL_LAUNCH((k_pv<TIO, E, DH, QT, OWN, QF>), fm_dim3((a.n_own + C::QW - 1) / C::QW, bh), fm_dim3(FM_THREADS), lds,
                    stream, a);
   return fm_launch_status();
 }
 
-template <typename TIO, typename E, int DH, int QT, int OWN, int DV = 0, int PREP = 0>
+template <typename TIO, typename E, int DH, int QT, int OWN, int DV = 0, int PREP = 0, int QF = 0>
 int launch_ds(const TokArgs<TIO, E>& a, int bh, int kernel_id, fm_stream_t stream) {
   typedef TokCfg<E, DH, QT> C;
   const size_t lds = tok_lds_bytes<E, DH, QT>(PREP ? 3 : (DV ? 2 : 1));
-  fm_allow_lds(reinterpret_cast<const void*>(&k_ds<TIO, E, DH, QT, OWN, DV, PREP>), lds);
+  fm_allow_lds(reinterpret_cast<const void*>(&k_ds<TIO, E, DH, QT, OWN, DV, PREP, QF>), lds);
   ProfScope prof(kernel_id, stream);
-  FM_KERNEL_LAUNCH((k_ds<TIO, E, DH, QT, OWN, DV, PREP>), fm_dim3((a.n_own + C::QW - 1) / C::QW, bh), fm_dim3(FM_THREADS), lds,
+  FM_KERNEL_LAUNCH((k_ds<TIO, E, DH, QT, OWN, DV, PREP, QF>), fm_dim3((a.n_own + C::QW - 1) / C::QW, bh), fm_dim3(FM_THREADS), lds,
                    stream, a);
   return fm_launch_status();
 }
@@ -380,7 +404,8 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   // the transposed copies feed the state walk and the fp32 kernels; the _Float16 token kernels read
   // transposed fragments out of row tiles
   if (sizeof(E) == 2 && (!p.use_state || p.rows_build)) { kt = nullptr; vt = nullptr; }
-  int st = launch_transpose2<TIO, E, DH>(v, d->sv, vt, vr, 1.0f, k, d->sk, kt, kr, p.sc, d->bh, d->nk, p.npad_k, stream);
+  int st = launch_transpose2<TIO, E, DH>(v, d->sv, vt, vr, 1.0f, no_fold, k, d->sk, kt, kr, p.sc, k_fold(d), d->bh, d->nk,
+                                         p.npad_k, stream);
   if (st) return st;
   if (p.use_state) {
     BuildArgs<E> b;
@@ -399,6 +424,7 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   TokArgs<TIO, E> a;
   tok_common(a, d, p);
   a.own_io = cref<TIO>(q, d->sq);
+  a.own_fold = q_fold(d);
   a.xr = kr; a.yr = vr; a.zt = vt; a.npad_own = p.npad_q; a.npad_str = p.npad_k;
   a.big = big; a.small = small;
   a.out = mref<TIO>(o, d->so);
@@ -408,6 +434,9 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   // at B*H = 16, N = 65536 on MI355X); without states one tile per wavefront and more workgroups per CU win
   if (sizeof(E) == 2 && p.use_state && p.quad)
     return launch_pv<TIO, E, DH, (sizeof(E) == 2 ? 2 : QT), FM_OWN_Q>(a, d->bh, FM_K_FWD, stream);
+  if constexpr (sizeof(E) == 2) {
+    if (p.qf) return launch_pv<TIO, E, DH, 1, FM_OWN_Q, 1>(a, d->bh, FM_K_FWD, stream);
+  }
   return launch_pv<TIO, E, DH, QT, FM_OWN_Q>(a, d->bh, FM_K_FWD, stream);
 }
 
@@ -678,6 +707,30 @@ size_t fastmax_normalize_stats_bytes(const FastmaxNormDesc* desc) {
 int fastmax_normalize(const FastmaxNormDesc* desc, const void* x, void* y, float* stats, void* hip_stream) {
   ProfScope prof(FM_K_NORM, static_cast<fm_stream_t>(hip_stream));   // the whole pass (its kernels together)
   return fm_normalize_dispatch(desc, x, y, stats, static_cast<fm_stream_t>(hip_stream));
+}
+
+size_t fastmax_maxnorm_stats_bytes(int32_t bh, int32_t n) {
+  if (bh <= 0 || n <= 0) return 0;
+  return size_t(bh) * size_t(fm_maxnorm_blocks(n)) * 8;
+}
+
+int fastmax_maxnorm_stats(const FastmaxNormDesc* desc0, const void* x0, void* keys0, const FastmaxNormDesc* desc1,
+                          const void* x1, void* keys1, void* hip_stream) {
+  if (!desc0 || !x0 || !keys0) return FASTMAX_ERR_NULL;
+  const bool two = desc1 != nullptr;
+  if (two && (!x1 || !keys1)) return FASTMAX_ERR_NULL;
+  for (const FastmaxNormDesc* d : {desc0, desc1}) {
+    if (!d) continue;
+    if (d->dtype != FASTMAX_F32 && d->dtype != FASTMAX_BF16) return FASTMAX_ERR_DTYPE;
+    if (d->bh <= 0 || d->n <= 0 || d->bh > 65535 || d->n > (1 << 30)) return FASTMAX_ERR_SHAPE;
+    if (d->d != 32 && d->d != 64) return FASTMAX_ERR_UNSUPPORTED;
+    if (d->sx.n < d->d && d->n > 1) return FASTMAX_ERR_SHAPE;
+  }
+  if (two && (desc1->bh != desc0->bh || desc1->d != desc0->d || desc1->dtype != desc0->dtype)) return FASTMAX_ERR_SHAPE;
+  if ((reinterpret_cast<uintptr_t>(keys0) | reinterpret_cast<uintptr_t>(keys1)) % 8) return FASTMAX_ERR_WORKSPACE;
+  fm_stream_t stream = static_cast<fm_stream_t>(hip_stream);
+  ProfScope prof(FM_K_NORM, stream);
+  return fm_maxnorm_dispatch(desc0, x0, keys0, desc1, x1, keys1, stream);
 }
 
 size_t fastmax_normalize_backward_stats_bytes(const FastmaxNormDesc* desc) {

@@ -200,6 +200,28 @@ FastmaxStrides gstrides_of(const torch::Tensor& g) {
   return FastmaxStrides{g.stride(0), g.stride(1), 0, 0, 0};
 }
 
+// Folded max-norm normalisation (FastmaxNormFold): the key tensors of maxnorm_stats, or undefined tensors for "off".
+struct NormArgs {
+  torch::Tensor q_keys, k_keys;
+  double lim = 1.0;
+  bool grad = false;
+};
+
+void apply_norm_args(FastmaxDesc& d, const NormArgs* na) {
+  if (!na) return;
+  auto check = [&](const torch::Tensor& t, int64_t n, const char* what) -> const void* {
+    if (!t.defined()) return nullptr;
+    TORCH_CHECK(t.is_cuda() && t.scalar_type() == torch::kInt64 && t.is_contiguous() &&
+                    t.numel() * 8 == int64_t(fastmax_maxnorm_stats_bytes(d.bh, static_cast<int32_t>(n))),
+                what, " must be the int64 tensor maxnorm_stats returned for this tensor");
+    return t.data_ptr();
+  };
+  d.norm.q_keys = check(na->q_keys, d.nq, "q_keys");
+  d.norm.k_keys = check(na->k_keys, d.nk, "k_keys");
+  d.norm.lim = float(na->lim);
+  d.norm.grad = na->grad ? 1 : 0;
+}
+
 FastmaxDesc ex_desc(const View& q, const View& k, const View& v, bool mask, double inv_tau, double a0, double a1,
                     double a2, int64_t p, int64_t chunk, int64_t flags) {
   FM_CHECK_CUDA(q.t); FM_CHECK_CUDA(k.t); FM_CHECK_CUDA(v.t);
@@ -221,9 +243,11 @@ FastmaxDesc ex_desc(const View& q, const View& k, const View& v, bool mask, doub
 }
 
 std::vector<torch::Tensor> forward_any(torch::Tensor q_, torch::Tensor k_, torch::Tensor v_, bool mask, double inv_tau,
-                                       double a0, double a1, double a2, int64_t p, int64_t chunk, int64_t flags) {
+                                       double a0, double a1, double a2, int64_t p, int64_t chunk, int64_t flags,
+                                       const NormArgs* na = nullptr) {
   const View q = view_of(q_, "q"), k = view_of(k_, "k"), v = view_of(v_, "v");
   FastmaxDesc d = ex_desc(q, k, v, mask, inv_tau, a0, a1, a2, p, chunk, flags);
+  apply_norm_args(d, na);
   torch::Tensor o = empty_like_layout(q.t, q.n, q.t.scalar_type());
   torch::Tensor g = q.t.dim() == 4 ? torch::empty({q.t.size(0), q.t.size(1), q.n}, q.t.options().dtype(torch::kFloat32))
                                    : torch::empty({q.bh, q.n}, q.t.options().dtype(torch::kFloat32));
@@ -257,10 +281,11 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> forward_save(torch::Tens
 std::vector<torch::Tensor> backward_any(torch::Tensor q_, torch::Tensor k_, torch::Tensor v_, torch::Tensor o_,
                                         torch::Tensor g_, torch::Tensor go_, const torch::Tensor* saved, bool mask,
                                         double inv_tau, double a0, double a1, double a2, int64_t p, int64_t chunk,
-                                        int64_t flags) {
+                                        int64_t flags, const NormArgs* na = nullptr) {
   const View q = view_of(q_, "q"), k = view_of(k_, "k"), v = view_of(v_, "v");
   const View o = view_of(o_, "o"), go = view_of(go_, "grad_output");
   FastmaxDesc d = ex_desc(q, k, v, mask, inv_tau, a0, a1, a2, p, chunk, flags);
+  apply_norm_args(d, na);
   TORCH_CHECK(o.t.scalar_type() == q.t.scalar_type() && go.t.scalar_type() == q.t.scalar_type(),
               "o and grad_output must match q");
   TORCH_CHECK(o.bh == q.bh && o.n == q.n && o.d == q.d && go.bh == q.bh && go.n == q.n && go.d == q.d,
@@ -307,6 +332,47 @@ std::vector<torch::Tensor> backward_saved(torch::Tensor q, torch::Tensor k, torc
                                           int64_t flags) {
   return backward_any(q, k, v, o, g, go, &saved, mask, inv_tau, a0, a1, a2, p, chunk,
                       flags | FASTMAX_FLAG_SAVE_FOR_BACKWARD);
+}
+
+// Statistics of the folded max-norm normalisation for q and k in one launch (fastmax_maxnorm_stats): two int64
+// tensors (bh, blocks of 256 tokens).
+std::tuple<torch::Tensor, torch::Tensor> maxnorm_stats(torch::Tensor q_, torch::Tensor k_) {
+  const View q = view_of(q_, "q"), k = view_of(k_, "k");
+  FM_CHECK_CUDA(q.t); FM_CHECK_CUDA(k.t);
+  TORCH_CHECK(k.bh == q.bh && k.d == q.d && k.t.scalar_type() == q.t.scalar_type(), "q and k must agree in batch*heads, head size and dtype");
+  FastmaxNormDesc dq{}, dk{};
+  dq.bh = static_cast<int32_t>(q.bh); dq.n = static_cast<int32_t>(q.n); dq.d = static_cast<int32_t>(q.d);
+  dq.dtype = dtype_code(q.t); dq.sx = q.s;
+  dk = dq; dk.n = static_cast<int32_t>(k.n); dk.sx = k.s;
+  auto keys = [&](int32_t n) {
+    return torch::empty({q.bh, int64_t(fastmax_maxnorm_stats_bytes(dq.bh, n) / 8 / q.bh)}, q.t.options().dtype(torch::kInt64));
+  };
+  torch::Tensor kq = keys(dq.n), kk = keys(dk.n);
+  check_status(fastmax_maxnorm_stats(&dq, q.t.data_ptr(), kq.data_ptr(), &dk, k.t.data_ptr(), kk.data_ptr(), stream_of(q.t)),
+               "fastmax_maxnorm_stats");
+  return {kq, kk};
+}
+
+// Forward with q and k normalised on load (x_hat = lim * x / max-norm); keeps its workspace for backward_norm.
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> forward_norm(torch::Tensor q, torch::Tensor k, torch::Tensor v,
+                                                                   torch::Tensor q_keys, torch::Tensor k_keys, double lim,
+                                                                   bool mask, double inv_tau, double a0, double a1,
+                                                                   double a2, int64_t p, int64_t chunk, int64_t flags) {
+  NormArgs na{q_keys, k_keys, lim, false};
+  std::vector<torch::Tensor> r = forward_any(q, k, v, mask, inv_tau, a0, a1, a2, p, chunk,
+                                             flags | FASTMAX_FLAG_SAVE_FOR_BACKWARD, &na);
+  return {r[0], r[1], r[2]};
+}
+
+// Its backward.  grad: true -> gradients with respect to the raw q and k (through the normalisation);
+// false -> with respect to the normalised tensors (what the reference's extension returns).
+std::vector<torch::Tensor> backward_norm(torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor o, torch::Tensor g,
+                                         torch::Tensor go, torch::Tensor saved, torch::Tensor q_keys, torch::Tensor k_keys,
+                                         double lim, bool grad, bool mask, double inv_tau, double a0, double a1, double a2,
+                                         int64_t p, int64_t chunk, int64_t flags) {
+  NormArgs na{q_keys, k_keys, lim, grad};
+  return backward_any(q, k, v, o, g, go, &saved, mask, inv_tau, a0, a1, a2, p, chunk,
+                      flags | FASTMAX_FLAG_SAVE_FOR_BACKWARD, &na);
 }
 
 // y = scale * (x - centre) / max_n ||x_n - centre||  (see fastmax_normalize in the C header)
@@ -365,6 +431,9 @@ PYBIND11_MODULE(fastmax_cuda, m) {
   m.def("backward_ex", &backward_ex, "strided backward: returns [dq, dk, dv]");
   m.def("forward_save", &forward_save, "strided forward keeping its workspace: returns (o, g, saved)");
   m.def("backward_saved", &backward_saved, "strided backward on a saved forward workspace: returns [dq, dk, dv]");
+  m.def("maxnorm_stats", &maxnorm_stats, "statistics of the folded max-norm normalisation of q and k: (q_keys, k_keys)");
+  m.def("forward_norm", &forward_norm, "strided forward with q, k normalised on load: returns (o, g, saved)");
+  m.def("backward_norm", &backward_norm, "backward of forward_norm: returns [dq, dk, dv]");
   m.def("normalize", &normalize, "fused normalisation pass");
   m.def("normalize_backward", &normalize_backward, "gradient of the normalisation pass with respect to its input");
   m.def("version", []() { return fastmax_version(); });

@@ -139,6 +139,47 @@ template <typename T> inline TRef<T> fm_ref(T* ptr, const FastmaxStrides& s) {
 }
 
 // ------------------------------------------------------------------------------
+// Max-norm normalisation folded into the loads:  x_hat = lim * x / max_n ||x_n||_2  per batch*head
+// (transformer/model.py:97-102; apply_norm of fastmax_cuda_forward.cu:326-338 makes this a pass of its own
+// that reads and rewrites the tensor).  One statistics pass (k_maxnorm_keys in fm_norm.h) leaves one 64-bit
+// key per 256 tokens: the bits of the largest squared token norm in the high half and ~token in the low
+// half, so that an integer maximum finds the largest norm and, among equal ones, the first token.  Every
+// kernel that loads such a tensor joins the keys of its batch*head (the same values in the same order
+// everywhere, so all agree on the bits) and multiplies by lim / max-norm as it converts the rows.
+// ------------------------------------------------------------------------------
+struct NormFold {
+  const unsigned long long* keys;   // [bh][nblk], or null: the tensor is taken as it is
+  int nblk;
+  float lim;
+};
+static constexpr int FM_MAXNORM_TOKENS = 256;
+inline int fm_maxnorm_blocks(int n) { return (n + FM_MAXNORM_TOKENS - 1) / FM_MAXNORM_TOKENS; }
+// A slice whose largest squared norm is not above this value (all zeros: padding) is mapped to zeros.
+static constexpr float FM_MAXNORM_FLOOR = 1e-30f;
+
+FM_DEVICE unsigned long long fm_shfl_xor_u64(unsigned long long v, int m) {
+  const int lo = fm_shfl_xor_i(int(uint32_t(v)), m), hi = fm_shfl_xor_i(int(uint32_t(v >> 32)), m);
+  return (static_cast<unsigned long long>(uint32_t(hi)) << 32) | uint32_t(lo);
+}
+// largest squared norm m2 and its token of one batch*head; every lane of the wavefront must call it
+FM_DEVICE void fm_maxnorm_join(const unsigned long long* keys, int nblk, int lane, float& m2, int& nstar) {
+  unsigned long long k = 0;
+  for (int i = lane; i < nblk; i += 64) { const unsigned long long x = keys[i]; k = x > k ? x : k; }
+#pragma unroll
+  for (int w = 1; w < 64; w <<= 1) { const unsigned long long o = fm_shfl_xor_u64(k, w); k = o > k ? o : k; }
+  const uint32_t bits = uint32_t(k >> 32);
+  __builtin_memcpy(&m2, &bits, 4);
+  nstar = int(~uint32_t(k));
+}
+// lim / max-norm of batch*head bh (1 when the fold is off, 0 for an all-zero slice)
+FM_DEVICE float fm_norm_factor(const NormFold& f, int bh, int lane) {
+  if (!f.keys) return 1.0f;
+  float m2; int nstar;
+  fm_maxnorm_join(f.keys + int64_t(bh) * f.nblk, f.nblk, lane, m2, nstar);
+  return m2 > FM_MAXNORM_FLOOR ? f.lim * fm_rsqrtf(m2) : 0.0f;
+}
+
+// ------------------------------------------------------------------------------
 // k_transpose: x (bh, n, DH) strided, interface type  ->  compute type, multiplied by
 // `scale`, zero for tokens >= n:  xt [bh][DH][npad] (transposed) and, when xr is not
 // null, xr [bh][npad][DH] (row-major); xt may be null as well (the _Float16 token kernels read
@@ -146,7 +187,7 @@ template <typename T> inline TRef<T> fm_ref(T* ptr, const FastmaxStrides& s) {
 // these copies with plain 16-byte moves.  Two tensors of the same length (k and v) go in one
 // launch: grid (npad/64, bh, 2), the second set of arguments serves z = 1.
 // ------------------------------------------------------------------------------
-template <typename TIO, typename E> struct TransposeJob { TRef<const TIO> x; E* xt; E* xr; float scale; };
+template <typename TIO, typename E> struct TransposeJob { TRef<const TIO> x; E* xt; E* xr; float scale; NormFold fold; };
 
 template <typename TIO, typename E, int DH>
 FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS)
@@ -159,7 +200,7 @@ k_transpose(TransposeJob<TIO, E> j0, TransposeJob<TIO, E> j1, int n, int npad) {
   const TRef<const TIO> x = second ? j1.x : j0.x;
   E* FM_RESTRICT xt = second ? j1.xt : j0.xt;
   E* FM_RESTRICT xr = second ? j1.xr : j0.xr;
-  const float scale = second ? j1.scale : j0.scale;
+  const float scale = (second ? j1.scale : j0.scale) * fm_norm_factor(second ? j1.fold : j0.fold, bh, tid & 63);
   const TIO* xb = x.base(bh);
   const int64_t s_n = x.s_n;
   const int vec = x.vec;
@@ -275,8 +316,8 @@ FM_DEVICE float fm_grad_scale(const float* part, int nblk, int lane) {
 template <typename TIO, typename E, int DH>
 FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS)
 k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, TRef<const float> g, int n, int npad, E* FM_RESTRICT gh, E* FM_RESTRICT ght,
-           E* FM_RESTRICT qt, E* FM_RESTRICT qct, E* FM_RESTRICT qr, E* FM_RESTRICT cv, float qscale,
-           const float* FM_RESTRICT gpart, int gnblk) {
+           E* FM_RESTRICT qt, E* FM_RESTRICT qct, E* FM_RESTRICT qr, E* FM_RESTRICT cv, float qscale0,
+           const float* FM_RESTRICT gpart, int gnblk, NormFold qfold) {
   constexpr int PT = 64 + Mma<E>::PAD;
   constexpr int VEC = Mma<E>::VEC;
   constexpr int EPT = DH / 4;                      // elements per thread (4 threads per token)
@@ -287,6 +328,7 @@ k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, TRef<const
   const int tok = tid >> 2, part = tid & 3, d0 = part * EPT;
   const int row = t0 + tok;
   const float gscale = fm_grad_scale(gpart ? gpart + int64_t(bh) * gnblk : nullptr, gnblk, tid & 63);
+  const float qscale = qscale0 * fm_norm_factor(qfold, bh, tid & 63);
   float vg[EPT], vq[EPT];
   float csum = 0.f;
   if (row < n) {
@@ -1087,10 +1129,11 @@ struct TokCfg {
   static constexpr int NZ = sizeof(E) == 2 ? 2 : 1; // hi/lo split of fp32 denominators
   static constexpr int SLAB = SA * DH * PS;         // elements per slab buffer
   static constexpr int PV_STAGE = M::HAS_TR ? 2 * KT_PV * PQ : KT_PV * PQ + DH * PV_PV;   // k_pv: two row tiles, or stream rows + stream transposed
-  static constexpr int DS_STAGE = 2 * KT_DS * PQ + (M::HAS_TR ? 0 : DH * PV_DS) + KT_DS;   // k_ds: two row tiles, (transposed tile,) c values
+  // c values of a stage: KT compute-type elements, or KT floats (the completed-square kernels stage -c in fp32)
+  static constexpr int DS_STAGE = 2 * KT_DS * PQ + (M::HAS_TR ? 0 : DH * PV_DS) + (M::HAS_TR ? 2 : 1) * KT_DS;   // k_ds: two row tiles, (transposed tile,) c values
   // k_ds with dV: two row tiles and the c values; the transposed fragments come from the row tiles
   // through transposing LDS reads where the type has them, from two more (transposed) tiles otherwise
-  static constexpr int DV_STAGE = 2 * KT_DV * PQ + (M::HAS_TR ? 0 : 2 * DH * PV_DV) + KT_DV;
+  static constexpr int DV_STAGE = 2 * KT_DV * PQ + (M::HAS_TR ? 0 : 2 * DH * PV_DV) + (M::HAS_TR ? 2 : 1) * KT_DV;
   static constexpr int DS_NBUF = sizeof(E) == 2 ? 2 : 1;
 };
 

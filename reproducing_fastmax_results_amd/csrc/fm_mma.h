@@ -233,6 +233,15 @@ template <> struct TileMath<float> {
   }
 };
 
+// Completed-square forms (order 2, _Float16, dense tiles without states).  With a2 != 0,
+//   f(s)  = a0 + a1 s + a2 s^2 = k1 * (h^2 + kc),   h = 2 a2 s + a1 = f'(s),   k1 = 1 / (4 a2),  kc = 4 a0 a2 - a1^2,
+// so when the score product itself delivers h (own fragments multiplied by 2 a2, accumulator seeded with a1) the
+// weight costs one packed multiply-add, W = h^2 + kc = f / k1, and the factor of the score gradient none; the
+// constant k1 is taken out of the sums (o = F / g does not see it; g and dV are multiplied by it when stored).
+// Likewise the accumulator of gh.v is seeded with -c, so dS = h * (gh.v - c) is one packed multiply.
+//   wq   : W and the lane's partial row sum of W                        (forward)
+//   dsq  : dS                                                           (dQ)
+//   bothq: W and dS                                                     (dK and dV in one pass)
 template <> struct TileMath<fm_half> {
   typedef fm_half8 frag;
   // every constant is one packed pair (one register); all arithmetic is written on pairs so
@@ -320,4 +329,58 @@ template <> struct TileMath<fm_half> {
       }
     if (edge) { FM_KEEP_BRANCH(); window_frags(pb, lo, hi, lh); window_frags(db, lo, hi, lh); }
   }
+  static FM_DEVICE float wq(const fm_f32x16& h, fm_half2 kc, bool edge, int lo, int hi, int lh, frag* pb) {
+    const fm_half2 one = {fm_half(1.f), fm_half(1.f)};
+#pragma unroll
+    for (int ss = 0; ss < 2; ++ss)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int e = 8 * ss + 2 * i;
+        const fm_half2 x = cvt2(h[e], h[e + 1]);
+        put2(pb[ss], i, x * x + kc);
+      }
+    if (edge) { FM_KEEP_BRANCH(); window_frags(pb, lo, hi, lh); }
+    float g = 0.f;
+#pragma unroll
+    for (int ss = 0; ss < 2; ++ss)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) g = fm_dot2(get2(pb[ss], i), one, g);
+    return g;
+  }
+  static FM_DEVICE void dsq(const fm_f32x16& h, const fm_f32x16& dpc, bool edge, int lo, int hi, int lh, frag* db) {
+#pragma unroll
+    for (int ss = 0; ss < 2; ++ss)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int e = 8 * ss + 2 * i;
+        put2(db[ss], i, cvt2(h[e], h[e + 1]) * cvt2(dpc[e], dpc[e + 1]));
+      }
+    if (edge) { FM_KEEP_BRANCH(); window_frags(db, lo, hi, lh); }
+  }
+  static FM_DEVICE void bothq(const fm_f32x16& h, const fm_f32x16& dpc, fm_half2 kc, bool edge, int lo, int hi, int lh,
+                              frag* pb, frag* db) {
+#pragma unroll
+    for (int ss = 0; ss < 2; ++ss)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int e = 8 * ss + 2 * i;
+        const fm_half2 x = cvt2(h[e], h[e + 1]);
+        put2(pb[ss], i, x * x + kc);
+        put2(db[ss], i, x * cvt2(dpc[e], dpc[e + 1]));
+      }
+    if (edge) { FM_KEEP_BRANCH(); window_frags(pb, lo, hi, lh); window_frags(db, lo, hi, lh); }
+  }
 };
+
+// The 16 accumulator entries of a lane, all equal to x, as a value the optimiser cannot take apart: kept in
+// registers across a loop and handed to the first matrix instruction of every tile as its addend (a seed the
+// compiler could see through would be rebuilt with 16 moves per tile).
+FM_DEVICE fm_f32x16 fm_seed16(float x) {
+  fm_f32x16 r;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) r[i] = x;
+#if !defined(FM_HOSTSIM)
+  asm volatile("" : "+v"(r));
+#endif
+  return r;
+}

@@ -415,3 +415,112 @@ inline int fm_normalize_bwd_dispatch(const FastmaxNormDesc* d, const void* x, co
   return d->d == 64 ? fm_normalize_bwd_run<float, 64>(d, x, dy, dx, stats, stream)
                     : fm_normalize_bwd_run<float, 32>(d, x, dy, dx, stats, stream);
 }
+
+// ------------------------------------------------------------------------------
+// The max-norm normalisation folded into the attention kernels (NormFold in fm_kernels.h): the one pass that
+// is left reads the tensor once.  k_maxnorm_keys: grid (ceil(n / 256), bh, tensors); four threads per token;
+// one 64-bit key per workgroup (bits of its largest squared token norm, ~token).  Two tensors (q and k) go
+// in one launch.
+// ------------------------------------------------------------------------------
+template <typename TIO> struct MaxnormJob { TRef<const TIO> x; unsigned long long* keys; int n; int nblk; };
+
+template <typename TIO, int DH>
+FM_GLOBAL void FM_LAUNCH_BOUNDS(256) k_maxnorm_keys(MaxnormJob<TIO> j0, MaxnormJob<TIO> j1) {
+  constexpr int EPT = DH / 4, NP = FM_MAXNORM_TOKENS / 64;
+  FM_SHARED unsigned long long wkey[4];
+  const MaxnormJob<TIO> J = FM_BID_Z ? j1 : j0;
+  const int tid = FM_TID_X, bh = FM_BID_Y;
+  if (int(FM_BID_X) >= J.nblk) return;                  // the shorter tensor of the two (workgroup-uniform)
+  const int n = J.n;
+  const int tok0 = FM_BID_X * FM_MAXNORM_TOKENS + (tid >> 2), d0 = (tid & 3) * EPT;
+  float v[NP][EPT];
+  // every lane takes part in the shuffles; rows past the end re-read the last row and do not count
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    const int tok = tok0 + 64 * p, tk = tok < n ? tok : n - 1;
+    fm_norm_load<TIO, DH>(J.x.base(bh) + int64_t(tk) * J.x.s_n, J.x.vec != 0, d0, v[p]);
+  }
+  float mx = -1.0f;
+  int cand = 0x7fffffff;
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    float nrm = 0.f;
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) nrm += v[p][j] * v[p][j];
+    nrm += fm_shfl_xor(nrm, 1);
+    nrm += fm_shfl_xor(nrm, 2);
+    const int tok = tok0 + 64 * p;
+    if (tok >= n) nrm = -1.0f;
+    if (nrm > mx) { mx = nrm; cand = tok; }             // ascending token order: the first token wins ties
+  }
+  float wmx = mx;
+#pragma unroll
+  for (int m = 4; m < 64; m <<= 1) wmx = fm_fmaxf(wmx, fm_shfl_xor(wmx, m));
+  int wc = (mx == wmx && mx >= 0.f) ? cand : 0x7fffffff;
+#pragma unroll
+  for (int m = 4; m < 64; m <<= 1) { const int o = fm_shfl_xor_i(wc, m); wc = o < wc ? o : wc; }
+  if ((tid & 63) == 0) {
+    unsigned long long key = 0;                          // no norm of this wavefront compares (all NaN)
+    if (wc != 0x7fffffff) {
+      uint32_t bits;
+      __builtin_memcpy(&bits, &wmx, 4);
+      key = (static_cast<unsigned long long>(bits) << 32) | uint32_t(~uint32_t(wc));
+    }
+    wkey[tid >> 6] = key;
+  }
+  FM_SYNC();
+  if (tid == 0) {
+    const unsigned long long a = wkey[0] > wkey[1] ? wkey[0] : wkey[1], b = wkey[2] > wkey[3] ? wkey[2] : wkey[3];
+    J.keys[int64_t(bh) * J.nblk + FM_BID_X] = a > b ? a : b;
+  }
+}
+
+// The rank-one term of the normalisation's Jacobian.  With y = (lim / m) x, m = ||x_n*|| the largest token norm,
+// dy the gradient with respect to y and B = sum_{n,d} dy * y over the whole slice:
+//     dx_n = (lim / m) dy_n - [n == n*] * B * x_n* / m^2 .
+// The attention kernels have stored (lim / m) dy and left B in parts (one per workgroup, added here in a fixed
+// order); this kernel corrects the one row n*.  grid (bh, tensors), 64 threads.
+template <typename TIO> struct NormFixJob {
+  TRef<const TIO> x; TRef<TIO> dx; const unsigned long long* keys; int nblk; const float* bpart; int nb; int n;
+};
+template <typename TIO, int DH>
+FM_GLOBAL void FM_LAUNCH_BOUNDS(64) k_norm_fix(NormFixJob<TIO> j0, NormFixJob<TIO> j1) {
+  const NormFixJob<TIO> J = FM_BID_Y ? j1 : j0;
+  const int lane = FM_TID_X, bh = FM_BID_X;
+  if (!J.keys) return;
+  float m2; int nstar;
+  fm_maxnorm_join(J.keys + int64_t(bh) * J.nblk, J.nblk, lane, m2, nstar);
+  if (!(m2 > FM_MAXNORM_FLOOR) || nstar < 0 || nstar >= J.n) return;
+  // the parts in a fixed order: lane l adds parts l, l + 64, ...; then the lanes pairwise
+  float b = 0.f;
+  for (int i = lane; i < J.nb; i += 64) b += J.bpart[int64_t(bh) * J.nb + i];
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) b += fm_shfl_xor(b, m);
+  if (lane < DH) {
+    const float xv = IO<TIO>::ld(J.x.base(bh) + int64_t(nstar) * J.x.s_n + lane);
+    TIO* p = J.dx.base(bh) + int64_t(nstar) * J.dx.s_n + lane;
+    IO<TIO>::st(p, IO<TIO>::ld(p) - b * xv / m2);
+  }
+}
+
+template <typename TIO, int DH>
+int fm_maxnorm_run(const FastmaxNormDesc* d0, const void* x0, void* keys0, const FastmaxNormDesc* d1, const void* x1,
+                   void* keys1, fm_stream_t stream) {
+  MaxnormJob<TIO> j0{fm_ref<const TIO>(static_cast<const TIO*>(x0), d0->sx), static_cast<unsigned long long*>(keys0), d0->n,
+                     fm_maxnorm_blocks(d0->n)};
+  MaxnormJob<TIO> j1 = j0;
+  if (d1) j1 = MaxnormJob<TIO>{fm_ref<const TIO>(static_cast<const TIO*>(x1), d1->sx), static_cast<unsigned long long*>(keys1),
+                               d1->n, fm_maxnorm_blocks(d1->n)};
+  const int nb = j0.nblk > j1.nblk ? j0.nblk : j1.nblk;
+  FM_KERNEL_LAUNCH((k_maxnorm_keys<TIO, DH>), fm_dim3(nb, d0->bh, d1 ? 2 : 1), fm_dim3(256), 0, stream, j0, j1);
+  return fm_after_launch() ? FASTMAX_ERR_LAUNCH : FASTMAX_OK;
+}
+
+inline int fm_maxnorm_dispatch(const FastmaxNormDesc* d0, const void* x0, void* keys0, const FastmaxNormDesc* d1,
+                               const void* x1, void* keys1, fm_stream_t stream) {
+  if (d0->dtype == FASTMAX_BF16)
+    return d0->d == 64 ? fm_maxnorm_run<fm_bf16, 64>(d0, x0, keys0, d1, x1, keys1, stream)
+                       : fm_maxnorm_run<fm_bf16, 32>(d0, x0, keys0, d1, x1, keys1, stream);
+  return d0->d == 64 ? fm_maxnorm_run<float, 64>(d0, x0, keys0, d1, x1, keys1, stream)
+                     : fm_maxnorm_run<float, 32>(d0, x0, keys0, d1, x1, keys1, stream);
+}

@@ -52,6 +52,13 @@ template <typename TIO, typename E> struct TokArgs {
   // partial maxima of |dO| / |g| ([bh][gnblk], see k_grad_scale) or null: the kernels that form gh multiply it by
   // fm_grad_scale of them, the kernels that store a gradient divide by it
   const float* gpart; int gnblk;
+  // Max-norm normalisation folded into the loads (see NormFold).  own_fold: of the own tokens' caller tensor
+  // (the kernels that read it: forward, and dQ with PREP); the compute-type copies are made with the factor in.
+  // Backward with the normalisation's own Jacobian (bpart != null): the stored gradient is multiplied by
+  // out_fold's factor and the workgroup leaves its part of B = sum dy . y (y = normalised rows, taken from
+  // the copy `brows` = sc * y) in bpart [bh][blocks]; k_norm_fix applies the rank-one term to one row later.
+  NormFold own_fold, out_fold;
+  const E* brows; float* bpart;
 };
 
 // Z (fp32, [DH][DH]) -> LDS in the compute type (hi/lo split for _Float16), va/vb -> vecs.
@@ -84,9 +91,12 @@ FM_DEVICE fm_f32x16 fm_zy(const E* Zs, const typename Mma<E>::frag* tf, int mt, 
 }
 
 // Accumulators (rows = feature, column = token of tile j) -> caller tensor rows, through LDS.
+// brows (optional): compute-type rows [n][DH] of the same tokens; the workgroup's sum over its stored values
+// times those rows, times bscale, goes to *bout (one workgroup-uniform address).
 template <typename TIO, typename E, int DH, int QT>
 FM_DEVICE void fm_store_tokens(fm_f32x16 (*acc)[DH / 32], const int* xrow, const float* addvec, float scale, float* Os,
-                               TRef<TIO> out, int bh, int row0, int nrows, int tid) {
+                               TRef<TIO> out, int bh, int row0, int nrows, int tid, const E* brows = nullptr,
+                               float bscale = 0.f, float* bout = nullptr) {
   typedef TokCfg<E, DH, QT> C;
   const int lane = tid & 63, lh = lane >> 5;
 #pragma unroll
@@ -100,16 +110,30 @@ FM_DEVICE void fm_store_tokens(fm_f32x16 (*acc)[DH / 32], const int* xrow, const
       }
   FM_SYNC();
   TIO* ob = out.base(bh);
+  float bsum = 0.f;
   for (int c = tid; c < C::QW * (DH / 8); c += FM_THREADS) {
     const int row = c / (DH / 8), col = (c % (DH / 8)) * 8;
     if (row0 + row < nrows) {
       float v[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i) v[i] = Os[row * (DH + 1) + col + i];
+      if (brows) {
+        const E* br = brows + int64_t(row0 + row) * DH + col;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) bsum += v[i] * float(br[i]);
+      }
       IO<TIO>::st8(ob + int64_t(row0 + row) * out.s_n + col, out.vec != 0, v);
     }
   }
   FM_SYNC();
+  if (bout) {
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) bsum += fm_shfl_xor(bsum, m);
+    if (lane == 0) Os[tid >> 6] = bsum;
+    FM_SYNC();
+    if (tid == 0) *bout = bscale * ((Os[0] + Os[1]) + (Os[2] + Os[3]));
+    FM_SYNC();
+  }
 }
 
 // Placement of the blocks of own tokens.  A causal block's work is its dense part (1 .. L/QW
@@ -209,8 +233,11 @@ template <int OWN> FM_DEVICE void fm_tile_window(bool causal, int s0, int lo, in
 // LDS: va, vb | own rows [QW][PQ] | region (Z, then state slabs); the two dense stages and the
 // output staging lie over the own rows and the region once they are spent.
 // ------------------------------------------------------------------------------
-template <typename TIO, typename E, int DH, int QT, int OWN>
+// QF = 1 (forward of an order-2 problem without states, _Float16): the weights in their completed-square
+// form (see TileMath<fm_half>::wq); the host picks it when a2 is of ordinary size.
+template <typename TIO, typename E, int DH, int QT, int OWN, int QF = 0>
 FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(TokArgs<TIO, E> A) {
+  static_assert(!QF || (QT == 1 && OWN == FM_OWN_Q && sizeof(E) == 2), "completed-square weights: forward, one tile per wavefront");
   typedef TokCfg<E, DH, QT> C;
   typedef Mma<E> M;
   typedef TileMath<E> TM;
@@ -232,7 +259,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
   if (OWN == FM_OWN_Q) {
     RowRegs<TIO, E, QW, DH> rq;
     rq.load(A.own_io.base(bh), A.own_io.s_n, A.own_io.vec != 0, t0, A.n_own, tid);
-    rq.store(Own, PQ, tid, A.sc);
+    rq.store(Own, PQ, tid, A.sc * fm_norm_factor(A.own_fold, bh, lane));
   } else {
     TileRegs<E, QW, DH> ro;
     ro.load(A.own_r + (int64_t(bh) * A.npad_own + t0) * DH, DH, tid);
@@ -257,6 +284,14 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
   for (int j = 0; j < QT; ++j)
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) of[j][ks] = M::load(Own + xrow[j] * PQ + ks * M::KSTEP + lh * M::KPL);
+  fm_f32x16 sseed = fm_zero16();
+  if constexpr (QF != 0) {
+    // the score products deliver h = 2 a2 s + a1
+    const frag t2 = M::splat(CE<E>::from(2.0f * A.a2));
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) of[0][ks] = of[0][ks] * t2;
+    sseed = fm_seed16(A.a1);
+  }
 
   fm_f32x16 acc[QT][NT];
 #pragma unroll
@@ -345,7 +380,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
         if (QT == 1) { FM_SCHED_MFMA_DS(0); }
         fm_f32x16 s[QT];
 #pragma unroll
-        for (int j = 0; j < QT; ++j) s[j] = fm_zero16();
+        for (int j = 0; j < QT; ++j) s[j] = QF ? sseed : fm_zero16();
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) {
           const frag xf = M::load(Xs + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL);
@@ -377,7 +412,9 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
           int wlo, whi;
           fm_tile_window<OWN>(causal, ss0, lo, lr, A.n_str, wlo, whi);
           frag pb[M::ACC_KSTEPS];
-          const float gs = TM::fwd(s[j], coef, edge, wlo, whi, lh, pb);
+          float gs;
+          if constexpr (QF != 0) gs = TM::wq(s[j], TM::pair(4.0f * A.a0 * A.a2 - A.a1 * A.a1), edge, wlo, whi, lh, pb);
+          else gs = TM::fwd(s[j], coef, edge, wlo, whi, lh, pb);
           if (OWN == FM_OWN_Q) gsum[j] += gs;
 #pragma unroll
           for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
@@ -400,6 +437,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
       float gt = gsum[j] + fm_shfl_xor(gsum[j], 32);
       if (G.use_state) gt += A.a0 * cnt;
       const float ginv = 1.0f / gt;
+      if (QF) gt *= 1.0f / (4.0f * A.a2);              // the constant taken out of the weights (o does not see it)
 #pragma unroll
       for (int ct = 0; ct < NT; ++ct)
 #pragma unroll
@@ -439,8 +477,11 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
 // score tiles it already has, P = f(S), dV^T += gh^T P, which saves the four score
 // products per tile that a separate k_pv launch would repeat.
 // ------------------------------------------------------------------------------
-template <typename TIO, typename E, int DH, int QT, int OWN, int DV, int PREP>
+// QF = 1 (order 2 without states, _Float16): completed-square weights and seeded accumulators (see
+// TileMath<fm_half>::dsq / bothq); the host picks it when a2 is of ordinary size.
+template <typename TIO, typename E, int DH, int QT, int OWN, int DV, int PREP, int QF = 0>
 FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS)) k_ds(TokArgs<TIO, E> A) {
+  static_assert(!QF || (QT == 1 && sizeof(E) == 2 && (DV != 0 || OWN == FM_OWN_Q)), "completed-square weights: dQ, or dK with dV, one tile per wavefront");
   typedef TokCfg<E, DH, QT> C;
   typedef Mma<E> M;
   typedef TileMath<E> TM;
@@ -476,6 +517,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
     float* cl = reinterpret_cast<float*>(R + QW * PQ);   // c per own query, behind the gh rows
     const int part = tid & 3, d0 = part * EPT;
     constexpr int NH = QW / 64;
+    const float qsc = A.sc * fm_norm_factor(A.own_fold, bh, lane);
     float ra[NH][EPT], rb[NH][EPT], rc[NH][EPT], gi[NH];
     // every load of the block is issued before the first result is used
 #pragma unroll
@@ -505,7 +547,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
       for (int j = 0; j < EPT; ++j) {
         vg[j] = ra[h][j] * ginv;
         csum += vg[j] * rb[h][j];
-        vq[j] = rc[h][j] * A.sc;
+        vq[j] = rc[h][j] * qsc;
       }
       csum += fm_shfl_xor(csum, 1);
       csum += fm_shfl_xor(csum, 2);
@@ -556,6 +598,15 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
       of2[j][ks] = M::load(o2 + ks * M::KSTEP);
     }
   }
+  fm_f32x16 sseed = fm_zero16(), dpseed = fm_zero16();
+  if constexpr (QF != 0) {
+    // the score products deliver h = 2 a2 s + a1; the gh.v products start from -c (own = queries: the lane's own c)
+    const frag t2 = M::splat(CE<E>::from(2.0f * A.a2));
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) of[0][ks] = of[0][ks] * t2;
+    sseed = fm_seed16(A.a1);
+    if (OWN == FM_OWN_Q) dpseed = fm_seed16(-ci[0]);
+  }
   fm_f32x16 acc[QT][NT], av[DV ? QT : 1][NT];
 #pragma unroll
   for (int j = 0; j < QT; ++j)
@@ -603,14 +654,17 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
       ry.load(yb + int64_t(sx) * DH, DH, tid);
       if (!TR) rz.load(zb + sx, A.npad_str, tid);
       if (DV && !TR) rz2.load(z2b + sx, A.npad_str, tid);
-      if (OWN == FM_OWN_K && tid < KT) creg = cvb[sx + tid];
+      // QF: c is staged as -c in fp32, tokens in their natural order (the copy holds them in `tperm` order)
+      if (OWN == FM_OWN_K && tid < KT) creg = cvb[sx + (QF ? M::tperm(tid) : tid)];
     };
     auto put = [&](int b) {                             // registers -> stage buffer b
       E* Xn = Own + b * STAGE; E* Yn = Xn + KT * PQ; E* Zn = Yn + KT * PQ; E* cn = Zn + (TR ? 0 : DH * PV);
       rx.store(Xn, PQ, tid); ry.store(Yn, PQ, tid);
       if (!TR) rz.store(Zn, PV, tid);
       if (DV && !TR) rz2.store(cn + KT, PV, tid);
-      if (OWN == FM_OWN_K && tid < KT) cn[tid] = creg;
+      if (OWN == FM_OWN_K && tid < KT) {
+        if (QF) reinterpret_cast<float*>(cn)[tid] = -float(creg); else cn[tid] = creg;
+      }
     };
     // Two buffers: the tiles of stage i+1 travel global memory -> registers during stage i-1 and
     // registers -> LDS in the middle of stage i (see k_pv).  One buffer (fp32): both at the top.
@@ -633,7 +687,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
         if (QT == 1) { FM_SCHED_MFMA_DS(DV ? 0 : 1); }   // two tiles per wavefront: measured slower with it
         fm_f32x16 s[QT];
 #pragma unroll
-        for (int j = 0; j < QT; ++j) s[j] = fm_zero16();
+        for (int j = 0; j < QT; ++j) s[j] = QF ? sseed : fm_zero16();
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) {
           const frag xf = M::load(Xs + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL);
@@ -643,7 +697,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
         frag zf[NT][M::ACC_KSTEPS], crow[M::ACC_KSTEPS];
 #pragma unroll
         for (int ss = 0; ss < M::ACC_KSTEPS; ++ss) {
-          if (OWN == FM_OWN_K) crow[ss] = M::load_perm(cs + 32 * st, ss, lh);
+          if (OWN == FM_OWN_K && !QF) crow[ss] = M::load_perm(cs + 32 * st, ss, lh);
 #pragma unroll
           for (int mt = 0; mt < NT; ++mt)
             zf[mt][ss] = TR ? M::load_tr(Xs, PQ, 32 * st + 16 * ss, 32 * mt, lane)
@@ -666,11 +720,26 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
           int wlo, whi;
           fm_tile_window<OWN>(causal, ss0, lo, lr, A.n_str, wlo, whi);
           fm_f32x16 dp = fm_zero16();
+          if constexpr (QF != 0) {
+            if (OWN == FM_OWN_Q) dp = dpseed;
+            else {
+              // -c of the tile's 32 queries, the lane's 16 accumulator rows: four 16-byte reads
+              const float* cf = reinterpret_cast<const float*>(cs) + 32 * st + 4 * lh;
+#pragma unroll
+              for (int gq = 0; gq < 4; ++gq) {
+                const fm_f32x4 t = *reinterpret_cast<const fm_f32x4*>(cf + 8 * gq);
+                dp[4 * gq] = t[0]; dp[4 * gq + 1] = t[1]; dp[4 * gq + 2] = t[2]; dp[4 * gq + 3] = t[3];
+              }
+            }
+          }
           const E* yrow = Ys + (32 * st + lr) * PQ + lh * M::KPL + (QT > 1 ? FM_OPAQUE_ZERO() : 0);
 #pragma unroll
           for (int ks = 0; ks < NKS; ++ks) dp = M::mma(M::load(yrow + ks * M::KSTEP), of2[j][ks], dp);
           frag db[M::ACC_KSTEPS], pb[M::ACC_KSTEPS];
-          if (DV) TM::both(s[j], dp, crow, coef, edge, wlo, whi, lh, pb, db);
+          if constexpr (QF != 0) {
+            if (DV) TM::bothq(s[j], dp, TM::pair(4.0f * A.a0 * A.a2 - A.a1 * A.a1), edge, wlo, whi, lh, pb, db);
+            else TM::dsq(s[j], dp, edge, wlo, whi, lh, db);
+          } else if (DV) TM::both(s[j], dp, crow, coef, edge, wlo, whi, lh, pb, db);
           else if (OWN == FM_OWN_Q) TM::dsc(s[j], dp, cs_own[j], coef, edge, wlo, whi, lh, db);
           else TM::dsr(s[j], dp, crow, coef, edge, wlo, whi, lh, db);
 #pragma unroll
@@ -688,9 +757,16 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
     }
     if (NBUF == 2) FM_SYNC();
   }
-  fm_store_tokens<TIO, E, DH, QT>(acc, xrow, nullptr, A.out_scale * ginv_sc, reinterpret_cast<float*>(Own), A.out, bh, t0,
-                                  A.n_own, tid);
+  {
+    // with the normalisation's Jacobian: the stored gradient carries lim / max-norm, and the workgroup's part of
+    // B = sum dy . y is left for k_norm_fix (the stored values are fac * dy, the copy's rows sc * y)
+    const float fac = A.bpart ? fm_norm_factor(A.out_fold, bh, lane) : 1.0f;
+    const E* brows = A.bpart ? (PREP ? A.w_qr : A.brows) + int64_t(bh) * A.npad_own * DH : nullptr;
+    float* bout = A.bpart ? A.bpart + int64_t(bh) * ((A.n_own + QW - 1) / QW) + t0 / QW : nullptr;
+    fm_store_tokens<TIO, E, DH, QT>(acc, xrow, nullptr, A.out_scale * ginv_sc * fac, reinterpret_cast<float*>(Own), A.out, bh, t0,
+                                    A.n_own, tid, brows, fac > 0.f ? 1.0f / (fac * A.sc) : 0.f, bout);
+  }
   if (DV)
-    fm_store_tokens<TIO, E, DH, QT>(av, xrow, nullptr, A.out2_scale * ginv_sc, reinterpret_cast<float*>(Own), A.out2, bh, t0,
-                                    A.n_own, tid);
+    fm_store_tokens<TIO, E, DH, QT>(av, xrow, nullptr, A.out2_scale * ginv_sc * (QF ? 1.0f / (4.0f * A.a2) : 1.0f),
+                                    reinterpret_cast<float*>(Own), A.out2, bh, t0, A.n_own, tid);
 }

@@ -20,11 +20,16 @@ import math
 import torch
 from torch import nn
 
-from ..attention_mechanisms.score_function import CENTRE_NONE, FASTMultiHeadAttention_Function, FastmaxNormalize
+from ..attention_mechanisms.score_function import (CENTRE_NONE, FASTMultiHeadAttention_Function, FastmaxNormalize,
+                                                    FastmaxNormAttention, _fold_possible)
 
 
 def fastmax_attention(q, k, v, *, mask, normalize, lim, temperature, a0, a1, a2, p):
     """``(b, h, n, d)`` views in, ``(b, h, n, d)`` out, on the HIP kernels."""
+    if normalize and _fold_possible(q, k, mask):
+        # the normalisation folded into the attention kernels, its gradient included
+        return FastmaxNormAttention.apply(q, k, v, bool(mask), float(lim), float(temperature), float(a0), float(a1),
+                                          float(a2), int(p))
     if normalize:
         q = FastmaxNormalize.apply(q, CENTRE_NONE, float(lim))
         k = FastmaxNormalize.apply(k, CENTRE_NONE, float(lim))

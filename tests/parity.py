@@ -87,3 +87,33 @@ def check_batch_head_strides(lib, b, h, n, d, dtype, device, *, mask, p, chunk=0
     for x4, x3 in zip(d4, d3):
         assert torch.equal(x4.contiguous().view(b * h, n, d), x3)
     return True
+
+
+def check_norm_fold(lib, bh, nq, d, dtype, device, *, mask, p, nk=None, chunk=0, lim=1.5, tau=1.0, seed=0, saved=True,
+                    jacobian=True, scale=1.0):
+    """The max-norm normalisation of q and k folded into the kernels (FastmaxNormFold) against the fp64 closed
+    form on lim * x / max_n ||x_n||: o, g, and either the gradients with respect to the raw q and k (torch
+    autograd through the normalisation: ``jacobian``) or those with respect to the normalised tensors (what the
+    reference's extension returns)."""
+    nk = nk or nq
+    q, k, v, go = make_inputs(bh, nq, nk, d, dtype, device, seed, scale)
+    qk, kk = lib.maxnorm_stats(q, k)
+    kw = dict(mask=mask, inv_tau=1.0 / tau, p=p, chunk=chunk, norm=(qk, kk, lim, jacobian))
+    if saved:
+        o, g, ws = lib.forward(q, k, v, save=True, **kw)
+        dq, dk, dv = lib.backward(q, k, v, o, g, go, saved=ws, **kw)
+    else:
+        o, g = lib.forward(q, k, v, **kw)
+        dq, dk, dv = lib.backward(q, k, v, o, g, go, **kw)
+    qd, kd, vd, gd = (t.detach().cpu().double() for t in (q, k, v, go))
+    if jacobian:
+        qd.requires_grad_(True); kd.requires_grad_(True); vd.requires_grad_(True)
+        oo, gg = O.closed_form_forward(O.normalize_lim(qd, lim), O.normalize_lim(kd, lim), vd, mask=mask, tau=tau, p=p)
+        rq, rk, rv = torch.autograd.grad(oo, (qd, kd, vd), gd)
+        ref = (oo.detach(), gg.detach(), rq, rk, rv)
+    else:
+        ref = oracle_all(O.normalize_lim(qd, lim), O.normalize_lim(kd, lim), vd, gd, mask=mask, tau=tau, p=p)
+    errs = {n: rel_err(x, r) for n, x, r in zip(("o", "g", "dq", "dk", "dv"), (o, g, dq, dk, dv), ref)}
+    for n, e in errs.items():
+        assert e < TOL[dtype], f"{n} rel-L2 {e:.3e} (all: {errs})"
+    return errs

@@ -100,6 +100,34 @@ def test_autograd_wrapper(sf, dtype, four_d):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_normalised_attention_function(sf, dtype):
+    """FastmaxNormAttention: normalisation folded into the kernels, gradients with respect to the raw q and k
+    (fp64 autograd through lim * x / max-norm and the closed form); and the reference-style wrapper with
+    normalize=True, whose gradients are those with respect to the normalised tensors."""
+    b, h, n, d, lim = 2, 3, 600, 64, 1.3
+    q, k, v, go = (rnd(b, n, h * d, seed=s).to(dtype).to(DEV).view(b, n, h, d).transpose(1, 2) for s in (44, 45, 46, 47))
+    qd, kd, vd = (x.detach().clone().requires_grad_(True) for x in (q, k, v))
+    o = sf.FastmaxNormAttention.apply(qd, kd, vd, True, lim, 1.0, 1.0, 1.0, 0.5, 2)
+    o.backward(go)
+    q64, k64, v64 = (x.double().cpu().contiguous().requires_grad_(True) for x in (q, k, v))
+    oo, _ = O.closed_form_forward(O.normalize_lim(q64, lim), O.normalize_lim(k64, lim), v64, mask=True, tau=1.0, p=2)
+    rq, rk, rv = torch.autograd.grad(oo, (q64, k64, v64), go.double().cpu())
+    assert rel_err(o, oo) < TOL[dtype]
+    for got, want in ((qd.grad, rq), (kd.grad, rk), (vd.grad, rv)):
+        assert rel_err(got, want) < TOL[dtype]
+    # the reference's call: normalize inside, gradients with respect to the normalised q and k
+    qe, ke, ve = (x.detach().clone().requires_grad_(True) for x in (q, k, v))
+    o2 = sf.FASTMultiHeadAttention_Function.apply(qe, ke, ve, None, None, True, 0.0, True, 1.0, 1.0, 1.0, 0.5, lim, 2)
+    o2.backward(go)
+    assert torch.equal(o2, o)
+    qn, kn = O.normalize_lim(q.double().cpu(), lim), O.normalize_lim(k.double().cpu(), lim)
+    ref = O.manual_backward_blocked(qn.contiguous(), kn.contiguous(), v.double().cpu().contiguous(), go.double().cpu().contiguous(),
+                                    mask=True, tau=1.0, p=2)
+    for got, want in ((qe.grad, ref[2]), (ke.grad, ref[3]), (ve.grad, ref[4])):
+        assert rel_err(got, want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_one_head_per_batch_projection_layout(sf, ext, dtype):
     """(b, n, 1*d) projections viewed as (b, 1, n, d): stride(1) of that view is d, not the distance between
     the batches; the binding must address batch i at i * n * d (heads_per_block = 1 in the model)."""

@@ -4,7 +4,7 @@ bf16-rounded inputs)."""
 import pytest
 import torch
 
-from tests.parity import check_batch_head_strides, check_forward, check_forward_backward
+from tests.parity import check_batch_head_strides, check_forward, check_forward_backward, check_norm_fold
 from reproducing_fastmax_results_amd._capi import FLAG_FORCE_DENSE, FLAG_FORCE_MOMENTS
 
 pytestmark = pytest.mark.gpu
@@ -205,6 +205,21 @@ def test_causal_more_keys_than_queries(lib, dtype, p, nq, nk):
     print(f"case causal nk>nq dtype={dtype} p={p} nq={nq} nk={nk}", flush=True)
     d = 64 if nq != 300 else 32
     check_forward_backward(lib, 3, nq, d, dtype, DEV, mask=True, p=p, nk=nk, seed=50)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("jacobian", [True, False])
+def test_normalisation_folded_into_the_loads(lib, dtype, jacobian):
+    """lim * x / max-norm of q and k applied as the kernels load the rows (one statistics pass, one read of q and
+    k); gradients with respect to the raw tensors (fp64 autograd through the normalisation) or, like the
+    reference's extension, with respect to the normalised ones."""
+    print(f"case folded normalisation dtype={dtype} jacobian={jacobian}", flush=True)
+    for p, chunk in ((2, 0), (2, 256), (1, 0), (1, 256)):
+        check_norm_fold(lib, 3, 1100, 64, dtype, DEV, mask=True, p=p, chunk=chunk, seed=70 + p, jacobian=jacobian)
+        check_norm_fold(lib, 2, 700, 32, dtype, DEV, mask=True, p=p, chunk=chunk, seed=72 + p, jacobian=jacobian, saved=False)
+    check_norm_fold(lib, 2, 300, 64, dtype, DEV, mask=False, p=2, nk=700, seed=75, jacobian=jacobian, saved=False)
+    check_norm_fold(lib, 2, 50, 32, dtype, DEV, mask=False, p=2, seed=76, jacobian=jacobian)
+    check_norm_fold(lib, 8, 4096, 64, dtype, DEV, mask=True, p=2, seed=77, jacobian=jacobian, lim=1.0, tau=1.0)
 
 
 @pytest.mark.parametrize("go_scale", [1e-7, 1e-4, 3e4])

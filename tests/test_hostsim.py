@@ -15,7 +15,7 @@ import pytest
 import torch
 
 from reproducing_fastmax_results_amd import _capi
-from tests.parity import (TOL, check_batch_head_strides, check_forward, check_forward_backward, make_inputs, oracle_all,
+from tests.parity import (TOL, check_batch_head_strides, check_norm_fold, check_forward, check_forward_backward, make_inputs, oracle_all,
                           rel_err)
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -201,3 +201,14 @@ def test_upstream_gradient_of_any_size(sim):
         check_forward_backward(sim, 1, 300, 32, torch.bfloat16, "cpu", mask=True, p=2, chunk=256, seed=21,
                                go_scale=go_scale, saved=True)
     check_forward_backward(sim, 1, 300, 32, torch.bfloat16, "cpu", mask=True, p=1, chunk=256, seed=22, go_scale=1e-7)
+
+
+def test_normalisation_folded_into_the_loads(sim):
+    # q and k normalised as they are loaded; gradients through the normalisation (one row gets the rank-one term)
+    check_norm_fold(sim, 2, 70, 32, torch.float32, "cpu", mask=True, p=2, seed=23)
+    check_norm_fold(sim, 2, 70, 32, torch.bfloat16, "cpu", mask=True, p=2, seed=24)
+    check_norm_fold(sim, 1, 300, 32, torch.bfloat16, "cpu", mask=True, p=2, chunk=256, seed=25)      # through states
+    check_norm_fold(sim, 1, 300, 32, torch.float32, "cpu", mask=True, p=1, chunk=256, seed=26, saved=False)
+    check_norm_fold(sim, 2, 40, 32, torch.float32, "cpu", mask=False, p=2, nk=75, seed=27, saved=False)
+    # the reference extension's gradients: with respect to the normalised tensors
+    check_norm_fold(sim, 2, 70, 32, torch.float32, "cpu", mask=True, p=2, seed=28, jacobian=False)
