@@ -157,6 +157,26 @@ int fastmax_backward_saved(const FastmaxDesc* desc, const void* q, const void* k
                            const void* forward_workspace, size_t forward_workspace_bytes,
                            void* workspace, size_t workspace_bytes, void* hip_stream);
 
+/* Incremental decoding on a persistent moment state (the running sums of fastmax_cuda_forward.cu:160-276
+ * kept between calls; the reference's generation loop, transformer/eval.py:8-32, re-runs the whole context
+ * for every new token).  The state of a batch*head is the fp32 sums over all keys so far of [1, k', k' x k']
+ * times [v, 1] with k' = k * inv_tau: fastmax_decode_state_bytes(desc) bytes for desc->bh of them (1.07 MB
+ * per batch*head at d = 64, order 2; 17 KB at order 1), whatever the number of keys.  A zero-filled buffer
+ * is the empty state.  desc: bh, d, dtype, p, a0..a2, inv_tau and the strides named below are used; mask,
+ * chunk, flags and norm are ignored (decoding is causal by construction and needs unnormalised q, k: the
+ * max-norm depends on every token).
+ *   fastmax_decode_absorb: adds desc->nk tokens (k, v: strides sk, sv) to the state, e.g. a prompt whose
+ *     own outputs come from fastmax_forward.
+ *   fastmax_decode_step: adds one token (k, v) and reads the state out for its query q (strides sq; the
+ *     query sees its own key, as in causal attention): o (strides so, one token) and g (sg).  scratch:
+ *     fastmax_decode_scratch_bytes(desc) bytes of device memory.  desc->nq and nk are ignored (one token).
+ * Both enqueue on the stream and allocate nothing; a step reads and writes the state once. */
+size_t fastmax_decode_state_bytes(const FastmaxDesc* desc);
+size_t fastmax_decode_scratch_bytes(const FastmaxDesc* desc);
+int fastmax_decode_absorb(const FastmaxDesc* desc, const void* k, const void* v, float* state, void* hip_stream);
+int fastmax_decode_step(const FastmaxDesc* desc, const void* q, const void* k, const void* v, float* state,
+                        void* o, float* g, float* scratch, void* hip_stream);
+
 /* Fused normalisation pass over one (bh, n, d) tensor.  Replaces apply_rpe_and_temp, calc_norms,
  * find_max and apply_norm (reference fastmax_cuda_forward.cu:282-338) with the semantics the
  * Python variants define:

@@ -62,6 +62,7 @@ EXPORTS = (
     "fastmax_probe_mfma_rate",
     "fastmax_profile_begin", "fastmax_profile_end", "fastmax_forward_static",
     "fastmax_maxnorm_stats", "fastmax_maxnorm_stats_bytes",
+    "fastmax_decode_state_bytes", "fastmax_decode_scratch_bytes", "fastmax_decode_absorb", "fastmax_decode_step",
 )
 STATIC_SCRATCH_BYTES = 64 << 20     # FASTMAX_STATIC_SCRATCH_BYTES
 
@@ -146,6 +147,13 @@ class FastmaxLib:
         L.fastmax_maxnorm_stats.argtypes = [C.POINTER(NormDesc), C.c_void_p, C.c_void_p, C.POINTER(NormDesc), C.c_void_p,
                                             C.c_void_p, C.c_void_p]
         L.fastmax_maxnorm_stats.restype = C.c_int
+        for fn in (L.fastmax_decode_state_bytes, L.fastmax_decode_scratch_bytes):
+            fn.argtypes = [C.POINTER(Desc)]
+            fn.restype = C.c_size_t
+        L.fastmax_decode_absorb.argtypes = [C.POINTER(Desc)] + [C.c_void_p] * 4
+        L.fastmax_decode_absorb.restype = C.c_int
+        L.fastmax_decode_step.argtypes = [C.POINTER(Desc)] + [C.c_void_p] * 8
+        L.fastmax_decode_step.restype = C.c_int
         L.fastmax_status_string.argtypes = [C.c_int]
         L.fastmax_status_string.restype = C.c_char_p
         L.fastmax_version.restype = C.c_int
@@ -269,6 +277,32 @@ class FastmaxLib:
                                              g.data_ptr(), self._stream(q))
         self.check(st, "fastmax_forward_static")
         return out, g
+
+    # -- incremental decoding on a persistent moment state ---------------------------
+    def decode_state(self, k, *, inv_tau, p=2, a0=1.0, a1=1.0, a2=0.5):
+        """An empty state for tensors shaped like k ((bh, n, d) or (b, h, n, d)): zero-filled float32."""
+        desc = self.make_desc(k, k, k, mask=True, inv_tau=inv_tau, a0=a0, a1=a1, a2=a2, p=p)
+        return torch.zeros(self.lib.fastmax_decode_state_bytes(C.byref(desc)) // 4, dtype=torch.float32, device=k.device)
+
+    def decode_absorb(self, k, v, state, *, inv_tau, p=2, a0=1.0, a1=1.0, a2=0.5):
+        """Adds all tokens of k, v to the state."""
+        desc = self.make_desc(k, k, v, mask=True, inv_tau=inv_tau, a0=a0, a1=a1, a2=a2, p=p)
+        st = self.lib.fastmax_decode_absorb(C.byref(desc), k.data_ptr(), v.data_ptr(), state.data_ptr(), self._stream(k))
+        self.check(st, "fastmax_decode_absorb")
+
+    def decode_step(self, q, k, v, state, *, inv_tau, p=2, a0=1.0, a1=1.0, a2=0.5):
+        """One token: q, k, v are (bh, 1, d) or (b, h, 1, d); returns (o, g) for it and updates the state."""
+        desc = self.make_desc(q, k, v, mask=True, inv_tau=inv_tau, a0=a0, a1=a1, a2=a2, p=p)
+        lead = tuple(q.shape[:-2])
+        o = torch.empty(lead + (1, desc.d), dtype=q.dtype, device=q.device)
+        g = torch.empty(lead + (1,), dtype=torch.float32, device=q.device)
+        desc.so, desc.sg = _strides(o), _gstrides(g)
+        scratch = torch.empty(max(self.lib.fastmax_decode_scratch_bytes(C.byref(desc)) // 4, 1), dtype=torch.float32,
+                              device=q.device)
+        st = self.lib.fastmax_decode_step(C.byref(desc), q.data_ptr(), k.data_ptr(), v.data_ptr(), state.data_ptr(),
+                                          o.data_ptr(), g.data_ptr(), scratch.data_ptr(), self._stream(q))
+        self.check(st, "fastmax_decode_step")
+        return o, g
 
     def backward(self, q, k, v, o, g, d_o, *, mask, inv_tau, a0=1.0, a1=1.0, a2=0.5, p=2, chunk=0, flags=0,
                  saved: Optional[torch.Tensor] = None, out=None, ws: Optional[torch.Tensor] = None, norm=None):

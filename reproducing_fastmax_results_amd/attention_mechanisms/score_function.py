@@ -29,7 +29,7 @@ from .. import fastmax_cuda as _ext   # the torch binding built by __graft_entry
 
 __all__ = [
     "FASTMultiHeadAttention_Function", "FASTMultiHeadAttention", "rpe_matrix_creator", "fastmax_custom",
-    "fastmax", "fastmax_einops", "FastmaxNormalize", "FastmaxNormAttention",
+    "fastmax", "fastmax_einops", "FastmaxNormalize", "FastmaxNormAttention", "FastmaxDecodeState",
 ]
 
 CENTRE_NONE, CENTRE_FEATURE, CENTRE_TOKEN = 0, 1, 2
@@ -171,6 +171,47 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
             grad_output = _pad_features(grad_output)
         gq, gk, gv = _ext.backward_saved(q, k, v, o, g, grad_output, saved, mask, inv_tau, a0, a1, a2, p, 0, 0)
         return (gq[..., :d], gk[..., :d], gv[..., :d]) + (None,) * 11
+
+
+class FastmaxDecodeState:
+    """The persistent moment state of incremental decoding for one attention layer: the sums the
+    reference's causal kernel runs along the sequence (``fastmax_cuda_forward.cu:160-276``), kept between
+    calls, so that a generation step costs the same whatever the number of tokens before it (the
+    reference's loop, ``transformer/eval.py:8-32``, runs the whole context for every token).
+    ``prompt(q, k, v)``: ordinary causal attention over a first block of tokens, whose keys and values are
+    then absorbed; ``step(q, k, v)``: one token.  Tensors are ``(b, h, n, d)`` or ``(b*h, n, d)``; no
+    gradients; q and k unnormalised (the max-norm depends on every token)."""
+
+    def __init__(self, temperature=1.0, a0=1.0, a1=1.0, a2=0.5, p=2):
+        self.args = (1.0 / float(temperature), float(a0), float(a1), float(a2), int(p))
+        self.state, self.tokens = None, 0
+
+    def _absorb(self, k, v):
+        if self.state is None:
+            self.state = _ext.decode_state(k, *self.args)
+        _ext.decode_absorb(k, v, self.state, *self.args)
+        self.tokens += k.shape[-2]
+
+    @torch.no_grad()
+    def prompt(self, q, k, v):
+        if self.tokens:
+            raise ValueError("the state takes a block of tokens only while it is empty; then single tokens")
+        d = q.shape[-1]
+        q, k, v = _pad_features(q), _pad_features(k), _pad_features(v)
+        inv_tau, a0, a1, a2, p = self.args
+        o, _ = _ext.forward_ex(q, k, v, True, inv_tau, a0, a1, a2, p, 0, 0)
+        self._absorb(k, v)
+        return o[..., :d]
+
+    @torch.no_grad()
+    def step(self, q, k, v):
+        d = q.shape[-1]
+        q, k, v = _pad_features(q), _pad_features(k), _pad_features(v)
+        if self.state is None:
+            self.state = _ext.decode_state(k, *self.args)
+        o, _ = _ext.decode_step(q, k, v, self.state, *self.args)
+        self.tokens += 1
+        return o[..., :d]
 
 
 def fastmax_function(q, k, v, mask=0, dropout_rate=0.0, normalize=0, temperature=1, a0=1, a1=1, a2=0.5, lim=1, p=2):

@@ -5,6 +5,7 @@
 #include "fm_tok.h"
 #include "fm_norm.h"
 #include "fm_split.h"
+#include "fm_decode.h"
 #include <atomic>
 #include <cmath>
 #include <mutex>
@@ -707,6 +708,49 @@ size_t fastmax_normalize_stats_bytes(const FastmaxNormDesc* desc) {
 int fastmax_normalize(const FastmaxNormDesc* desc, const void* x, void* y, float* stats, void* hip_stream) {
   ProfScope prof(FM_K_NORM, static_cast<fm_stream_t>(hip_stream));   // the whole pass (its kernels together)
   return fm_normalize_dispatch(desc, x, y, stats, static_cast<fm_stream_t>(hip_stream));
+}
+
+static int decode_validate(const FastmaxDesc* d) {
+  if (!d) return FASTMAX_ERR_NULL;
+  if (d->dtype != FASTMAX_F32 && d->dtype != FASTMAX_BF16) return FASTMAX_ERR_DTYPE;
+  if (d->bh <= 0 || d->bh > 65535) return FASTMAX_ERR_SHAPE;
+  if (d->p != 1 && d->p != 2) return FASTMAX_ERR_UNSUPPORTED;
+  if (d->d != 32 && d->d != 64) return FASTMAX_ERR_UNSUPPORTED;
+  if (!(d->inv_tau > 0.0f) || !(d->inv_tau < 3.0e38f)) return FASTMAX_ERR_SHAPE;
+  return FASTMAX_OK;
+}
+
+size_t fastmax_decode_state_bytes(const FastmaxDesc* desc) {
+  if (decode_validate(desc)) return 0;
+  return size_t(desc->bh) * size_t(fm_decode_state_floats(desc->d, desc->p == 2 && desc->a2 != 0.0f)) * 4;
+}
+
+size_t fastmax_decode_scratch_bytes(const FastmaxDesc* desc) {
+  if (decode_validate(desc)) return 0;
+  return size_t(desc->bh) * size_t(fm_decode_blocks(desc->d, desc->p == 2 && desc->a2 != 0.0f)) * (desc->d + 1) * 4;
+}
+
+int fastmax_decode_absorb(const FastmaxDesc* desc, const void* k, const void* v, float* state, void* hip_stream) {
+  const int st = decode_validate(desc);
+  if (st) return st;
+  if (!k || !v || !state) return FASTMAX_ERR_NULL;
+  if (desc->nk <= 0 || desc->nk > (1 << 30)) return FASTMAX_ERR_SHAPE;
+  if (!strides_ok(desc->sk, desc->bh, desc->nk, desc->d) || !strides_ok(desc->sv, desc->bh, desc->nk, desc->d))
+    return FASTMAX_ERR_SHAPE;
+  return fm_decode_dispatch(desc, nullptr, k, v, desc->nk, state, nullptr, nullptr, nullptr, static_cast<fm_stream_t>(hip_stream));
+}
+
+int fastmax_decode_step(const FastmaxDesc* desc, const void* q, const void* k, const void* v, float* state, void* o, float* g,
+                        float* scratch, void* hip_stream) {
+  const int st = decode_validate(desc);
+  if (st) return st;
+  if (!q || !k || !v || !state || !o || !g) return FASTMAX_ERR_NULL;
+  if (!scratch) return FASTMAX_ERR_WORKSPACE;
+  if (!strides_ok(desc->sq, desc->bh, 1, desc->d) || !strides_ok(desc->sk, desc->bh, 1, desc->d) ||
+      !strides_ok(desc->sv, desc->bh, 1, desc->d) || !strides_ok(desc->so, desc->bh, 1, desc->d) ||
+      !strides_ok(desc->sg, desc->bh, 1, 1))
+    return FASTMAX_ERR_SHAPE;
+  return fm_decode_dispatch(desc, q, k, v, 1, state, o, g, scratch, static_cast<fm_stream_t>(hip_stream));
 }
 
 size_t fastmax_maxnorm_stats_bytes(int32_t bh, int32_t n) {

@@ -375,6 +375,47 @@ std::vector<torch::Tensor> backward_norm(torch::Tensor q, torch::Tensor k, torch
                       flags | FASTMAX_FLAG_SAVE_FOR_BACKWARD, &na);
 }
 
+// Incremental decoding on a persistent moment state (fastmax_decode_* in the C header).
+FastmaxDesc decode_desc(const View& q, const View& k, const View& v, double inv_tau, double a0, double a1, double a2,
+                        int64_t p) {
+  return ex_desc(q, k, v, true, inv_tau, a0, a1, a2, p, 0, 0);
+}
+
+// an empty state for keys shaped like k: zero-filled float32
+torch::Tensor decode_state(torch::Tensor k_, double inv_tau, double a0, double a1, double a2, int64_t p) {
+  const View k = view_of(k_, "k");
+  FastmaxDesc d = decode_desc(k, k, k, inv_tau, a0, a1, a2, p);
+  return torch::zeros({int64_t(fastmax_decode_state_bytes(&d) / 4)}, k.t.options().dtype(torch::kFloat32));
+}
+
+void decode_absorb(torch::Tensor k_, torch::Tensor v_, torch::Tensor state, double inv_tau, double a0, double a1, double a2,
+                   int64_t p) {
+  const View k = view_of(k_, "k"), v = view_of(v_, "v");
+  FastmaxDesc d = decode_desc(k, k, v, inv_tau, a0, a1, a2, p);
+  TORCH_CHECK(state.is_cuda() && state.scalar_type() == torch::kFloat32 && state.is_contiguous() &&
+                  size_t(state.numel()) * 4 == fastmax_decode_state_bytes(&d), "state must come from decode_state for this shape");
+  check_status(fastmax_decode_absorb(&d, k.t.data_ptr(), v.t.data_ptr(), state.data_ptr<float>(), stream_of(k.t)),
+               "fastmax_decode_absorb");
+}
+
+std::tuple<torch::Tensor, torch::Tensor> decode_step(torch::Tensor q_, torch::Tensor k_, torch::Tensor v_, torch::Tensor state,
+                                                    double inv_tau, double a0, double a1, double a2, int64_t p) {
+  const View q = view_of(q_, "q"), k = view_of(k_, "k"), v = view_of(v_, "v");
+  TORCH_CHECK(q.n == 1 && k.n == 1, "decode_step takes one token");
+  FastmaxDesc d = decode_desc(q, k, v, inv_tau, a0, a1, a2, p);
+  TORCH_CHECK(state.is_cuda() && state.scalar_type() == torch::kFloat32 && state.is_contiguous() &&
+                  size_t(state.numel()) * 4 == fastmax_decode_state_bytes(&d), "state must come from decode_state for this shape");
+  torch::Tensor o = empty_like_layout(q.t, 1, q.t.scalar_type());
+  torch::Tensor g = q.t.dim() == 4 ? torch::empty({q.t.size(0), q.t.size(1), 1}, q.t.options().dtype(torch::kFloat32))
+                                   : torch::empty({q.bh, 1}, q.t.options().dtype(torch::kFloat32));
+  d.so = view_of(o, "o").s;
+  d.sg = gstrides_of(g);
+  torch::Tensor scratch = torch::empty({int64_t(fastmax_decode_scratch_bytes(&d) / 4)}, q.t.options().dtype(torch::kFloat32));
+  check_status(fastmax_decode_step(&d, q.t.data_ptr(), k.t.data_ptr(), v.t.data_ptr(), state.data_ptr<float>(), o.data_ptr(),
+                                   g.data_ptr<float>(), scratch.data_ptr<float>(), stream_of(q.t)), "fastmax_decode_step");
+  return {o, g};
+}
+
 // y = scale * (x - centre) / max_n ||x_n - centre||  (see fastmax_normalize in the C header)
 torch::Tensor normalize(torch::Tensor x_, int64_t centre, bool max_norm, double scale) {
   const View x = view_of(x_, "x");
@@ -434,6 +475,9 @@ PYBIND11_MODULE(fastmax_cuda, m) {
   m.def("maxnorm_stats", &maxnorm_stats, "statistics of the folded max-norm normalisation of q and k: (q_keys, k_keys)");
   m.def("forward_norm", &forward_norm, "strided forward with q, k normalised on load: returns (o, g, saved)");
   m.def("backward_norm", &backward_norm, "backward of forward_norm: returns [dq, dk, dv]");
+  m.def("decode_state", &decode_state, "empty decoding state (zeros) for keys shaped like k");
+  m.def("decode_absorb", &decode_absorb, "add all tokens of k, v to a decoding state");
+  m.def("decode_step", &decode_step, "one decoding step on the state: returns (o, g) of the new token");
   m.def("normalize", &normalize, "fused normalisation pass");
   m.def("normalize_backward", &normalize_backward, "gradient of the normalisation pass with respect to its input");
   m.def("version", []() { return fastmax_version(); });

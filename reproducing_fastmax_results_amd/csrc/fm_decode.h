@@ -1,0 +1,154 @@
+// Incremental decoding on a persistent moment state: what makes Fastmax generation O(1) per token.
+//
+// The causal kernel of the reference keeps running sums over the keys and adds one key per query
+// (fastmax_cuda_forward.cu:160-276: the first nk - nq keys are summed before the first query, then one
+// more per query).  Kept between calls, those sums are the whole memory of the sequence: a decoding step
+// adds the new token's key and value to them and reads them out with the new query, without touching any
+// earlier key (the reference's generation loop, transformer/eval.py:8-32, runs the whole context through the
+// model for every new token).
+//
+// State of one batch*head, fp32, with k' = k * inv_tau and R = 1 + D (+ D*D for order 2) moment rows:
+//     num [R][D]   row 0: sum v        rows 1 + m: sum k'_m v        rows 1 + D + m*D + l: sum k'_m k'_l v
+//     den [R]      the same sums with v replaced by 1 (row 0: the number of keys)
+// Readout for a query q:  F = a0 num[0] + a1 sum_m q_m num[1+m] + a2 sum_{m,l} q_m q_l num[1+D+mD+l],
+// g likewise from den, o = F / g.
+//
+// k_decode_absorb: grid (ceil(R / 256), bh), 256 threads.  A workgroup owns 256 moment rows; thread (wave w,
+// lane c) keeps column c of the rows w, w + 4, ... of that block in registers (64 values), adds the new
+// tokens one after the other (their k', v staged through LDS), writes the rows back and, when a query is
+// given (one new token), leaves its part of F and g in `part` [bh][blocks][D + 1]; k_decode_finish adds the
+// parts in a fixed order and divides.  Bandwidth bound: a step reads and writes the state once.
+#pragma once
+#include "fm_kernels.h"
+
+static constexpr int FM_DEC_ROWS = 256;     // moment rows per workgroup
+inline int64_t fm_decode_rows(int d, bool quad) { return 1 + int64_t(d) + (quad ? int64_t(d) * d : 0); }
+inline int fm_decode_blocks(int d, bool quad) { return int((fm_decode_rows(d, quad) + FM_DEC_ROWS - 1) / FM_DEC_ROWS); }
+// floats of one batch*head's state: num [R][D] then den [R], R rounded up to whole blocks
+inline int64_t fm_decode_state_floats(int d, bool quad) {
+  return int64_t(fm_decode_blocks(d, quad)) * FM_DEC_ROWS * (d + 1);
+}
+
+// the two key features a moment row multiplies (index DH stands for the constant 1)
+template <int DH> FM_DEVICE void fm_decode_row(int r, bool quad, int& m, int& l, bool& live) {
+  live = true;
+  if (r == 0) { m = DH; l = DH; }
+  else if (r <= DH) { m = r - 1; l = DH; }
+  else if (quad && r < 1 + DH + DH * DH) { m = (r - 1 - DH) / DH; l = (r - 1 - DH) % DH; }
+  else { m = DH; l = DH; live = false; }
+}
+
+template <typename TIO, int DH>
+FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS)
+k_decode_absorb(TRef<const TIO> k, TRef<const TIO> v, TRef<const TIO> q, int n_new, int quad, float inv_tau, float a0,
+                float a1, float a2, float* FM_RESTRICT state, float* FM_RESTRICT part) {
+  constexpr int RPT = FM_DEC_ROWS / 4;                  // rows per thread (one column each)
+  constexpr int TB = 16;                                 // new tokens staged at a time
+  FM_SHARED float ks[TB][DH + 1];                        // k' of the staged tokens, [DH] = 1
+  FM_SHARED float vs[TB][DH];
+  FM_SHARED float qs[DH + 1];
+  FM_SHARED float red[4][DH + 1];
+  const int tid = FM_TID_X, lane = tid & 63, wave = tid >> 6, bh = FM_BID_Y, blk = FM_BID_X;
+  const int64_t R = int64_t(FM_GDIM_X) * FM_DEC_ROWS;
+  float* num = state + int64_t(bh) * R * (DH + 1);
+  float* den = num + R * DH;
+  const int r0 = blk * FM_DEC_ROWS;
+  const bool col_live = lane < DH;                       // D = 32: half of the lanes hold no column
+  // this thread's rows and their feature pairs
+  float acc[RPT];
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) acc[i] = col_live ? num[int64_t(r0 + wave + 4 * i) * DH + lane] : 0.f;
+  // denominators: thread t owns row r0 + t
+  float dsum = den[r0 + tid];
+  int dm, dl; bool dlive;
+  fm_decode_row<DH>(r0 + tid, quad != 0, dm, dl, dlive);
+  for (int t0 = 0; t0 < n_new; t0 += TB) {
+    FM_SYNC();
+    for (int i = tid; i < TB * (DH + 1); i += FM_THREADS) {
+      const int t = i / (DH + 1), f = i % (DH + 1);
+      float x = 0.f;
+      if (t0 + t < n_new) x = f < DH ? IO<TIO>::ld(k.base(bh) + int64_t(t0 + t) * k.s_n + f) * inv_tau : 1.0f;
+      ks[t][f] = x;
+    }
+    for (int i = tid; i < TB * DH; i += FM_THREADS) {
+      const int t = i / DH, f = i % DH;
+      vs[t][f] = (t0 + t < n_new) ? IO<TIO>::ld(v.base(bh) + int64_t(t0 + t) * v.s_n + f) : 0.f;
+    }
+    FM_SYNC();
+    const int nt = n_new - t0 < TB ? n_new - t0 : TB;
+    for (int t = 0; t < nt; ++t) {
+      const float vc = col_live ? vs[t][lane] : 0.f;
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) {
+        int m, l; bool live;
+        fm_decode_row<DH>(r0 + wave + 4 * i, quad != 0, m, l, live);
+        if (live) acc[i] += ks[t][m] * ks[t][l] * vc;
+      }
+      if (dlive) dsum += ks[t][dm] * ks[t][dl];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < RPT; ++i)
+    if (col_live) num[int64_t(r0 + wave + 4 * i) * DH + lane] = acc[i];
+  den[r0 + tid] = dsum;
+  if (!part) return;
+  // readout of the new token's query against the rows of this block
+  FM_SYNC();
+  if (tid <= DH) qs[tid] = tid < DH ? IO<TIO>::ld(q.base(bh) + tid) : 1.0f;
+  FM_SYNC();
+  float f = 0.f;
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) {
+    int m, l; bool live;
+    const int r = r0 + wave + 4 * i;
+    fm_decode_row<DH>(r, quad != 0, m, l, live);
+    const float coef = r == 0 ? a0 : (r <= DH ? a1 : a2);
+    if (live) f += coef * qs[m] * qs[l] * acc[i];
+  }
+  float gsum = dlive ? (r0 + tid == 0 ? a0 : (r0 + tid <= DH ? a1 : a2)) * qs[dm] * qs[dl] * dsum : 0.f;
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) gsum += fm_shfl_xor(gsum, m);
+  if (col_live) red[wave][lane] = f;
+  if (lane == 0) red[wave][DH] = gsum;
+  FM_SYNC();
+  if (tid <= DH)
+    part[(int64_t(bh) * FM_GDIM_X + blk) * (DH + 1) + tid] = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
+}
+
+// o = F / g from the parts of k_decode_absorb.  grid (bh), 64 threads.
+template <typename TIO, int DH>
+FM_GLOBAL void FM_LAUNCH_BOUNDS(64) k_decode_finish(const float* FM_RESTRICT part, int nblk, TRef<TIO> o, TRef<float> g) {
+  const int bh = FM_BID_X, lane = FM_TID_X;
+  const float* p = part + int64_t(bh) * nblk * (DH + 1);
+  float gs = 0.f, f = 0.f;
+  for (int b = 0; b < nblk; ++b) {
+    gs += p[b * (DH + 1) + DH];
+    if (lane < DH) f += p[b * (DH + 1) + lane];
+  }
+  if (lane < DH) IO<TIO>::st(o.base(bh) + lane, f / gs);
+  if (lane == 0) g.base(bh)[0] = gs;
+}
+
+template <typename TIO, int DH>
+int fm_decode_run(const FastmaxDesc* d, const void* q, const void* k, const void* v, int n_new, float* state, void* o,
+                  float* g, float* scratch, fm_stream_t stream) {
+  const bool quad = d->p == 2 && d->a2 != 0.0f;
+  const int nblk = fm_decode_blocks(DH, quad);
+  const TRef<const TIO> kr = fm_ref<const TIO>(static_cast<const TIO*>(k), d->sk), vr = fm_ref<const TIO>(static_cast<const TIO*>(v), d->sv);
+  const TRef<const TIO> qr = q ? fm_ref<const TIO>(static_cast<const TIO*>(q), d->sq) : kr;
+  FM_KERNEL_LAUNCH((k_decode_absorb<TIO, DH>), fm_dim3(nblk, d->bh), fm_dim3(FM_THREADS), 0, stream, kr, vr, qr, n_new, quad ? 1 : 0,
+                   d->inv_tau, d->a0, d->a1, quad ? d->a2 : 0.0f, state, q ? scratch : nullptr);
+  if (q)
+    FM_KERNEL_LAUNCH((k_decode_finish<TIO, DH>), fm_dim3(d->bh), fm_dim3(64), 0, stream, scratch, nblk,
+                     fm_ref<TIO>(static_cast<TIO*>(o), d->so), fm_ref<float>(g, d->sg));
+  return fm_after_launch() ? FASTMAX_ERR_LAUNCH : FASTMAX_OK;
+}
+
+inline int fm_decode_dispatch(const FastmaxDesc* d, const void* q, const void* k, const void* v, int n_new, float* state,
+                              void* o, float* g, float* scratch, fm_stream_t stream) {
+  if (d->dtype == FASTMAX_BF16)
+    return d->d == 64 ? fm_decode_run<fm_bf16, 64>(d, q, k, v, n_new, state, o, g, scratch, stream)
+                      : fm_decode_run<fm_bf16, 32>(d, q, k, v, n_new, state, o, g, scratch, stream);
+  return d->d == 64 ? fm_decode_run<float, 64>(d, q, k, v, n_new, state, o, g, scratch, stream)
+                    : fm_decode_run<float, 32>(d, q, k, v, n_new, state, o, g, scratch, stream);
+}

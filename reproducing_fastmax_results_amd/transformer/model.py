@@ -20,8 +20,8 @@ import math
 import torch
 from torch import nn
 
-from ..attention_mechanisms.score_function import (CENTRE_NONE, FASTMultiHeadAttention_Function, FastmaxNormalize,
-                                                    FastmaxNormAttention, _fold_possible)
+from ..attention_mechanisms.score_function import (CENTRE_NONE, FASTMultiHeadAttention_Function, FastmaxDecodeState,
+                                                    FastmaxNormalize, FastmaxNormAttention, _fold_possible)
 
 
 def fastmax_attention(q, k, v, *, mask, normalize, lim, temperature, a0, a1, a2, p):
@@ -61,9 +61,24 @@ class Attention(nn.Module):
         b, n, _ = x.shape
         q = self.query_transform(x).view(b, n, self.h, self.d_head).transpose(1, 2)   # (b, h, n, d) views
         kp, vp = self.key_transform(x), self.value_transform(x)
+        if cache is not None and self.normalize:
+            raise ValueError("cached decoding needs normalize=False: the max-norm scaling looks at every token")
+        if cache is not None and cache.get("kind") == "state":
+            # O(1) decoding: the layer keeps the moment state instead of the keys and values (needs the causal mask)
+            if not self.use_masking:
+                raise ValueError("the decoding state is causal attention's; this layer is unmasked")
+            if "state" not in cache:
+                a0, a1, a2 = self.coefficients
+                cache["state"] = FastmaxDecodeState(self.temperature, a0, a1, a2, self.p)
+            k = kp.view(b, n, self.h, self.d_head).transpose(1, 2)
+            v = vp.view(b, n, self.h, self.d_head).transpose(1, 2)
+            st = cache["state"]
+            o = st.step(q, k, v) if (n == 1 and st.tokens) else st.prompt(q, k, v)
+            cache["n"] = st.tokens
+            o = o.transpose(1, 2).reshape(b, n, self.h * self.d_head)
+            return self.dropout(self.linear(o))
         if cache is not None:
-            if self.normalize:
-                raise ValueError("cached keys need normalize=False: the max-norm scaling looks at every token")
+            cache["n"] = cache.get("n", 0) + n
             if "k" in cache:
                 kp, vp = torch.cat((cache["k"], kp), dim=1), torch.cat((cache["v"], vp), dim=1)
             cache["k"], cache["v"] = kp, vp
@@ -158,7 +173,7 @@ class Transformer(nn.Module):
         x = self.token_embedding(tokens)
         if self.classifier.kind == "cls_token":
             x = torch.cat((self.class_token.expand(x.shape[0], 1, -1), x), dim=1)
-        past = caches[0]["k"].shape[1] if caches and "k" in caches[0] else 0
+        past = caches[0].get("n", 0) if caches else 0
         x = x + self.pos_embedding(torch.arange(past, past + x.shape[1], device=x.device))
         for i, block in enumerate(self.blocks):
             x = block(x, caches[i] if caches is not None else None)
@@ -168,13 +183,18 @@ class Transformer(nn.Module):
     def generate(self, tokens, max_new_tokens, sample=False, use_cache=True):
         """Next-token generation (reference ``transformer/eval.py:8-32``): ``tokens`` ``(b, n)`` grows
         by ``max_new_tokens``.  The reference runs the whole context through the model for every
-        new token.  With ``use_cache`` the key and value projections of every block are kept and a
+        new token.  With ``use_cache="state"`` every layer keeps the O(1) moment state of its keys and values
+        (``FastmaxDecodeState``) and a step costs the same whatever the context length; with
+        ``use_cache=True`` the key and value projections of every block are kept and a
         step runs the new token only; its attention is one causal call with one query and all the
         keys so far.  That is exact for ``normalize=False`` models (the max-norm scaling of the
         others depends on every token, so they take the reference's route).  Contexts longer than
         the position table are not handled (the reference crops to the last ``max_tokens``)."""
-        cached = use_cache and not any(b.attention_subblock.normalize for b in self.blocks)
-        caches = [dict() for _ in self.blocks] if cached else None
+        cached = bool(use_cache) and not any(b.attention_subblock.normalize for b in self.blocks)
+        # use_cache = "state": every layer keeps its O(1) moment state (the prompt goes through ordinary causal
+        # attention once and is absorbed); True: keys and values are kept and re-read every step
+        kind = "state" if use_cache == "state" else "kv"
+        caches = [dict(kind=kind) for _ in self.blocks] if cached else None
         logits = self(tokens, caches)[:, -1, :]
         for _ in range(max_new_tokens):
             nxt = torch.multinomial(torch.softmax(logits, -1), 1) if sample else logits.argmax(-1, keepdim=True)

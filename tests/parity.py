@@ -117,3 +117,29 @@ def check_norm_fold(lib, bh, nq, d, dtype, device, *, mask, p, nk=None, chunk=0,
     for n, e in errs.items():
         assert e < TOL[dtype], f"{n} rel-L2 {e:.3e} (all: {errs})"
     return errs
+
+
+def check_decode(lib, bh, n, n0, d, dtype, device, *, p, tau_mult=8.0, a=(1.0, 1.0, 0.5), seed=0, four_d=False):
+    """Incremental decoding on the persistent moment state: the first n0 tokens are absorbed as a prompt, the
+    others go through one step each; every step's o and g against the fp64 closed form of causal attention over
+    the whole sequence (the state is fp32, so the bar is the fp32 one for fp32 tensors, the bf16 one for bf16)."""
+    q, k, v, _ = make_inputs(bh, n, n, d, dtype, device, seed)
+    tau = tau_mult * math.sqrt(d)
+    kw = dict(inv_tau=1.0 / tau, p=p, a0=a[0], a1=a[1], a2=a[2])
+    if four_d:                                   # (b, h, n, d) views of a (b, n, h*d) layout, two heads per batch
+        assert bh % 2 == 0
+        q, k, v = (t.view(bh // 2, 2, n, d).transpose(1, 2).contiguous().transpose(1, 2) for t in (q, k, v))
+    state = lib.decode_state(k, **kw)
+    if n0:
+        lib.decode_absorb(k[..., :n0, :], v[..., :n0, :], state, **kw)
+    outs, gs = [], []
+    for t in range(n0, n):
+        o, g = lib.decode_step(q[..., t:t + 1, :], k[..., t:t + 1, :], v[..., t:t + 1, :], state, **kw)
+        outs.append(o); gs.append(g)
+    o = torch.cat(outs, dim=-2).reshape(bh, n - n0, d)
+    g = torch.cat(gs, dim=-1).reshape(bh, n - n0)
+    q3, k3, v3 = (t.reshape(bh, n, d).detach().cpu().double() for t in (q, k, v))
+    ro, rg = O.closed_form_forward(q3, k3, v3, mask=True, tau=tau, p=p, a0=a[0], a1=a[1], a2=a[2])
+    eo, eg = rel_err(o, ro[:, n0:]), rel_err(g, rg[:, n0:])
+    assert eo < TOL[dtype] and eg < TOL[dtype], f"decode o {eo:.3e} g {eg:.3e}"
+    return eo, eg

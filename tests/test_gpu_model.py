@@ -223,6 +223,15 @@ def test_cached_generation_matches_full_recompute():
         step = hip(fast[:, 50:51], caches)[:, -1, :]
         want = ref(fast[:, :51])[:, -1, :]
     assert float((step - want).norm() / want.norm()) < 1e-4
+    # O(1) decoding state per layer (prompt through ordinary causal attention, then one step per token): the same
+    # tokens, and the step logits against the oracle again
+    state_tokens = hip.generate(prompt, 24, use_cache="state")
+    assert torch.equal(state_tokens, slow)
+    with torch.no_grad():
+        caches = [dict(kind="state") for _ in hip.blocks]
+        hip(fast[:, :50], caches)
+        step = hip(fast[:, 50:51], caches)[:, -1, :]
+    assert float((step - want).norm() / want.norm()) < 1e-4
     # models that normalise q and k cannot cache (the scaling sees every token): same route as the reference
     norm_model = gpt_for_c5(**dict(cfg, normalize=True, temperature=1.0)).to(DEV).eval()
     assert norm_model.generate(prompt, 3).shape == (3, 43)

@@ -4,7 +4,8 @@ bf16-rounded inputs)."""
 import pytest
 import torch
 
-from tests.parity import check_batch_head_strides, check_forward, check_forward_backward, check_norm_fold
+from tests.parity import (check_batch_head_strides, check_decode, check_forward, check_forward_backward,
+                          check_norm_fold)
 from reproducing_fastmax_results_amd._capi import FLAG_FORCE_DENSE, FLAG_FORCE_MOMENTS
 
 pytestmark = pytest.mark.gpu
@@ -220,6 +221,29 @@ def test_normalisation_folded_into_the_loads(lib, dtype, jacobian):
     check_norm_fold(lib, 2, 300, 64, dtype, DEV, mask=False, p=2, nk=700, seed=75, jacobian=jacobian, saved=False)
     check_norm_fold(lib, 2, 50, 32, dtype, DEV, mask=False, p=2, seed=76, jacobian=jacobian)
     check_norm_fold(lib, 8, 4096, 64, dtype, DEV, mask=True, p=2, seed=77, jacobian=jacobian, lim=1.0, tau=1.0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("p", [1, 2])
+@pytest.mark.parametrize("d", [32, 64])
+def test_incremental_decoding_on_the_moment_state(lib, dtype, p, d):
+    """fastmax_decode_absorb / fastmax_decode_step: a prompt absorbed into the persistent state, then one step per
+    token, every step against the fp64 closed form of causal attention over the whole sequence; also decoding
+    from the empty state, the reference's own test temperature, and the cached-keys route on the same tokens."""
+    print(f"case decode state dtype={dtype} p={p} d={d}", flush=True)
+    check_decode(lib, 6, 700, 640, d, dtype, DEV, p=p, seed=90)
+    check_decode(lib, 4, 48, 0, d, dtype, DEV, p=p, seed=91, tau_mult=1.0)
+    check_decode(lib, 4, 300, 290, d, dtype, DEV, p=p, seed=92, four_d=True)
+    # one step against the library's own route over cached keys (causal, one query, all keys)
+    import math
+    from tests.parity import make_inputs, rel_err, TOL
+    q, k, v, _ = make_inputs(3, 513, 513, d, dtype, DEV, seed=93)
+    kw = dict(inv_tau=1.0 / (8.0 * math.sqrt(d)), p=p)
+    state = lib.decode_state(k, **kw)
+    lib.decode_absorb(k[:, :512], v[:, :512], state, **kw)
+    o, g = lib.decode_step(q[:, 512:], k[:, 512:], v[:, 512:], state, **kw)
+    o2, g2 = lib.forward(q[:, 512:].contiguous(), k, v, mask=True, **kw)
+    assert rel_err(o, o2) < TOL[dtype] and rel_err(g, g2) < TOL[dtype]
 
 
 @pytest.mark.parametrize("go_scale", [1e-7, 1e-4, 3e4])

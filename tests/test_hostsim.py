@@ -15,7 +15,7 @@ import pytest
 import torch
 
 from reproducing_fastmax_results_amd import _capi
-from tests.parity import (TOL, check_batch_head_strides, check_norm_fold, check_forward, check_forward_backward, make_inputs, oracle_all,
+from tests.parity import (TOL, check_batch_head_strides, check_decode, check_norm_fold, check_forward, check_forward_backward, make_inputs, oracle_all,
                           rel_err)
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -212,3 +212,10 @@ def test_normalisation_folded_into_the_loads(sim):
     check_norm_fold(sim, 2, 40, 32, torch.float32, "cpu", mask=False, p=2, nk=75, seed=27, saved=False)
     # the reference extension's gradients: with respect to the normalised tensors
     check_norm_fold(sim, 2, 70, 32, torch.float32, "cpu", mask=True, p=2, seed=28, jacobian=False)
+
+
+def test_incremental_decoding_on_the_moment_state(sim):
+    # a prompt absorbed into the state, then one step per token; and decoding from the empty state
+    check_decode(sim, 2, 40, 33, 32, torch.float32, "cpu", p=2, seed=30)
+    check_decode(sim, 2, 12, 0, 32, torch.bfloat16, "cpu", p=2, seed=31, tau_mult=1.0)
+    check_decode(sim, 2, 30, 20, 32, torch.float32, "cpu", p=1, seed=32, four_d=True)
