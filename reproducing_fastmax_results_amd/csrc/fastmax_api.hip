@@ -6,6 +6,7 @@
 #include "fm_norm.h"
 #include "fm_split.h"
 #include "fm_decode.h"
+#include "fm_o1.h"
 #include <atomic>
 #include <cmath>
 #include <mutex>
@@ -167,7 +168,8 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
     // beyond; order 1 (one D x D state per segment): one segment up to 1024 tokens (0.150 against 0.159 ms
     // per step at B*H = 128; at 1536 tokens, B*H = 96: 0.209 against 0.190),
     // 256-token segments beyond.
-    const int auto_L = p.quad ? (d->nq > 6144 ? 1024 : p.npad_q) : (d->nq > 1024 ? 256 : p.npad_q);
+    // Order 1 on _Float16: 128-token segments, so that the backward of a segment is one workgroup's work (k_o1_bwd).
+    const int auto_L = p.quad ? (d->nq > 6144 ? 1024 : p.npad_q) : (d->nq > 1024 ? (p.half ? 128 : 256) : p.npad_q);
     int L = d->chunk > 0 ? (d->chunk >= d->nq ? p.npad_q : int(round_up(d->chunk, 256))) : auto_L;
     if (force_dense || L > p.npad_q) L = p.npad_q;
     p.L = L;

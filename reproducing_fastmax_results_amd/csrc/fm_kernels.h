@@ -164,7 +164,14 @@ FM_DEVICE unsigned long long fm_shfl_xor_u64(unsigned long long v, int m) {
 // largest squared norm m2 and its token of one batch*head; every lane of the wavefront must call it
 FM_DEVICE void fm_maxnorm_join(const unsigned long long* keys, int nblk, int lane, float& m2, int& nstar) {
   unsigned long long k = 0;
-  for (int i = lane; i < nblk; i += 64) { const unsigned long long x = keys[i]; k = x > k ? x : k; }
+  constexpr int UB = 4;                                  // loads in flight per round (see fm_grad_scale)
+  for (int i0 = lane; i0 < nblk; i0 += 64 * UB) {
+    unsigned long long x[UB];
+#pragma unroll
+    for (int u = 0; u < UB; ++u) x[u] = (i0 + 64 * u < nblk) ? keys[i0 + 64 * u] : 0ull;
+#pragma unroll
+    for (int u = 0; u < UB; ++u) k = x[u] > k ? x[u] : k;
+  }
 #pragma unroll
   for (int w = 1; w < 64; w <<= 1) { const unsigned long long o = fm_shfl_xor_u64(k, w); k = o > k ? o : k; }
   const uint32_t bits = uint32_t(k >> 32);
@@ -283,7 +290,16 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_grad_scale(TRef<const TIO> d_o, TR
 FM_DEVICE float fm_grad_scale(const float* part, int nblk, int lane) {
   if (!part) return 1.0f;
   float m = 0.f;
-  for (int i = lane; i < nblk; i += 64) { const float x = part[i]; if (x < 3.0e38f) m = fm_fmaxf(m, x); }
+  // eight loads in flight per round: a long sequence has a thousand parts, and one load per round trip would
+  // make this a chain of memory latencies at the start of every workgroup
+  constexpr int UB = 8;
+  for (int i0 = lane; i0 < nblk; i0 += 64 * UB) {
+    float x[UB];
+#pragma unroll
+    for (int u = 0; u < UB; ++u) x[u] = (i0 + 64 * u < nblk) ? part[i0 + 64 * u] : 0.f;
+#pragma unroll
+    for (int u = 0; u < UB; ++u) if (x[u] < 3.0e38f) m = fm_fmaxf(m, x[u]);
+  }
 #pragma unroll
   for (int w = 1; w < 64; w <<= 1) m = fm_fmaxf(m, fm_shfl_xor(m, w));
   if (!(m > 0.f)) return 1.0f;

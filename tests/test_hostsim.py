@@ -219,3 +219,10 @@ def test_incremental_decoding_on_the_moment_state(sim):
     check_decode(sim, 2, 40, 33, 32, torch.float32, "cpu", p=2, seed=30)
     check_decode(sim, 2, 12, 0, 32, torch.bfloat16, "cpu", p=2, seed=31, tau_mult=1.0)
     check_decode(sim, 2, 30, 20, 32, torch.float32, "cpu", p=1, seed=32, four_d=True)
+
+
+def test_order1_segment_backward_in_one_pass(sim):
+    # beyond 1024 tokens order 1 on _Float16 runs in 128-token segments and k_o1_bwd makes dq, dk, dv of a segment
+    # in one workgroup (9 segments here, the last one ragged); also with the folded normalisation's Jacobian
+    check_forward_backward(sim, 1, 1100, 32, torch.bfloat16, "cpu", mask=True, p=1, seed=40, saved=True)
+    check_norm_fold(sim, 1, 1100, 32, torch.bfloat16, "cpu", mask=True, p=1, seed=41)
