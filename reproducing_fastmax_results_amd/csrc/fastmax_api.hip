@@ -95,6 +95,7 @@ struct Plan {
   int L, nseg, nslots;
   bool use_state, quad;
   bool rows_build;      // order-1 segment sums read the row-major copies: no transposed copy is written
+  bool o1;              // order 1, causal, _Float16, 128-token segments: the path of fm_o1.h (reads the caller's tensors, no copies)
   bool qf;              // dense _Float16 kernels evaluate the order-2 weights in completed-square form (see TileMath)
   int npad_q, npad_k;
   float a0, a1, a2;     // polynomial on the score s = (q.k) / tau
@@ -183,6 +184,7 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
     p.use_state = force_m || (!force_dense && int64_t(d->nk) > int64_t(d->d) * d->d + d->d);
     p.nslots = p.use_state ? 1 : 0;
   }
+  p.o1 = p.half && p.use_state && !p.quad && d->mask && p.L == FM_O1_SEG && d->nq == d->nk;
   p.rows_build = p.half && p.use_state && !p.quad && d->mask;
   {
     // f = (h^2 + kc) / (4 a2) with h = 2 a2 s + a1: worth it, and safe in _Float16, when a2 and kc are of ordinary size
@@ -193,8 +195,8 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   const size_t slots = size_t(d->bh) * p.nslots;
   const size_t bigarr = d->d == 64 ? big_array_bytes<64>(p.esz, p.quad, slots) : big_array_bytes<32>(p.esz, p.quad, slots);
   const size_t smallsz = size_t(d->d == 64 ? StateDims<64>::SMALL : StateDims<32>::SMALL) * 4;
-  const size_t tq = size_t(d->bh) * d->d * p.npad_q * p.esz;
-  const size_t tk = size_t(d->bh) * d->d * p.npad_k * p.esz;
+  const size_t tq = p.o1 ? 0 : size_t(d->bh) * d->d * p.npad_q * p.esz;
+  const size_t tk = p.o1 ? 0 : size_t(d->bh) * d->d * p.npad_k * p.esz;
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off = align256(off + bytes); return o; };
   // transposed copies: only the order-2 state walk, the one-total order-1 walk and the fp32 kernels read them
@@ -207,16 +209,16 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   p.small = take(size_t(d->bh) * p.nslots * smallsz);
   p.save = (d->flags & FASTMAX_FLAG_SAVE_FOR_BACKWARD) != 0;
   p.vr = take(p.save || p.half ? tk : 0);      // _Float16: the forward stages v rows (transposing LDS reads)
-  p.big2 = take(p.save ? bigarr : 0);
+  p.big2 = take(p.save && !p.o1 ? bigarr : 0);
   p.fwd_bytes = off ? off : 256;
   off = 0;
   p.b_kt = take(tkt); p.b_vt = take(tkt); p.b_qt = take(tqt); p.b_qct = take(tqt);
   p.b_kr = take(tk); p.b_vr = take(tk); p.b_qr = take(tq);
   p.b_gh = take(tq); p.b_ght = take(tqt);
-  p.b_cv = take(size_t(d->bh) * p.npad_q * 4);
+  p.b_cv = take(p.o1 ? 0 : size_t(d->bh) * p.npad_q * 4);
   p.b_bigq = take(bigarr); p.b_smallq = take(size_t(d->bh) * p.nslots * smallsz);
   p.b_bigk = take(bigarr); p.b_smallk = take(size_t(d->bh) * p.nslots * smallsz);
-  p.b_bigv = take(bigarr);
+  p.b_bigv = take(p.o1 ? 0 : bigarr);
   p.b_gpart = take(p.half ? size_t(d->bh) * fm_grad_scale_blocks(d->nq) * 4 : 0);   // see k_grad_scale
   // parts of B = sum dy . y per workgroup of the dQ and dK kernels (128 own tokens at least), see k_norm_fix
   const bool jac = d->norm.grad != 0;
@@ -395,9 +397,62 @@ int launch_ds(const TokArgs<TIO, E>& a, int bh, int kernel_id, fm_stream_t strea
   return fm_launch_status();
 }
 
+// ---- order 1 in 128-token segments on the caller's tensors (fm_o1.h) -------------------------
+// Sums of every segment but the last (QG = 0: keys and values, prefix walk) or but the first (QG = 1: queries and
+// gh, suffix walk), then the scan that turns them into prefix / suffix sums.
+template <typename TIO, int DH, int QG>
+int launch_o1_sums(O1SumArgs<TIO>& a, int bh, fm_stream_t stream) {
+  const int nsteps = a.b.nseg - 1;
+  if (nsteps <= 0) return FASTMAX_OK;
+  ProfScope prof(FM_K_BUILD, stream);
+  const size_t lds = fm_o1_sums_lds<DH>();
+  fm_allow_lds(reinterpret_cast<const void*>(&k_o1_sums<TIO, DH, QG>), lds);
+  FM_KERNEL_LAUNCH((k_o1_sums<TIO, DH, QG>), fm_dim3(1, bh, nsteps), fm_dim3(FM_THREADS), lds, stream, a);
+  const int st = fm_launch_status();
+  return (st || nsteps < 2) ? st : launch_scan<fm_half, DH>(a.b, bh, nsteps, stream);
+}
+
+// key / value sums of the forward (and of a backward that has no saved forward): big [v][k']
+template <typename TIO, int DH>
+int o1_key_sums(const FastmaxDesc* d, const Plan& p, const void* k, const void* v, fm_half* big, float* small,
+                fm_stream_t stream) {
+  O1SumArgs<TIO> a;
+  a.x0 = cref<TIO>(k, d->sk); a.x1 = cref<TIO>(v, d->sv); a.o = a.x0; a.g = TRef<const float>{nullptr, 0, 0, 0, 0, 0};
+  a.scale0 = p.sc; a.fold0 = k_fold(d); a.gpart = nullptr; a.gnblk = 0; a.n = d->nk;
+  BuildArgs<fm_half>& b = a.b;
+  b.xt = nullptr; b.pt = nullptr; b.rt = nullptr; b.zt = nullptr; b.pr = nullptr; b.rr = nullptr; b.cw = nullptr;
+  b.za_sel = FM_SRC_R; b.zb_sel = FM_SRC_R; b.vb_from_r = 0; b.seg_parallel = 1;
+  b.npad = p.npad_k; b.nseg = p.nseg; b.L = p.L; b.mode = FM_WALK_PREFIX; b.quad = 0;
+  b.big = big; b.big2 = nullptr; b.small = small; b.nslots = p.nslots;
+  b.coef2 = 0.f; b.coef2b = 0.f; b.coefz = 0.f; b.coef1 = p.a1; b.coef1b = p.a1; b.coefva = p.a1; b.coefvb = p.a0;
+  return launch_o1_sums<TIO, DH, 0>(a, d->bh, stream);
+}
+
+template <typename TIO, int DH>
+int run_forward_o1(const FastmaxDesc* d, const Plan& p, const void* q, const void* k, const void* v, void* o, float* g,
+                   char* ws, fm_stream_t stream) {
+  fm_half* big = reinterpret_cast<fm_half*>(ws + p.big);
+  float* small = reinterpret_cast<float*>(ws + p.small);
+  int st = o1_key_sums<TIO, DH>(d, p, k, v, big, small, stream);   // the backward reads the same state: nothing else to save
+  if (st) return st;
+  O1FwdArgs<TIO> a;
+  a.q = cref<TIO>(q, d->sq); a.k = cref<TIO>(k, d->sk); a.v = cref<TIO>(v, d->sv);
+  a.o = mref<TIO>(o, d->so); a.g = mref<float>(g, d->sg);
+  a.n = d->nq; a.nseg = p.nseg; a.nslots = p.nslots; a.big = big; a.small = small;
+  a.a0 = p.a0; a.a1 = p.a1; a.sc = p.sc; a.q_fold = q_fold(d); a.k_fold = k_fold(d);
+  const size_t lds = fm_o1_fwd_lds<DH>();
+  fm_allow_lds(reinterpret_cast<const void*>(&k_o1_fwd<TIO, DH>), lds);
+  ProfScope prof(FM_K_FWD, stream);
+  FM_KERNEL_LAUNCH((k_o1_fwd<TIO, DH>), fm_dim3(p.nseg, d->bh), fm_dim3(FM_THREADS), lds, stream, a);
+  return fm_launch_status();
+}
+
 template <typename TIO, typename E, int DH, int QT>
 int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* k, const void* v, void* o,
                 float* g, char* ws, fm_stream_t stream) {
+  if constexpr (sizeof(E) == 2) {
+    if (p.o1) return run_forward_o1<TIO, DH>(d, p, q, k, v, o, g, ws, stream);
+  }
   E* kt = reinterpret_cast<E*>(ws + p.kt);
   E* vt = reinterpret_cast<E*>(ws + p.vt);
   E* big = reinterpret_cast<E*>(ws + p.big);

@@ -290,9 +290,9 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_grad_scale(TRef<const TIO> d_o, TR
 FM_DEVICE float fm_grad_scale(const float* part, int nblk, int lane) {
   if (!part) return 1.0f;
   float m = 0.f;
-  // eight loads in flight per round: a long sequence has a thousand parts, and one load per round trip would
+  // sixteen loads in flight per round: a long sequence has a thousand parts, and one load per round trip would
   // make this a chain of memory latencies at the start of every workgroup
-  constexpr int UB = 8;
+  constexpr int UB = 16;
   for (int i0 = lane; i0 < nblk; i0 += 64 * UB) {
     float x[UB];
 #pragma unroll

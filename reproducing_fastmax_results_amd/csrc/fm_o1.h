@@ -1,79 +1,413 @@
-// Order 1, long sequences: the three gradients of one 128-token segment in one pass.
+// Order 1 on long sequences (bf16 tensors, _Float16 arithmetic, causal, 128-token segments): a path of its
+// own that reads the caller's tensors directly and is bound by the bytes it moves.
 //
-// With f(s) = a0 + a1 s the score gradient does not depend on the score, dS_ij = a1 (gh_i.v_j - c_i), and every
-// term that crosses a segment boundary is a D x D sum:
+// With f(s) = a0 + a1 s every term that crosses a segment boundary is a D x D sum, and the score gradient
+// does not depend on the score, dS_ij = a1 (gh_i.v_j - c_i):
+//     F_i   = a0 sum_{j<=i} v_j + a1 (sum_{j<=i} v_j k'_j^T) q'_i          g_i = a0 (i + 1) + a1 q'_i . sum_{j<=i} k'_j
 //     dq'_i = a1 [ (sum_{j<=i} k'_j v_j^T) gh_i - c_i sum_{j<=i} k'_j ]
 //     dk'_j = a1 [ (sum_{i>=j} q'_i gh_i^T) v_j - sum_{i>=j} c_i q'_i ]
 //     dv_j  = a0 sum_{i>=j} gh_i + a1 (sum_{i>=j} gh_i q'_i^T) k'_j
-// so a segment needs its own 128 rows of q', k', v, gh (and c), the prefix sums of (k', v) before it and the
-// suffix sums of (q', gh) after it, and nothing else.  One workgroup per segment stages the four row tiles in
-// LDS once (74 KB: two workgroups per CU, so one loads while the other computes), each wavefront owns 32 tokens
-// and accumulates dq, dk and dv for them: the dense causal tiles inside the segment (8 matrix instructions per
-// tile pair for dq, 16 for dk and dv), then the three state products.  The kernel is bound by the bytes it
-// moves: four tensors in, three out, 16 KB of states per segment; the separate dQ, dK and dV kernels read the
-// four tensors three times over and stream every tile of a segment again per 128 own tokens.
-// Replaces, for this case, calc_gradq/k/v_masked (fastmax_cuda_backward.cu:101-188, 272-358, 430-491).
+// so a segment needs its own 128 rows, the sums over the segments before it (keys, values) and after it
+// (queries, gh), and nothing else.  Four kernels, one workgroup per segment each:
+//   k_o1_sums<KV>  k, v            -> the segment's sums       (k_state_scan then makes prefix sums)
+//   k_o1_fwd       q, k, v, prefix -> o, g
+//   k_o1_sums<QG>  q, dO, o, g     -> the segment's sums       (k_state_scan: suffix sums)
+//   k_o1_bwd       q, k, v, dO, o, g, prefix, suffix -> dq, dk, dv
+// No converted or transposed copy of any tensor is written: rows are converted (and scaled: 1/tau, the
+// folded normalisation, the gradient scale) in registers on their way into LDS.  The general kernels need a
+// conversion pass per tensor, read the four operand copies once per gradient and stream every tile of a
+// segment again per 128 own tokens.  Replaces, for this case, calc_masked (fastmax_cuda_forward.cu:146-280)
+// and calc_gradq/k/v_masked (fastmax_cuda_backward.cu:101-188, 272-358, 430-491).
 #pragma once
 #include "fm_tok.h"
 
-template <typename TIO, typename E> struct O1BwdArgs {
-  const E* qr; const E* gh; const E* kr; const E* vr;   // [bh][npad][DH] compute-type rows (q', gh, k', v)
-  const E* cv;                                          // [bh][npad] c, 16-token groups in `tperm` order
-  int npad, n, nseg, nslots;
-  const E* bigq; const float* smallq;                   // prefix sums of (k', v): slab [f][c] = a1 sum k'_f v_c; va = a1 sum k'
-  const E* bigk; const float* smallk;                   // suffix sums of (q', gh): slab [f][c] = a1 sum q'_f gh_c; va = a1 sum c q'; vb = a0 sum gh
-  const E* bigv;                                        // the same slab transposed: [c][f]
-  TRef<TIO> dq, dk, dv;
-  float a0, a1, sc;
-  const float* gpart; int gnblk;                        // see k_grad_scale
-  NormFold q_fold, k_fold;                              // Jacobian of a folded normalisation: see TokArgs
-  float* bq; float* bk;
+static constexpr int FM_O1_SEG = 128;
+
+// One 128-token segment of a bf16 caller tensor as raw 16-byte chunks: with CPR = DH / 8 chunks per row,
+// thread t holds chunk t % CPR of the rows t / CPR + (256 / CPR) i.  Rows past the end are zeros.
+template <int DH> struct O1Raw {
+  static constexpr int CPR = DH / 8, N = FM_O1_SEG * CPR / FM_THREADS, RSTEP = FM_THREADS / CPR;
+  fm_u32x4 r[N];
+  FM_DEVICE void load(const TRef<const fm_bf16>& x, int bh, int t0, int n, int tid) {
+    const fm_bf16* base = x.base(bh);
+    const int col = (tid % CPR) * 8;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int row = t0 + tid / CPR + RSTEP * i;
+      fm_u32x4 z = {0u, 0u, 0u, 0u};
+      if (row < n) {
+        const fm_bf16* p = base + int64_t(row) * x.s_n + col;
+        if (x.vec) z = *reinterpret_cast<const fm_u32x4*>(p);
+        else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) z[j] = uint32_t(p[2 * j]) | (uint32_t(p[2 * j + 1]) << 16);
+        }
+      }
+      r[i] = z;
+    }
+  }
+  // chunk i as eight floats
+  FM_DEVICE void unpack(int i, float out[8]) const {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t lo = r[i][j] << 16, hi = r[i][j] & 0xffff0000u;
+      __builtin_memcpy(&out[2 * j], &lo, 4);
+      __builtin_memcpy(&out[2 * j + 1], &hi, 4);
+    }
+  }
+  static FM_DEVICE int row_of(int i, int tid) { return tid / CPR + RSTEP * i; }     // inside the segment
+  static FM_DEVICE int col_of(int tid) { return (tid % CPR) * 8; }
+  // converted (times scale) into an LDS tile [128][pitch]
+  FM_DEVICE void store(fm_half* lds, int pitch, int tid, float scale) const {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      float f[8];
+      unpack(i, f);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) f[j] *= scale;
+      CE<fm_half>::st8(lds + row_of(i, tid) * pitch + col_of(tid), f);
+    }
+  }
 };
 
-template <typename TIO, typename E, int DH>
-FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO, E> A) {
+// gh = gscale * dO / g and c = gh . o of the segment's rows, from raw dO and o chunks and the denominators gi of
+// the thread's rows (1 past the end): gh rows go to the LDS
+// tile Gs, c (compute type, 16-token groups in `tperm` order) to cs.  Every lane takes part in the shuffles.
+template <int DH>
+FM_DEVICE void fm_o1_gh_rows(const O1Raw<DH>& rdo, const O1Raw<DH>& ro, const float* gi, float gscale, fm_half* Gs,
+                             int pitch, fm_half* cs, int tid) {
+  typedef O1Raw<DH> R;
+#pragma unroll
+  for (int i = 0; i < R::N; ++i) {
+    const int row = R::row_of(i, tid);
+    const float ginv = gscale / gi[i];
+    float a[8], b[8];
+    rdo.unpack(i, a);
+    ro.unpack(i, b);
+    float csum = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) { a[j] *= ginv; csum += a[j] * b[j]; }
+#pragma unroll
+    for (int m = 1; m < R::CPR; m <<= 1) csum += fm_shfl_xor(csum, m);
+    CE<fm_half>::st8(Gs + row * pitch + R::col_of(tid), a);
+    if (tid % R::CPR == 0) cs[Mma<fm_half>::tperm(row)] = CE<fm_half>::from(csum);
+  }
+}
+
+// ------------------------------------------------------------------------------
+// k_o1_sums: the sums of one segment.  grid (1, bh, steps): step w of the walk (fm_walk_step) is segment w of
+// a prefix walk, segment nseg - 1 - w of a suffix walk.
+//   QG = 0: operands p = v, r = k':   slab [r][c] = coef1 sum p_r r_c (and its transpose in big2),
+//           va = coefva sum k', vb = coefvb sum v
+//   QG = 1: operands p = q', r = gh:  the same slab, va = coefva sum c q', vb = coefvb sum gh
+// The eight 32x32 tiles of the sums (D = 64) are dealt to the wavefronts as in k_build1_rows.
+// ------------------------------------------------------------------------------
+template <typename TIO> struct O1SumArgs {
+  TRef<const TIO> x0, x1;            // QG = 0: k, v          QG = 1: q, dO
+  TRef<const TIO> o; TRef<const float> g;     // QG = 1
+  float scale0;                      // on x0: sqrt(1/tau)
+  NormFold fold0;                    // folded normalisation of x0
+  const float* gpart; int gnblk;     // QG = 1: see k_grad_scale
+  int n;
+  BuildArgs<fm_half> b;              // where the sums go and their coefficients (big, big2, small, nslots, nseg, L, npad, mode, coef*)
+};
+
+template <typename TIO, int DH, int QG>
+FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_o1_sums(O1SumArgs<TIO> A) {
+  typedef fm_half E;
+  typedef Mma<E> M;
+  typedef typename M::frag frag;
+  constexpr int NT = DH / 32, NTILE = NT * NT + 2 * NT, NS = (NTILE + 3) / 4;
+  constexpr int TT = FM_O1_SEG, PQ = DH + M::PAD;
+  FM_DYN_SMEM(smem);
+  E* Lp = reinterpret_cast<E*>(smem);                  // [TT][PQ] each
+  E* Lr = Lp + TT * PQ;
+  E* Lc = Lr + TT * PQ;                                // [TT] weights (QG)
+  const int tid = FM_TID_X, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int wave = FM_UNIFORM(tid >> 6);
+  const int bh = FM_BID_Y;
+  int tb, te, slot;
+  fm_walk_step(A.b.mode, A.b.nseg, A.b.L, A.b.npad, FM_BID_Z, tb, te, slot);
+  E* big = A.b.big + int64_t(bh) * A.b.nslots * StateDims<DH>::stride(false);
+  E* big2 = A.b.big2 ? A.b.big2 + int64_t(bh) * A.b.nslots * StateDims<DH>::stride(false) : nullptr;
+  float* ds = A.b.small + (int64_t(bh) * A.b.nslots + slot) * StateDims<DH>::SMALL;
+  {
+    O1Raw<DH> r0, r1;
+    r0.load(A.x0, bh, tb, A.n, tid);
+    r1.load(A.x1, bh, tb, A.n, tid);
+    const float s0 = A.scale0 * fm_norm_factor(A.fold0, bh, lane);
+    if (QG) {
+      O1Raw<DH> ro;
+      ro.load(A.o, bh, tb, A.n, tid);
+      float gi[O1Raw<DH>::N];
+#pragma unroll
+      for (int i = 0; i < O1Raw<DH>::N; ++i) {
+        const int row = tb + O1Raw<DH>::row_of(i, tid);
+        gi[i] = row < A.n ? A.g.base(bh)[int64_t(row) * A.g.s_n] : 1.0f;
+      }
+      const float gscale = fm_grad_scale(A.gpart ? A.gpart + int64_t(bh) * A.gnblk : nullptr, A.gnblk, lane);
+      r0.store(Lp, PQ, tid, s0);                                       // p = q'
+      fm_o1_gh_rows<DH>(r1, ro, gi, gscale, Lr, PQ, Lc, tid);          // r = gh, weights c
+    } else {
+      r1.store(Lp, PQ, tid, 1.0f);                                     // p = v
+      r0.store(Lr, PQ, tid, s0);                                       // r = k'
+    }
+  }
+  FM_SYNC();
+  // tiles of this wavefront: A operand (tile, feature offset), B operand (tile, or null = weights / ones)
+  const frag ones = M::splat(E(1.0f));
+  fm_f32x16 acc[NS];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) {
+    acc[s] = fm_zero16();
+    const int t = wave + 4 * s;
+    if (t >= NTILE) continue;
+    const E* ta = Lp; const E* tbt = nullptr;
+    int fa = 0, fb = 0;
+    bool wsum = false;
+    if (t < NT * NT) { fa = 32 * (t / NT); tbt = Lr; fb = 32 * (t % NT); }
+    else if (t < NT * NT + NT) { fa = 32 * (t - NT * NT); if (QG) wsum = true; else ta = Lr; }    // va: sum c q' | sum k'
+    else { fa = 32 * (t - NT * NT - NT); if (QG) ta = Lr; }                                       // vb: sum gh   | sum v
+#pragma unroll 4
+    for (int k = 0; k < TT; k += M::KSTEP) {
+      const frag a = M::load_tr(ta, PQ, k, fa, lane);
+      const frag b = tbt ? M::load_tr(tbt, PQ, k, fb, lane) : (wsum ? M::load_perm(Lc + k, 0, lh) : ones);
+      acc[s] = M::mma(a, b, acc[s]);
+    }
+  }
+#pragma unroll
+  for (int s = 0; s < NS; ++s) {
+    const int t = wave + 4 * s;
+    if (t < NTILE) {
+      float v[16];
+#pragma unroll
+      for (int e = 0; e < 16; ++e) v[e] = acc[s][e];
+      fm_put_small<E, DH>(A.b, big, big2, ds, slot, t < NT * NT ? t : t + NT * NT, v, lr, lh);
+    }
+  }
+}
+template <int DH> inline size_t fm_o1_sums_lds() { return (size_t(2) * FM_O1_SEG * (DH + Mma<fm_half>::PAD) + FM_O1_SEG) * 2; }
+
+// ------------------------------------------------------------------------------
+// k_o1_fwd: o and g of one segment.  grid (nseg, bh); wavefront w owns the 32 queries of tile w.
+// big: prefix sums, slab [r][c] = a1 sum v_r k'_c; small: va = a1 sum k', vb = a0 sum v (slot s: segments < s).
+// ------------------------------------------------------------------------------
+template <typename TIO> struct O1FwdArgs {
+  TRef<const TIO> q, k, v;
+  TRef<TIO> o; TRef<float> g;
+  int n, nseg, nslots;
+  const fm_half* big; const float* small;
+  float a0, a1, sc;
+  NormFold q_fold, k_fold;
+};
+
+template <typename TIO, int DH>
+FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 3) k_o1_fwd(O1FwdArgs<TIO> A) {
+  typedef fm_half E;
   typedef TokCfg<E, DH, 1> C;
   typedef Mma<E> M;
   typedef TileMath<E> TM;
   typedef typename M::frag frag;
-  static_assert(M::HAS_TR, "this kernel reads transposed fragments out of row tiles");
-  constexpr int NT = C::NT, NKS = C::NKS, QW = C::QW, PQ = C::PQ;   // QW = 128 tokens = one segment
+  constexpr int NT = C::NT, NKS = C::NKS, QW = C::QW, PQ = C::PQ;
+  static_assert(QW == FM_O1_SEG, "one workgroup per segment");
   FM_DYN_SMEM(smem);
-  E* Qs = reinterpret_cast<E*>(smem);                   // [QW][PQ] each
-  E* Gs = Qs + QW * PQ;
-  E* Ks = Gs + QW * PQ;
+  E* Ks = reinterpret_cast<E*>(smem);                   // [QW][PQ] each; Q' lies in the first tile until its fragments are taken
   E* Vs = Ks + QW * PQ;
-  E* cs = Vs + QW * PQ;                                  // [QW] c in `tperm` order
-  float* vecs = reinterpret_cast<float*>(cs + QW);       // va of the prefix sums | va, vb of the suffix sums: 3 * DH
+  float* vecs = reinterpret_cast<float*>(Vs + QW * PQ);  // va, vb of the prefix sums
+  E* Qs = Ks;
   const int tid = FM_TID_X, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   const int wave = FM_UNIFORM(tid >> 6);
   int seg, bh;
   fm_xcd_map(A.nseg, FM_GDIM_Y, seg, bh);
   const int t0 = seg * QW;
-  const int64_t rows = (int64_t(bh) * A.npad + t0) * DH;
+  const int own = wave * 32 + lr;
+  // every load first: the three row tiles, the vector sums, this lane's fragments of the prefix state
+  O1Raw<DH> rk, rv;
+  frag sf[NT][NKS];
   {
-    TileRegs<E, QW, DH> rq, rg, rk, rv;
-    rq.load(A.qr + rows, DH, tid); rg.load(A.gh + rows, DH, tid);
-    rk.load(A.kr + rows, DH, tid); rv.load(A.vr + rows, DH, tid);
-    if (tid < QW) cs[tid] = A.cv[int64_t(bh) * A.npad + t0 + tid];
+    O1Raw<DH> rq;
+    rq.load(A.q, bh, t0, A.n, tid); rk.load(A.k, bh, t0, A.n, tid); rv.load(A.v, bh, t0, A.n, tid);
+    float vsum = 0.f;
+    if (tid < 2 * DH && seg > 0) vsum = A.small[(int64_t(bh) * A.nslots + seg) * StateDims<DH>::SMALL + DH * DH + tid];
+    const E* sl = A.big + (int64_t(bh) * A.nslots + (seg > 0 ? seg : 1)) * StateDims<DH>::SLAB + lr * DH + lh * M::KPL;
+#pragma unroll
+    for (int ct = 0; ct < NT; ++ct)
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) sf[ct][ks] = M::load(sl + 32 * ct * DH + ks * M::KSTEP);
+    if (tid < 2 * DH) vecs[tid] = vsum;
+    rq.store(Qs, PQ, tid, A.sc * fm_norm_factor(A.q_fold, bh, lane));
+  }
+  FM_SYNC();
+  frag qf[NKS];
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) qf[ks] = M::load(Qs + own * PQ + ks * M::KSTEP + lh * M::KPL);
+  FM_SYNC();                                             // every wavefront has its fragments of Q': K' takes the tile
+  rk.store(Ks, PQ, tid, A.sc * fm_norm_factor(A.k_fold, bh, lane));
+  rv.store(Vs, PQ, tid, 1.0f);
+  FM_SYNC();
+  fm_f32x16 acc[NT];
+#pragma unroll
+  for (int ct = 0; ct < NT; ++ct) acc[ct] = fm_zero16();
+  float gsum = 0.f;
+  if (seg > 0) {
+    // the keys of the earlier segments: F += slab q', g += q' . va (this lane's half of the row; the halves meet below)
+#pragma unroll
+    for (int ct = 0; ct < NT; ++ct)
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) acc[ct] = M::mma(sf[ct][ks], qf[ks], acc[ct]);
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks)
+#pragma unroll
+      for (int i = 0; i < M::KPL; ++i) gsum += vecs[ks * M::KSTEP + lh * M::KPL + i] * M::elem(qf[ks], i);
+  }
+  const typename TM::Coef coef = TM::coef(A.a0, A.a1, 0.0f);
+  for (int jt = 0; jt <= wave; ++jt) {
+    fm_f32x16 s = fm_zero16();
+    const E* krow = Ks + (32 * jt + lr) * PQ + lh * M::KPL;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) s = M::mma(M::load(krow + ks * M::KSTEP), qf[ks], s);
+    frag pb[M::ACC_KSTEPS];
+    // keys past the end of the sequence are zero rows, which the weight a0 would still count: the window ends at n - 1
+    const int last = A.n - 1 - t0 - 32 * jt;
+    const int hi = jt == wave ? (lr < last ? lr : last) : last;
+    gsum += TM::fwd(s, coef, jt == wave || last < 31, 0, hi, lh, pb);
+#pragma unroll
+    for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
+#pragma unroll
+      for (int ct = 0; ct < NT; ++ct) acc[ct] = M::mma(M::load_tr(Vs, PQ, 32 * jt + 16 * ss, 32 * ct, lane), pb[ss], acc[ct]);
+  }
+  FM_SYNC();                                             // the tiles are spent: the output staging lies over them
+  float* Os = reinterpret_cast<float*>(smem);           // [QW][DH + 1]
+  float gt = gsum + fm_shfl_xor(gsum, 32) + A.a0 * float(t0);
+  const float ginv = 1.0f / gt;
+#pragma unroll
+  for (int ct = 0; ct < NT; ++ct)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int c = 32 * ct + fm_acc_row(e, lh);
+      Os[own * (DH + 1) + c] = (acc[ct][e] + vecs[DH + c]) * ginv;
+    }
+  if (lh == 0 && t0 + own < A.n) A.g.base(bh)[int64_t(t0 + own) * A.g.s_n] = gt;
+  FM_SYNC();
+  TIO* ob = A.o.base(bh);
+  for (int c = tid; c < QW * (DH / 8); c += FM_THREADS) {
+    const int row = c / (DH / 8), col = (c % (DH / 8)) * 8;
+    if (t0 + row < A.n) {
+      float v[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = Os[row * (DH + 1) + col + i];
+      IO<TIO>::st8(ob + int64_t(t0 + row) * A.o.s_n + col, A.o.vec != 0, v);
+    }
+  }
+}
+template <int DH> inline size_t fm_o1_fwd_lds() {
+  // two row tiles and the two vectors behind them; the output staging lies over the tiles
+  const size_t tiles = size_t(2) * FM_O1_SEG * (DH + Mma<fm_half>::PAD) * 2 + size_t(2) * DH * 4;
+  return tiles;
+}
+
+// ------------------------------------------------------------------------------
+// k_o1_bwd: dq, dk and dv of one segment.  grid (nseg, bh); wavefront w owns the 32 tokens of tile w for all
+// three.  First the tiles K', V, GH are in LDS (the raw q rows wait in registers): the prefix product and the
+// dense tiles of dq; then Q' takes the place of K' for the dense tiles of dk and dv and the suffix products.
+//   bigq (prefix, slot s: segments < s): slab [c][f] = a1 sum v_c k'_f, the forward's own state; smallq: va = a1 sum k'
+//   bigk (suffix, slot s: segments > s): slab [f][c] = a1 sum q'_f gh_c;  smallk: va = a1 sum c q', vb = a0 sum gh
+// dq contracts the prefix slab over its first index and dv the suffix slab over its first index: a slab is staged
+// in LDS with its rows in `tperm` order and those fragments are transposing reads, so no transposed copy of any
+// state is ever written.
+// ------------------------------------------------------------------------------
+template <typename TIO> struct O1BwdArgs {
+  TRef<const TIO> q, k, v, o, d_o; TRef<const float> g;
+  TRef<TIO> dq, dk, dv;
+  int n, nseg, nslots;
+  const fm_half* bigq; const float* smallq;
+  const fm_half* bigk; const float* smallk;
+  float a0, a1, sc;
+  const float* gpart; int gnblk;                        // see k_grad_scale
+  NormFold q_fold, k_fold;                              // folded normalisation; bq / bk != null: its Jacobian (see TokArgs)
+  float* bq; float* bk;
+};
+
+template <typename TIO, int DH>
+FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
+  typedef fm_half E;
+  typedef TokCfg<E, DH, 1> C;
+  typedef Mma<E> M;
+  typedef TileMath<E> TM;
+  typedef typename M::frag frag;
+  constexpr int NT = C::NT, NKS = C::NKS, QW = C::QW, PQ = C::PQ;
+  FM_DYN_SMEM(smem);
+  E* Ks = reinterpret_cast<E*>(smem);                   // [QW][PQ] each; Q' later lies over K'
+  E* Vs = Ks + QW * PQ;
+  E* Gs = Vs + QW * PQ;
+  E* cs = Gs + QW * PQ;                                  // [QW] c in `tperm` order
+  float* vecs = reinterpret_cast<float*>(cs + QW);       // va of the prefix sums | va, vb of the suffix sums: 3 * DH
+  E* Sl = reinterpret_cast<E*>(vecs + 3 * DH);           // one state slab [DH][PS], rows in `tperm` order
+  E* Qs = Ks;
+  constexpr int PS = C::PS;
+  const int tid = FM_TID_X, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int wave = FM_UNIFORM(tid >> 6);
+  int seg, bh;
+  fm_xcd_map(A.nseg, FM_GDIM_Y, seg, bh);
+  const int t0 = seg * QW;
+  // a state slab (DH x DH, contiguous) as 16-byte chunks, DH / 32 per thread; into LDS with row r at tperm(r)
+  constexpr int SCH = DH * DH / 8, SN = (SCH + FM_THREADS - 1) / FM_THREADS;
+  auto slab_load = [&](const E* src, fm_u32x4* r) {
+#pragma unroll
+    for (int i = 0; i < SN; ++i) {
+      const int c = tid + FM_THREADS * i;
+      if (SCH % FM_THREADS == 0 || c < SCH) r[i] = *reinterpret_cast<const fm_u32x4*>(src + c * 8);
+    }
+  };
+  auto slab_store = [&](const fm_u32x4* r) {
+#pragma unroll
+    for (int i = 0; i < SN; ++i) {
+      const int c = tid + FM_THREADS * i, row = c / (DH / 8), col = (c % (DH / 8)) * 8;
+      if (SCH % FM_THREADS == 0 || c < SCH) *reinterpret_cast<fm_u32x4*>(Sl + M::tperm(row) * PS + col) = r[i];
+    }
+  };
+  // Every load of the workgroup is issued before the first result is used: the five row tiles, the vector sums, the
+  // fragments of the prefix state (this lane's rows of it), then the parts of the gradient scale and of the folds.
+  O1Raw<DH> rq;
+  fm_u32x4 rs[SN];
+  float gsc, qsc, ksc;
+  {
+    O1Raw<DH> rk, rv, rdo, ro;
+    rk.load(A.k, bh, t0, A.n, tid); rv.load(A.v, bh, t0, A.n, tid);
+    rdo.load(A.d_o, bh, t0, A.n, tid); ro.load(A.o, bh, t0, A.n, tid);
+    rq.load(A.q, bh, t0, A.n, tid);
+    float gi[O1Raw<DH>::N];
+#pragma unroll
+    for (int i = 0; i < O1Raw<DH>::N; ++i) {
+      const int row = t0 + O1Raw<DH>::row_of(i, tid);
+      gi[i] = row < A.n ? A.g.base(bh)[int64_t(row) * A.g.s_n] : 1.0f;
+    }
+    float vsum = 0.f;
     if (tid < 3 * DH) {
       // the vector sums of the two states this segment reads (a segment at either end reads zeros instead)
       const bool pre = tid < DH;
       const float* src = (pre ? A.smallq : A.smallk) + (int64_t(bh) * A.nslots + seg) * StateDims<DH>::SMALL + DH * DH +
                          (pre ? tid : tid - DH);
-      vecs[tid] = (pre ? seg > 0 : seg < A.nseg - 1) ? *src : 0.f;
+      if (pre ? seg > 0 : seg < A.nseg - 1) vsum = *src;
     }
-    rq.store(Qs, PQ, tid); rg.store(Gs, PQ, tid); rk.store(Ks, PQ, tid); rv.store(Vs, PQ, tid);
+    slab_load(A.bigq + (int64_t(bh) * A.nslots + (seg > 0 ? seg : 1)) * StateDims<DH>::SLAB, rs);
+    gsc = fm_grad_scale(A.gpart ? A.gpart + int64_t(bh) * A.gnblk : nullptr, A.gnblk, lane);
+    qsc = A.sc * fm_norm_factor(A.q_fold, bh, lane);
+    ksc = A.sc * fm_norm_factor(A.k_fold, bh, lane);
+    if (tid < 3 * DH) vecs[tid] = vsum;
+    slab_store(rs);
+    rk.store(Ks, PQ, tid, ksc);
+    rv.store(Vs, PQ, tid, 1.0f);
+    fm_o1_gh_rows<DH>(rdo, ro, gi, gsc, Gs, PQ, cs, tid);
   }
-  const float gsc = fm_grad_scale(A.gpart ? A.gpart + int64_t(bh) * A.gnblk : nullptr, A.gnblk, lane);
   FM_SYNC();
 
   const int own = wave * 32 + lr;                        // the lane's token inside the segment
-  frag qf[NKS], gf[NKS], kf[NKS], vf[NKS];
+  frag gf[NKS], kf[NKS], vf[NKS];
 #pragma unroll
   for (int ks = 0; ks < NKS; ++ks) {
     const int off = own * PQ + ks * M::KSTEP + lh * M::KPL;
-    qf[ks] = M::load(Qs + off); gf[ks] = M::load(Gs + off); kf[ks] = M::load(Ks + off); vf[ks] = M::load(Vs + off);
+    gf[ks] = M::load(Gs + off); kf[ks] = M::load(Ks + off); vf[ks] = M::load(Vs + off);
   }
   const float ci = float(cs[wave * 32 + M::tperm(lr)]);
   const typename TM::CSplat csp = TM::splat_c(ci);
@@ -83,38 +417,19 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO, E> A) {
   for (int mt = 0; mt < NT; ++mt) { dq[mt] = fm_zero16(); dk[mt] = fm_zero16(); dv[mt] = fm_zero16(); }
   const fm_f32x16 zero = fm_zero16();
 
-  // ---- the sums over the other segments first (their loads have the longest way): fragments straight from
-  // the states, which the L2 holds ----
-  const int frag_off = lr * DH + lh * M::KPL;
+  // the suffix slab travels to registers meanwhile; it takes the prefix slab's place after the first phase
+  slab_load(A.bigk + (int64_t(bh) * A.nslots + (seg < A.nseg - 1 ? seg : 0)) * StateDims<DH>::SLAB, rs);
+  // ---- dq: the keys of the earlier segments: sum_c slab[c][f] gh_c, transposing reads of the staged slab ----
   if (seg > 0) {
-    const E* sq = A.bigq + (int64_t(bh) * A.nslots + seg) * StateDims<DH>::SLAB + frag_off;
 #pragma unroll
     for (int mt = 0; mt < NT; ++mt) {
 #pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) dq[mt] = M::mma(M::load(sq + 32 * mt * DH + ks * M::KSTEP), gf[ks], dq[mt]);
+      for (int ks = 0; ks < NKS; ++ks) dq[mt] = M::mma(M::load_tr(Sl, PS, 16 * ks, 32 * mt, lane), gf[ks], dq[mt]);
 #pragma unroll
       for (int e = 0; e < 16; ++e) dq[mt][e] -= ci * vecs[32 * mt + fm_acc_row(e, lh)];
     }
   }
-  if (seg < A.nseg - 1) {
-    const E* sk = A.bigk + (int64_t(bh) * A.nslots + seg) * StateDims<DH>::SLAB + frag_off;
-    const E* sv = A.bigv + (int64_t(bh) * A.nslots + seg) * StateDims<DH>::SLAB + frag_off;
-#pragma unroll
-    for (int mt = 0; mt < NT; ++mt) {
-#pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) {
-        dk[mt] = M::mma(M::load(sk + 32 * mt * DH + ks * M::KSTEP), vf[ks], dk[mt]);
-        dv[mt] = M::mma(M::load(sv + 32 * mt * DH + ks * M::KSTEP), kf[ks], dv[mt]);
-      }
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int f = 32 * mt + fm_acc_row(e, lh);
-        dk[mt][e] -= vecs[DH + f];
-        dv[mt][e] += vecs[2 * DH + f];
-      }
-    }
-  }
-  // ---- dense tiles: own tokens as queries against the keys at or before them ----
+  // ---- dq: dense tiles, own tokens as queries against the keys at or before them ----
   for (int jt = 0; jt <= wave; ++jt) {
     fm_f32x16 dp = fm_zero16();
     const E* vrow = Vs + (32 * jt + lr) * PQ + lh * M::KPL;
@@ -127,7 +442,11 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO, E> A) {
 #pragma unroll
       for (int mt = 0; mt < NT; ++mt) dq[mt] = M::mma(M::load_tr(Ks, PQ, 32 * jt + 16 * ss, 32 * mt, lane), db[ss], dq[mt]);
   }
-  // ---- dense tiles: own tokens as keys against the queries at or after them ----
+  FM_SYNC();                                             // K' and the prefix slab are spent
+  rq.store(Qs, PQ, tid, qsc);
+  slab_store(rs);
+  FM_SYNC();
+  // ---- dk, dv: dense tiles, own tokens as keys against the queries at or after them ----
   for (int it = wave; it < QW / 32; ++it) {
     fm_f32x16 s = fm_zero16(), dp = fm_zero16();
     const E* qrow = Qs + (32 * it + lr) * PQ + lh * M::KPL;
@@ -149,30 +468,56 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO, E> A) {
         dv[mt] = M::mma(M::load_tr(Gs, PQ, 32 * it + 16 * ss, 32 * mt, lane), pb[ss], dv[mt]);
       }
   }
-  FM_SYNC();                                             // the row tiles are spent: the output staging lies over them
-  // ---- stores, through LDS; with a folded normalisation the Jacobian's pieces as in k_ds ----
-  float* Os = reinterpret_cast<float*>(smem);
-  const int xrow[1] = {own};
+  // ---- dk, dv: the queries of the later segments ----
+  if (seg < A.nseg - 1) {
+#pragma unroll
+    for (int mt = 0; mt < NT; ++mt) {
+      // dk: sum_c slab[f][c] v_c (rows of the staged slab, at their permuted places); dv: sum_f slab[f][c] k'_f
+      const E* srow = Sl + M::tperm(32 * mt + lr) * PS + lh * M::KPL;
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        dk[mt] = M::mma(M::load(srow + ks * M::KSTEP), vf[ks], dk[mt]);
+        dv[mt] = M::mma(M::load_tr(Sl, PS, 16 * ks, 32 * mt, lane), kf[ks], dv[mt]);
+      }
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int f = 32 * mt + fm_acc_row(e, lh);
+        dk[mt][e] -= vecs[DH + f];
+        dv[mt][e] += vecs[2 * DH + f];
+      }
+    }
+  }
+  // ---- stores, through LDS.  With the Jacobian of a folded normalisation (bq / bk): the stored gradient carries
+  // lim / max-norm and the workgroup's part of B = sum dy . y is left for k_norm_fix; the rows y * sc are the tiles
+  // still in LDS (Q', and K' which is written back first) ----
   const float ginv = 1.0f / gsc;
   const int nblk = (A.n + QW - 1) / QW;
+  const int xrow[1] = {own};
+  float* Os = reinterpret_cast<float*>(Vs);              // over V and GH: [QW][DH + 1] floats
+  FM_SYNC();                                             // GH, V and c are spent
   {
     const float fac = A.bq ? fm_norm_factor(A.q_fold, bh, lane) : 1.0f;
     fm_store_tokens<TIO, E, DH, 1>(&dq, xrow, nullptr, A.sc * ginv * fac, Os, A.dq, bh, t0, A.n, tid,
-                                   A.bq ? A.qr + int64_t(bh) * A.npad * DH : nullptr, fac > 0.f ? 1.0f / (fac * A.sc) : 0.f,
-                                   A.bq ? A.bq + int64_t(bh) * nblk + seg : nullptr);
+                                   A.bq ? Qs : nullptr, fac > 0.f ? 1.0f / (fac * A.sc) : 0.f,
+                                   A.bq ? A.bq + int64_t(bh) * nblk + seg : nullptr, PQ, t0);
+  }
+  if (A.bk) {
+    // K' rows back into the tile (from the fragments every lane kept): the Jacobian part of dk needs them
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) *reinterpret_cast<frag*>(Ks + own * PQ + ks * M::KSTEP + lh * M::KPL) = kf[ks];
+    FM_SYNC();
   }
   {
     const float fac = A.bk ? fm_norm_factor(A.k_fold, bh, lane) : 1.0f;
     fm_store_tokens<TIO, E, DH, 1>(&dk, xrow, nullptr, A.sc * ginv * fac, Os, A.dk, bh, t0, A.n, tid,
-                                   A.bk ? A.kr + int64_t(bh) * A.npad * DH : nullptr, fac > 0.f ? 1.0f / (fac * A.sc) : 0.f,
-                                   A.bk ? A.bk + int64_t(bh) * nblk + seg : nullptr);
+                                   A.bk ? Ks : nullptr, fac > 0.f ? 1.0f / (fac * A.sc) : 0.f,
+                                   A.bk ? A.bk + int64_t(bh) * nblk + seg : nullptr, PQ, t0);
   }
   fm_store_tokens<TIO, E, DH, 1>(&dv, xrow, nullptr, ginv, Os, A.dv, bh, t0, A.n, tid);
 }
-
-template <typename E, int DH> inline size_t fm_o1_bwd_lds() {
-  typedef TokCfg<E, DH, 1> C;
-  const size_t tiles = (size_t(4) * C::QW * C::PQ + C::QW) * sizeof(E) + size_t(3) * DH * 4;
-  const size_t outst = size_t(C::QW) * (DH + 1) * 4;
+template <int DH> inline size_t fm_o1_bwd_lds() {
+  const size_t tile = size_t(FM_O1_SEG) * (DH + Mma<fm_half>::PAD) * 2;
+  const size_t tiles = 3 * tile + size_t(FM_O1_SEG) * 2 + size_t(3) * DH * 4 + size_t(DH) * (DH + Mma<fm_half>::PAD) * 2;
+  const size_t outst = tile + size_t(FM_O1_SEG) * (DH + 1) * 4;      // Q' / K' tile kept, staging over V and GH
   return tiles > outst ? tiles : outst;
 }

@@ -91,12 +91,13 @@ FM_DEVICE fm_f32x16 fm_zy(const E* Zs, const typename Mma<E>::frag* tf, int mt, 
 }
 
 // Accumulators (rows = feature, column = token of tile j) -> caller tensor rows, through LDS.
-// brows (optional): compute-type rows [n][DH] of the same tokens; the workgroup's sum over its stored values
-// times those rows, times bscale, goes to *bout (one workgroup-uniform address).
+// brows (optional): compute-type rows of the same tokens (row t at brows + (t - brow0) * bpitch: a copy in
+// memory, or a tile still in LDS); the workgroup's sum over its stored values times those rows, times bscale,
+// goes to *bout (one workgroup-uniform address).
 template <typename TIO, typename E, int DH, int QT>
 FM_DEVICE void fm_store_tokens(fm_f32x16 (*acc)[DH / 32], const int* xrow, const float* addvec, float scale, float* Os,
                                TRef<TIO> out, int bh, int row0, int nrows, int tid, const E* brows = nullptr,
-                               float bscale = 0.f, float* bout = nullptr) {
+                               float bscale = 0.f, float* bout = nullptr, int bpitch = DH, int brow0 = 0) {
   typedef TokCfg<E, DH, QT> C;
   const int lane = tid & 63, lh = lane >> 5;
 #pragma unroll
@@ -118,7 +119,7 @@ FM_DEVICE void fm_store_tokens(fm_f32x16 (*acc)[DH / 32], const int* xrow, const
 #pragma unroll
       for (int i = 0; i < 8; ++i) v[i] = Os[row * (DH + 1) + col + i];
       if (brows) {
-        const E* br = brows + int64_t(row0 + row) * DH + col;
+        const E* br = brows + int64_t(row0 + row - brow0) * bpitch + col;
 #pragma unroll
         for (int i = 0; i < 8; ++i) bsum += v[i] * float(br[i]);
       }
