@@ -361,6 +361,14 @@ def score_function_fastmax(q, k, v, mask=None, denum_term=8, normalize=0, p=1,
         raise ValueError("the oracle covers dropout_rate=0 only")
     if create_attn_matrix:
         tau = denum_term * math.sqrt(q.shape[-1])
+        if torch.is_tensor(mask):
+            # the reference's own reading of `mask` in this branch (``:243-244``): a tensor whose zero
+            # entries are removed, `torch.where(mask == 0, 0, attn)`, before the rows are normalised
+            s = torch.matmul(q, k.transpose(-1, -2)) / tau
+            a = 1 + s + 0.5 * s * s
+            a = torch.where(mask == 0, torch.zeros((), dtype=a.dtype), a)
+            a = a / a.sum(-1, keepdim=True)
+            return torch.matmul(a, v), a
         o, _, a = closed_form_forward(q, k, v, mask=bool(mask is not None and mask), tau=tau,
                                       p=2, return_attn=True)
         return o, a

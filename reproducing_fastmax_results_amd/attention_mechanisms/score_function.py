@@ -258,10 +258,15 @@ fastmax_custom = FASTMultiHeadAttention()
 
 def _attn_matrix(q, k, mask, tau, p):
     """Quadratic debug path (reference ``score_function.py:226-247``): explicit attention
-    matrix in torch; not a hot path."""
+    matrix in torch; not a hot path.  ``mask`` is what the reference takes there, a tensor
+    broadcastable to ``(b, h, nq, nk)`` whose zero entries are removed
+    (``torch.where(mask == 0, 0, attn)``, ``:243-244``); ``True`` is accepted as a shorthand
+    for the lower-triangular mask, ``None`` / ``False`` remove nothing."""
     s = torch.matmul(q.float(), k.float().transpose(-1, -2)) / tau
     f = 1 + s + (0.5 * s * s if p == 2 else 0)
-    if mask:
+    if torch.is_tensor(mask):
+        f = torch.where(mask.to(f.device) == 0, torch.zeros((), dtype=f.dtype, device=f.device), f)
+    elif mask:
         f = f * torch.ones_like(f).tril()
     return f / f.sum(-1, keepdim=True)
 
@@ -275,11 +280,11 @@ def fastmax(q, k, v, mask=None, denum_term=8, normalize=0, p=1, create_attn_matr
     random feature dropout has no seeded counterpart)."""
     if dropout_rate:
         raise NotImplementedError("fastmax: dropout_rate != 0 is not supported by the HIP path")
-    masked = False if mask is None else bool(mask)      # reference: `if mask is None or not mask` -> unmasked
     d = q.shape[-1]
     if create_attn_matrix:
-        a = _attn_matrix(q, k, masked, denum_term * math.sqrt(d), 2)
+        a = _attn_matrix(q, k, mask, denum_term * math.sqrt(d), 2)
         return torch.matmul(a, v.float()).to(q.dtype), a
+    masked = False if mask is None else bool(mask)      # reference: `if mask is None or not mask` -> unmasked
     if normalize == 1:
         q = FastmaxNormalize.apply(q, CENTRE_TOKEN, 1.0)
         k = FastmaxNormalize.apply(k, CENTRE_TOKEN, 1.0)

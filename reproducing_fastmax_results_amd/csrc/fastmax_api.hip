@@ -287,29 +287,14 @@ int launch_build(const BuildArgs<E>& args, int bh, fm_stream_t stream) {
     // MI355X than two values per wavefront at one workgroup per CU (0.092 vs 0.115 ms at
     // B*H = 32, N = 4096, D = 64).
     constexpr int G = DH / 4;
-#ifndef FM_TUNE_QSP
-#define FM_TUNE_QSP 256
-#endif
-#ifndef FM_TUNE_BUILD_TT
-#define FM_TUNE_BUILD_TT 64
-#endif
-    a.seg_parallel = nsteps > 1 && bh * G < FM_TUNE_QSP;
-#ifndef FM_TUNE_BUILD_TT_SMALL
-#define FM_TUNE_BUILD_TT_SMALL 128
-#endif
-#ifndef FM_TUNE_KB_SMALL
-#define FM_TUNE_KB_SMALL 8
-#endif
+    a.seg_parallel = nsteps > 1 && bh * G < 256;
     // the one-workgroup-per-CU variant on _Float16: 128-token tiles, all eight k-steps of fragments requested at once
-    constexpr int TTS = sizeof(E) == 2 ? FM_TUNE_BUILD_TT_SMALL : FM_TUNE_BUILD_TT;
-    constexpr int KBS = sizeof(E) == 2 ? FM_TUNE_KB_SMALL : 4;
-#ifndef FM_TUNE_KB_LARGE
-#define FM_TUNE_KB_LARGE 2
-#endif
+    constexpr int TTS = sizeof(E) == 2 ? 128 : 64;
+    constexpr int KBS = sizeof(E) == 2 ? 8 : 4;
     // at most one workgroup per CU: all the registers are its own, every fragment of a tile is in flight at once
     if (bh * G * (a.seg_parallel ? nsteps : 1) <= 256)
       return launch_build_cfg<E, DH, 1, TTS, (NSMALL + G - 1) / G, KBS>(a, G, bh, nsteps, stream);
-    return launch_build_cfg<E, DH, 1, FM_TUNE_BUILD_TT, (NSMALL + G - 1) / G, FM_TUNE_KB_LARGE>(a, G, bh, nsteps, stream);
+    return launch_build_cfg<E, DH, 1, 64, (NSMALL + G - 1) / G, 2>(a, G, bh, nsteps, stream);
   }
   // Order 1: the sums are a few 32x32 tiles per segment, far too little work per token tile for
   // a staged walk.  One workgroup per (segment, batch*head) sums its segment from fragments loaded

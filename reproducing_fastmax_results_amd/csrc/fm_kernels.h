@@ -1104,15 +1104,6 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_SCAN_THREADS) k_state_scan(E* FM_RESTRICT big
 // tiles only (its transposed fragments come from transposing LDS reads), so 64-token stages cost it
 // no occupancy and halve its barriers (dQ 0.117 -> 0.114 ms at B*H = 32, N = 4096 on MI355X); k_pv
 // measured slower with them (0.092 vs 0.087 ms).
-#ifndef FM_TUNE_KT_PV
-#define FM_TUNE_KT_PV 32
-#endif
-#ifndef FM_TUNE_KT_DS
-#define FM_TUNE_KT_DS 64
-#endif
-#ifndef FM_TUNE_KT_DV
-#define FM_TUNE_KT_DV 64
-#endif
 template <typename E, int DH, int QT>
 struct TokCfg {
   typedef Mma<E> M;
@@ -1128,17 +1119,14 @@ struct TokCfg {
   // _Float16, QT = 2: two tiles per wavefront share every state fragment read from LDS and halve
   // the state bytes staged per token; used by k_ds when there are states to read (dQ + dK
   // 0.20 vs 0.23 ms at the same shape with 1024-token segments).
-#ifndef FM_TUNE_OCC_PV
-#define FM_TUNE_OCC_PV 4
-#endif
-  static constexpr int OCC_PV = sizeof(E) == 2 ? (QT == 1 ? FM_TUNE_OCC_PV : 2) : 1;   // workgroups per CU the kernels are sized for
+  static constexpr int OCC_PV = sizeof(E) == 2 ? (QT == 1 ? 4 : 2) : 1;   // workgroups per CU the kernels are sized for
   static constexpr int OCC_DS = sizeof(E) == 2 ? (QT == 1 ? 3 : 2) : 1;
   static constexpr int SA = sizeof(E) == 2 ? QT : 2;                      // values of a per state slab
-  static constexpr int KT_PV = sizeof(E) == 2 ? FM_TUNE_KT_PV : 64;   // stream tokens per stage of the dense loop, k_pv
-  static constexpr int KT_DS = sizeof(E) == 2 ? FM_TUNE_KT_DS : 64;   //                                           k_ds
+  static constexpr int KT_PV = sizeof(E) == 2 ? 32 : 64;   // stream tokens per stage of the dense loop, k_pv
+  static constexpr int KT_DS = 64;                        //                                           k_ds
   // the dK + dV pass runs two workgroups per CU whatever its stages are, and 64-token stages
   // halve its barriers (0.163 vs 0.173 ms at the shape above)
-  static constexpr int KT_DV = sizeof(E) == 2 ? FM_TUNE_KT_DV : 64;   //                                           k_ds with dV
+  static constexpr int KT_DV = 64;                        //                                           k_ds with dV
   static constexpr int PV_PV = KT_PV + M::PAD;      // pitch of the transposed token tiles
   static constexpr int PV_DS = KT_DS + M::PAD;
   static constexpr int PV_DV = KT_DV + M::PAD;

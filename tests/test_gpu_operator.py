@@ -196,6 +196,22 @@ def test_score_function_front(sf, normalize, mask, p):
         assert rel_err(got, want) < 2e-5      # the fp32 normalisation backward pass on top of the kernels
 
 
+def test_rpe_matrix_structured(sf):
+    """Sinusoidal relative-position table (reference transformer/model.py:230-241): row n - 1 + t holds
+    position -t, row n - 1 - t position +t; checked against the closed form entry by entry."""
+    n, d = 9, 32
+    rpe = sf.rpe_matrix_creator(n, d, DEV, torch.float32, structured=True).cpu()
+    assert rpe.shape == (2 * n - 1, d)
+    for row in range(2 * n - 1):
+        pos = float(n - 1 - row)
+        for c in range(0, d, 2):
+            w = math.exp(-c * math.log(10000.0) / d)
+            assert abs(float(rpe[row, c]) - math.sin(pos * w)) < 1e-5
+            assert abs(float(rpe[row, c + 1]) - math.cos(pos * w)) < 1e-5
+    rnd_rpe = sf.rpe_matrix_creator(n, d, DEV, torch.float32, structured=False, is_zero=False)
+    assert rnd_rpe.shape == (2 * n - 1, d) and float(rnd_rpe.abs().sum()) > 0
+
+
 def test_create_attn_matrix_debug_path(sf):
     q, k, v = (rnd(1, 2, 40, 32, seed=s).to(DEV) for s in (19, 20, 21))
     o, a = sf.fastmax(q, k, v, mask=True, p=2, create_attn_matrix=True)
@@ -203,6 +219,16 @@ def test_create_attn_matrix_debug_path(sf):
     assert torch.allclose(a.sum(-1), torch.ones_like(a.sum(-1)), atol=1e-5)
     o2 = sf.fastmax(q, k, v, mask=True, denum_term=8, p=2)
     assert rel_err(o, o2) < 1e-5
+    # the reference passes the mask of this branch as a tensor (score_function.py:243-244)
+    tril = torch.ones(40, 40, device=DEV).tril()
+    o3, a3 = sf.fastmax(q, k, v, mask=tril, p=2, create_attn_matrix=True)
+    assert torch.equal(a3, a)
+    m = (torch.rand(40, 40, generator=torch.Generator().manual_seed(3)) < 0.5).float()
+    m[:, 0] = 1
+    o4, a4 = sf.fastmax(q, k, v, mask=m.to(DEV), p=2, create_attn_matrix=True)
+    ow, aw = O.score_function_fastmax(q.double().cpu(), k.double().cpu(), v.double().cpu(), mask=m.double(),
+                                      create_attn_matrix=True)
+    assert rel_err(a4, aw) < 1e-5 and rel_err(o4, ow) < 1e-5
 
 
 @pytest.mark.parametrize("centre", [0, 1, 2])

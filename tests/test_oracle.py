@@ -244,3 +244,29 @@ def test_score_function_front():
     o, a = O.score_function_fastmax(q, k, v, mask=None, create_attn_matrix=True)
     assert torch.allclose(a.sum(-1), torch.ones(1, 2, 6, dtype=torch.float64))
     assert torch.allclose(a @ v, o)
+
+
+def test_attn_matrix_tensor_mask():
+    """The debug branch takes the mask as a tensor (reference score_function.py:243-244): a lower-triangular
+    one reproduces the causal closed form, an arbitrary one is checked entry by entry with plain loops."""
+    q, k, v = rnd(1, 2, 6, 4, seed=41), rnd(1, 2, 6, 4, seed=42), rnd(1, 2, 6, 4, seed=43)
+    tril = torch.ones(6, 6).tril()
+    o, a = O.score_function_fastmax(q, k, v, mask=tril, create_attn_matrix=True)
+    o_ref, _ = O.closed_form_forward(q, k, v, mask=True, tau=8 * 2.0, p=2)
+    assert torch.allclose(o, o_ref, atol=1e-12)
+    g = torch.Generator().manual_seed(5)
+    m = (torch.rand(6, 6, generator=g) < 0.6).float()
+    m[:, 0] = 1                                            # no empty row
+    o, a = O.score_function_fastmax(q, k, v, mask=m, create_attn_matrix=True)
+    for h in range(2):
+        for i in range(6):
+            w = []
+            for j in range(6):
+                s = sum(float(q[0, h, i, c]) * float(k[0, h, j, c]) for c in range(4)) / 16.0
+                w.append((1 + s + 0.5 * s * s) if m[i, j] != 0 else 0.0)
+            tot = sum(w)
+            for j in range(6):
+                assert abs(float(a[0, h, i, j]) - w[j] / tot) < 1e-12
+            for c in range(4):
+                want = sum(w[j] * float(v[0, h, j, c]) for j in range(6)) / tot
+                assert abs(float(o[0, h, i, c]) - want) < 1e-12
