@@ -43,11 +43,9 @@ PEAK_HBM_GBS = 8000.0
 # (N, order, dtype, --chunk, kernel).  A constant, not a live measurement: it belongs to the kernels as they
 # were when the named summary was made.
 TRAFFIC = {
-    (4096, 2, "bf16", 0, "dkv"): {"bytes": 115648 * 1024, "source": "profiles/bench_c2_bf16_hbm_traffic.md"},
-    (65536, 1, "bf16", 0, "fwd"): {"bytes": (593327 + 135168) * 1024, "source": "profiles/bench_long_order1_bf16_hbm_traffic.md"},
-    (65536, 1, "bf16", 0, "dq"): {"bytes": (562733 + 131072) * 1024, "source": "profiles/bench_long_order1_bf16_hbm_traffic.md"},
-    (65536, 1, "bf16", 0, "dk"): {"bytes": (601611 + 176955) * 1024, "source": "profiles/bench_long_order1_bf16_hbm_traffic.md"},
-    (65536, 1, "bf16", 0, "dv"): {"bytes": (428990 + 131072) * 1024, "source": "profiles/bench_long_order1_bf16_hbm_traffic.md"},
+    (4096, 2, "bf16", 0, "dkv"): {"bytes": (44173 * 2 + 32770) * 1024, "source": "profiles/c2_bf16_hbm_traffic.md"},
+    (65536, 1, "bf16", 0, "dkv"): {"bytes": (398600 * 2 + 393200) * 1024, "source": "profiles/long_order1_bf16_hbm_traffic.md"},
+    (65536, 2, "bf16", 0, "build"): {"bytes": (209300 * 2 + 982300) * 1024, "source": "profiles/long_order2_bf16_hbm_traffic.md"},
 }
 
 WORKLOAD = dict(name="configs[1]: causal order-2 fwd+bwd", B=4, H=8, N=4096, D=64, p=2, mask=True, scale=1.0)
@@ -327,18 +325,20 @@ def operator_line(lib, dev, W, dtype, args, steps, warmup, full):
         tot, cnt = per_kernel.get(name, (0.0, 0))
         per_kernel[name] = (tot + ms, cnt + 1)
     units = UNITS_STATE if "build" in per_kernel else UNITS_DENSE
-    heavy = {nme: v for nme, v in per_kernel.items() if nme in units}
+    # tensors (bh * N * D elements each) a kernel of an order-1 step has to read and write once
+    k_tensors = {"fwd": 4, "dq": 5, "dk": 5, "dv": 4, "dkv": 8, "build": 2}
+    heavy = {nme: v for nme, v in per_kernel.items() if nme in (k_tensors if p == 1 else units)}
     dominant = max(heavy, key=lambda nme: heavy[nme][0] / heavy[nme][1])
     avg_ms = per_kernel[dominant][0] / per_kernel[dominant][1]
     unit = alg_flops_unit(bh, N, D, p)
-    achieved = units[dominant] * unit / (avg_ms * 1e-3) / 1e12
+    achieved = units.get(dominant, 0) * unit / (avg_ms * 1e-3) / 1e12
     peak = PEAK_TFLOPS[dtype]
     # `achieved` / `frac`: ALGORITHMIC flop of the moment formulation per launch of the dominant kernel (the
     # definition the metric fixes, whatever form the kernel computes in); `executed`: what its matrix
     # instructions actually execute (set below when the kernel runs dense causal tiles only)
     roofline = {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
                 "frac": achieved / peak, "traffic": None, "avg_ms": avg_ms,
-                "algorithmic_flop_per_launch": units[dominant] * unit,
+                "algorithmic_flop_per_launch": units.get(dominant, 0) * unit,
                 "whole_step": {"achieved": 7 * unit / (ms_per_step * 1e-3) / 1e12,
                                "frac": 7 * unit / (ms_per_step * 1e-3) / 1e12 / peak},
                 "kernels_ms_per_step": {nme: tot / nprof for nme, (tot, cnt) in sorted(per_kernel.items())}}
@@ -348,8 +348,7 @@ def operator_line(lib, dev, W, dtype, args, steps, warmup, full):
         # writes dq, dk, dv; per kernel, the tensors it must read and write once.
         esz_io = 2 if dtype == "bf16" else 4
         tensor_b = bh * N * D * esz_io
-        k_tensors = {"fwd": 4, "dq": 5, "dk": 5, "dv": 4, "dkv": 7, "build": 2}
-        dom_b = k_tensors.get(dominant, 4) * tensor_b
+        dom_b = k_tensors[dominant] * tensor_b
         roofline = {"bound": "hbm", "kernel": dominant, "achieved": dom_b / (avg_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
                     "unit": "GB/s", "frac": dom_b / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None, "avg_ms": avg_ms,
                     "whole_step": {"achieved": 12 * tensor_b / (ms_per_step * 1e-3) / 1e9,

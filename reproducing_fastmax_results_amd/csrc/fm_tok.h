@@ -197,7 +197,13 @@ struct TokGeom {
       unit = id % nblk;
       bh = id / nblk;
     }
-    const int blk = A.causal ? fm_block_of_rank<OWN>(unit, nblk, A.L / QW) : unit;
+    // Many segments (a long sequence): the blocks of one segment read the same state, 557 KB at order 2, so
+    // they are launched next to each other and run at the same time: the state comes from HBM once and from
+    // the L2 for the others (ordered by weight, the blocks of a segment ran far apart and each fetched it
+    // again).  With hundreds of blocks per batch*head the dispatcher evens the weights out by itself.
+    const bool seg_major = A.causal && A.use_state && A.nseg >= 8;
+    const int blk = !A.causal ? unit : seg_major ? (OWN == FM_OWN_Q ? nblk - 1 - unit : unit)
+                                                 : fm_block_of_rank<OWN>(unit, nblk, A.L / QW);
     t0 = blk * QW;
     seg = A.causal ? t0 / A.L : 0;
     slot = A.causal ? seg : 0;
