@@ -95,15 +95,16 @@ struct Plan {
   int L, nseg, nslots;
   bool use_state, quad;
   bool rows_build;      // order-1 segment sums read the row-major copies: no transposed copy is written
+  int o1_run;           // order-1 path: segments per run (see k_o1_sums)
   bool o1;              // order 1, causal, _Float16, 128-token segments: the path of fm_o1.h (reads the caller's tensors, no copies)
   bool qf;              // dense _Float16 kernels evaluate the order-2 weights in completed-square form (see TileMath)
   int npad_q, npad_k;
   float a0, a1, a2;     // polynomial on the score s = (q.k) / tau
   float sc;             // sqrt(1/tau), folded into q and k when they are converted
   // workspace offsets (bytes)
-  size_t kt, vt, kr, vr, big, big2, small, fwd_bytes;
+  size_t kt, vt, kr, vr, big, big2, small, run, runh, fwd_bytes;   // run, runh: see k_o1_sums
   bool save;
-  size_t b_kr, b_vr, b_qr, b_kt, b_vt, b_qt, b_qct, b_gh, b_ght, b_cv, b_bigq, b_smallq, b_bigk, b_smallk, b_bigv, b_gpart, b_bq, b_bk, bwd_bytes;
+  size_t b_kr, b_vr, b_qr, b_kt, b_vt, b_qt, b_qct, b_gh, b_ght, b_cv, b_bigq, b_smallq, b_bigk, b_smallk, b_bigv, b_gpart, b_bq, b_bk, b_runq, b_runqh, b_runk, b_runkh, bwd_bytes;
 };
 
 bool strides_ok(const FastmaxStrides& s, int bh, int n, int d) {
@@ -210,6 +211,12 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   p.save = (d->flags & FASTMAX_FLAG_SAVE_FOR_BACKWARD) != 0;
   p.vr = take(p.save || p.half ? tk : 0);      // _Float16: the forward stages v rows (transposing LDS reads)
   p.big2 = take(p.save && !p.o1 ? bigarr : 0);
+  // the order-1 path sums runs of segments: per batch*head and run one fp32 total and its compute-type slab
+  p.o1_run = fm_o1_run_len(p.nseg, d->bh);
+  const size_t nruns = p.o1 ? size_t(fm_o1_runs(p.nseg, p.o1_run)) : 0;
+  const size_t runarr = size_t(d->bh) * nruns * (d->d == 64 ? O1Run<64>::RS : O1Run<32>::RS) * 4;
+  const size_t runharr = size_t(d->bh) * nruns * d->d * d->d * 2;
+  p.run = take(runarr); p.runh = take(runharr);
   p.fwd_bytes = off ? off : 256;
   off = 0;
   p.b_kt = take(tkt); p.b_vt = take(tkt); p.b_qt = take(tqt); p.b_qct = take(tqt);
@@ -224,6 +231,7 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   const bool jac = d->norm.grad != 0;
   p.b_bq = take(jac && d->norm.q_keys ? size_t(d->bh) * ((d->nq + 127) / 128) * 4 : 0);
   p.b_bk = take(jac && d->norm.k_keys ? size_t(d->bh) * ((d->nk + 127) / 128) * 4 : 0);
+  p.b_runq = take(runarr); p.b_runqh = take(runharr); p.b_runk = take(runarr); p.b_runkh = take(runharr);
   p.bwd_bytes = off ? off : 256;
   return FASTMAX_OK;
 }
@@ -383,34 +391,36 @@ int launch_ds(const TokArgs<TIO, E>& a, int bh, int kernel_id, fm_stream_t strea
 }
 
 // ---- order 1 in 128-token segments on the caller's tensors (fm_o1.h) -------------------------
-// Sums of every segment but the last (QG = 0: keys and values, prefix walk) or but the first (QG = 1: queries and
-// gh, suffix walk), then the scan that turns them into prefix / suffix sums.
+// The sums inside every run of segments (QG = 0: keys and values, prefix walk; QG = 1: queries and gh, suffix
+// walk), then the scan over the runs' totals.
 template <typename TIO, int DH, int QG>
-int launch_o1_sums(O1SumArgs<TIO>& a, int bh, fm_stream_t stream) {
-  const int nsteps = a.b.nseg - 1;
-  if (nsteps <= 0) return FASTMAX_OK;
+int launch_o1_sums(O1SumArgs<TIO>& a, fm_half* runhalf, int bh, fm_stream_t stream) {
+  const int nruns = fm_o1_runs(a.b.nseg, a.run_len);
   ProfScope prof(FM_K_BUILD, stream);
   const size_t lds = fm_o1_sums_lds<DH>();
   fm_allow_lds(reinterpret_cast<const void*>(&k_o1_sums<TIO, DH, QG>), lds);
-  FM_KERNEL_LAUNCH((k_o1_sums<TIO, DH, QG>), fm_dim3(1, bh, nsteps), fm_dim3(FM_THREADS), lds, stream, a);
+  FM_KERNEL_LAUNCH((k_o1_sums<TIO, DH, QG>), fm_dim3(1, bh, nruns), fm_dim3(FM_THREADS), lds, stream, a);
   const int st = fm_launch_status();
-  return (st || nsteps < 2) ? st : launch_scan<fm_half, DH>(a.b, bh, nsteps, stream);
+  if (st) return st;
+  FM_KERNEL_LAUNCH((k_o1_runscan<DH>), fm_dim3((O1Run<DH>::RS + FM_THREADS - 1) / FM_THREADS, bh), fm_dim3(FM_THREADS), 0, stream,
+                   a.runtot, runhalf, nruns, a.b.mode == FM_WALK_SUFFIX ? 1 : 0);
+  return fm_launch_status();
 }
 
 // key / value sums of the forward (and of a backward that has no saved forward): big [v][k']
 template <typename TIO, int DH>
 int o1_key_sums(const FastmaxDesc* d, const Plan& p, const void* k, const void* v, fm_half* big, float* small,
-                fm_stream_t stream) {
+                float* runtot, fm_half* runhalf, fm_stream_t stream) {
   O1SumArgs<TIO> a;
   a.x0 = cref<TIO>(k, d->sk); a.x1 = cref<TIO>(v, d->sv); a.o = a.x0; a.g = TRef<const float>{nullptr, 0, 0, 0, 0, 0};
-  a.scale0 = p.sc; a.fold0 = k_fold(d); a.gpart = nullptr; a.gnblk = 0; a.n = d->nk;
+  a.scale0 = p.sc; a.fold0 = k_fold(d); a.gpart = nullptr; a.gnblk = 0; a.n = d->nk; a.runtot = runtot; a.run_len = p.o1_run;
   BuildArgs<fm_half>& b = a.b;
   b.xt = nullptr; b.pt = nullptr; b.rt = nullptr; b.zt = nullptr; b.pr = nullptr; b.rr = nullptr; b.cw = nullptr;
   b.za_sel = FM_SRC_R; b.zb_sel = FM_SRC_R; b.vb_from_r = 0; b.seg_parallel = 1;
   b.npad = p.npad_k; b.nseg = p.nseg; b.L = p.L; b.mode = FM_WALK_PREFIX; b.quad = 0;
   b.big = big; b.big2 = nullptr; b.small = small; b.nslots = p.nslots;
   b.coef2 = 0.f; b.coef2b = 0.f; b.coefz = 0.f; b.coef1 = p.a1; b.coef1b = p.a1; b.coefva = p.a1; b.coefvb = p.a0;
-  return launch_o1_sums<TIO, DH, 0>(a, d->bh, stream);
+  return launch_o1_sums<TIO, DH, 0>(a, runhalf, d->bh, stream);
 }
 
 template <typename TIO, int DH>
@@ -418,12 +428,15 @@ int run_forward_o1(const FastmaxDesc* d, const Plan& p, const void* q, const voi
                    char* ws, fm_stream_t stream) {
   fm_half* big = reinterpret_cast<fm_half*>(ws + p.big);
   float* small = reinterpret_cast<float*>(ws + p.small);
-  int st = o1_key_sums<TIO, DH>(d, p, k, v, big, small, stream);   // the backward reads the same state: nothing else to save
+  float* runtot = reinterpret_cast<float*>(ws + p.run);
+  fm_half* runhalf = reinterpret_cast<fm_half*>(ws + p.runh);
+  int st = o1_key_sums<TIO, DH>(d, p, k, v, big, small, runtot, runhalf, stream);   // the backward reads the same sums: nothing else to save
   if (st) return st;
   O1FwdArgs<TIO> a;
   a.q = cref<TIO>(q, d->sq); a.k = cref<TIO>(k, d->sk); a.v = cref<TIO>(v, d->sv);
   a.o = mref<TIO>(o, d->so); a.g = mref<float>(g, d->sg);
   a.n = d->nq; a.nseg = p.nseg; a.nslots = p.nslots; a.big = big; a.small = small;
+  a.runbig = runhalf; a.runtot = runtot; a.run_len = p.o1_run; a.nruns = fm_o1_runs(p.nseg, p.o1_run);
   a.a0 = p.a0; a.a1 = p.a1; a.sc = p.sc; a.q_fold = q_fold(d); a.k_fold = k_fold(d);
   const size_t lds = fm_o1_fwd_lds<DH>();
   fm_allow_lds(reinterpret_cast<const void*>(&k_o1_fwd<TIO, DH>), lds);

@@ -9,9 +9,9 @@
 //     dv_j  = a0 sum_{i>=j} gh_i + a1 (sum_{i>=j} gh_i q'_i^T) k'_j
 // so a segment needs its own 128 rows, the sums over the segments before it (keys, values) and after it
 // (queries, gh), and nothing else.  Four kernels, one workgroup per segment each:
-//   k_o1_sums<KV>  k, v            -> the segment's sums       (k_state_scan then makes prefix sums)
+//   k_o1_sums<KV>  k, v            -> sums inside runs of segments (k_o1_runscan: sums over whole runs)
 //   k_o1_fwd       q, k, v, prefix -> o, g
-//   k_o1_sums<QG>  q, dO, o, g     -> the segment's sums       (k_state_scan: suffix sums)
+//   k_o1_sums<QG>  q, dO, o, g     -> the same, walking backwards
 //   k_o1_bwd       q, k, v, dO, o, g, prefix, suffix -> dq, dk, dv
 // No converted or transposed copy of any tensor is written: rows are converted (and scaled: 1/tau, the
 // folded normalisation, the gradient scale) in registers on their way into LDS.  The general kernels need a
@@ -95,13 +95,28 @@ FM_DEVICE void fm_o1_gh_rows(const O1Raw<DH>& rdo, const O1Raw<DH>& ro, const fl
 }
 
 // ------------------------------------------------------------------------------
-// k_o1_sums: the sums of one segment.  grid (1, bh, steps): step w of the walk (fm_walk_step) is segment w of
-// a prefix walk, segment nseg - 1 - w of a suffix walk.
-//   QG = 0: operands p = v, r = k':   slab [r][c] = coef1 sum p_r r_c (and its transpose in big2),
-//           va = coefva sum k', vb = coefvb sum v
+// k_o1_sums: the sums over a run of `run_len` consecutive segments, one workgroup per run.  grid (1, bh, runs).
+// A prefix walk takes the run's segments in ascending order, a suffix walk in descending order; before a segment
+// is added, the sums so far go to the segment's slot (the state of the segments before / after it INSIDE its
+// run), and at the end the run's total goes to `runtot`.  k_o1_runscan then turns the totals into the sums over
+// the runs before / after each run; a consumer adds the two.  (Per-segment sums followed by a scan over all
+// segments moved every state three times more and ran the scan on a handful of wavefronts.)
+//   QG = 0: operands p = v, r = k':   slab [r][c] = coef1 sum p_r r_c, va = coefva sum k', vb = coefvb sum v
 //   QG = 1: operands p = q', r = gh:  the same slab, va = coefva sum c q', vb = coefvb sum gh
-// The eight 32x32 tiles of the sums (D = 64) are dealt to the wavefronts as in k_build1_rows.
+// The eight 32x32 tiles of the sums (D = 64) are dealt to the wavefronts, two each; the next segment's rows travel
+// from global memory to registers while this one's products run.
+// A run total (and `runtot` after the scan): DH * DH + 2 * DH floats, the slab, then va, then vb.
 // ------------------------------------------------------------------------------
+template <int DH> struct O1Run { static constexpr int RS = DH * DH + 2 * DH; };
+// Segments per run: enough runs to give every CU two workgroups, runs as long as that allows (measured on
+// MI355X, B*H = 16, 512 segments each: 16 segments per run 0.19 ms for both sums passes of a step, 8: 0.205,
+// 32: 0.215, 64: 0.38).
+inline int fm_o1_run_len(int nseg, int bh) {
+  const int64_t r = int64_t(nseg) * bh / 512;
+  return r < 2 ? 2 : (r > 32 ? 32 : int(r));
+}
+inline int fm_o1_runs(int nseg, int run_len) { return (nseg + run_len - 1) / run_len; }
+
 template <typename TIO> struct O1SumArgs {
   TRef<const TIO> x0, x1;            // QG = 0: k, v          QG = 1: q, dO
   TRef<const TIO> o; TRef<const float> g;     // QG = 1
@@ -109,14 +124,17 @@ template <typename TIO> struct O1SumArgs {
   NormFold fold0;                    // folded normalisation of x0
   const float* gpart; int gnblk;     // QG = 1: see k_grad_scale
   int n;
-  BuildArgs<fm_half> b;              // where the sums go and their coefficients (big, big2, small, nslots, nseg, L, npad, mode, coef*)
+  BuildArgs<fm_half> b;              // where the segments' states go and their coefficients (big, small, nslots = nseg, mode, coef*)
+  float* runtot;                     // [bh][runs][O1Run::RS]
+  int run_len;                       // segments per run
 };
 
 template <typename TIO, int DH, int QG>
-FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_o1_sums(O1SumArgs<TIO> A) {
+FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_sums(O1SumArgs<TIO> A) {
   typedef fm_half E;
   typedef Mma<E> M;
   typedef typename M::frag frag;
+  typedef O1Raw<DH> R;
   constexpr int NT = DH / 32, NTILE = NT * NT + 2 * NT, NS = (NTILE + 3) / 4;
   constexpr int TT = FM_O1_SEG, PQ = DH + M::PAD;
   FM_DYN_SMEM(smem);
@@ -125,64 +143,116 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_o1_sums(O1SumArgs<TIO> A) {
   E* Lc = Lr + TT * PQ;                                // [TT] weights (QG)
   const int tid = FM_TID_X, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   const int wave = FM_UNIFORM(tid >> 6);
-  const int bh = FM_BID_Y;
-  int tb, te, slot;
-  fm_walk_step(A.b.mode, A.b.nseg, A.b.L, A.b.npad, FM_BID_Z, tb, te, slot);
+  const int bh = FM_BID_Y, run = FM_BID_Z, nruns = FM_GDIM_Z;
+  const int s_lo = run * A.run_len, s_hi = s_lo + A.run_len < A.b.nseg ? s_lo + A.run_len : A.b.nseg;
+  const int cnt = s_hi - s_lo;
+  const bool suffix = A.b.mode == FM_WALK_SUFFIX;
   E* big = A.b.big + int64_t(bh) * A.b.nslots * StateDims<DH>::stride(false);
-  E* big2 = A.b.big2 ? A.b.big2 + int64_t(bh) * A.b.nslots * StateDims<DH>::stride(false) : nullptr;
-  float* ds = A.b.small + (int64_t(bh) * A.b.nslots + slot) * StateDims<DH>::SMALL;
-  {
-    O1Raw<DH> r0, r1;
+  float* sml = A.b.small + int64_t(bh) * A.b.nslots * StateDims<DH>::SMALL;
+  R r0, r1, ro;
+  float gi[R::N];
+  auto fetch = [&](int seg) FM_ALWAYS_INLINE {
+    const int tb = seg * TT;
     r0.load(A.x0, bh, tb, A.n, tid);
     r1.load(A.x1, bh, tb, A.n, tid);
-    const float s0 = A.scale0 * fm_norm_factor(A.fold0, bh, lane);
     if (QG) {
-      O1Raw<DH> ro;
       ro.load(A.o, bh, tb, A.n, tid);
-      float gi[O1Raw<DH>::N];
 #pragma unroll
-      for (int i = 0; i < O1Raw<DH>::N; ++i) {
-        const int row = tb + O1Raw<DH>::row_of(i, tid);
+      for (int i = 0; i < R::N; ++i) {
+        const int row = tb + R::row_of(i, tid);
         gi[i] = row < A.n ? A.g.base(bh)[int64_t(row) * A.g.s_n] : 1.0f;
       }
-      const float gscale = fm_grad_scale(A.gpart ? A.gpart + int64_t(bh) * A.gnblk : nullptr, A.gnblk, lane);
+    }
+  };
+  fetch(suffix ? s_hi - 1 : s_lo);
+  const float s0 = A.scale0 * fm_norm_factor(A.fold0, bh, lane);
+  const float gscale = QG ? fm_grad_scale(A.gpart ? A.gpart + int64_t(bh) * A.gnblk : nullptr, A.gnblk, lane) : 1.0f;
+  const frag ones = M::splat(E(1.0f));
+  fm_f32x16 acc[NS];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) acc[s] = fm_zero16();
+  for (int i = 0; i < cnt; ++i) {
+    const int seg = suffix ? s_hi - 1 - i : s_lo + i;
+    FM_SYNC();                                                         // the products of the segment before are done with the tiles
+    if (QG) {
       r0.store(Lp, PQ, tid, s0);                                       // p = q'
       fm_o1_gh_rows<DH>(r1, ro, gi, gscale, Lr, PQ, Lc, tid);          // r = gh, weights c
     } else {
       r1.store(Lp, PQ, tid, 1.0f);                                     // p = v
       r0.store(Lr, PQ, tid, s0);                                       // r = k'
     }
-  }
-  FM_SYNC();
-  // tiles of this wavefront: A operand (tile, feature offset), B operand (tile, or null = weights / ones)
-  const frag ones = M::splat(E(1.0f));
-  fm_f32x16 acc[NS];
+    if (i + 1 < cnt) fetch(suffix ? seg - 1 : seg + 1);
+    FM_SYNC();
+    float* ds = sml + int64_t(seg) * StateDims<DH>::SMALL;
 #pragma unroll
-  for (int s = 0; s < NS; ++s) {
-    acc[s] = fm_zero16();
-    const int t = wave + 4 * s;
-    if (t >= NTILE) continue;
-    const E* ta = Lp; const E* tbt = nullptr;
-    int fa = 0, fb = 0;
-    bool wsum = false;
-    if (t < NT * NT) { fa = 32 * (t / NT); tbt = Lr; fb = 32 * (t % NT); }
-    else if (t < NT * NT + NT) { fa = 32 * (t - NT * NT); if (QG) wsum = true; else ta = Lr; }    // va: sum c q' | sum k'
-    else { fa = 32 * (t - NT * NT - NT); if (QG) ta = Lr; }                                       // vb: sum gh   | sum v
-#pragma unroll 4
-    for (int k = 0; k < TT; k += M::KSTEP) {
-      const frag a = M::load_tr(ta, PQ, k, fa, lane);
-      const frag b = tbt ? M::load_tr(tbt, PQ, k, fb, lane) : (wsum ? M::load_perm(Lc + k, 0, lh) : ones);
-      acc[s] = M::mma(a, b, acc[s]);
-    }
-  }
-#pragma unroll
-  for (int s = 0; s < NS; ++s) {
-    const int t = wave + 4 * s;
-    if (t < NTILE) {
+    for (int s = 0; s < NS; ++s) {
+      const int t = wave + 4 * s;
+      if (t >= NTILE) continue;
+      // the sums of the run so far are this segment's state inside the run
       float v[16];
 #pragma unroll
       for (int e = 0; e < 16; ++e) v[e] = acc[s][e];
-      fm_put_small<E, DH>(A.b, big, big2, ds, slot, t < NT * NT ? t : t + NT * NT, v, lr, lh);
+      fm_put_small<E, DH>(A.b, big, nullptr, ds, seg, t < NT * NT ? t : t + NT * NT, v, lr, lh);
+      // tiles of this wavefront: A operand (tile, feature offset), B operand (tile, or null = weights / ones)
+      const E* ta = Lp; const E* tbt = nullptr;
+      int fa = 0, fb = 0;
+      bool wsum = false;
+      if (t < NT * NT) { fa = 32 * (t / NT); tbt = Lr; fb = 32 * (t % NT); }
+      else if (t < NT * NT + NT) { fa = 32 * (t - NT * NT); if (QG) wsum = true; else ta = Lr; }    // va: sum c q' | sum k'
+      else { fa = 32 * (t - NT * NT - NT); if (QG) ta = Lr; }                                       // vb: sum gh   | sum v
+#pragma unroll 4
+      for (int k = 0; k < TT; k += M::KSTEP) {
+        const frag a = M::load_tr(ta, PQ, k, fa, lane);
+        const frag b = tbt ? M::load_tr(tbt, PQ, k, fb, lane) : (wsum ? M::load_perm(Lc + k, 0, lh) : ones);
+        acc[s] = M::mma(a, b, acc[s]);
+      }
+    }
+  }
+  // the run's total, fp32
+  float* tot = A.runtot + (int64_t(bh) * nruns + run) * O1Run<DH>::RS;
+#pragma unroll
+  for (int s = 0; s < NS; ++s) {
+    const int t = wave + 4 * s;
+    if (t >= NTILE) continue;
+    if (t < NT * NT) {
+      const int rr = 32 * (t / NT), c = 32 * (t % NT) + lr;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) tot[(rr + fm_acc_row(e, lh)) * DH + c] = A.b.coef1 * acc[s][e];
+    } else if (lr == 0) {
+      const bool is_va = t < NT * NT + NT;
+      float* dv = tot + DH * DH + (is_va ? 32 * (t - NT * NT) : DH + 32 * (t - NT * NT - NT));
+      const float cf = is_va ? A.b.coefva : A.b.coefvb;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) dv[fm_acc_row(e, lh)] = cf * acc[s][e];
+    }
+  }
+}
+
+// Run totals -> for every run the sum over the runs before it (prefix) or after it (suffix), in place, and a
+// compute-type copy of the slab part for the consumers' matrix operands.  grid (ceil(RS / 256), bh).
+template <int DH>
+FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_o1_runscan(float* FM_RESTRICT runtot, fm_half* FM_RESTRICT runhalf, int nruns, int suffix) {
+  constexpr int RS = O1Run<DH>::RS, UB = 8;
+  const int e = FM_BID_X * FM_THREADS + FM_TID_X, bh = FM_BID_Y;
+  if (e >= RS) return;
+  float* p = runtot + int64_t(bh) * nruns * RS + e;
+  fm_half* h = runhalf + int64_t(bh) * nruns * DH * DH + e;
+  float sum = 0.f;
+  for (int b0 = 0; b0 < nruns; b0 += UB) {
+    float t[UB];
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+      const int i = b0 + u, r = suffix ? nruns - 1 - i : i;
+      t[u] = i < nruns ? p[int64_t(r) * RS] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+      const int i = b0 + u, r = suffix ? nruns - 1 - i : i;
+      if (i < nruns) {
+        p[int64_t(r) * RS] = sum;
+        if (e < DH * DH) h[int64_t(r) * DH * DH] = CE<fm_half>::from(sum);
+        sum += t[u];
+      }
     }
   }
 }
@@ -190,13 +260,16 @@ template <int DH> inline size_t fm_o1_sums_lds() { return (size_t(2) * FM_O1_SEG
 
 // ------------------------------------------------------------------------------
 // k_o1_fwd: o and g of one segment.  grid (nseg, bh); wavefront w owns the 32 queries of tile w.
-// big: prefix sums, slab [r][c] = a1 sum v_r k'_c; small: va = a1 sum k', vb = a0 sum v (slot s: segments < s).
+// The sums over the keys before the segment are two parts (see k_o1_sums): big / small, slot s: the segments before s
+// inside its run; runbig / runtot, entry s / run_len: the runs before.  Slab [r][c] = a1 sum v_r k'_c, va = a1 sum k',
+// vb = a0 sum v.
 // ------------------------------------------------------------------------------
 template <typename TIO> struct O1FwdArgs {
   TRef<const TIO> q, k, v;
   TRef<TIO> o; TRef<float> g;
   int n, nseg, nslots;
   const fm_half* big; const float* small;
+  const fm_half* runbig; const float* runtot; int nruns, run_len;
   float a0, a1, sc;
   NormFold q_fold, k_fold;
 };
@@ -208,12 +281,13 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 3) k_o1_fwd(O1FwdArgs<TIO> A) {
   typedef Mma<E> M;
   typedef TileMath<E> TM;
   typedef typename M::frag frag;
-  constexpr int NT = C::NT, NKS = C::NKS, QW = C::QW, PQ = C::PQ;
+  constexpr int NT = C::NT, NKS = C::NKS, QW = C::QW, PQ = C::PQ, PS = C::PS;
   static_assert(QW == FM_O1_SEG, "one workgroup per segment");
   FM_DYN_SMEM(smem);
   E* Ks = reinterpret_cast<E*>(smem);                   // [QW][PQ] each; Q' lies in the first tile until its fragments are taken
   E* Vs = Ks + QW * PQ;
   float* vecs = reinterpret_cast<float*>(Vs + QW * PQ);  // va, vb of the prefix sums
+  E* Sl = reinterpret_cast<E*>(vecs + 2 * DH);           // the prefix slab [DH][PS]
   E* Qs = Ks;
   const int tid = FM_TID_X, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   const int wave = FM_UNIFORM(tid >> 6);
@@ -221,21 +295,35 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 3) k_o1_fwd(O1FwdArgs<TIO> A) {
   fm_xcd_map(A.nseg, FM_GDIM_Y, seg, bh);
   const int t0 = seg * QW;
   const int own = wave * 32 + lr;
-  // every load first: the three row tiles, the vector sums, this lane's fragments of the prefix state
+  // every load first: the three row tiles, the vector sums, the two parts of the prefix slab (16-byte chunks)
+  constexpr int SCH = DH * DH / 8, SN = (SCH + FM_THREADS - 1) / FM_THREADS;
   O1Raw<DH> rk, rv;
-  frag sf[NT][NKS];
   {
     O1Raw<DH> rq;
+    frag rs[SN], rs2[SN];
     rq.load(A.q, bh, t0, A.n, tid); rk.load(A.k, bh, t0, A.n, tid); rv.load(A.v, bh, t0, A.n, tid);
+    const int run = seg / A.run_len;
     float vsum = 0.f;
-    if (tid < 2 * DH && seg > 0) vsum = A.small[(int64_t(bh) * A.nslots + seg) * StateDims<DH>::SMALL + DH * DH + tid];
-    const E* sl = A.big + (int64_t(bh) * A.nslots + (seg > 0 ? seg : 1)) * StateDims<DH>::SLAB + lr * DH + lh * M::KPL;
+    if (tid < 2 * DH && seg > 0)
+      vsum = A.small[(int64_t(bh) * A.nslots + seg) * StateDims<DH>::SMALL + DH * DH + tid] +
+             A.runtot[(int64_t(bh) * A.nruns + run) * O1Run<DH>::RS + DH * DH + tid];
+    const E* sl = A.big + (int64_t(bh) * A.nslots + seg) * StateDims<DH>::SLAB;
+    const E* rl = A.runbig + (int64_t(bh) * A.nruns + run) * StateDims<DH>::SLAB;
 #pragma unroll
-    for (int ct = 0; ct < NT; ++ct)
-#pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) sf[ct][ks] = M::load(sl + 32 * ct * DH + ks * M::KSTEP);
+    for (int i = 0; i < SN; ++i) {
+      const int c = tid + FM_THREADS * i;
+      if (SCH % FM_THREADS == 0 || c < SCH) {
+        rs[i] = *reinterpret_cast<const frag*>(sl + c * 8);
+        rs2[i] = *reinterpret_cast<const frag*>(rl + c * 8);
+      }
+    }
     if (tid < 2 * DH) vecs[tid] = vsum;
     rq.store(Qs, PQ, tid, A.sc * fm_norm_factor(A.q_fold, bh, lane));
+#pragma unroll
+    for (int i = 0; i < SN; ++i) {
+      const int c = tid + FM_THREADS * i, row = c / (DH / 8), col = (c % (DH / 8)) * 8;
+      if (SCH % FM_THREADS == 0 || c < SCH) *reinterpret_cast<frag*>(Sl + row * PS + col) = rs[i] + rs2[i];
+    }
   }
   FM_SYNC();
   frag qf[NKS];
@@ -254,7 +342,8 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 3) k_o1_fwd(O1FwdArgs<TIO> A) {
 #pragma unroll
     for (int ct = 0; ct < NT; ++ct)
 #pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) acc[ct] = M::mma(sf[ct][ks], qf[ks], acc[ct]);
+      for (int ks = 0; ks < NKS; ++ks)
+        acc[ct] = M::mma(M::load(Sl + (32 * ct + lr) * PS + ks * M::KSTEP + lh * M::KPL), qf[ks], acc[ct]);
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
@@ -301,8 +390,9 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 3) k_o1_fwd(O1FwdArgs<TIO> A) {
   }
 }
 template <int DH> inline size_t fm_o1_fwd_lds() {
-  // two row tiles and the two vectors behind them; the output staging lies over the tiles
-  const size_t tiles = size_t(2) * FM_O1_SEG * (DH + Mma<fm_half>::PAD) * 2 + size_t(2) * DH * 4;
+  // two row tiles, the two vectors and the prefix slab behind them; the output staging lies over the tiles
+  const size_t tiles = size_t(2) * FM_O1_SEG * (DH + Mma<fm_half>::PAD) * 2 + size_t(2) * DH * 4 +
+                       size_t(DH) * (DH + Mma<fm_half>::PAD) * 2;
   return tiles;
 }
 
@@ -312,6 +402,7 @@ template <int DH> inline size_t fm_o1_fwd_lds() {
 // dense tiles of dq; then Q' takes the place of K' for the dense tiles of dk and dv and the suffix products.
 //   bigq (prefix, slot s: segments < s): slab [c][f] = a1 sum v_c k'_f, the forward's own state; smallq: va = a1 sum k'
 //   bigk (suffix, slot s: segments > s): slab [f][c] = a1 sum q'_f gh_c;  smallk: va = a1 sum c q', vb = a0 sum gh
+// each in two parts, the segments inside the run (big*, small*) and the whole runs (run*, see k_o1_sums), added on load.
 // dq contracts the prefix slab over its first index and dv the suffix slab over its first index: a slab is staged
 // in LDS with its rows in `tperm` order and those fragments are transposing reads, so no transposed copy of any
 // state is ever written.
@@ -322,6 +413,9 @@ template <typename TIO> struct O1BwdArgs {
   int n, nseg, nslots;
   const fm_half* bigq; const float* smallq;
   const fm_half* bigk; const float* smallk;
+  const fm_half* runbigq; const float* runtotq;         // sums over whole runs: before the segment's run (q side) ...
+  const fm_half* runbigk; const float* runtotk;         // ... and after it (k side)
+  int nruns, run_len;
   float a0, a1, sc;
   const float* gpart; int gnblk;                        // see k_grad_scale
   NormFold q_fold, k_fold;                              // folded normalisation; bq / bk != null: its Jacobian (see TokArgs)
@@ -352,25 +446,27 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
   const int t0 = seg * QW;
   // a state slab (DH x DH, contiguous) as 16-byte chunks, DH / 32 per thread; into LDS with row r at tperm(r)
   constexpr int SCH = DH * DH / 8, SN = (SCH + FM_THREADS - 1) / FM_THREADS;
-  auto slab_load = [&](const E* src, fm_u32x4* r) {
+  auto slab_load = [&](const E* src, frag* r) {
 #pragma unroll
     for (int i = 0; i < SN; ++i) {
       const int c = tid + FM_THREADS * i;
-      if (SCH % FM_THREADS == 0 || c < SCH) r[i] = *reinterpret_cast<const fm_u32x4*>(src + c * 8);
+      if (SCH % FM_THREADS == 0 || c < SCH) r[i] = *reinterpret_cast<const frag*>(src + c * 8);
     }
   };
-  auto slab_store = [&](const fm_u32x4* r) {
+  // the two parts of a state, added
+  auto slab_store = [&](const frag* r, const frag* r2) {
 #pragma unroll
     for (int i = 0; i < SN; ++i) {
       const int c = tid + FM_THREADS * i, row = c / (DH / 8), col = (c % (DH / 8)) * 8;
-      if (SCH % FM_THREADS == 0 || c < SCH) *reinterpret_cast<fm_u32x4*>(Sl + M::tperm(row) * PS + col) = r[i];
+      if (SCH % FM_THREADS == 0 || c < SCH) *reinterpret_cast<frag*>(Sl + M::tperm(row) * PS + col) = r[i] + r2[i];
     }
   };
   // Every load of the workgroup is issued before the first result is used: the five row tiles, the vector sums, the
   // fragments of the prefix state (this lane's rows of it), then the parts of the gradient scale and of the folds.
   O1Raw<DH> rq;
-  fm_u32x4 rs[SN];
+  frag rs[SN], rs2[SN];
   float gsc, qsc, ksc;
+  const int run = seg / A.run_len;
   {
     O1Raw<DH> rk, rv, rdo, ro;
     rk.load(A.k, bh, t0, A.n, tid); rv.load(A.v, bh, t0, A.n, tid);
@@ -386,16 +482,18 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
     if (tid < 3 * DH) {
       // the vector sums of the two states this segment reads (a segment at either end reads zeros instead)
       const bool pre = tid < DH;
-      const float* src = (pre ? A.smallq : A.smallk) + (int64_t(bh) * A.nslots + seg) * StateDims<DH>::SMALL + DH * DH +
-                         (pre ? tid : tid - DH);
-      if (pre ? seg > 0 : seg < A.nseg - 1) vsum = *src;
+      const int f = pre ? tid : tid - DH;
+      const float* src = (pre ? A.smallq : A.smallk) + (int64_t(bh) * A.nslots + seg) * StateDims<DH>::SMALL + DH * DH + f;
+      const float* src2 = (pre ? A.runtotq : A.runtotk) + (int64_t(bh) * A.nruns + run) * O1Run<DH>::RS + DH * DH + f;
+      if (pre ? seg > 0 : seg < A.nseg - 1) vsum = *src + *src2;
     }
-    slab_load(A.bigq + (int64_t(bh) * A.nslots + (seg > 0 ? seg : 1)) * StateDims<DH>::SLAB, rs);
+    slab_load(A.bigq + (int64_t(bh) * A.nslots + seg) * StateDims<DH>::SLAB, rs);
+    slab_load(A.runbigq + (int64_t(bh) * A.nruns + run) * StateDims<DH>::SLAB, rs2);
     gsc = fm_grad_scale(A.gpart ? A.gpart + int64_t(bh) * A.gnblk : nullptr, A.gnblk, lane);
     qsc = A.sc * fm_norm_factor(A.q_fold, bh, lane);
     ksc = A.sc * fm_norm_factor(A.k_fold, bh, lane);
     if (tid < 3 * DH) vecs[tid] = vsum;
-    slab_store(rs);
+    slab_store(rs, rs2);
     rk.store(Ks, PQ, tid, ksc);
     rv.store(Vs, PQ, tid, 1.0f);
     fm_o1_gh_rows<DH>(rdo, ro, gi, gsc, Gs, PQ, cs, tid);
@@ -418,7 +516,8 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
   const fm_f32x16 zero = fm_zero16();
 
   // the suffix slab travels to registers meanwhile; it takes the prefix slab's place after the first phase
-  slab_load(A.bigk + (int64_t(bh) * A.nslots + (seg < A.nseg - 1 ? seg : 0)) * StateDims<DH>::SLAB, rs);
+  slab_load(A.bigk + (int64_t(bh) * A.nslots + seg) * StateDims<DH>::SLAB, rs);
+  slab_load(A.runbigk + (int64_t(bh) * A.nruns + run) * StateDims<DH>::SLAB, rs2);
   // ---- dq: the keys of the earlier segments: sum_c slab[c][f] gh_c, transposing reads of the staged slab ----
   if (seg > 0) {
 #pragma unroll
@@ -444,7 +543,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
   }
   FM_SYNC();                                             // K' and the prefix slab are spent
   rq.store(Qs, PQ, tid, qsc);
-  slab_store(rs);
+  slab_store(rs, rs2);
   FM_SYNC();
   // ---- dk, dv: dense tiles, own tokens as keys against the queries at or after them ----
   for (int it = wave; it < QW / 32; ++it) {

@@ -43,6 +43,7 @@ typedef hostsim::Dim3 fm_dim3;
 #define FM_BID_Z (int(hostsim::g_t.bid.z))
 #define FM_GDIM_X (int(hostsim::g_t.gdim.x))
 #define FM_GDIM_Y (int(hostsim::g_t.gdim.y))
+#define FM_GDIM_Z (int(hostsim::g_t.gdim.z))
 #define FM_SYNC() hostsim::syncthreads()
 #define FM_DYN_SMEM(name) unsigned char* name = hostsim::g_t.blk->dyn_smem
 #define FM_KERNEL_LAUNCH(kern, grid, block, smem, stream, ...) \
@@ -120,6 +121,7 @@ typedef dim3 fm_dim3;
 #define FM_BID_Z (int(blockIdx.z))
 #define FM_GDIM_X (int(gridDim.x))
 #define FM_GDIM_Y (int(gridDim.y))
+#define FM_GDIM_Z (int(gridDim.z))
 #define FM_SYNC() __syncthreads()
 #define FM_DYN_SMEM(name) extern __shared__ __align__(16) unsigned char name[]
 // A launch the runtime refuses leaves its error as the calling thread's last error.  Only an error that
