@@ -75,6 +75,28 @@ struct TileRegs {
       }
     }
   }
+  // one chunk of the thread at a time (tiles of a whole number of chunks per thread)
+  FM_DEVICE void load_part(const E* src, int row_stride, int tid, int i) {
+    static_assert(TOTAL % FM_THREADS == 0 || TOTAL <= FM_THREADS, "whole chunks per thread");
+    const int c = TOTAL <= FM_THREADS ? tid % TOTAL : tid + FM_THREADS * i;
+    r[i] = *reinterpret_cast<const fm_u32x4*>(src + uint32_t(c / CPR) * uint32_t(row_stride) + uint32_t((c % CPR) * VEC));
+  }
+  FM_DEVICE void store_part(E* lds, int pitch, int tid, int i) const {
+    const int c = TOTAL <= FM_THREADS ? tid % TOTAL : tid + FM_THREADS * i;
+    *reinterpret_cast<fm_u32x4*>(lds + (c / CPR) * pitch + (c % CPR) * VEC) = r[i];
+  }
+  // The same without a branch, for a tile of fewer chunks than threads: the surplus threads repeat the work of the
+  // first ones (same addresses, same data), so the instructions can be scheduled among others.
+  FM_DEVICE void load_wrapped(const E* src, int row_stride, int tid) {
+    static_assert(N == 1 && TOTAL <= FM_THREADS, "a tile of at most one chunk per thread");
+    const int c = tid % TOTAL;
+    r[0] = *reinterpret_cast<const fm_u32x4*>(src + uint32_t(c / CPR) * uint32_t(row_stride) + uint32_t((c % CPR) * VEC));
+  }
+  FM_DEVICE void store_wrapped(E* lds, int pitch, int tid) const {
+    static_assert(N == 1 && TOTAL <= FM_THREADS, "a tile of at most one chunk per thread");
+    const int c = tid % TOTAL;
+    *reinterpret_cast<fm_u32x4*>(lds + (c / CPR) * pitch + (c % CPR) * VEC) = r[0];
+  }
 };
 
 // Rows of a caller tensor (interface type, strided, bounds-checked) -> LDS in the
@@ -586,9 +608,214 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <
       for (int k = 0; k < NT; ++k) acc[i][j][k] = fm_zero16();
 #pragma unroll
   for (int s = 0; s < SPW; ++s) sacc[s] = fm_zero16();
+  // _Float16 walk that has the CU to itself: two LDS buffers of token tiles (see below)
+  constexpr bool DB = sizeof(E) == 2 && KB >= 4;
   fetch(R0, pf);
   advance(pf);
-  if (pf.valid) { fetch(R1, pf); advance(pf); }
+  if (!DB && pf.valid) { fetch(R1, pf); advance(pf); }
+  // End of a segment: the snapshot of the order-2 slice and the reduced lower-order tiles go to the state of `slot`.
+  // mem: LDS that no wavefront reads any more once all of them have arrived here (staging for the stores).
+  auto finish_segment = [&](int slot, unsigned char* mem) FM_ALWAYS_INLINE {
+#if !defined(FM_HOSTSIM)
+    // The accumulators live in the accumulation registers while the products run; without this the
+    // compiler copies all of them to vector registers at the end of every tile, ahead of this branch.
+#pragma unroll
+    for (int i = 0; i < NA; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int k = 0; k < NT; ++k)
+          if (sizeof(E) == 2 && KB >= 4) asm volatile("" : "+a"(acc[i][j][k]));    // the one-workgroup-per-CU variant
+#endif
+    if (quad) {
+      // snapshot through LDS (the token tiles are spent): accumulators -> staged tiles ->
+      // coalesced 16-byte stores; a second pass writes the transposed tiles
+      constexpr int SP = DH + M::PAD;
+      constexpr int VEC = M::VEC;
+      E* stg = reinterpret_cast<E*>(mem);                  // [AW][DH][SP]
+      FM_SYNC();
+#pragma unroll
+      for (int i = 0; i < NA; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+          for (int k = 0; k < NT; ++k)
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+              stg[((wave * NA + i) * DH + 32 * j + fm_acc_row(e, lh)) * SP + 32 * k + lr] =
+                  CE<E>::from(A.coef2 * acc[i][j][k][e]);
+      FM_SYNC();
+      E* dst = big + int64_t(slot) * StateDims<DH>::BIG + int64_t(a0) * DH * DH;
+      for (int c = tid; c < AW * DH * (DH / VEC); c += FM_THREADS) {
+        const int row = c / (DH / VEC), col = (c % (DH / VEC)) * VEC;
+        *reinterpret_cast<fm_u32x4*>(dst + row * DH + col) = *reinterpret_cast<const fm_u32x4*>(stg + row * SP + col);
+      }
+      if (big2) {
+        FM_SYNC();
+#pragma unroll
+        for (int i = 0; i < NA; ++i)
+#pragma unroll
+          for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int k = 0; k < NT; ++k)
+#pragma unroll
+              for (int e = 0; e < 16; ++e)
+                stg[((wave * NA + i) * DH + 32 * k + lr) * SP + 32 * j + fm_acc_row(e, lh)] =
+                    CE<E>::from(A.coef2b * acc[i][j][k][e]);
+        FM_SYNC();
+        E* dst2 = big2 + int64_t(slot) * StateDims<DH>::BIG + int64_t(a0) * DH * DH;
+        for (int c = tid; c < AW * DH * (DH / VEC); c += FM_THREADS) {
+          const int row = c / (DH / VEC), col = (c % (DH / VEC)) * VEC;
+          *reinterpret_cast<fm_u32x4*>(dst2 + row * DH + col) = *reinterpret_cast<const fm_u32x4*>(stg + row * SP + col);
+        }
+      }
+    }
+    // reduce the four wavefronts' partial lower-order tiles through LDS (the token tiles are
+    // spent), RC tiles per pass: every wavefront stores its part of each, then wavefront u adds
+    // the four parts of tile u and writes it
+    constexpr int RC = SPW < 4 ? SPW : 4;
+    float* red = reinterpret_cast<float*>(mem);            // [RC][4 waves][16][64 lanes]
+    float* ds = sml + int64_t(slot) * StateDims<DH>::SMALL;
+#pragma unroll
+    for (int sb = 0; sb < SPW; sb += RC) {
+      FM_SYNC();
+#pragma unroll
+      for (int u = 0; u < RC; ++u)
+        if (sb + u < SPW) {
+#pragma unroll
+          for (int e = 0; e < 16; ++e) red[((u * 4 + wave) * 16 + e) * 64 + lane] = sacc[sb + u][e];
+        }
+      FM_SYNC();
+      const int tl = grp + (sb + wave) * G;
+      if (wave < RC && sb + wave < SPW && tl < NSMALL && (quad || tl < NT * NT || tl >= 2 * NT * NT)) {
+        float v[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          v[e] = red[((wave * 4 + 0) * 16 + e) * 64 + lane] + red[((wave * 4 + 1) * 16 + e) * 64 + lane] +
+                 red[((wave * 4 + 2) * 16 + e) * 64 + lane] + red[((wave * 4 + 3) * 16 + e) * 64 + lane];
+        fm_put_small<E, DH>(A, big, big2, ds, slot, tl, v, lr, lh);
+      }
+    }
+  };
+  if constexpr (DB) {
+    // Measured with cycle counters around the phases of the single-buffered loop below (one wavefront per SIMD, so
+    // nothing else runs meanwhile): of 4100 cycles per 128-token tile the products and their fragment reads took 40 %,
+    // the stores of the next tile into LDS 12 %, issuing its global loads 12 %, the lower-order tiles 8 %, the two
+    // barriers and the loop 12 %, the snapshots 16 % -- one after the other.  Here the token tiles have two LDS buffers
+    // and two register sets: the stores of tile t + 1 (other buffer) and the global loads of tile t + 2 (other
+    // registers) depend on nothing the products of tile t touch, the whole tile is one branch-free block, and the
+    // scheduler is told to issue one store or load behind each matrix instruction; one barrier per tile is left.
+    static_assert(KB == NSTEP, "all fragments of a tile are requested at once");
+    constexpr int TILE_E = (3 * DH + AW) * PT;                 // elements of one buffer: p, r, x, third operand
+    unsigned char* const stage_mem = smem + size_t(2) * TILE_E * sizeof(E);
+    auto walk = [&](auto hz_tag) FM_ALWAYS_INLINE {
+      constexpr bool HZ = decltype(hz_tag)::value;
+      // tile 0 -> buffer 0; tile 1 -> R1
+      R0.p.store(s0, PT, tid); R0.r.store(s1, PT, tid); R0.x.store(s2, PT, tid);
+      if (HZ) R0.z.store(s3, PT, tid);
+      auto fetch_next = [&](Regs& R) FM_ALWAYS_INLINE {
+        // the tile `pf` names, or (nothing left to load) the current one again: same instructions either way
+        const int t = pf.valid ? pf.t : cur.t;
+        R.p.load(A.pt + tb_off + t, A.npad, tid);
+        R.r.load(A.rt + tb_off + t, A.npad, tid);
+        R.x.load_wrapped(A.xt + tb_off + int64_t(a0) * A.npad + t, A.npad, tid);
+        if (HZ) R.z.load(A.zt + tb_off + t, A.npad, tid);
+      };
+      fetch_next(R1);
+      if (pf.valid) advance(pf);
+      FM_SYNC();
+      // items of a tile: chunk i of p, of r, the x chunk, chunk i of the third operand
+      constexpr int NP = TileRegs<E, DH, TT>::N, NITEM = 2 * NP + 1 + (HZ ? NP : 0);
+      auto body = [&](const Regs& Rs, Regs& Rf, E* cb, E* nb) FM_ALWAYS_INLINE {
+        const E* pb_ = cb + lr * PT + lh * M::KPL;
+        const E* rb_ = cb + DH * PT + lr * PT + lh * M::KPL;
+        const E* xb_ = cb + 2 * DH * PT + (wave * NA) * PT + lh * M::KPL;
+        const int tn = pf.valid ? pf.t : cur.t;     // the tile to load: the one `pf` names, or (none left) the current one again
+        frag fb[KB][NT], fp[KB][NT], fx[KB][NA];
+        // The fragments of three k-steps are requested ahead of their products (the counter a wavefront waits on
+        // for LDS ends at 15 outstanding operations: with all 40 reads of a tile in flight the first product would
+        // wait for 26 of them).
+        constexpr int AHEAD = 3;
+        auto frags = [&](int u) FM_ALWAYS_INLINE {
+#pragma unroll
+          for (int i = 0; i < NA; ++i) fx[u][i] = M::load(xb_ + i * PT + u * M::KSTEP);
+#pragma unroll
+          for (int j = 0; j < NT; ++j) {
+            fp[u][j] = M::load(pb_ + 32 * j * PT + u * M::KSTEP);
+            fb[u][j] = M::load(rb_ + 32 * j * PT + u * M::KSTEP);
+          }
+        };
+#pragma unroll
+        for (int u = 0; u < AHEAD; ++u) frags(u);
+#pragma unroll
+        for (int u = 0; u < KB; ++u) {
+#if !defined(FM_HOSTSIM)
+          __builtin_amdgcn_sched_barrier(0);       // the reads, stores and loads below stay with the products of their k-step
+#endif
+          if (u + AHEAD < KB) frags(u + AHEAD);
+#pragma unroll
+          for (int i = 0; i < NA; ++i)
+#pragma unroll
+            for (int j = 0; j < NT; ++j) {
+              const frag fa = fp[u][j] * fx[u][i];
+#pragma unroll
+              for (int k = 0; k < NT; ++k) acc[i][j][k] = M::mma(fa, fb[u][k], acc[i][j][k]);
+            }
+          // this k-step's share of the next tile's stores (registers -> other buffer) and of the loads of the tile after it
+#pragma unroll
+          for (int it = u * NITEM / KB; it < (u + 1) * NITEM / KB; ++it) {
+            if (it < NP) {
+              Rs.p.store_part(nb, PT, tid, it);
+              Rf.p.load_part(A.pt + tb_off + tn, A.npad, tid, it);
+            } else if (it < 2 * NP) {
+              Rs.r.store_part(nb + DH * PT, PT, tid, it - NP);
+              Rf.r.load_part(A.rt + tb_off + tn, A.npad, tid, it - NP);
+            } else if (it == 2 * NP) {
+              Rs.x.store_part(nb + 2 * DH * PT, PT, tid, 0);
+              Rf.x.load_part(A.xt + tb_off + int64_t(a0) * A.npad + tn, A.npad, tid, 0);
+            } else {
+              Rs.z.store_part(nb + (2 * DH + AW) * PT, PT, tid, it - 2 * NP - 1);
+              Rf.z.load_part(A.zt + tb_off + tn, A.npad, tid, it - 2 * NP - 1);
+            }
+          }
+        }
+#if !defined(FM_HOSTSIM)
+        __builtin_amdgcn_sched_barrier(0);
+#endif
+      };
+      auto tail = [&](const E* cb) FM_ALWAYS_INLINE {
+        // the lower-order tiles: this wavefront takes the k-steps ks = wave (mod 4)
+#pragma unroll
+        for (int s = 0; s < SPW; ++s) {
+          if (sm_id[s] >= 0) {
+            for (int ks = wave; ks < NSTEP; ks += 4) {
+              const frag fa = M::load(cb + sm_a[s] + ks * M::KSTEP);
+              const frag fo = sm_b[s] >= 0 ? M::load(cb + sm_b[s] + ks * M::KSTEP) : M::splat(E(1.0f));
+              sacc[s] = M::mma(fa, fo, sacc[s]);
+            }
+          }
+        }
+        const bool last = cur.t + TT >= cur.te;
+        if (last) finish_segment(cur.slot, stage_mem);
+        advance(cur);
+        if (pf.valid) advance(pf);
+      };
+      E* const b0 = s0;
+      E* const b1 = s0 + TILE_E;
+      while (true) {
+        body(R1, R0, b0, b1);
+        tail(b0);
+        if (!cur.valid) break;
+        FM_SYNC();
+        body(R0, R1, b1, b0);
+        tail(b1);
+        if (!cur.valid) break;
+        FM_SYNC();
+      }
+    };
+    if (has_z) walk(std::true_type()); else walk(std::false_type());
+    return;
+  }
   auto stage = [&](Regs& R) FM_ALWAYS_INLINE {
     FM_SYNC();
     R.p.store(s0, PT, tid); R.r.store(s1, PT, tid);
@@ -674,88 +901,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <
         }
       }
     }
-    if (last) {
-#if !defined(FM_HOSTSIM)
-      // The accumulators live in the accumulation registers while the products run; without this the
-      // compiler copies all of them to vector registers at the end of every tile, ahead of this branch.
-#pragma unroll
-      for (int i = 0; i < NA; ++i)
-#pragma unroll
-        for (int j = 0; j < NT; ++j)
-#pragma unroll
-          for (int k = 0; k < NT; ++k)
-            if (sizeof(E) == 2 && KB >= 4) asm volatile("" : "+a"(acc[i][j][k]));    // the one-workgroup-per-CU variant
-#endif
-      if (quad) {
-        // snapshot through LDS (the token tiles are spent): accumulators -> staged tiles ->
-        // coalesced 16-byte stores; a second pass writes the transposed tiles
-        constexpr int SP = DH + M::PAD;
-        constexpr int VEC = M::VEC;
-        E* stg = reinterpret_cast<E*>(smem);                 // [AW][DH][SP]
-        FM_SYNC();
-#pragma unroll
-        for (int i = 0; i < NA; ++i)
-#pragma unroll
-          for (int j = 0; j < NT; ++j)
-#pragma unroll
-            for (int k = 0; k < NT; ++k)
-#pragma unroll
-              for (int e = 0; e < 16; ++e)
-                stg[((wave * NA + i) * DH + 32 * j + fm_acc_row(e, lh)) * SP + 32 * k + lr] =
-                    CE<E>::from(A.coef2 * acc[i][j][k][e]);
-        FM_SYNC();
-        E* dst = big + int64_t(slot) * StateDims<DH>::BIG + int64_t(a0) * DH * DH;
-        for (int c = tid; c < AW * DH * (DH / VEC); c += FM_THREADS) {
-          const int row = c / (DH / VEC), col = (c % (DH / VEC)) * VEC;
-          *reinterpret_cast<fm_u32x4*>(dst + row * DH + col) = *reinterpret_cast<const fm_u32x4*>(stg + row * SP + col);
-        }
-        if (big2) {
-          FM_SYNC();
-#pragma unroll
-          for (int i = 0; i < NA; ++i)
-#pragma unroll
-            for (int j = 0; j < NT; ++j)
-#pragma unroll
-              for (int k = 0; k < NT; ++k)
-#pragma unroll
-                for (int e = 0; e < 16; ++e)
-                  stg[((wave * NA + i) * DH + 32 * k + lr) * SP + 32 * j + fm_acc_row(e, lh)] =
-                      CE<E>::from(A.coef2b * acc[i][j][k][e]);
-          FM_SYNC();
-          E* dst2 = big2 + int64_t(slot) * StateDims<DH>::BIG + int64_t(a0) * DH * DH;
-          for (int c = tid; c < AW * DH * (DH / VEC); c += FM_THREADS) {
-            const int row = c / (DH / VEC), col = (c % (DH / VEC)) * VEC;
-            *reinterpret_cast<fm_u32x4*>(dst2 + row * DH + col) = *reinterpret_cast<const fm_u32x4*>(stg + row * SP + col);
-          }
-        }
-      }
-      // reduce the four wavefronts' partial lower-order tiles through LDS (the token tiles are
-      // spent), RC tiles per pass: every wavefront stores its part of each, then wavefront u adds
-      // the four parts of tile u and writes it
-      constexpr int RC = SPW < 4 ? SPW : 4;
-      float* red = reinterpret_cast<float*>(smem);           // [RC][4 waves][16][64 lanes]
-      float* ds = sml + int64_t(slot) * StateDims<DH>::SMALL;
-#pragma unroll
-      for (int sb = 0; sb < SPW; sb += RC) {
-        FM_SYNC();
-#pragma unroll
-        for (int u = 0; u < RC; ++u)
-          if (sb + u < SPW) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) red[((u * 4 + wave) * 16 + e) * 64 + lane] = sacc[sb + u][e];
-          }
-        FM_SYNC();
-        const int tl = grp + (sb + wave) * G;
-        if (wave < RC && sb + wave < SPW && tl < NSMALL && (quad || tl < NT * NT || tl >= 2 * NT * NT)) {
-          float v[16];
-#pragma unroll
-          for (int e = 0; e < 16; ++e)
-            v[e] = red[((wave * 4 + 0) * 16 + e) * 64 + lane] + red[((wave * 4 + 1) * 16 + e) * 64 + lane] +
-                   red[((wave * 4 + 2) * 16 + e) * 64 + lane] + red[((wave * 4 + 3) * 16 + e) * 64 + lane];
-          fm_put_small<E, DH>(A, big, big2, ds, slot, tl, v, lr, lh);
-        }
-      }
-    }
+    if (last) finish_segment(slot, smem);
     advance(cur);
   };
   while (true) {
