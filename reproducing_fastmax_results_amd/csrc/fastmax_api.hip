@@ -275,7 +275,7 @@ int launch_build_cfg(const BuildArgs<E>& a, int groups, int bh, int nsteps, fm_s
   if (lds < red) lds = red;
   if (lds < snap) lds = snap;
   // the _Float16 walk with a CU to itself keeps two buffers of token tiles and stages its stores behind them
-  if (sizeof(E) == 2 && KB >= 4) lds = 2 * size_t(3 * DH + AW) * PT * sizeof(E) + (red > snap ? red : snap);
+  if (sizeof(E) == 2 && KB >= 4) lds = 2 * size_t(3 * DH + AW) * PT * sizeof(E) + (red > snap ? red : snap) + 16;   // + eight ones
   fm_allow_lds(reinterpret_cast<const void*>(&k_build<E, DH, NA, TT, SPW, KB>), lds);
   FM_KERNEL_LAUNCH((k_build<E, DH, NA, TT, SPW, KB>), fm_dim3(groups, bh, a.seg_parallel ? nsteps : 1),
                    fm_dim3(FM_THREADS), lds, stream, a);

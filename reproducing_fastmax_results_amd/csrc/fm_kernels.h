@@ -708,6 +708,8 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <
     static_assert(KB == NSTEP, "all fragments of a tile are requested at once");
     constexpr int TILE_E = (3 * DH + AW) * PT;                 // elements of one buffer: p, r, x, third operand
     unsigned char* const stage_mem = smem + size_t(2) * TILE_E * sizeof(E);
+    constexpr size_t RED_BYTES = size_t(SPW < 4 ? SPW : 4) * 4 * 64 * 16 * 4, SNAP_BYTES = size_t(AW) * DH * (DH + M::PAD) * sizeof(E);
+    constexpr size_t STAGE_BYTES = RED_BYTES > SNAP_BYTES ? RED_BYTES : SNAP_BYTES;
     auto walk = [&](auto hz_tag) FM_ALWAYS_INLINE {
       constexpr bool HZ = decltype(hz_tag)::value;
       // tile 0 -> buffer 0; tile 1 -> R1
@@ -723,6 +725,9 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <
       };
       fetch_next(R1);
       if (pf.valid) advance(pf);
+      // eight ones for the lower-order tiles whose second operand is a column of ones: a fragment like any other
+      E* const ones_lds = reinterpret_cast<E*>(stage_mem + STAGE_BYTES);
+      if (tid < 8) ones_lds[tid] = E(1.0f);
       FM_SYNC();
       // items of a tile: chunk i of p, of r, the x chunk, chunk i of the third operand
       constexpr int NP = TileRegs<E, DH, TT>::N, NITEM = 2 * NP + 1 + (HZ ? NP : 0);
@@ -747,12 +752,26 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <
         };
 #pragma unroll
         for (int u = 0; u < AHEAD; ++u) frags(u);
+        // the lower-order tiles: this wavefront takes the k-steps wave and wave + 4; their fragments travel with the
+        // others (a tile that does not exist for this workgroup is computed on valid operands and never stored)
+        constexpr int SK = NSTEP / 4;
+        frag sa[SPW][SK], sb[SPW][SK];
 #pragma unroll
         for (int u = 0; u < KB; ++u) {
 #if !defined(FM_HOSTSIM)
           __builtin_amdgcn_sched_barrier(0);       // the reads, stores and loads below stay with the products of their k-step
 #endif
           if (u + AHEAD < KB) frags(u + AHEAD);
+          if (u == KB - AHEAD) {
+#pragma unroll
+            for (int s = 0; s < SPW; ++s)
+#pragma unroll
+              for (int q = 0; q < SK; ++q) {
+                const int ks = wave + 4 * q;
+                sa[s][q] = M::load(cb + sm_a[s] + ks * M::KSTEP);
+                sb[s][q] = M::load(sm_b[s] >= 0 ? cb + sm_b[s] + ks * M::KSTEP : ones_lds);
+              }
+          }
 #pragma unroll
           for (int i = 0; i < NA; ++i)
 #pragma unroll
@@ -779,22 +798,15 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <
             }
           }
         }
+#pragma unroll
+        for (int s = 0; s < SPW; ++s)
+#pragma unroll
+          for (int q = 0; q < SK; ++q) sacc[s] = M::mma(sa[s][q], sb[s][q], sacc[s]);
 #if !defined(FM_HOSTSIM)
         __builtin_amdgcn_sched_barrier(0);
 #endif
       };
-      auto tail = [&](const E* cb) FM_ALWAYS_INLINE {
-        // the lower-order tiles: this wavefront takes the k-steps ks = wave (mod 4)
-#pragma unroll
-        for (int s = 0; s < SPW; ++s) {
-          if (sm_id[s] >= 0) {
-            for (int ks = wave; ks < NSTEP; ks += 4) {
-              const frag fa = M::load(cb + sm_a[s] + ks * M::KSTEP);
-              const frag fo = sm_b[s] >= 0 ? M::load(cb + sm_b[s] + ks * M::KSTEP) : M::splat(E(1.0f));
-              sacc[s] = M::mma(fa, fo, sacc[s]);
-            }
-          }
-        }
+      auto tail = [&](const E*) FM_ALWAYS_INLINE {
         const bool last = cur.t + TT >= cur.te;
         if (last) finish_segment(cur.slot, stage_mem);
         advance(cur);
