@@ -43,9 +43,10 @@ PEAK_HBM_GBS = 8000.0
 # (N, order, dtype, --chunk, kernel).  A constant, not a live measurement: it belongs to the kernels as they
 # were when the named summary was made.
 TRAFFIC = {
-    (4096, 2, "bf16", 0, "dkv"): {"bytes": (44173 * 2 + 32770) * 1024, "source": "profiles/c2_bf16_hbm_traffic.md"},
-    (65536, 1, "bf16", 0, "dkv"): {"bytes": (398600 * 2 + 393200) * 1024, "source": "profiles/long_order1_bf16_hbm_traffic.md"},
-    (65536, 2, "bf16", 0, "build"): {"bytes": (209300 * 2 + 982300) * 1024, "source": "profiles/long_order2_bf16_hbm_traffic.md"},
+    (4096, 2, "bf16", 0, "dkv"): {"bytes": (44092 * 2 + 32770) * 1024, "source": "profiles/c2_bf16_hbm_traffic.md"},
+    (65536, 1, "bf16", 0, "dkv"): {"bytes": (402970 * 2 + 393240) * 1024, "source": "profiles/long_order1_bf16_hbm_traffic.md"},
+    (65536, 2, "bf16", 0, "build"): {"bytes": (161374 * 2 + 982214) * 1024, "source": "profiles/long_order2_bf16_hbm_traffic.md"},
+    (65536, 2, "bf16", 0, "dk"): {"bytes": (619174 * 2 + 199579) * 1024, "source": "profiles/long_order2_bf16_hbm_traffic.md"},
 }
 
 WORKLOAD = dict(name="configs[1]: causal order-2 fwd+bwd", B=4, H=8, N=4096, D=64, p=2, mask=True, scale=1.0)

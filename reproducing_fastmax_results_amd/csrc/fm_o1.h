@@ -8,11 +8,13 @@
 //     dk'_j = a1 [ (sum_{i>=j} q'_i gh_i^T) v_j - sum_{i>=j} c_i q'_i ]
 //     dv_j  = a0 sum_{i>=j} gh_i + a1 (sum_{i>=j} gh_i q'_i^T) k'_j
 // so a segment needs its own 128 rows, the sums over the segments before it (keys, values) and after it
-// (queries, gh), and nothing else.  Four kernels, one workgroup per segment each:
-//   k_o1_sums<KV>  k, v            -> sums inside runs of segments (k_o1_runscan: sums over whole runs)
-//   k_o1_fwd       q, k, v, prefix -> o, g
+// (queries, gh), and nothing else.  Four kernels:
+//   k_o1_sums<KV>  k, v            -> one workgroup per run of segments: for every segment the sums over the segments
+//                                     before it inside the run, and the run's total (k_o1_runscan: totals -> sums over
+//                                     the runs before); a consumer adds the two parts
+//   k_o1_fwd       q, k, v, prefix -> o, g            (one workgroup per segment)
 //   k_o1_sums<QG>  q, dO, o, g     -> the same, walking backwards
-//   k_o1_bwd       q, k, v, dO, o, g, prefix, suffix -> dq, dk, dv
+//   k_o1_bwd       q, k, v, dO, o, g, prefix, suffix -> dq, dk, dv      (one workgroup per segment)
 // No converted or transposed copy of any tensor is written: rows are converted (and scaled: 1/tau, the
 // folded normalisation, the gradient scale) in registers on their way into LDS.  The general kernels need a
 // conversion pass per tensor, read the four operand copies once per gradient and stream every tile of a
