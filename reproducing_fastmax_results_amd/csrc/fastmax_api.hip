@@ -569,7 +569,7 @@ int add_rows(const FastmaxDesc* d, const SplitPlan& sp, const void* dqa, void* d
 
 extern "C" {
 
-int fastmax_version(void) { return 105; }
+int fastmax_version(void) { return 200; }   // 0.2.0: FastmaxDesc gained `norm`; decode, static-scratch and statistics entry points
 
 const char* fastmax_status_string(int status) {
   switch (status) {

@@ -116,7 +116,7 @@ def test_forward_backward_reject_bad_arguments_before_launching(lib):
     assert lib.lib.fastmax_probe_mfma_rate(1, 1, None, None) == 1
     assert lib.lib.fastmax_probe_mfma_rate(0, 1, one, None) == 2
     assert lib.lib.fastmax_probe_mfma_rate(1, (1 << 20) + 1, one, None) == 2
-    assert lib.lib.fastmax_version() >= 105
+    assert lib.lib.fastmax_version() >= 200
 
 
 def test_static_scratch_entry_rejects_before_touching_the_device(lib):
