@@ -403,12 +403,11 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
                             : M::load_perm(Zt + (32 * ct + lr) * PV + 32 * st, ss, lh);
         if (st == KT / 32 - 1) {
           // next stage: registers -> the other buffer (its readers finished before this stage's
-          // barrier), then the stage after it: global memory -> registers
-          const int sn = s0 + s_step;
-          if (more(sn)) {
-            put(buf ^ 1);
-            if (more(sn + s_step)) fetch(sn + s_step);
-          }
+          // barrier), then the stage after it: global memory -> registers.  No branch (see k_ds): past the last
+          // stage the registers go where nobody reads and the current stage is loaded once more.
+          const int sn = s0 + s_step, sf = more(sn) && more(sn + s_step) ? sn + s_step : s0;
+          put(buf ^ 1);
+          fetch(sf);
         }
 #pragma unroll
         for (int j = 0; j < QT; ++j) {
@@ -661,16 +660,17 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
       ry.load(yb + int64_t(sx) * DH, DH, tid);
       if (!TR) rz.load(zb + sx, A.npad_str, tid);
       if (DV && !TR) rz2.load(z2b + sx, A.npad_str, tid);
-      // QF: c is staged as -c in fp32, tokens in their natural order (the copy holds them in `tperm` order)
-      if (OWN == FM_OWN_K && tid < KT) creg = cvb[sx + (QF ? M::tperm(tid) : tid)];
+      // QF: c is staged as -c in fp32, tokens in their natural order (the copy holds them in `tperm` order).
+      // Every thread takes part (the threads past KT repeat the first ones): no branch in the stage loop.
+      if (OWN == FM_OWN_K) creg = cvb[sx + (QF ? M::tperm(tid % KT) : tid % KT)];
     };
     auto put = [&](int b) {                             // registers -> stage buffer b
       E* Xn = Own + b * STAGE; E* Yn = Xn + KT * PQ; E* Zn = Yn + KT * PQ; E* cn = Zn + (TR ? 0 : DH * PV);
       rx.store(Xn, PQ, tid); ry.store(Yn, PQ, tid);
       if (!TR) rz.store(Zn, PV, tid);
       if (DV && !TR) rz2.store(cn + KT, PV, tid);
-      if (OWN == FM_OWN_K && tid < KT) {
-        if (QF) reinterpret_cast<float*>(cn)[tid] = -float(creg); else cn[tid] = creg;
+      if (OWN == FM_OWN_K) {
+        if (QF) reinterpret_cast<float*>(cn)[tid % KT] = -float(creg); else cn[tid % KT] = creg;
       }
     };
     // Two buffers: the tiles of stage i+1 travel global memory -> registers during stage i-1 and
@@ -711,11 +711,11 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
                             : M::load_perm(Zt + (32 * mt + lr) * PV + 32 * st, ss, lh);
         }
         if (NBUF == 2 && st == KT / 32 - 1) {
-          const int sn = s0 + s_step;
-          if (more(sn)) {
-            put(buf ^ 1);
-            if (more(sn + s_step)) fetch(sn + s_step);
-          }
+          // the next stage's tiles into the other buffer and the loads of the stage after it, without a branch: past
+          // the last stage the registers are stored where nobody reads and the current stage is loaded once more
+          const int sn = s0 + s_step, sf = more(sn) && more(sn + s_step) ? sn + s_step : s0;
+          put(buf ^ 1);
+          fetch(sf);
         }
 #pragma unroll
         for (int j = 0; j < QT; ++j) {
