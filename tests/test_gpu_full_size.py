@@ -120,10 +120,21 @@ def test_config2_all_slices_through_states(lib, chunk):
 def test_config3_all_slices(lib, p):
     # causal long context, B*H = 16, N = 65536, D = 64, bf16, inputs scaled by 0.5
     print(f"case full config3 p={p}", flush=True)
-    # the library's segments at this length: 256 tokens (order 1), 1024 tokens (order 2); a row with an
-    # upstream gradient in every 256 tokens covers every segment of either (256 + rows per slice)
-    _check_sparse_rows(lib, 16, 65536, 64, torch.bfloat16, p, seed=110 + p, scale=0.5, seg=256)
+    # the library's segments at this length: 128 tokens (order 1), 1024 tokens (order 2); a row with an
+    # upstream gradient in every 128 (256) tokens covers every segment (512 / 256 + rows per slice)
+    _check_sparse_rows(lib, 16, 65536, 64, torch.bfloat16, p, seed=110 + p, scale=0.5, seg=128 if p == 1 else 256)
     _check_running_mean(lib, 16, 65536, 64, torch.bfloat16, p, seed=120 + p)
+
+
+@pytest.mark.parametrize("bh,n", [(40, 5000), (7, 9000), (96, 2304)])
+def test_order1_runs_of_segments(lib, bh, n):
+    """Order 1 on bf16 beyond 1024 tokens sums its 128-token segments in runs whose length follows the number of
+    segments and batch*heads (3, 2 and 3 segments per run here; ragged last segment, last run of one or two
+    segments, a whole number of runs): every segment holds a row with upstream gradient, so the part of every
+    segment's state that comes from inside its run and the part that comes from the runs before / after it both
+    enter o, dq, dk and dv."""
+    print(f"case order-1 runs bh={bh} n={n}", flush=True)
+    _check_sparse_rows(lib, bh, n, 64, torch.bfloat16, 1, seed=90 + bh, scale=0.7, seg=128)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -138,7 +149,7 @@ def test_config2_all_slices_sharp_temperature(lib, dtype):
 @pytest.mark.parametrize("p", [1, 2])
 def test_config3_all_slices_sharp_temperature(lib, p):
     print(f"case full config3 tau=sqrt(D) p={p}", flush=True)
-    _check_sparse_rows(lib, 16, 65536, 64, torch.bfloat16, p, seed=150 + p, scale=0.5, seg=256, tau_mult=1.0)
+    _check_sparse_rows(lib, 16, 65536, 64, torch.bfloat16, p, seed=150 + p, scale=0.5, seg=128 if p == 1 else 256, tau_mult=1.0)
 
 
 @pytest.mark.parametrize("p", [1, 2])
