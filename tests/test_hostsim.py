@@ -4,8 +4,9 @@ The very same kernel templates the GPU runs are compiled as plain C++ with
 -DFM_HOSTSIM (work-items are OS threads, MFMA tiles are emulated with the lane
 layout the GPU probe test pins) and driven through the same C ABI.  This checks
 indexing, lane layouts, masks and ragged sizes without a GPU and, with
-FASTMAX_HOSTSIM_ASAN=1, under AddressSanitizer.  It is a test build only: the
-package never loads it.  Sizes are tiny because every work-item is a thread.
+FASTMAX_HOSTSIM_ASAN=1 (minutes of compile and run time, so not by default), under
+AddressSanitizer through a driver of its own (tests/hostsim/asan_driver.cpp).  It is a test build
+only: the package never loads it.  Sizes are tiny because every work-item is a thread.
 """
 import os
 import shutil
@@ -226,3 +227,18 @@ def test_order1_segment_backward_in_one_pass(sim):
     # in one workgroup (9 segments here, the last one ragged); also with the folded normalisation's Jacobian
     check_forward_backward(sim, 1, 1100, 32, torch.bfloat16, "cpu", mask=True, p=1, seed=40, saved=True)
     check_norm_fold(sim, 1, 1100, 32, torch.bfloat16, "cpu", mask=True, p=1, seed=41)
+
+
+@pytest.mark.skipif(os.environ.get("FASTMAX_HOSTSIM_ASAN") != "1", reason="set FASTMAX_HOSTSIM_ASAN=1 (several minutes)")
+def test_kernel_sources_under_address_sanitizer(tmp_path):
+    # the state walk with two tile buffers, order 1 in runs of segments, the dense kernels, fp32: forward and backward
+    exe = str(tmp_path / "asan_driver")
+    cmd = [CLANG, "-x", "c++", "-std=c++17", "-O1", "-g", "-DFM_HOSTSIM", "-Wno-psabi", "-pthread", "-fsanitize=address",
+           "-fno-omit-frame-pointer", "-I", os.path.join(ROOT, "include"), "-I", os.path.join(ROOT, "tests", "hostsim"),
+           "-I", os.path.join(ROOT, "reproducing_fastmax_results_amd", "csrc"),
+           os.path.join(ROOT, "reproducing_fastmax_results_amd", "csrc", "fastmax_api.hip"),
+           os.path.join(ROOT, "tests", "hostsim", "asan_driver.cpp"), "-o", exe]
+    subprocess.run(cmd, check=True, capture_output=True)
+    run = subprocess.run([exe], capture_output=True, text=True, env=dict(os.environ, ASAN_OPTIONS="detect_leaks=0"))
+    assert run.returncode == 0, run.stdout[-2000:] + run.stderr[-4000:]
+    assert "AddressSanitizer" not in run.stderr
