@@ -737,10 +737,11 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <
         const E* xb_ = cb + 2 * DH * PT + (wave * NA) * PT + lh * M::KPL;
         const int tn = pf.valid ? pf.t : cur.t;     // the tile to load: the one `pf` names, or (none left) the current one again
         frag fb[KB][NT], fp[KB][NT], fx[KB][NA];
-        // The fragments of three k-steps are requested ahead of their products (the counter a wavefront waits on
+        // The fragments of two k-steps are requested ahead of their products (the counter a wavefront waits on
         // for LDS ends at 15 outstanding operations: with all 40 reads of a tile in flight the first product would
-        // wait for 26 of them).
-        constexpr int AHEAD = 3;
+        // wait for 26 of them; both walks of a step at the long shape: all at once 1.79 - 1.88 ms, four ahead 1.64,
+        // three 1.56, two 1.54).
+        constexpr int AHEAD = 2;
         auto frags = [&](int u) FM_ALWAYS_INLINE {
 #pragma unroll
           for (int i = 0; i < NA; ++i) fx[u][i] = M::load(xb_ + i * PT + u * M::KSTEP);
