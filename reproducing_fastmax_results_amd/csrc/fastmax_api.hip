@@ -195,7 +195,8 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   }
   const size_t slots = size_t(d->bh) * p.nslots;
   const size_t bigarr = d->d == 64 ? big_array_bytes<64>(p.esz, p.quad, slots) : big_array_bytes<32>(p.esz, p.quad, slots);
-  const size_t smallsz = size_t(d->d == 64 ? StateDims<64>::SMALL : StateDims<32>::SMALL) * 4;
+  // fp32 part of a slot: Z and the two vector sums; the order-1 path of fm_o1.h keeps the two vectors only
+  const size_t smallsz = p.o1 ? size_t(2) * d->d * 4 : size_t(d->d == 64 ? StateDims<64>::SMALL : StateDims<32>::SMALL) * 4;
   const size_t tq = p.o1 ? 0 : size_t(d->bh) * d->d * p.npad_q * p.esz;
   const size_t tk = p.o1 ? 0 : size_t(d->bh) * d->d * p.npad_k * p.esz;
   size_t off = 0;

@@ -109,7 +109,10 @@ FM_DEVICE void fm_o1_gh_rows(const O1Raw<DH>& rdo, const O1Raw<DH>& ro, const fl
 // from global memory to registers while this one's products run.
 // A run total (and `runtot` after the scan): DH * DH + 2 * DH floats, the slab, then va, then vb.
 // ------------------------------------------------------------------------------
-template <int DH> struct O1Run { static constexpr int RS = DH * DH + 2 * DH; };
+template <int DH> struct O1Run {
+  static constexpr int RS = DH * DH + 2 * DH;      // floats of a run total
+  static constexpr int VS = 2 * DH;                // floats of a segment's vector sums (`small`: [bh][segments][VS], va then vb)
+};
 // Segments per run: enough runs to give every CU two workgroups, runs as long as that allows (measured on
 // MI355X, B*H = 16, 512 segments each: 16 segments per run 0.19 ms for both sums passes of a step, 8: 0.205,
 // 32: 0.215, 64: 0.38).
@@ -150,7 +153,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_sums(O1SumArgs<TIO> A) {
   const int cnt = s_hi - s_lo;
   const bool suffix = A.b.mode == FM_WALK_SUFFIX;
   E* big = A.b.big + int64_t(bh) * A.b.nslots * StateDims<DH>::stride(false);
-  float* sml = A.b.small + int64_t(bh) * A.b.nslots * StateDims<DH>::SMALL;
+  float* sml = A.b.small + int64_t(bh) * A.b.nslots * O1Run<DH>::VS;
   R r0, r1, ro;
   float gi[R::N];
   auto fetch = [&](int seg) FM_ALWAYS_INLINE {
@@ -185,16 +188,24 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_sums(O1SumArgs<TIO> A) {
     }
     if (i + 1 < cnt) fetch(suffix ? seg - 1 : seg + 1);
     FM_SYNC();
-    float* ds = sml + int64_t(seg) * StateDims<DH>::SMALL;
+    float* ds = sml + int64_t(seg) * O1Run<DH>::VS;
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
       const int t = wave + 4 * s;
       if (t >= NTILE) continue;
       // the sums of the run so far are this segment's state inside the run
-      float v[16];
+      if (t < NT * NT) {
+        float v[16];
 #pragma unroll
-      for (int e = 0; e < 16; ++e) v[e] = acc[s][e];
-      fm_put_small<E, DH>(A.b, big, nullptr, ds, seg, t < NT * NT ? t : t + NT * NT, v, lr, lh);
+        for (int e = 0; e < 16; ++e) v[e] = acc[s][e];
+        fm_put_small<E, DH>(A.b, big, nullptr, nullptr, seg, t, v, lr, lh);
+      } else if (lr == 0) {
+        const bool is_va = t < NT * NT + NT;
+        float* dv = ds + (is_va ? 32 * (t - NT * NT) : DH + 32 * (t - NT * NT - NT));
+        const float cf = is_va ? A.b.coefva : A.b.coefvb;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) dv[fm_acc_row(e, lh)] = cf * acc[s][e];
+      }
       // tiles of this wavefront: A operand (tile, feature offset), B operand (tile, or null = weights / ones)
       const E* ta = Lp; const E* tbt = nullptr;
       int fa = 0, fb = 0;
@@ -307,7 +318,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 3) k_o1_fwd(O1FwdArgs<TIO> A) {
     const int run = seg / A.run_len;
     float vsum = 0.f;
     if (tid < 2 * DH && seg > 0)
-      vsum = A.small[(int64_t(bh) * A.nslots + seg) * StateDims<DH>::SMALL + DH * DH + tid] +
+      vsum = A.small[(int64_t(bh) * A.nslots + seg) * O1Run<DH>::VS + tid] +
              A.runtot[(int64_t(bh) * A.nruns + run) * O1Run<DH>::RS + DH * DH + tid];
     const E* sl = A.big + (int64_t(bh) * A.nslots + seg) * StateDims<DH>::SLAB;
     const E* rl = A.runbig + (int64_t(bh) * A.nruns + run) * StateDims<DH>::SLAB;
@@ -485,7 +496,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
       // the vector sums of the two states this segment reads (a segment at either end reads zeros instead)
       const bool pre = tid < DH;
       const int f = pre ? tid : tid - DH;
-      const float* src = (pre ? A.smallq : A.smallk) + (int64_t(bh) * A.nslots + seg) * StateDims<DH>::SMALL + DH * DH + f;
+      const float* src = (pre ? A.smallq : A.smallk) + (int64_t(bh) * A.nslots + seg) * O1Run<DH>::VS + f;
       const float* src2 = (pre ? A.runtotq : A.runtotk) + (int64_t(bh) * A.nruns + run) * O1Run<DH>::RS + DH * DH + f;
       if (pre ? seg > 0 : seg < A.nseg - 1) vsum = *src + *src2;
     }
