@@ -448,6 +448,10 @@ def operator_line(lib, dev, W, dtype, args, steps, warmup, full):
     e1.record()
     e1.synchronize()
     out["measured_on_this_box"] = {"mfma_f16_loop_TFLOPs": lib.mfma_rate(dev),
+                                   # the same products fed from LDS with the dense kernels' instruction mix: what a
+                                   # kernel of this structure can reach (one / two own tiles per wavefront)
+                                   "mfma_f16_lds_fed_mix_TFLOPs": lib.mix_rate(dev, 1),
+                                   "mfma_f16_lds_fed_mix_two_tiles_TFLOPs": lib.mix_rate(dev, 2),
                                    "hbm_copy_GBps": 5 * 2 * float(1 << 30) / (e0.elapsed_time(e1) * 1e-3) / 1e9,
                                    "published": {"mfma_bf16_TFLOPs": PEAK_TFLOPS["bf16"], "mfma_f32_TFLOPs": PEAK_TFLOPS["f32"],
                                                  "hbm_GBps": PEAK_HBM_GBS}}

@@ -251,6 +251,15 @@ int fastmax_probe_mfma(float* out_f16, float* out_f32, void* hip_stream);
  * out: workgroups * 256 floats (device memory, checksums).  workgroups <= 65536, iters <= 2^20. */
 int fastmax_probe_mfma_rate(int workgroups, int iters, float* out, void* hip_stream);
 
+/* Second yardstick (no counterpart in the reference): the same, with the operands coming out of LDS the way the
+ * dense kernels' do.  Per round and own tile a wavefront issues the 16 products of one 32x32 tile pair of the
+ * dK + dV pass, fed by 8 sixteen-byte LDS reads and 16 transposing eight-byte reads per round (shared by the
+ * wavefront's own_tiles = 1 or 2 tiles) and accompanied by 64 packed-half vector instructions per own tile;
+ * workgroups * 4 * iters * 16 * own_tiles * 32768 flop.  Timed by the caller, it gives the matrix rate this
+ * instruction mix can reach on the device, which is what the dense kernels' own rate is to be held against.
+ * out: workgroups * 256 floats.  own_tiles = 1 is built for two workgroups per CU, 2 for one. */
+int fastmax_probe_mix_rate(int workgroups, int iters, int own_tiles, float* out, void* hip_stream);
+
 /* Self-check of the transposing LDS read (ds_read_b64_tr_b16) the _Float16 kernels use for transposed
  * fragments: one wavefront reads a 16 x 64 tile holding 64 * row + col; lane l addresses the four
  * values at (row l % 16, columns 4 * (l / 16) ..).  out: 256 floats (device memory), four per lane.

@@ -59,7 +59,7 @@ EXPORTS = (
     "fastmax_workspace_bytes", "fastmax_forward", "fastmax_backward", "fastmax_backward_saved", "fastmax_normalize",
     "fastmax_normalize_stats_bytes", "fastmax_normalize_backward", "fastmax_normalize_backward_stats_bytes",
     "fastmax_status_string", "fastmax_version", "fastmax_probe_mfma", "fastmax_probe_lds_transpose",
-    "fastmax_probe_mfma_rate",
+    "fastmax_probe_mfma_rate", "fastmax_probe_mix_rate",
     "fastmax_profile_begin", "fastmax_profile_end", "fastmax_forward_static",
     "fastmax_maxnorm_stats", "fastmax_maxnorm_stats_bytes",
     "fastmax_decode_state_bytes", "fastmax_decode_scratch_bytes", "fastmax_decode_absorb", "fastmax_decode_step",
@@ -163,6 +163,8 @@ class FastmaxLib:
         L.fastmax_probe_lds_transpose.restype = C.c_int
         L.fastmax_probe_mfma_rate.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p]
         L.fastmax_probe_mfma_rate.restype = C.c_int
+        L.fastmax_probe_mix_rate.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+        L.fastmax_probe_mix_rate.restype = C.c_int
         L.fastmax_profile_begin.restype = C.c_int
         L.fastmax_profile_end.argtypes = [C.POINTER(C.c_int), C.POINTER(C.c_float), C.c_int]
         L.fastmax_profile_end.restype = C.c_int
@@ -408,6 +410,21 @@ class FastmaxLib:
         e1.record()
         e1.synchronize()
         return workgroups * 4 * iters * 8 * 32768.0 / (e0.elapsed_time(e1) * 1e-3) / 1e12
+
+    def mix_rate(self, device, own_tiles: int = 1, iters: int = 4000) -> float:
+        """TFLOP/s of the matrix products of a loop with the dense kernels' instruction mix (operands read
+        out of LDS, packed-half vector work beside them; see fastmax_probe_mix_rate), every CU filled the
+        way the dK + dV pass fills it."""
+        workgroups = 512 if own_tiles == 1 else 256
+        out = torch.empty(workgroups * 256, dtype=torch.float32, device=device)
+        stream = torch.cuda.current_stream(out.device).cuda_stream
+        self.check(self.lib.fastmax_probe_mix_rate(workgroups, 10, own_tiles, out.data_ptr(), stream), "fastmax_probe_mix_rate")
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        self.check(self.lib.fastmax_probe_mix_rate(workgroups, iters, own_tiles, out.data_ptr(), stream), "fastmax_probe_mix_rate")
+        e1.record()
+        e1.synchronize()
+        return workgroups * 4 * iters * 16 * own_tiles * 32768.0 / (e0.elapsed_time(e1) * 1e-3) / 1e12
 
 
 _lock = threading.Lock()

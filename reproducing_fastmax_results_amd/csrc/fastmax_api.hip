@@ -888,6 +888,16 @@ int fastmax_probe_mfma_rate(int workgroups, int iters, float* out, void* hip_str
   return fm_launch_status();
 }
 
+int fastmax_probe_mix_rate(int workgroups, int iters, int own_tiles, float* out, void* hip_stream) {
+  if (!out) return FASTMAX_ERR_NULL;
+  if (workgroups <= 0 || workgroups > 65536 || iters <= 0 || iters > (1 << 20)) return FASTMAX_ERR_SHAPE;
+  if (own_tiles != 1 && own_tiles != 2) return FASTMAX_ERR_UNSUPPORTED;
+  fm_stream_t st = static_cast<fm_stream_t>(hip_stream);
+  if (own_tiles == 1) FM_KERNEL_LAUNCH(k_probe_mix<1>, fm_dim3(workgroups), fm_dim3(FM_THREADS), 0, st, out, iters);
+  else FM_KERNEL_LAUNCH(k_probe_mix<2>, fm_dim3(workgroups), fm_dim3(FM_THREADS), 0, st, out, iters);
+  return fm_launch_status();
+}
+
 int fastmax_probe_lds_transpose(float* out, void* hip_stream) {
   if (!out) return FASTMAX_ERR_NULL;
   FM_KERNEL_LAUNCH(k_probe_lds_tr, fm_dim3(1), fm_dim3(64), 0, static_cast<fm_stream_t>(hip_stream), out);
