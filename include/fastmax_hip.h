@@ -225,6 +225,24 @@ size_t fastmax_normalize_backward_stats_bytes(const FastmaxNormDesc* desc);
 int fastmax_normalize_backward(const FastmaxNormDesc* desc, const void* x, const void* dy, void* dx,
                                float* stats, void* hip_stream);
 
+/* The two element-wise steps the reference's forward_cuda carries switched off, for callers that switch
+ * them on.  desc: bh, n, d, dtype; sx: strides of the input (and of `noise`), sy: strides of the output,
+ * which may be the input buffer itself when the strides agree.
+ *
+ * fastmax_key_rpe replaces the addition in apply_rpe_and_temp (reference fastmax_cuda_forward.cu:282-292,
+ * commented out at :289):  k[l][m] = k[l][m] / tau + rpe[(l + n) % (2 n - 1)][m], rpe a contiguous fp32
+ * (2 n - 1, d) table (rpe_matrix_creator, transformer/model.py:218-247).  The operator divides by tau in
+ * its loads, so this writes k_out = k + temperature * rpe[..]; pass the result as k with the same inv_tau.
+ * dk of the operator is then also the gradient with respect to the k given here.
+ *
+ * fastmax_output_noise replaces apply_dropout (fastmax_cuda_forward.cu:340-349, called with scale 0 at
+ * :443):  o_out = o * (1 + scale * noise), noise of o's type and strides.  Applied to dO with the same
+ * noise it is the step's backward. */
+int fastmax_key_rpe(const FastmaxNormDesc* desc, const void* k, const float* rpe, void* k_out, float temperature,
+                    void* hip_stream);
+int fastmax_output_noise(const FastmaxNormDesc* desc, const void* o, const void* noise, void* o_out, float scale,
+                         void* hip_stream);
+
 const char* fastmax_status_string(int status);
 
 /* Library version: major * 10000 + minor * 100 + patch. */

@@ -43,7 +43,7 @@ __all__ = [
     "tau_einops", "closed_form_forward", "closed_form_forward_backward",
     "manual_backward_blocked", "sampled_rows_forward_backward", "factorised_forward", "factorised_backward",
     "extension_forward", "extension_backward", "score_function_fastmax",
-    "normalize_feature_mean", "normalize_token_mean", "normalize_lim",
+    "normalize_feature_mean", "normalize_token_mean", "normalize_lim", "apply_rpe_and_temp", "apply_dropout",
     "rel_l2",
 ]
 
@@ -347,6 +347,28 @@ def normalize_lim(x, lim: float = 1.0):
     """Intended semantics of the extension's ``normalize`` flag as written out in
     ``transformer/model.py:97-102``: ``lim * x / max_n ||x_n||_2``, no centring."""
     return lim * x / torch.linalg.vector_norm(x, dim=-1).amax(-1)[..., None, None]
+
+
+def apply_rpe_and_temp(k, rpe, temperature: float, add_rpe: bool = True):
+    """``apply_rpe_and_temp`` with its commented-out addition switched on
+    (``fastmax_cuda_forward.cu:282-292``): token by token, as the kernel loops,
+    ``k[l] = k[l] / temperature + rpe[(l + nk) % (2 nk - 1)]``.  k ``(..., nk, d)``,
+    rpe ``(2 nk - 1, d)``.  Pinned by a hand-worked case (the row order for nk = 3
+    is 3, 4, 0) and by ``add_rpe=False`` being the plain division."""
+    nk = k.shape[-2]
+    out = k.double() / float(temperature)
+    if add_rpe:
+        out = out.clone()
+        for l in range(nk):
+            out[..., l, :] += rpe[(l + nk) % (2 * nk - 1)].double()
+    return out
+
+
+def apply_dropout(o, drop_noise, scale: float):
+    """``apply_dropout`` (``fastmax_cuda_forward.cu:340-349``):
+    ``o *= 1 + scale * drop_noise`` element by element; the reference calls it with
+    scale 0 (``:443``)."""
+    return o.double() * (1.0 + float(scale) * drop_noise.double())
 
 
 def score_function_fastmax(q, k, v, mask=None, denum_term=8, normalize=0, p=1,

@@ -59,7 +59,7 @@ EXPORTS = (
     "fastmax_workspace_bytes", "fastmax_forward", "fastmax_backward", "fastmax_backward_saved", "fastmax_normalize",
     "fastmax_normalize_stats_bytes", "fastmax_normalize_backward", "fastmax_normalize_backward_stats_bytes",
     "fastmax_status_string", "fastmax_version", "fastmax_probe_mfma", "fastmax_probe_lds_transpose",
-    "fastmax_probe_mfma_rate", "fastmax_probe_mix_rate",
+    "fastmax_probe_mfma_rate", "fastmax_probe_mix_rate", "fastmax_key_rpe", "fastmax_output_noise",
     "fastmax_profile_begin", "fastmax_profile_end", "fastmax_forward_static",
     "fastmax_maxnorm_stats", "fastmax_maxnorm_stats_bytes",
     "fastmax_decode_state_bytes", "fastmax_decode_scratch_bytes", "fastmax_decode_absorb", "fastmax_decode_step",
@@ -165,6 +165,10 @@ class FastmaxLib:
         L.fastmax_probe_mfma_rate.restype = C.c_int
         L.fastmax_probe_mix_rate.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
         L.fastmax_probe_mix_rate.restype = C.c_int
+        L.fastmax_key_rpe.argtypes = [C.POINTER(NormDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p]
+        L.fastmax_key_rpe.restype = C.c_int
+        L.fastmax_output_noise.argtypes = [C.POINTER(NormDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p]
+        L.fastmax_output_noise.restype = C.c_int
         L.fastmax_profile_begin.restype = C.c_int
         L.fastmax_profile_end.argtypes = [C.POINTER(C.c_int), C.POINTER(C.c_float), C.c_int]
         L.fastmax_profile_end.restype = C.c_int
@@ -373,6 +377,40 @@ class FastmaxLib:
                                                  self._stream(x))
         self.check(st, "fastmax_normalize_backward")
         return dx
+
+    def _pointwise_desc(self, x, out):
+        nd = NormDesc()
+        nd.bh, nd.n, nd.d = _dims(x)
+        nd.dtype = _dtype_code(x)
+        nd.sx, nd.sy = _strides(x), _strides(out)
+        return nd
+
+    def key_rpe(self, k, rpe, temperature: float, out: Optional[torch.Tensor] = None):
+        """k (bh, n, d) view, rpe (2n-1, d): k + temperature * rpe[(l + n) % (2n - 1)], the keys that make the
+        operator see k / temperature + rpe (the addition the reference leaves commented out)."""
+        bh, n, d = _dims(k)
+        if tuple(rpe.shape) != (2 * n - 1, d):
+            raise ValueError(f"rpe must be ({2 * n - 1}, {d}), got {tuple(rpe.shape)}")
+        table = rpe.detach().to(device=k.device, dtype=torch.float32).contiguous()
+        if out is None:
+            out = torch.empty(tuple(k.shape), dtype=k.dtype, device=k.device)
+        nd = self._pointwise_desc(k, out)
+        st = self.lib.fastmax_key_rpe(C.byref(nd), k.data_ptr(), table.data_ptr(), out.data_ptr(), float(temperature),
+                                      self._stream(k))
+        self.check(st, "fastmax_key_rpe")
+        return out
+
+    def output_noise(self, o, noise, scale: float, out: Optional[torch.Tensor] = None):
+        """o * (1 + scale * noise); o and noise (bh, n, d) views of one type and layout."""
+        if noise.dtype != o.dtype or tuple(noise.shape) != tuple(o.shape) or noise.stride() != o.stride():
+            raise ValueError("noise must have o's type, shape and strides")
+        if out is None:
+            out = torch.empty(tuple(o.shape), dtype=o.dtype, device=o.device)
+        nd = self._pointwise_desc(o, out)
+        st = self.lib.fastmax_output_noise(C.byref(nd), o.data_ptr(), noise.data_ptr(), out.data_ptr(), float(scale),
+                                           self._stream(o))
+        self.check(st, "fastmax_output_noise")
+        return out
 
     KERNEL_NAMES = ("transpose", "prep_bwd", "build", "fwd", "dq", "dk", "normalize", "dv", "dkv")
 

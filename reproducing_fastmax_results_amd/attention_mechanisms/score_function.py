@@ -30,6 +30,7 @@ from .. import fastmax_cuda as _ext   # the torch binding built by __graft_entry
 __all__ = [
     "FASTMultiHeadAttention_Function", "FASTMultiHeadAttention", "rpe_matrix_creator", "fastmax_custom",
     "fastmax", "fastmax_einops", "FastmaxNormalize", "FastmaxNormAttention", "FastmaxDecodeState",
+    "FastmaxOutputNoise", "FastmaxKeyRpe", "fastmax_with_dormant_steps",
 ]
 
 CENTRE_NONE, CENTRE_FEATURE, CENTRE_TOKEN = 0, 1, 2
@@ -110,6 +111,61 @@ class FastmaxNormAttention(torch.autograd.Function):
         gq, gk, gv = _ext.backward_norm(q, k, v, o, g, grad_output, saved, qk, kk, ctx.lim, True, *ctx.cfg, 0, 0)
         d = ctx.d
         return (gq[..., :d], gk[..., :d], gv[..., :d]) + (None,) * 7
+
+
+class FastmaxOutputNoise(torch.autograd.Function):
+    """``o * (1 + scale * noise)``: the reference's ``apply_dropout`` (``fastmax_cuda_forward.cu:340-349``),
+    which its ``forward_cuda`` calls with scale 0 (``:443``).  The backward is the same pass on dO."""
+
+    @staticmethod
+    def forward(ctx, o, noise, scale):
+        d = o.shape[-1]
+        noise = _pad_features(noise.to(o.dtype))
+        ctx.save_for_backward(noise)
+        ctx.scale, ctx.d = float(scale), d
+        return _ext.output_noise(_pad_features(o), noise, float(scale))[..., :d]
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        (noise,) = ctx.saved_tensors
+        return _ext.output_noise(_pad_features(grad_y), noise, ctx.scale)[..., :ctx.d], None, None
+
+
+class FastmaxKeyRpe(torch.autograd.Function):
+    """``k + temperature * rpe[(l + n) % (2n - 1)]``: keys that make the operator see ``k / temperature +
+    rpe``, the addition the reference leaves commented out (``fastmax_cuda_forward.cu:289``).  The gradient
+    with respect to k passes through; the table gets none (the reference never trains through it)."""
+
+    @staticmethod
+    def forward(ctx, k, rpe, temperature):
+        d = k.shape[-1]
+        ctx.d = d
+        kp = _pad_features(k)
+        table = torch.nn.functional.pad(rpe, (0, kp.shape[-1] - d))
+        return _ext.key_rpe(kp, table, float(temperature))[..., :d]
+
+    @staticmethod
+    def backward(ctx, grad_k):
+        return grad_k, None, None
+
+
+def fastmax_with_dormant_steps(q, k, v, drop_noise=None, rpe_matrix=None, mask=False, noise_scale=0.0, rpe_on_keys=False,
+                               normalize=False, temperature=1.0, a0=1.0, a1=1.0, a2=0.5, lim=1.0, p=2):
+    """The operator with the two steps switched on that the reference's ``forward_cuda`` carries switched off:
+    ``rpe_on_keys`` adds ``rpe_matrix`` rows to ``k / temperature`` (``fastmax_cuda_forward.cu:289``) and a non-zero
+    ``noise_scale`` multiplies the output by ``1 + noise_scale * drop_noise`` (``:340-349``).  With both off
+    this is ``FASTMultiHeadAttention_Function.apply``; the order of the steps is the reference's
+    (temperature and RPE, normalisation, attention, noise)."""
+    if rpe_on_keys:
+        if rpe_matrix is None:
+            raise ValueError("rpe_on_keys needs rpe_matrix (rpe_matrix_creator)")
+        k = FastmaxKeyRpe.apply(k, rpe_matrix, temperature)
+    o = FASTMultiHeadAttention_Function.apply(q, k, v, None, None, mask, 0.0, normalize, temperature, a0, a1, a2, lim, p)
+    if noise_scale:
+        if drop_noise is None:
+            raise ValueError("a non-zero noise_scale needs drop_noise")
+        o = FastmaxOutputNoise.apply(o, drop_noise, noise_scale)
+    return o
 
 
 class FASTMultiHeadAttention_Function(torch.autograd.Function):

@@ -7,6 +7,7 @@
 #include "fm_split.h"
 #include "fm_decode.h"
 #include "fm_o1.h"
+#include "fm_pointwise.h"
 #include <atomic>
 #include <cmath>
 #include <mutex>
@@ -766,6 +767,22 @@ size_t fastmax_normalize_stats_bytes(const FastmaxNormDesc* desc) {
 int fastmax_normalize(const FastmaxNormDesc* desc, const void* x, void* y, float* stats, void* hip_stream) {
   ProfScope prof(FM_K_NORM, static_cast<fm_stream_t>(hip_stream));   // the whole pass (its kernels together)
   return fm_normalize_dispatch(desc, x, y, stats, static_cast<fm_stream_t>(hip_stream));
+}
+
+int fastmax_key_rpe(const FastmaxNormDesc* desc, const void* k, const float* rpe, void* k_out, float temperature,
+                    void* hip_stream) {
+  if (!(temperature > 0.0f) || !(temperature < 3.0e38f)) return FASTMAX_ERR_SHAPE;
+  PointwiseArgs a;
+  a.n = desc ? desc->n : 0; a.mode = 0; a.factor = temperature; a.table = rpe;
+  return fm_pointwise_dispatch(desc, k, nullptr, k_out, a, static_cast<fm_stream_t>(hip_stream));
+}
+
+int fastmax_output_noise(const FastmaxNormDesc* desc, const void* o, const void* noise, void* o_out, float scale,
+                         void* hip_stream) {
+  if (!(scale == scale) || scale > 3.0e38f || scale < -3.0e38f) return FASTMAX_ERR_SHAPE;
+  PointwiseArgs a;
+  a.n = desc ? desc->n : 0; a.mode = 1; a.factor = scale; a.table = nullptr;
+  return fm_pointwise_dispatch(desc, o, noise, o_out, a, static_cast<fm_stream_t>(hip_stream));
 }
 
 static int decode_validate(const FastmaxDesc* d) {

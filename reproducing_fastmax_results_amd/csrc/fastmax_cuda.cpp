@@ -463,6 +463,40 @@ torch::Tensor normalize_backward(torch::Tensor x_, torch::Tensor dy_, int64_t ce
   return dx;
 }
 
+// k + temperature * rpe[(l + n) % (2n - 1)]  (see fastmax_key_rpe in the C header)
+torch::Tensor key_rpe(torch::Tensor k_, torch::Tensor rpe, double temperature) {
+  const View k = view_of(k_, "k");
+  FM_CHECK_CUDA(k.t);
+  TORCH_CHECK(rpe.dim() == 2 && rpe.size(0) == 2 * k.n - 1 && rpe.size(1) == k.d, "rpe must be (2n-1, d) = (", 2 * k.n - 1,
+              ", ", k.d, ")");
+  torch::Tensor table = rpe.to(k.t.device(), torch::kFloat32).contiguous();
+  FastmaxNormDesc nd{};
+  nd.bh = static_cast<int32_t>(k.bh); nd.n = static_cast<int32_t>(k.n); nd.d = static_cast<int32_t>(k.d);
+  nd.dtype = dtype_code(k.t);
+  torch::Tensor y = empty_like_layout(k.t, k.n, k.t.scalar_type());
+  nd.sx = k.s; nd.sy = view_of(y, "y").s;
+  check_status(fastmax_key_rpe(&nd, k.t.data_ptr(), table.data_ptr<float>(), y.data_ptr(), float(temperature), stream_of(k.t)),
+               "fastmax_key_rpe");
+  return y;
+}
+
+// o * (1 + scale * noise)  (see fastmax_output_noise in the C header)
+torch::Tensor output_noise(torch::Tensor o_, torch::Tensor noise_, double scale) {
+  const View o = view_of(o_, "o");
+  FM_CHECK_CUDA(o.t);
+  TORCH_CHECK(noise_.sizes() == o_.sizes() && noise_.scalar_type() == o_.scalar_type() && noise_.device() == o_.device(),
+              "noise must have o's shape, dtype and device");
+  torch::Tensor noise = noise_.strides() == o.t.strides() ? noise_ : torch::empty_strided(o.t.sizes(), o.t.strides(), o.t.options()).copy_(noise_);
+  FastmaxNormDesc nd{};
+  nd.bh = static_cast<int32_t>(o.bh); nd.n = static_cast<int32_t>(o.n); nd.d = static_cast<int32_t>(o.d);
+  nd.dtype = dtype_code(o.t);
+  torch::Tensor y = empty_like_layout(o.t, o.n, o.t.scalar_type());
+  nd.sx = o.s; nd.sy = view_of(y, "y").s;
+  check_status(fastmax_output_noise(&nd, o.t.data_ptr(), noise.data_ptr(), y.data_ptr(), float(scale), stream_of(o.t)),
+               "fastmax_output_noise");
+  return y;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(fastmax_cuda, m) {
@@ -480,5 +514,7 @@ PYBIND11_MODULE(fastmax_cuda, m) {
   m.def("decode_step", &decode_step, "one decoding step on the state: returns (o, g) of the new token");
   m.def("normalize", &normalize, "fused normalisation pass");
   m.def("normalize_backward", &normalize_backward, "gradient of the normalisation pass with respect to its input");
+  m.def("key_rpe", &key_rpe, "keys with the relative-position rows added (the reference's commented-out step)");
+  m.def("output_noise", &output_noise, "output times (1 + scale * noise) (the reference's apply_dropout)");
   m.def("version", []() { return fastmax_version(); });
 }

@@ -359,3 +359,69 @@ def test_other_head_sizes_run_padded(sf, d, normalize):
     with pytest.raises(RuntimeError, match="unsupported head size"):
         sf.FASTMultiHeadAttention_Function.apply(*(rnd(1, 1, 8, 80).to(DEV) for _ in range(3)))
 
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(2, 3, 333, 64), (5, 700, 32), (1, 1, 1, 64)])
+def test_dormant_steps_kernels(dtype, shape):
+    """fastmax_key_rpe / fastmax_output_noise through the C ABI against the oracle's restatement of the
+    reference's switched-off steps (fastmax_cuda_forward.cu:282-292, :340-349), on packed tensors, on the
+    projection layout and in place."""
+    from reproducing_fastmax_results_amd._capi import get_lib
+    lib = get_lib()
+    n, d, t = shape[-2], shape[-1], 3.5
+    k = rnd(*shape, seed=71).to(dtype)
+    rpe = rnd(2 * n - 1, d, seed=72)
+    want = O.apply_rpe_and_temp(k.double(), rpe, t) * t          # the pass leaves the division to the operator
+    got = lib.key_rpe(k.to(DEV), rpe.to(DEV), t)
+    assert rel_err(got, want) < (1e-6 if dtype == torch.float32 else 4e-3)
+    noise = rnd(*shape, seed=73).to(dtype)
+    want = O.apply_dropout(k.double(), noise.double(), 0.3)
+    got = lib.output_noise(k.to(DEV), noise.to(DEV), 0.3)
+    assert rel_err(got, want) < (1e-6 if dtype == torch.float32 else 4e-3)
+    assert torch.equal(lib.output_noise(k.to(DEV), noise.to(DEV), 0.0).cpu(), k)
+    if len(shape) == 4 and shape[1] > 1:
+        # (b, n, h, d) memory seen as (b, h, n, d), written in place
+        kp = k.permute(0, 2, 1, 3).contiguous().to(DEV).permute(0, 2, 1, 3)
+        np_ = noise.permute(0, 2, 1, 3).contiguous().to(DEV).permute(0, 2, 1, 3)
+        out = lib.output_noise(kp, np_, 0.3, out=kp)
+        assert out.data_ptr() == kp.data_ptr()
+        assert rel_err(kp, want) < (1e-6 if dtype == torch.float32 else 4e-3)
+
+
+def test_dormant_steps_errors():
+    from reproducing_fastmax_results_amd._capi import FastmaxError, get_lib
+    lib = get_lib()
+    k = torch.zeros(2, 10, 64, device=DEV)
+    with pytest.raises(ValueError):
+        lib.key_rpe(k, torch.zeros(20, 64, device=DEV), 1.0)          # 2n-1 = 19 rows
+    with pytest.raises(FastmaxError):
+        lib.key_rpe(k, torch.zeros(19, 64, device=DEV), 0.0)          # temperature must be positive
+    with pytest.raises(ValueError):
+        lib.output_noise(k, torch.zeros(2, 10, 64, device=DEV, dtype=torch.bfloat16), 0.1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("d", [64, 48])
+def test_operator_with_dormant_steps(sf, dtype, d):
+    """The operator with key RPE and output noise on, gradients included, against the closed form on the
+    keys and output the oracle's restatement of the two steps gives."""
+    b, h, n, t, scale = 2, 2, 300, 6.0, 0.25
+    q, k, v, go, noise = (rnd(b, h, n, d, seed=s).to(dtype) for s in (81, 82, 83, 84, 85))
+    rpe = rnd(2 * n - 1, d, seed=86)
+    qd, kd, vd = (x.to(DEV).requires_grad_(True) for x in (q, k, v))
+    o = sf.fastmax_with_dormant_steps(qd, kd, vd, noise.to(DEV), rpe.to(DEV), mask=True, noise_scale=scale,
+                                      rpe_on_keys=True, temperature=t, p=2)
+    o.backward(go.to(DEV))
+    q64, k64, v64 = (x.double().requires_grad_(True) for x in (q, k, v))
+    keys = O.apply_rpe_and_temp(k64, rpe, t)                      # already divided by the temperature
+    o64, _ = O.closed_form_forward(q64, keys, v64, mask=True, tau=1.0, p=2)
+    o64 = O.apply_dropout(o64, noise, scale)
+    o64.backward(go.double())
+    assert rel_err(o, o64) < TOL[dtype]
+    for got, want in ((qd.grad, q64.grad), (kd.grad, k64.grad), (vd.grad, v64.grad)):
+        assert rel_err(got, want) < TOL[dtype]
+    # both switched off: the plain operator
+    o_plain = sf.fastmax_with_dormant_steps(qd, kd, vd, noise.to(DEV), rpe.to(DEV), mask=True, temperature=t, p=2)
+    o_ref = sf.FASTMultiHeadAttention_Function.apply(qd, kd, vd, None, None, True, 0.0, False, t, 1.0, 1.0, 0.5, 1.0, 2)
+    assert torch.equal(o_plain, o_ref)

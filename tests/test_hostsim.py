@@ -105,6 +105,21 @@ def test_normalize(sim):
     assert O.rel_l2(sim.normalize(x, centre=2, max_norm=False, scale=2.0), 2.0 * (x - x.mean(1, keepdim=True)).double()) < 1e-6
 
 
+def test_dormant_steps(sim):
+    """Key RPE and output noise (the reference's switched-off steps) on ragged sizes and both types."""
+    from oracle import fastmax_oracle as O
+    for shape, dtype in (((2, 70, 32), torch.float32), ((1, 2, 129, 64), torch.bfloat16), ((1, 1, 64), torch.float32)):
+        n, d = shape[-2], shape[-1]
+        gen = torch.Generator().manual_seed(61)
+        k = torch.randn(*shape, generator=gen).to(dtype)
+        rpe = torch.randn(2 * n - 1, d, generator=gen)
+        noise = torch.randn(*shape, generator=gen).to(dtype)
+        tol = 1e-6 if dtype == torch.float32 else 4e-3
+        assert O.rel_l2(sim.key_rpe(k, rpe, 2.5), O.apply_rpe_and_temp(k.double(), rpe, 2.5) * 2.5) < tol
+        assert O.rel_l2(sim.output_noise(k, noise, -0.4), O.apply_dropout(k, noise, -0.4)) < tol
+        assert torch.equal(sim.output_noise(k, noise, 0.0), k)
+
+
 def test_normalize_backward(sim):
     from oracle import fastmax_oracle as O
     g = torch.Generator().manual_seed(12)

@@ -270,3 +270,22 @@ def test_attn_matrix_tensor_mask():
             for c in range(4):
                 want = sum(w[j] * float(v[0, h, j, c]) for j in range(6)) / tot
                 assert abs(float(o[0, h, i, c]) - want) < 1e-12
+
+
+def test_dormant_steps_known_answers():
+    """The two steps the reference ships switched off (fastmax_cuda_forward.cu:289, :340-349, :443), worked by hand:
+    for nk = 3 the table rows met by tokens 0, 1, 2 are (l + 3) % 5 = 3, 4, 0."""
+    k = torch.tensor([[[2.0, 4.0], [6.0, 8.0], [10.0, 12.0]]])
+    rpe = torch.tensor([[0.5, 0.25], [100.0, 100.0], [100.0, 100.0], [1.0, 2.0], [3.0, 4.0]])
+    got = O.apply_rpe_and_temp(k, rpe, temperature=2.0)
+    want = torch.tensor([[[1.0 + 1.0, 2.0 + 2.0], [3.0 + 3.0, 4.0 + 4.0], [5.0 + 0.5, 6.0 + 0.25]]], dtype=torch.float64)
+    assert torch.equal(got, want)
+    assert torch.equal(O.apply_rpe_and_temp(k, rpe, temperature=2.0, add_rpe=False), k.double() / 2.0)
+    # every table row but one is met at most once, and rows nk .. 2nk-2 come first
+    n = 7
+    idx = [(l + n) % (2 * n - 1) for l in range(n)]
+    assert idx == list(range(n, 2 * n - 1)) + [0]
+    o = torch.tensor([[1.0, -2.0], [4.0, 0.5]])
+    noise = torch.tensor([[0.5, 1.0], [-1.0, 2.0]])
+    assert torch.equal(O.apply_dropout(o, noise, 0.0), o.double())
+    assert torch.equal(O.apply_dropout(o, noise, 0.5), torch.tensor([[1.25, -3.0], [2.0, 1.0]], dtype=torch.float64))
