@@ -1366,6 +1366,107 @@ FM_DEVICE void fm_readout(const E* FM_RESTRICT state, bool quad, const E* xs, co
   FM_SYNC();
 }
 
+// The same readout when x and y are one vector and T[a][c][b] = T[b][c][a] (the forward's (k, v, k) sums read with
+// q, and the (q, gh, q) sums dV reads with k): sum_{a, b} = the 16 x 16 blocks on the diagonal of (a, b) once plus
+// twice the blocks above it, so a value of `a` in block KB meets the k-steps KB .. NKS - 1 only -- 10 of 16
+// products and 10 of 16 bytes of every slab, whose unused columns are neither loaded nor staged.
+constexpr int FM_SYM_BLOCK = 16;
+template <typename E, int DH, int QT, int NACC, int KB>
+FM_DEVICE void fm_readout_products(const E* sb, const E* xs, const int* xrow, int as, int na, bool ones,
+                                   const typename Mma<E>::frag (*yb)[TokCfg<E, DH, QT>::NKS], fm_f32x16 (*acc)[NACC],
+                                   int lane_off) {
+  typedef TokCfg<E, DH, QT> C;
+  typedef Mma<E> M;
+  typedef typename M::frag frag;
+  constexpr int KPB = FM_SYM_BLOCK / M::KSTEP;       // k-steps per block of (a, b)
+  constexpr int K0 = KB * KPB;                       // first k-step met
+  const E* sl = sb + lane_off;
+  frag fa[C::NT];
+#pragma unroll
+  for (int ct = 0; ct < C::NT; ++ct) fa[ct] = M::load(sl + (32 * ct) * C::PS + K0 * M::KSTEP);
+  E xv[QT];
+#pragma unroll
+  for (int j = 0; j < QT; ++j) xv[j] = ones ? E(1.0f) : xs[xrow[j] * C::PQ + as];
+  for (int al = 0; al < na; ++al) {
+    frag xr[QT], xr2[QT];
+#pragma unroll
+    for (int j = 0; j < QT; ++j) { xr[j] = M::splat(xv[j]); xr2[j] = ones ? xr[j] : xr[j] + xr[j]; }
+    const int an = (al + 1 < na) ? as + al + 1 : as + al;
+#pragma unroll
+    for (int j = 0; j < QT; ++j) xv[j] = ones ? E(1.0f) : xs[xrow[j] * C::PQ + an];
+#pragma unroll
+    for (int ks = K0; ks < C::NKS; ++ks) {
+      const int nks = (ks + 1 < C::NKS) ? ks + 1 : K0;
+      const int nal = (ks + 1 < C::NKS) ? al : (al + 1 < na ? al + 1 : al);
+      frag fn[C::NT];
+#pragma unroll
+      for (int ct = 0; ct < C::NT; ++ct) fn[ct] = M::load(sl + (nal * DH + 32 * ct) * C::PS + nks * M::KSTEP);
+#pragma unroll
+      for (int j = 0; j < QT; ++j) {
+        const frag fb = yb[j][ks] * (ks < K0 + KPB ? xr[j] : xr2[j]);
+#pragma unroll
+        for (int ct = 0; ct < C::NT; ++ct) acc[j][ct] = M::mma(fa[ct], fb, acc[j][ct]);
+      }
+#pragma unroll
+      for (int ct = 0; ct < C::NT; ++ct) fa[ct] = fn[ct];
+    }
+  }
+}
+
+template <typename E, int DH, int QT, int NACC, int KB>
+FM_DEVICE void fm_readout_sym_block(const E* FM_RESTRICT state, TileRegs<E, TokCfg<E, DH, QT>::SA * DH, DH - KB * FM_SYM_BLOCK>& cur,
+                                    const E* xs, const int* xrow, const typename Mma<E>::frag (*yb)[TokCfg<E, DH, QT>::NKS],
+                                    E* slab, fm_f32x16 (*acc)[NACC], int tid, int lane_off, int& buf) {
+  typedef TokCfg<E, DH, QT> C;
+  typedef Mma<E> M;
+  constexpr int C0 = KB * FM_SYM_BLOCK, A_END = C0 + FM_SYM_BLOCK;
+  constexpr bool LASTB = A_END == DH;
+  static_assert(FM_SYM_BLOCK % C::SA == 0 && FM_SYM_BLOCK % M::KSTEP == 0 && DH % FM_SYM_BLOCK == 0, "whole slabs and k-steps per block");
+  // after the last block: the order-1 slab (DH rows, every column)
+  TileRegs<E, LASTB ? DH : C::SA * DH, LASTB ? DH : DH - A_END> nxt;
+  for (int as = C0; as < A_END; as += C::SA) {
+    E* sb = slab + buf * C::SLAB;
+    cur.store(sb + C0, C::PS, tid);
+    FM_SYNC();
+    if (as + C::SA < A_END) cur.load(state + int64_t(as + C::SA) * DH * DH + C0, DH, tid);
+    else nxt.load(state + int64_t(as + C::SA) * DH * DH + (LASTB ? 0 : A_END), DH, tid);
+    fm_readout_products<E, DH, QT, NACC, KB>(sb, xs, xrow, as, C::SA, false, yb, acc, lane_off);
+    buf ^= 1;
+  }
+  if constexpr (!LASTB) {
+    fm_readout_sym_block<E, DH, QT, NACC, KB + 1>(state, nxt, xs, xrow, yb, slab, acc, tid, lane_off, buf);
+  } else {
+    E* sb = slab + buf * C::SLAB;
+    nxt.store(sb, C::PS, tid);
+    FM_SYNC();
+    fm_readout_products<E, DH, QT, NACC, 0>(sb, xs, xrow, DH, 1, true, yb, acc, lane_off);
+  }
+}
+
+template <typename E, int DH, int QT, int NACC>
+FM_DEVICE void fm_readout_sym(const E* FM_RESTRICT state, bool quad, const E* xs, const int* xrow,
+                              const typename Mma<E>::frag (*yb)[TokCfg<E, DH, QT>::NKS],
+                              E* slab, fm_f32x16 (*acc)[NACC], int tid) {
+  typedef TokCfg<E, DH, QT> C;
+  typedef Mma<E> M;
+  const int lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int lane_off = lr * C::PS + lh * M::KPL;
+  int buf = 0;
+  if (quad) {
+    TileRegs<E, C::SA * DH, DH> first;
+    first.load(state, DH, tid);
+    fm_readout_sym_block<E, DH, QT, NACC, 0>(state, first, xs, xrow, yb, slab, acc, tid, lane_off, buf);
+  } else {
+    // `state` is the order-1 slab itself
+    TileRegs<E, DH, DH> one;
+    one.load(state, DH, tid);
+    one.store(slab, C::PS, tid);
+    FM_SYNC();
+    fm_readout_products<E, DH, QT, NACC, 0>(slab, xs, xrow, DH, 1, true, yb, acc, lane_off);
+  }
+  FM_SYNC();
+}
+
 // ------------------------------------------------------------------------------
 // k_probe_mfma: one wavefront; A[i][k] = i + 1 (k = 0) else 0 ... chosen so that
 // D[i][j] = (i + 1) * 100 + (j + 1) identifies which (row, col) every lane/register

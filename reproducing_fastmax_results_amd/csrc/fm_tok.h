@@ -336,7 +336,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
           for (int i = 0; i < M::KPL; ++i) gsum[j] += vecs[ks * M::KSTEP + lh * M::KPL + i] * M::elem(of[j][ks], i);
     }
     const E* state = A.big + (int64_t(bh) * A.nslots + G.slot) * StateDims<DH>::stride(A.quad != 0);
-    fm_readout<E, DH, QT, NT>(state, A.quad != 0, Own, xrow, of, R, acc, tid);
+    fm_readout_sym<E, DH, QT, NT>(state, A.quad != 0, Own, xrow, of, R, acc, tid);   // x = y = the own rows, sums symmetric in (a, b)
   } else {
     FM_SYNC();                                         // own rows are overwritten by the dense stages
   }
