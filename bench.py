@@ -58,7 +58,7 @@ LONG_WORKLOAD = dict(name="configs[2]: causal long-context fwd+bwd", B=1, H=16, 
 # With moment states: two state walks (forward, backward) of one unit each, the readouts one
 # each, and dQ also carries the unit of the prefix rebuild it is spared by reading the forward's.
 # Without (a sequence short enough for one segment) each kernel carries its walk as well.
-UNITS_STATE = {"build": 1, "fwd": 1, "dq": 2, "dk": 1, "dv": 1}
+UNITS_STATE = {"build": 1, "fwd": 1, "dq": 2, "dk": 1, "dv": 1, "dkv": 2}
 UNITS_DENSE = {"fwd": 2, "dq": 2, "dk": 2, "dv": 1, "dkv": 3}
 # 32x32x16 MFMA instructions per 32x32 score tile in the dense loops of each kernel
 MFMA_PER_TILE = {"fwd": 8, "dv": 8, "dq": 12, "dk": 12, "dkv": 16}

@@ -335,7 +335,7 @@ int launch_build(const BuildArgs<E>& args, int bh, fm_stream_t stream) {
 }
 
 // Dynamic LDS of a token kernel (kind 0: k_pv, 1: k_ds, 2: k_ds with dV, 3: k_ds with the fused
-// preparation): va, vb | own rows | region, where the dense stages and the output staging lie over
+// preparation, 4: k_ds with dV and states): va, vb | own rows | region, where the dense stages and the output staging lie over
 // the own rows and the region.
 template <typename E, int DH, int QT> size_t tok_lds_bytes(int kind) {
   typedef TokCfg<E, DH, QT> C;
@@ -345,7 +345,8 @@ template <typename E, int DH, int QT> size_t tok_lds_bytes(int kind) {
   size_t body = size_t(C::QW) * C::PQ * sizeof(E) + region;
   const size_t outst = size_t(C::QW) * (DH + 1) * 4;
   const size_t stage = kind == 0 ? size_t(2) * C::PV_STAGE * sizeof(E)
-                                 : size_t(C::DS_NBUF) * (kind == 2 ? C::DV_STAGE : C::DS_STAGE) * sizeof(E);
+                                 : size_t(C::DS_NBUF) * (kind == 2 || kind == 4 ? C::DV_STAGE : C::DS_STAGE) * sizeof(E);
+  if (kind == 4) body += size_t(C::QW) * (DH + 1) * 4;      // dK of the fused state readout, behind the slabs
   const size_t prep = size_t(2) * C::QW * C::PQ * sizeof(E) + size_t(C::QW) * 4;   // own q' rows, gh rows, c
   if (outst > body) body = outst;
   if (stage > body) body = stage;
@@ -363,7 +364,7 @@ const NormFold no_fold{nullptr, 0, 1.0f};
 template <typename TIO, typename E> void tok_common(TokArgs<TIO, E>& a, const FastmaxDesc* d, const Plan& p) {
   a.own_fold = no_fold; a.out_fold = no_fold; a.brows = nullptr; a.bpart = nullptr;
   a.own_io = TRef<const TIO>{nullptr, 0, 0, 0, 0, 0};
-  a.own_r = nullptr; a.own2_r = nullptr; a.cv = nullptr; a.xr = nullptr; a.yr = nullptr; a.zt = nullptr; a.zt2 = nullptr;
+  a.own_r = nullptr; a.own2_r = nullptr; a.cv = nullptr; a.xr = nullptr; a.yr = nullptr; a.zt = nullptr; a.zt2 = nullptr; a.bigb = nullptr;
   a.out2 = TRef<TIO>{nullptr, 0, 0, 0, 0, 0}; a.out2_scale = 1.0f;
   a.g = TRef<float>{nullptr, 0, 0, 0, 0, 0};
   a.nslots = p.nslots; a.L = p.L; a.nseg = p.nseg; a.causal = d->mask != 0; a.use_state = p.use_state;
@@ -386,7 +387,7 @@ int launch_pv(const TokArgs<TIO, E>& a, int bh, int kernel_id, fm_stream_t strea
 template <typename TIO, typename E, int DH, int QT, int OWN, int DV = 0, int PREP = 0, int QF = 0>
 int launch_ds(const TokArgs<TIO, E>& a, int bh, int kernel_id, fm_stream_t stream) {
   typedef TokCfg<E, DH, QT> C;
-  const size_t lds = tok_lds_bytes<E, DH, QT>(PREP ? 3 : (DV ? 2 : 1));
+  const size_t lds = tok_lds_bytes<E, DH, QT>(PREP ? 3 : (DV ? (a.use_state ? 4 : 2) : 1));
   fm_allow_lds(reinterpret_cast<const void*>(&k_ds<TIO, E, DH, QT, OWN, DV, PREP, QF>), lds);
   ProfScope prof(kernel_id, stream);
   FM_KERNEL_LAUNCH((k_ds<TIO, E, DH, QT, OWN, DV, PREP, QF>), fm_dim3((a.n_own + C::QW - 1) / C::QW, bh), fm_dim3(FM_THREADS), lds,

@@ -35,6 +35,7 @@ template <typename TIO, typename E> struct TokArgs {
   const E* zt2;             // k_ds with dV: gh transposed           [bh][DH][npad_str]
   int npad_own, npad_str;
   const E* big; const float* small; int nslots;
+  const E* bigb;            // k_ds with dV and order-2 states: the tile-transposed copy of `big` (dV's layout)
   TRef<TIO> out;
   TRef<TIO> out2;           // k_ds with dV: dV
   TRef<float> g;                        // k_pv, own = queries: denominators (bh, n)
@@ -475,6 +476,64 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
 }
 
 // ------------------------------------------------------------------------------
+// Order-2 suffix state read once for dK and dV of the own keys (one 32-token tile per wavefront).  With
+// U[a][c][b] = a2 sum_i q'_a gh_c q'_b (the transposed-tile copy of the state, slab a = rows c, columns b):
+//   Y_a[c] = sum_b U[a][c][b] k'_b            8 matrix instructions per slab, B fragments = the key's own rows
+//   dV[c] += k'_a Y_a[c]                      the accumulator entries of the lane, fp32
+//   dK[a]  = 2 sum_c v_c Y_a[c]               v in accumulator layout; the two halves of a wavefront hold 32 values of c
+//                                             each and meet through one cross-lane add; the sum goes to dks[token][a]
+// which is half of the matrix instructions of the two separate readouts (8 instead of 8 + 5 per slab and tile), no
+// Khatri-Rao products, and one staging of the state instead of two.
+// slab: two buffers of DH * PS elements; dks: [QW][DH + 1] floats, rows of the wavefront's own tokens only (no barrier
+// between its writes here and the reads of the same wavefront later).  All 256 threads must call this.
+// ------------------------------------------------------------------------------
+template <typename E, int DH>
+FM_DEVICE void fm_readout_kv(const E* FM_RESTRICT state2, const E* xs, int xrow, const typename Mma<E>::frag* kf,
+                             const float (*vacc)[16], E* slab, float* dks, fm_f32x16* av, int tid) {
+  typedef TokCfg<E, DH, 1> C;
+  typedef Mma<E> M;
+  typedef typename M::frag frag;
+  constexpr int NT = C::NT, NKS = C::NKS, PS = C::PS;
+  constexpr int SLAB1 = DH * PS;
+  const int lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int lane_off = lr * PS + lh * M::KPL;
+  TileRegs<E, DH, DH> regs;
+  regs.load(state2, DH, tid);
+  int buf = 0;
+  float ka = float(xs[xrow * C::PQ]);
+  for (int a = 0; a < DH; ++a) {
+    E* sb = slab + buf * SLAB1;
+    regs.store(sb, PS, tid);
+    FM_SYNC();
+    const int an = a + 1 < DH ? a + 1 : a;
+    if (a + 1 < DH) regs.load(state2 + int64_t(a + 1) * DH * DH, DH, tid);
+    const float kan = float(xs[xrow * C::PQ + an]);
+    frag fa[NT][NKS];
+#pragma unroll
+    for (int ct = 0; ct < NT; ++ct)
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) fa[ct][ks] = M::load(sb + lane_off + (32 * ct) * PS + ks * M::KSTEP);
+    float dot = 0.f;
+#pragma unroll
+    for (int ct = 0; ct < NT; ++ct) {
+      fm_f32x16 y = fm_zero16();
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) y = M::mma(fa[ct][ks], kf[ks], y);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        av[ct][e] += ka * y[e];
+        dot += vacc[ct][e] * y[e];
+      }
+    }
+    dot += fm_shfl_xor(dot, 32);
+    if (lh == 0) dks[xrow * (DH + 1) + a] = 2.0f * dot;
+    ka = kan;
+    buf ^= 1;
+  }
+  FM_SYNC();
+}
+
+// ------------------------------------------------------------------------------
 // k_ds: dQ (own = queries) and dK (own = keys).  grid (ceil(n_own / QW), bh).
 // LDS: va, vb | own rows [QW][PQ] | region (Z, then state slabs); the dense stages
 // (stream rows for the scores, stream rows for gh.v, stream transposed, c values)
@@ -635,7 +694,48 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
       }
     FM_SYNC();                                         // Z is overwritten by the slabs
     const E* state = A.big + (int64_t(bh) * A.nslots + G.slot) * StateDims<DH>::stride(A.quad != 0);
-    fm_readout<E, DH, QT, NT>(state, A.quad != 0, Own, xrow, of2, R, acc, tid);
+    if constexpr (DV != 0 && QT == 1 && sizeof(E) == 2) {
+      // dK and dV from one pass over the order-2 state (the host launches this instantiation with states only for
+      // order 2); then the two order-1 slabs, each in its own layout, staged side by side
+      const E* state2 = A.bigb + (int64_t(bh) * A.nslots + G.slot) * StateDims<DH>::stride(true);
+      float* dks = reinterpret_cast<float*>(R + 2 * C::SLAB);
+      float vacc[NT][16];
+      {
+        const E* vrow = A.own2_r + (int64_t(bh) * A.npad_own + t0 + xrow[0]) * DH;
+#pragma unroll
+        for (int ct = 0; ct < NT; ++ct)
+#pragma unroll
+          for (int g4 = 0; g4 < 4; ++g4) {
+            struct alignas(8) Four { E v[4]; };
+            const Four f = *reinterpret_cast<const Four*>(vrow + 32 * ct + fm_acc_row(4 * g4, lh));
+#pragma unroll
+            for (int u = 0; u < 4; ++u) vacc[ct][4 * g4 + u] = float(f.v[u]);
+          }
+      }
+      fm_readout_kv<E, DH>(state2, Own, xrow[0], of[0], vacc, R, dks, av[0], tid);
+      {
+        TileRegs<E, DH, DH> s1, s1b;
+        s1.load(state + int64_t(DH) * DH * DH, DH, tid);
+        s1b.load(state2 + int64_t(DH) * DH * DH, DH, tid);
+        s1.store(R, C::PS, tid);
+        s1b.store(R + C::SLAB, C::PS, tid);
+        FM_SYNC();
+        const int lane_off = lr * C::PS + lh * M::KPL;
+#pragma unroll
+        for (int mt = 0; mt < NT; ++mt) {
+#pragma unroll
+          for (int ks = 0; ks < NKS; ++ks) {
+            acc[0][mt] = M::mma(M::load(R + lane_off + (32 * mt) * C::PS + ks * M::KSTEP), of2[0][ks], acc[0][mt]);
+            av[0][mt] = M::mma(M::load(R + C::SLAB + lane_off + (32 * mt) * C::PS + ks * M::KSTEP), of[0][ks], av[0][mt]);
+          }
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc[0][mt][e] += dks[xrow[0] * (DH + 1) + 32 * mt + fm_acc_row(e, lh)];
+        }
+        FM_SYNC();                                     // the slabs and dks are overwritten by the dense stages
+      }
+    } else {
+      fm_readout<E, DH, QT, NT>(state, A.quad != 0, Own, xrow, of2, R, acc, tid);
+    }
   } else {
     FM_SYNC();                                         // own rows are overwritten by the dense stages
   }
@@ -774,6 +874,6 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
                                     A.n_own, tid, brows, fac > 0.f ? 1.0f / (fac * A.sc) : 0.f, bout);
   }
   if (DV)
-    fm_store_tokens<TIO, E, DH, QT>(av, xrow, nullptr, A.out2_scale * ginv_sc * (QF ? 1.0f / (4.0f * A.a2) : 1.0f),
+    fm_store_tokens<TIO, E, DH, QT>(av, xrow, G.use_state ? vecs + DH : nullptr, A.out2_scale * ginv_sc * (QF ? 1.0f / (4.0f * A.a2) : 1.0f),
                                     reinterpret_cast<float*>(Own), A.out2, bh, t0, A.n_own, tid);
 }
