@@ -45,8 +45,8 @@ PEAK_HBM_GBS = 8000.0
 TRAFFIC = {
     (4096, 2, "bf16", 0, "dkv"): {"bytes": (44092 * 2 + 32770) * 1024, "source": "profiles/c2_bf16_hbm_traffic.md"},
     (65536, 1, "bf16", 0, "dkv"): {"bytes": (402970 * 2 + 393240) * 1024, "source": "profiles/long_order1_bf16_hbm_traffic.md"},
-    (65536, 2, "bf16", 0, "build"): {"bytes": (161374 * 2 + 982214) * 1024, "source": "profiles/long_order2_bf16_hbm_traffic.md"},
-    (65536, 2, "bf16", 0, "dk"): {"bytes": (619174 * 2 + 199579) * 1024, "source": "profiles/long_order2_bf16_hbm_traffic.md"},
+    (65536, 2, "bf16", 0, "build"): {"bytes": (160828 * 2 + 982268) * 1024, "source": "profiles/long_order2_bf16_hbm_traffic.md"},
+    (65536, 2, "bf16", 0, "dkv"): {"bytes": (564148 * 2 + 262171) * 1024, "source": "profiles/long_order2_bf16_hbm_traffic.md"},
 }
 
 WORKLOAD = dict(name="configs[1]: causal order-2 fwd+bwd", B=4, H=8, N=4096, D=64, p=2, mask=True, scale=1.0)

@@ -300,6 +300,7 @@ int launch_build(const BuildArgs<E>& args, int bh, fm_stream_t stream) {
     // B*H = 32, N = 4096, D = 64).
     constexpr int G = DH / 4;
     a.seg_parallel = nsteps > 1 && bh * G < 256;
+    if (a.seg_parallel) a.skip_big = 0;                // the scan that follows treats both copies alike
     // the one-workgroup-per-CU variant on _Float16: 128-token tiles, all eight k-steps of fragments requested at once
     constexpr int TTS = sizeof(E) == 2 ? 128 : 64;
     constexpr int KBS = sizeof(E) == 2 ? 8 : 4;
@@ -421,7 +422,7 @@ int o1_key_sums(const FastmaxDesc* d, const Plan& p, const void* k, const void* 
   a.scale0 = p.sc; a.fold0 = k_fold(d); a.gpart = nullptr; a.gnblk = 0; a.n = d->nk; a.runtot = runtot; a.run_len = p.o1_run;
   BuildArgs<fm_half>& b = a.b;
   b.xt = nullptr; b.pt = nullptr; b.rt = nullptr; b.zt = nullptr; b.pr = nullptr; b.rr = nullptr; b.cw = nullptr;
-  b.za_sel = FM_SRC_R; b.zb_sel = FM_SRC_R; b.vb_from_r = 0; b.seg_parallel = 1;
+  b.za_sel = FM_SRC_R; b.zb_sel = FM_SRC_R; b.vb_from_r = 0; b.seg_parallel = 1; b.skip_big = 0;
   b.npad = p.npad_k; b.nseg = p.nseg; b.L = p.L; b.mode = FM_WALK_PREFIX; b.quad = 0;
   b.big = big; b.big2 = nullptr; b.small = small; b.nslots = p.nslots;
   b.coef2 = 0.f; b.coef2b = 0.f; b.coefz = 0.f; b.coef1 = p.a1; b.coef1b = p.a1; b.coefva = p.a1; b.coefvb = p.a0;
@@ -470,7 +471,7 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   if (st) return st;
   if (p.use_state) {
     BuildArgs<E> b;
-    b.seg_parallel = 0;
+    b.seg_parallel = 0; b.skip_big = 0;
     b.xt = kt; b.pt = vt; b.rt = kt; b.zt = nullptr; b.za_sel = FM_SRC_R; b.zb_sel = FM_SRC_R;
     b.pr = p.rows_build ? vr : nullptr; b.rr = p.rows_build ? kr : nullptr; b.cw = nullptr;
     b.npad = p.npad_k; b.nseg = p.nseg; b.L = p.L; b.mode = d->mask ? FM_WALK_PREFIX : FM_WALK_TOTAL;

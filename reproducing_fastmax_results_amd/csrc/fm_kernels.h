@@ -454,6 +454,8 @@ template <typename E> struct BuildArgs {
   int vb_from_r;                           // vb sums the r operand instead of p
   float coef2, coef1, coefz, coefva, coefvb;
   float coef2b, coef1b;                    // coefficients of the transposed copy
+  int skip_big;                            // order 2: the snapshot goes to big2 only (nobody reads the first layout); the
+                                           // order-1 tile and the lower-order sums are written as always
   int seg_parallel;                        // grid z = walk step: every workgroup sums one segment only and
                                            // k_state_scan turns the per-segment sums into prefix / suffix states
   // Order-1 sums from row-major operands (k_build1_rows; null: the transposed operands above are read):
@@ -634,24 +636,26 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (NA == 1 && sizeof(E) == 2 && SPW <
       constexpr int VEC = M::VEC;
       E* stg = reinterpret_cast<E*>(mem);                  // [AW][DH][SP]
       FM_SYNC();
+      if (!A.skip_big) {
 #pragma unroll
-      for (int i = 0; i < NA; ++i)
+        for (int i = 0; i < NA; ++i)
 #pragma unroll
-        for (int j = 0; j < NT; ++j)
+          for (int j = 0; j < NT; ++j)
 #pragma unroll
-          for (int k = 0; k < NT; ++k)
+            for (int k = 0; k < NT; ++k)
 #pragma unroll
-            for (int e = 0; e < 16; ++e)
-              stg[((wave * NA + i) * DH + 32 * j + fm_acc_row(e, lh)) * SP + 32 * k + lr] =
-                  CE<E>::from(A.coef2 * acc[i][j][k][e]);
-      FM_SYNC();
-      E* dst = big + int64_t(slot) * StateDims<DH>::BIG + int64_t(a0) * DH * DH;
-      for (int c = tid; c < AW * DH * (DH / VEC); c += FM_THREADS) {
-        const int row = c / (DH / VEC), col = (c % (DH / VEC)) * VEC;
-        *reinterpret_cast<fm_u32x4*>(dst + row * DH + col) = *reinterpret_cast<const fm_u32x4*>(stg + row * SP + col);
+              for (int e = 0; e < 16; ++e)
+                stg[((wave * NA + i) * DH + 32 * j + fm_acc_row(e, lh)) * SP + 32 * k + lr] =
+                    CE<E>::from(A.coef2 * acc[i][j][k][e]);
+        FM_SYNC();
+        E* dst = big + int64_t(slot) * StateDims<DH>::BIG + int64_t(a0) * DH * DH;
+        for (int c = tid; c < AW * DH * (DH / VEC); c += FM_THREADS) {
+          const int row = c / (DH / VEC), col = (c % (DH / VEC)) * VEC;
+          *reinterpret_cast<fm_u32x4*>(dst + row * DH + col) = *reinterpret_cast<const fm_u32x4*>(stg + row * SP + col);
+        }
+        if (big2) FM_SYNC();
       }
       if (big2) {
-        FM_SYNC();
 #pragma unroll
         for (int i = 0; i < NA; ++i)
 #pragma unroll
