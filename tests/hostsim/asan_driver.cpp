@@ -34,8 +34,23 @@ static int run(int bh, int n, int d, int p, int chunk, int dtype, int save) {
   printf("bh=%d n=%d d=%d p=%d chunk=%d dtype=%d save=%d -> status %d, sum g %.3f\n", bh, n, d, p, chunk, dtype, save, st, sum);
   return st;
 }
+// the two element-wise passes (key RPE, output noise) on a ragged shape, in place
+static int run_pointwise(int bh, int n, int d, int dtype) {
+  FastmaxNormDesc N{};
+  N.bh = bh; N.n = n; N.d = d; N.dtype = dtype;
+  N.sx.bh = int64_t(n) * d; N.sx.n = d; N.sy = N.sx;
+  const size_t esz = dtype == FASTMAX_BF16 ? 2 : 4;
+  std::vector<unsigned char> x(size_t(bh) * n * d * esz, 0), noise(x.size(), 0);
+  std::vector<float> rpe(size_t(2 * n - 1) * d, 0.25f);
+  int st = fastmax_key_rpe(&N, x.data(), rpe.data(), x.data(), 2.0f, nullptr);
+  if (!st) st = fastmax_output_noise(&N, x.data(), noise.data(), x.data(), 0.5f, nullptr);
+  printf("pointwise bh=%d n=%d d=%d dtype=%d -> status %d\n", bh, n, d, dtype, st);
+  return st;
+}
 int main() {
   int bad = 0;
+  bad |= run_pointwise(3, 333, 64, FASTMAX_BF16);
+  bad |= run_pointwise(2, 70, 32, FASTMAX_F32);
   bad |= run(1, 600, 32, 2, 256, FASTMAX_BF16, 1);    // order-2 walk (a CU to itself: two buffers), both walks
   bad |= run(1, 600, 32, 2, 256, FASTMAX_BF16, 0);
   bad |= run(1, 520, 64, 2, 256, FASTMAX_BF16, 1);
