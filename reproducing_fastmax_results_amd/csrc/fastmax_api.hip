@@ -340,7 +340,7 @@ int launch_build(const BuildArgs<E>& args, int bh, fm_stream_t stream) {
 // the own rows and the region.
 template <typename E, int DH, int QT> size_t tok_lds_bytes(int kind) {
   typedef TokCfg<E, DH, QT> C;
-  size_t region = size_t(2) * C::SLAB * sizeof(E);
+  size_t region = size_t(2) * (kind == 0 ? C::SLAB_SYM : C::SLAB) * sizeof(E);   // k_pv reads its states with fm_readout_sym
   const size_t zs = size_t(C::NZ) * DH * C::PS * sizeof(E);
   if (zs > region) region = zs;
   size_t body = size_t(C::QW) * C::PQ * sizeof(E) + region;

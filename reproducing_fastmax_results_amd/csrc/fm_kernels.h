@@ -1295,6 +1295,8 @@ struct TokCfg {
   static constexpr int PV_DV = KT_DV + M::PAD;
   static constexpr int NZ = sizeof(E) == 2 ? 2 : 1; // hi/lo split of fp32 denominators
   static constexpr int SLAB = SA * DH * PS;         // elements per slab buffer
+  // the symmetric readout's narrow blocks stage twice the values of a in compact rows (see SymBlk)
+  static constexpr int SLAB_SYM = (sizeof(E) == 2 && 2 * SA * DH * (DH / 2 + M::PAD) > SLAB) ? 2 * SA * DH * (DH / 2 + M::PAD) : SLAB;
   static constexpr int PV_STAGE = M::HAS_TR ? 2 * KT_PV * PQ : KT_PV * PQ + DH * PV_PV;   // k_pv: two row tiles, or stream rows + stream transposed
   // c values of a stage: KT compute-type elements, or KT floats (the completed-square kernels stage -c in fp32)
   static constexpr int DS_STAGE = 2 * KT_DS * PQ + (M::HAS_TR ? 0 : DH * PV_DS) + (M::HAS_TR ? 2 : 1) * KT_DS;   // k_ds: two row tiles, (transposed tile,) c values
@@ -1374,20 +1376,32 @@ FM_DEVICE void fm_readout(const E* FM_RESTRICT state, bool quad, const E* xs, co
 // q, and the (q, gh, q) sums dV reads with k): sum_{a, b} = the 16 x 16 blocks on the diagonal of (a, b) once plus
 // twice the blocks above it, so a value of `a` in block KB meets the k-steps KB .. NKS - 1 only -- 10 of 16
 // products and 10 of 16 bytes of every slab, whose unused columns are neither loaded nor staged.
+// Blocks of half the full width or less hold twice the values of `a` per slab, in compact rows (as many bytes per
+// stage as the full-width slabs: the barrier and the slab's way into LDS are paid per stage).
 constexpr int FM_SYM_BLOCK = 16;
-template <typename E, int DH, int QT, int NACC, int KB>
+template <typename E, int DH, int QT, int KB> struct SymBlk {
+  typedef TokCfg<E, DH, QT> C;
+  static constexpr int C0 = KB * FM_SYM_BLOCK, W = DH - C0;             // first column and columns met
+  static constexpr bool TALL = sizeof(E) == 2 && 2 * W <= DH;
+  static constexpr int SAB = TALL ? 2 * C::SA : C::SA;                  // values of a per slab
+  static constexpr int PSB = TALL ? W + Mma<E>::PAD : C::PS;            // row pitch of the staged slab
+  static constexpr int OFF = TALL ? 0 : C0;                             // where column C0 lies in a staged row
+  static_assert(SAB * DH * PSB <= C::SLAB_SYM, "a slab fits its buffer");
+};
+// products of one staged slab: values as .. as + na - 1 of a (rows [al][c] at pitch PSB, column C0 at OFF)
+template <typename E, int DH, int QT, int NACC, int KB, int PSB, int OFF>
 FM_DEVICE void fm_readout_products(const E* sb, const E* xs, const int* xrow, int as, int na, bool ones,
                                    const typename Mma<E>::frag (*yb)[TokCfg<E, DH, QT>::NKS], fm_f32x16 (*acc)[NACC],
-                                   int lane_off) {
+                                   int lr, int lh) {
   typedef TokCfg<E, DH, QT> C;
   typedef Mma<E> M;
   typedef typename M::frag frag;
   constexpr int KPB = FM_SYM_BLOCK / M::KSTEP;       // k-steps per block of (a, b)
   constexpr int K0 = KB * KPB;                       // first k-step met
-  const E* sl = sb + lane_off;
+  const E* sl = sb + lr * PSB + lh * M::KPL + OFF - K0 * M::KSTEP;      // column col of row 0 of the lane: sl + col
   frag fa[C::NT];
 #pragma unroll
-  for (int ct = 0; ct < C::NT; ++ct) fa[ct] = M::load(sl + (32 * ct) * C::PS + K0 * M::KSTEP);
+  for (int ct = 0; ct < C::NT; ++ct) fa[ct] = M::load(sl + (32 * ct) * PSB + K0 * M::KSTEP);
   E xv[QT];
 #pragma unroll
   for (int j = 0; j < QT; ++j) xv[j] = ones ? E(1.0f) : xs[xrow[j] * C::PQ + as];
@@ -1404,7 +1418,7 @@ FM_DEVICE void fm_readout_products(const E* sb, const E* xs, const int* xrow, in
       const int nal = (ks + 1 < C::NKS) ? al : (al + 1 < na ? al + 1 : al);
       frag fn[C::NT];
 #pragma unroll
-      for (int ct = 0; ct < C::NT; ++ct) fn[ct] = M::load(sl + (nal * DH + 32 * ct) * C::PS + nks * M::KSTEP);
+      for (int ct = 0; ct < C::NT; ++ct) fn[ct] = M::load(sl + (nal * DH + 32 * ct) * PSB + nks * M::KSTEP);
 #pragma unroll
       for (int j = 0; j < QT; ++j) {
         const frag fb = yb[j][ks] * (ks < K0 + KPB ? xr[j] : xr2[j]);
@@ -1418,32 +1432,36 @@ FM_DEVICE void fm_readout_products(const E* sb, const E* xs, const int* xrow, in
 }
 
 template <typename E, int DH, int QT, int NACC, int KB>
-FM_DEVICE void fm_readout_sym_block(const E* FM_RESTRICT state, TileRegs<E, TokCfg<E, DH, QT>::SA * DH, DH - KB * FM_SYM_BLOCK>& cur,
+FM_DEVICE void fm_readout_sym_block(const E* FM_RESTRICT state,
+                                    TileRegs<E, SymBlk<E, DH, QT, KB>::SAB * DH, SymBlk<E, DH, QT, KB>::W>& cur,
                                     const E* xs, const int* xrow, const typename Mma<E>::frag (*yb)[TokCfg<E, DH, QT>::NKS],
-                                    E* slab, fm_f32x16 (*acc)[NACC], int tid, int lane_off, int& buf) {
+                                    E* slab, fm_f32x16 (*acc)[NACC], int tid, int& buf) {
   typedef TokCfg<E, DH, QT> C;
   typedef Mma<E> M;
-  constexpr int C0 = KB * FM_SYM_BLOCK, A_END = C0 + FM_SYM_BLOCK;
+  typedef SymBlk<E, DH, QT, KB> B;
+  constexpr int C0 = B::C0, A_END = C0 + FM_SYM_BLOCK;
   constexpr bool LASTB = A_END == DH;
-  static_assert(FM_SYM_BLOCK % C::SA == 0 && FM_SYM_BLOCK % M::KSTEP == 0 && DH % FM_SYM_BLOCK == 0, "whole slabs and k-steps per block");
+  static_assert(FM_SYM_BLOCK % B::SAB == 0 && FM_SYM_BLOCK % M::KSTEP == 0 && DH % FM_SYM_BLOCK == 0, "whole slabs and k-steps per block");
+  typedef SymBlk<E, DH, QT, LASTB ? 0 : KB + 1> BN;
+  const int lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   // after the last block: the order-1 slab (DH rows, every column)
-  TileRegs<E, LASTB ? DH : C::SA * DH, LASTB ? DH : DH - A_END> nxt;
-  for (int as = C0; as < A_END; as += C::SA) {
-    E* sb = slab + buf * C::SLAB;
-    cur.store(sb + C0, C::PS, tid);
+  TileRegs<E, LASTB ? DH : BN::SAB * DH, LASTB ? DH : BN::W> nxt;
+  for (int as = C0; as < A_END; as += B::SAB) {
+    E* sb = slab + buf * C::SLAB_SYM;
+    cur.store(sb + B::OFF, B::PSB, tid);
     FM_SYNC();
-    if (as + C::SA < A_END) cur.load(state + int64_t(as + C::SA) * DH * DH + C0, DH, tid);
-    else nxt.load(state + int64_t(as + C::SA) * DH * DH + (LASTB ? 0 : A_END), DH, tid);
-    fm_readout_products<E, DH, QT, NACC, KB>(sb, xs, xrow, as, C::SA, false, yb, acc, lane_off);
+    if (as + B::SAB < A_END) cur.load(state + int64_t(as + B::SAB) * DH * DH + C0, DH, tid);
+    else nxt.load(state + int64_t(as + B::SAB) * DH * DH + (LASTB ? 0 : A_END), DH, tid);
+    fm_readout_products<E, DH, QT, NACC, KB, B::PSB, B::OFF>(sb, xs, xrow, as, B::SAB, false, yb, acc, lr, lh);
     buf ^= 1;
   }
   if constexpr (!LASTB) {
-    fm_readout_sym_block<E, DH, QT, NACC, KB + 1>(state, nxt, xs, xrow, yb, slab, acc, tid, lane_off, buf);
+    fm_readout_sym_block<E, DH, QT, NACC, KB + 1>(state, nxt, xs, xrow, yb, slab, acc, tid, buf);
   } else {
-    E* sb = slab + buf * C::SLAB;
+    E* sb = slab + buf * C::SLAB_SYM;
     nxt.store(sb, C::PS, tid);
     FM_SYNC();
-    fm_readout_products<E, DH, QT, NACC, 0>(sb, xs, xrow, DH, 1, true, yb, acc, lane_off);
+    fm_readout_products<E, DH, QT, NACC, 0, C::PS, 0>(sb, xs, xrow, DH, 1, true, yb, acc, lr, lh);
   }
 }
 
@@ -1452,21 +1470,19 @@ FM_DEVICE void fm_readout_sym(const E* FM_RESTRICT state, bool quad, const E* xs
                               const typename Mma<E>::frag (*yb)[TokCfg<E, DH, QT>::NKS],
                               E* slab, fm_f32x16 (*acc)[NACC], int tid) {
   typedef TokCfg<E, DH, QT> C;
-  typedef Mma<E> M;
   const int lane = tid & 63, lr = lane & 31, lh = lane >> 5;
-  const int lane_off = lr * C::PS + lh * M::KPL;
   int buf = 0;
   if (quad) {
-    TileRegs<E, C::SA * DH, DH> first;
+    TileRegs<E, SymBlk<E, DH, QT, 0>::SAB * DH, DH> first;
     first.load(state, DH, tid);
-    fm_readout_sym_block<E, DH, QT, NACC, 0>(state, first, xs, xrow, yb, slab, acc, tid, lane_off, buf);
+    fm_readout_sym_block<E, DH, QT, NACC, 0>(state, first, xs, xrow, yb, slab, acc, tid, buf);
   } else {
     // `state` is the order-1 slab itself
     TileRegs<E, DH, DH> one;
     one.load(state, DH, tid);
     one.store(slab, C::PS, tid);
     FM_SYNC();
-    fm_readout_products<E, DH, QT, NACC, 0>(slab, xs, xrow, DH, 1, true, yb, acc, lane_off);
+    fm_readout_products<E, DH, QT, NACC, 0, C::PS, 0>(slab, xs, xrow, DH, 1, true, yb, acc, lr, lh);
   }
   FM_SYNC();
 }
