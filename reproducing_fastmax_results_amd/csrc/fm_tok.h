@@ -795,11 +795,36 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
         fm_f32x16 s[QT];
 #pragma unroll
         for (int j = 0; j < QT; ++j) s[j] = QF ? sseed : fm_zero16();
+        // One tile per wavefront: the score products and the gh.v products are two chains of dependent matrix
+        // instructions that do not depend on each other; issued in turn, each hides the other's latency.
+        fm_f32x16 dp1 = fm_zero16();
+        if constexpr (QT == 1) {
+          if constexpr (QF != 0) {
+            if (OWN == FM_OWN_Q) dp1 = dpseed;
+            else {
+              // -c of the tile's 32 queries, the lane's 16 accumulator rows: four 16-byte reads
+              const float* cf = reinterpret_cast<const float*>(cs) + 32 * st + 4 * lh;
 #pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) {
-          const frag xf = M::load(Xs + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL);
+              for (int gq = 0; gq < 4; ++gq) {
+                const fm_f32x4 t = *reinterpret_cast<const fm_f32x4*>(cf + 8 * gq);
+                dp1[4 * gq] = t[0]; dp1[4 * gq + 1] = t[1]; dp1[4 * gq + 2] = t[2]; dp1[4 * gq + 3] = t[3];
+              }
+            }
+          }
 #pragma unroll
-          for (int j = 0; j < QT; ++j) s[j] = M::mma(xf, of[j][ks], s[j]);
+          for (int ks = 0; ks < NKS; ++ks) {
+            const frag xf = M::load(Xs + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL);
+            const frag yf = M::load(Ys + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL);
+            s[0] = M::mma(xf, of[0][ks], s[0]);
+            dp1 = M::mma(yf, of2[0][ks], dp1);
+          }
+        } else {
+#pragma unroll
+          for (int ks = 0; ks < NKS; ++ks) {
+            const frag xf = M::load(Xs + (32 * st + lr) * PQ + ks * M::KSTEP + lh * M::KPL);
+#pragma unroll
+            for (int j = 0; j < QT; ++j) s[j] = M::mma(xf, of[j][ks], s[j]);
+          }
         }
         frag zf[NT][M::ACC_KSTEPS], crow[M::ACC_KSTEPS];
 #pragma unroll
@@ -826,22 +851,24 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
           const bool edge = fm_tile_edge<OWN>(causal, ss0, lo, A.n_str);
           int wlo, whi;
           fm_tile_window<OWN>(causal, ss0, lo, lr, A.n_str, wlo, whi);
-          fm_f32x16 dp = fm_zero16();
-          if constexpr (QF != 0) {
-            if (OWN == FM_OWN_Q) dp = dpseed;
-            else {
-              // -c of the tile's 32 queries, the lane's 16 accumulator rows: four 16-byte reads
-              const float* cf = reinterpret_cast<const float*>(cs) + 32 * st + 4 * lh;
+          fm_f32x16 dp = dp1;
+          if constexpr (QT > 1) {
+            if constexpr (QF != 0) {
+              if (OWN == FM_OWN_Q) dp = dpseed;
+              else {
+                // -c of the tile's 32 queries, the lane's 16 accumulator rows: four 16-byte reads
+                const float* cf = reinterpret_cast<const float*>(cs) + 32 * st + 4 * lh;
 #pragma unroll
-              for (int gq = 0; gq < 4; ++gq) {
-                const fm_f32x4 t = *reinterpret_cast<const fm_f32x4*>(cf + 8 * gq);
-                dp[4 * gq] = t[0]; dp[4 * gq + 1] = t[1]; dp[4 * gq + 2] = t[2]; dp[4 * gq + 3] = t[3];
+                for (int gq = 0; gq < 4; ++gq) {
+                  const fm_f32x4 t = *reinterpret_cast<const fm_f32x4*>(cf + 8 * gq);
+                  dp[4 * gq] = t[0]; dp[4 * gq + 1] = t[1]; dp[4 * gq + 2] = t[2]; dp[4 * gq + 3] = t[3];
+                }
               }
             }
-          }
-          const E* yrow = Ys + (32 * st + lr) * PQ + lh * M::KPL + (QT > 1 ? FM_OPAQUE_ZERO() : 0);
+            const E* yrow = Ys + (32 * st + lr) * PQ + lh * M::KPL + FM_OPAQUE_ZERO();
 #pragma unroll
-          for (int ks = 0; ks < NKS; ++ks) dp = M::mma(M::load(yrow + ks * M::KSTEP), of2[j][ks], dp);
+            for (int ks = 0; ks < NKS; ++ks) dp = M::mma(M::load(yrow + ks * M::KSTEP), of2[j][ks], dp);
+          }
           frag db[M::ACC_KSTEPS], pb[M::ACC_KSTEPS];
           if constexpr (QF != 0) {
             if (DV) TM::bothq(s[j], dp, TM::pair(4.0f * A.a0 * A.a2 - A.a1 * A.a1), edge, wlo, whi, lh, pb, db);
