@@ -43,7 +43,7 @@ PEAK_HBM_GBS = 8000.0
 # (N, order, dtype, --chunk, kernel).  A constant, not a live measurement: it belongs to the kernels as they
 # were when the named summary was made.
 TRAFFIC = {
-    (4096, 2, "bf16", 0, "dkv"): {"bytes": (44092 * 2 + 32770) * 1024, "source": "profiles/c2_bf16_hbm_traffic.md"},
+    (4096, 2, "bf16", 0, "dkv"): {"bytes": (44639 * 2 + 32770) * 1024, "source": "profiles/c2_bf16_hbm_traffic.md"},
     (65536, 1, "bf16", 0, "dkv"): {"bytes": (402970 * 2 + 393240) * 1024, "source": "profiles/long_order1_bf16_hbm_traffic.md"},
     (65536, 2, "bf16", 0, "build"): {"bytes": (160828 * 2 + 982268) * 1024, "source": "profiles/long_order2_bf16_hbm_traffic.md"},
     (65536, 2, "bf16", 0, "dkv"): {"bytes": (564148 * 2 + 262171) * 1024, "source": "profiles/long_order2_bf16_hbm_traffic.md"},
