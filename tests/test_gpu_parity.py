@@ -45,6 +45,23 @@ def test_matrix_rate_probe_runs(lib):
     assert lib.mfma_rate(DEV, workgroups=256, iters=200) > 0.0
 
 
+def test_lds_fed_mix_probe_runs(lib):
+    """The second yardstick (matrix products fed from LDS with the dense kernels' instruction mix): runs for one and
+    two own tiles, writes every checksum, rejects anything else."""
+    import ctypes as C
+    stream = torch.cuda.current_stream().cuda_stream
+    for tiles in (1, 2):
+        out = torch.full((8 * 256,), float("nan"), device=DEV)
+        assert lib.lib.fastmax_probe_mix_rate(8, 16, tiles, C.c_void_p(out.data_ptr()), C.c_void_p(stream)) == 0
+        torch.cuda.synchronize()
+        assert bool(torch.isfinite(out).all())
+    out = torch.zeros(8 * 256, device=DEV)
+    assert lib.lib.fastmax_probe_mix_rate(8, 16, 3, C.c_void_p(out.data_ptr()), C.c_void_p(stream)) != 0
+    assert lib.lib.fastmax_probe_mix_rate(0, 16, 1, C.c_void_p(out.data_ptr()), C.c_void_p(stream)) != 0
+    assert lib.lib.fastmax_probe_mix_rate(8, 16, 1, None, C.c_void_p(stream)) != 0
+    assert lib.mix_rate(DEV, 1, iters=100) > 0.0
+
+
 def test_lds_transpose_read_layout(lib):
     """The kernels (and the host simulator) assume: inside each group of 16 lanes, lane i receives
     element i % 4 of the four-value words addressed by lanes i/4, 4 + i/4, 8 + i/4, 12 + i/4."""
