@@ -482,8 +482,8 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
 //   dV[c] += k'_a Y_a[c]                      the accumulator entries of the lane, fp32
 //   dK[a]  = 2 sum_c v_c Y_a[c]               v in accumulator layout; the two halves of a wavefront hold 32 values of c
 //                                             each and meet through one cross-lane add; the sum goes to dks[token][a]
-// which is half of the matrix instructions of the two separate readouts (8 instead of 8 + 5 per slab and tile), no
-// Khatri-Rao products, and one staging of the state instead of two.
+// which takes 8 matrix instructions per slab and tile where the two separate readouts take 8 + 5, no Khatri-Rao
+// products, and one staging of the state instead of two.
 // slab: two buffers of DH * PS elements; dks: [QW][DH + 1] floats, rows of the wavefront's own tokens only (no barrier
 // between its writes here and the reads of the same wavefront later).  All 256 threads must call this.
 // ------------------------------------------------------------------------------
