@@ -223,9 +223,55 @@ def main() -> int:
             extra[key] = {"workload": r["config"]["workload"], "dtype": dt, "ms_per_step": r["ms_per_step"],
                           "step_ms": r["step_ms"], "tokens_per_s": r["value"], "forward_only_ms": r["forward_only"]["ms"],
                           "roofline": r["roofline"], "hbm_bound_helpers": r["hbm_bound_helpers"]}
+        extra["decode_state_order2_bf16"] = decode_line(lib, dev)
         out["extra"] = extra
     print(json.dumps(out))
     return 0
+
+
+def decode_line(lib, dev, bh=16, d=64, prompt=4096, steps=200):
+    """Incremental decoding on the persistent moment state (the long shape's heads, order 2): a prompt is absorbed,
+    then one token per call; a step reads and writes the state once, so it is priced against HBM."""
+    import torch
+    gen = torch.Generator().manual_seed(5)
+    q, k, v = ((torch.randn(bh, prompt + steps, d, generator=gen)).to(torch.bfloat16).to(dev) for _ in range(3))
+    kw = dict(inv_tau=1.0 / (8.0 * math.sqrt(d)), p=2)
+    state = lib.decode_state(k, **kw)
+    lib.decode_absorb(k[:, :prompt], v[:, :prompt], state, **kw)
+    # the C entry point itself, on buffers made once (the Python front allocates o, g and the scratch per call)
+    import ctypes as C
+    from reproducing_fastmax_results_amd._capi import _strides, _gstrides
+    q1, k1, v1 = q[:, :1], k[:, :1], v[:, :1]
+    desc = lib.make_desc(q1, k1, v1, mask=True, a0=1.0, a1=1.0, a2=0.5, **kw)
+    o = torch.empty(bh, 1, d, dtype=q.dtype, device=dev)
+    g = torch.empty(bh, 1, dtype=torch.float32, device=dev)
+    desc.so, desc.sg = _strides(o), _gstrides(g)
+    scratch = torch.empty(max(lib.lib.fastmax_decode_scratch_bytes(C.byref(desc)) // 4, 1), dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    row = q.stride(1) * q.element_size()
+
+    def one(t):
+        st = lib.lib.fastmax_decode_step(C.byref(desc), q.data_ptr() + t * row, k.data_ptr() + t * row, v.data_ptr() + t * row,
+                                         state.data_ptr(), o.data_ptr(), g.data_ptr(), scratch.data_ptr(), stream)
+        lib.check(st, "fastmax_decode_step")
+
+    for t in range(prompt, prompt + 10):
+        one(t)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    n = steps - 10
+    e0.record()
+    for t in range(prompt + 10, prompt + steps):
+        one(t)
+    e1.record()
+    e1.synchronize()
+    us = 1e3 * e0.elapsed_time(e1) / n
+    state_bytes = state.numel() * 4
+    return {"workload": f"one token per call on the moment state, B*H={bh}, D={d}, after a {prompt}-token prompt",
+            "us_per_token": us, "tokens_per_s": 1e6 / us, "state_bytes": state_bytes,
+            "roofline": {"bound": "hbm", "achieved": 2 * state_bytes / (us * 1e-6) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": 2 * state_bytes / (us * 1e-6) / 1e9 / PEAK_HBM_GBS,
+                         "what": "state read and written once per step; two launches per token, back to back"}}
 
 
 def percentiles(xs):

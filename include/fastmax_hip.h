@@ -160,8 +160,8 @@ int fastmax_backward_saved(const FastmaxDesc* desc, const void* q, const void* k
 /* Incremental decoding on a persistent moment state (the running sums of fastmax_cuda_forward.cu:160-276
  * kept between calls; the reference's generation loop, transformer/eval.py:8-32, re-runs the whole context
  * for every new token).  The state of a batch*head is the fp32 sums over all keys so far of [1, k', k' x k']
- * times [v, 1] with k' = k * inv_tau: fastmax_decode_state_bytes(desc) bytes for desc->bh of them (1.07 MB
- * per batch*head at d = 64, order 2; 17 KB at order 1), whatever the number of keys.  A zero-filled buffer
+ * times [v, 1] with k' = k * inv_tau: fastmax_decode_state_bytes(desc) bytes for desc->bh of them (1.10 MB
+ * per batch*head at d = 64, order 2; 33 KB at order 1), whatever the number of keys.  A zero-filled buffer
  * is the empty state.  desc: bh, d, dtype, p, a0..a2, inv_tau and the strides named below are used; mask,
  * chunk, flags and norm are ignored (decoding is causal by construction and needs unnormalised q, k: the
  * max-norm depends on every token).

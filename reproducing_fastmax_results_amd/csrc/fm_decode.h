@@ -13,15 +13,17 @@
 // Readout for a query q:  F = a0 num[0] + a1 sum_m q_m num[1+m] + a2 sum_{m,l} q_m q_l num[1+D+mD+l],
 // g likewise from den, o = F / g.
 //
-// k_decode_absorb: grid (ceil(R / 256), bh), 256 threads.  A workgroup owns 256 moment rows; thread (wave w,
-// lane c) keeps column c of the rows w, w + 4, ... of that block in registers (64 values), adds the new
-// tokens one after the other (their k', v staged through LDS), writes the rows back and, when a query is
-// given (one new token), leaves its part of F and g in `part` [bh][blocks][D + 1]; k_decode_finish adds the
-// parts in a fixed order and divides.  Bandwidth bound: a step reads and writes the state once.
+// k_decode_absorb: grid (ceil(R / 64), bh), 256 threads.  A workgroup owns 64 moment rows; a thread keeps four
+// consecutive columns of FM_DEC_ROWS * D / 1024 of them in registers (16-byte loads and stores: D / 4 threads per
+// row), adds the new tokens one after the other (their k', v staged through LDS), writes the rows back and, when
+// a query is given (one new token), leaves its part of F and g in `part` [bh][blocks][D + 1]; k_decode_finish adds
+// the parts in a fixed order and divides.  Bandwidth bound: a step reads and writes the state once (a thousand
+// workgroups at the long shape's 16 heads; 256-row workgroups with one column per thread were a quarter as many and
+// took 30 us for the 36 MB of a step).
 #pragma once
 #include "fm_kernels.h"
 
-static constexpr int FM_DEC_ROWS = 256;     // moment rows per workgroup
+static constexpr int FM_DEC_ROWS = 64;      // moment rows per workgroup
 inline int64_t fm_decode_rows(int d, bool quad) { return 1 + int64_t(d) + (quad ? int64_t(d) * d : 0); }
 inline int fm_decode_blocks(int d, bool quad) { return int((fm_decode_rows(d, quad) + FM_DEC_ROWS - 1) / FM_DEC_ROWS); }
 // floats of one batch*head's state: num [R][D] then den [R], R rounded up to whole blocks
@@ -42,26 +44,37 @@ template <typename TIO, int DH>
 FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS)
 k_decode_absorb(TRef<const TIO> k, TRef<const TIO> v, TRef<const TIO> q, int n_new, int quad, float inv_tau, float a0,
                 float a1, float a2, float* FM_RESTRICT state, float* FM_RESTRICT part) {
-  constexpr int RPT = FM_DEC_ROWS / 4;                  // rows per thread (one column each)
+  constexpr int TPR = DH / 4;                            // threads per row (four columns each)
+  constexpr int RPP = FM_THREADS / TPR;                  // rows per pass of the workgroup
+  constexpr int RPT = FM_DEC_ROWS / RPP;                 // rows per thread
   constexpr int TB = 16;                                 // new tokens staged at a time
+  static_assert(FM_DEC_ROWS % RPP == 0 && FM_DEC_ROWS <= FM_THREADS, "whole passes; one thread per denominator row");
   FM_SHARED float ks[TB][DH + 1];                        // k' of the staged tokens, [DH] = 1
-  FM_SHARED float vs[TB][DH];
+  FM_SHARED __attribute__((aligned(16))) float vs[TB][DH];
   FM_SHARED float qs[DH + 1];
-  FM_SHARED float red[4][DH + 1];
-  const int tid = FM_TID_X, lane = tid & 63, wave = tid >> 6, bh = FM_BID_Y, blk = FM_BID_X;
+  FM_SHARED __attribute__((aligned(16))) float red[RPP][DH];
+  FM_SHARED float redg[FM_THREADS / 64];
+  const int tid = FM_TID_X, lane = tid & 63, bh = FM_BID_Y, blk = FM_BID_X;
+  const int c4 = (tid % TPR) * 4, rsub = tid / TPR;
   const int64_t R = int64_t(FM_GDIM_X) * FM_DEC_ROWS;
   float* num = state + int64_t(bh) * R * (DH + 1);
   float* den = num + R * DH;
   const int r0 = blk * FM_DEC_ROWS;
-  const bool col_live = lane < DH;                       // D = 32: half of the lanes hold no column
-  // this thread's rows and their feature pairs
-  float acc[RPT];
+  // this thread's rows (r0 + rsub + RPP * i), four columns of each, and their feature pairs
+  fm_f32x4 acc[RPT];
+  int rm[RPT], rl[RPT];
+  bool rlive[RPT];
 #pragma unroll
-  for (int i = 0; i < RPT; ++i) acc[i] = col_live ? num[int64_t(r0 + wave + 4 * i) * DH + lane] : 0.f;
-  // denominators: thread t owns row r0 + t
-  float dsum = den[r0 + tid];
-  int dm, dl; bool dlive;
-  fm_decode_row<DH>(r0 + tid, quad != 0, dm, dl, dlive);
+  for (int i = 0; i < RPT; ++i) {
+    const int r = r0 + rsub + RPP * i;
+    acc[i] = *reinterpret_cast<const fm_f32x4*>(num + int64_t(r) * DH + c4);
+    fm_decode_row<DH>(r, quad != 0, rm[i], rl[i], rlive[i]);
+  }
+  // denominators: thread t < FM_DEC_ROWS owns row r0 + t
+  const bool down = tid < FM_DEC_ROWS;
+  float dsum = down ? den[r0 + tid] : 0.f;
+  int dm = DH, dl = DH; bool dlive = false;
+  if (down) fm_decode_row<DH>(r0 + tid, quad != 0, dm, dl, dlive);
   for (int t0 = 0; t0 < n_new; t0 += TB) {
     FM_SYNC();
     for (int i = tid; i < TB * (DH + 1); i += FM_THREADS) {
@@ -77,56 +90,80 @@ k_decode_absorb(TRef<const TIO> k, TRef<const TIO> v, TRef<const TIO> q, int n_n
     FM_SYNC();
     const int nt = n_new - t0 < TB ? n_new - t0 : TB;
     for (int t = 0; t < nt; ++t) {
-      const float vc = col_live ? vs[t][lane] : 0.f;
+      const fm_f32x4 vc = *reinterpret_cast<const fm_f32x4*>(&vs[t][c4]);
 #pragma unroll
       for (int i = 0; i < RPT; ++i) {
-        int m, l; bool live;
-        fm_decode_row<DH>(r0 + wave + 4 * i, quad != 0, m, l, live);
-        if (live) acc[i] += ks[t][m] * ks[t][l] * vc;
+        const float w = rlive[i] ? ks[t][rm[i]] * ks[t][rl[i]] : 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] += w * vc[j];
       }
       if (dlive) dsum += ks[t][dm] * ks[t][dl];
     }
   }
 #pragma unroll
   for (int i = 0; i < RPT; ++i)
-    if (col_live) num[int64_t(r0 + wave + 4 * i) * DH + lane] = acc[i];
-  den[r0 + tid] = dsum;
+    *reinterpret_cast<fm_f32x4*>(num + int64_t(r0 + rsub + RPP * i) * DH + c4) = acc[i];
+  if (down) den[r0 + tid] = dsum;
   if (!part) return;
   // readout of the new token's query against the rows of this block
   FM_SYNC();
   if (tid <= DH) qs[tid] = tid < DH ? IO<TIO>::ld(q.base(bh) + tid) : 1.0f;
   FM_SYNC();
-  float f = 0.f;
+  fm_f32x4 f = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int i = 0; i < RPT; ++i) {
-    int m, l; bool live;
-    const int r = r0 + wave + 4 * i;
-    fm_decode_row<DH>(r, quad != 0, m, l, live);
+    const int r = r0 + rsub + RPP * i;
     const float coef = r == 0 ? a0 : (r <= DH ? a1 : a2);
-    if (live) f += coef * qs[m] * qs[l] * acc[i];
+    const float w = rlive[i] ? coef * qs[rm[i]] * qs[rl[i]] : 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) f[j] += w * acc[i][j];
   }
   float gsum = dlive ? (r0 + tid == 0 ? a0 : (r0 + tid <= DH ? a1 : a2)) * qs[dm] * qs[dl] * dsum : 0.f;
 #pragma unroll
   for (int m = 1; m < 64; m <<= 1) gsum += fm_shfl_xor(gsum, m);
-  if (col_live) red[wave][lane] = f;
-  if (lane == 0) red[wave][DH] = gsum;
+  *reinterpret_cast<fm_f32x4*>(&red[rsub][c4]) = f;
+  if (lane == 0) redg[tid >> 6] = gsum;
   FM_SYNC();
-  if (tid <= DH)
-    part[(int64_t(bh) * FM_GDIM_X + blk) * (DH + 1) + tid] = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
+  if (tid < DH) {
+    // the row groups in a fixed order
+    float sum = 0.f;
+#pragma unroll
+    for (int r = 0; r < RPP; ++r) sum += red[r][tid];
+    part[(int64_t(bh) * FM_GDIM_X + blk) * (DH + 1) + tid] = sum;
+  } else if (tid == DH) {
+    float gs = 0.f;
+#pragma unroll
+    for (int w = 0; w < FM_THREADS / 64; ++w) gs += redg[w];
+    part[(int64_t(bh) * FM_GDIM_X + blk) * (DH + 1) + DH] = gs;
+  }
 }
 
-// o = F / g from the parts of k_decode_absorb.  grid (bh), 64 threads.
+// o = F / g from the parts of k_decode_absorb.  grid (bh), 256 threads: every wavefront adds a quarter of the
+// blocks' parts, in order, and the four sums are added in a fixed order.
 template <typename TIO, int DH>
-FM_GLOBAL void FM_LAUNCH_BOUNDS(64) k_decode_finish(const float* FM_RESTRICT part, int nblk, TRef<TIO> o, TRef<float> g) {
-  const int bh = FM_BID_X, lane = FM_TID_X;
+FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_decode_finish(const float* FM_RESTRICT part, int nblk, TRef<TIO> o, TRef<float> g) {
+  FM_SHARED float red[FM_THREADS / 64][DH + 1];
+  const int bh = FM_BID_X, tid = FM_TID_X, lane = tid & 63, wave = tid >> 6;
   const float* p = part + int64_t(bh) * nblk * (DH + 1);
-  float gs = 0.f, f = 0.f;
-  for (int b = 0; b < nblk; ++b) {
-    gs += p[b * (DH + 1) + DH];
+  float f = 0.f, f2 = 0.f;
+  const int per = (nblk + FM_THREADS / 64 - 1) / (FM_THREADS / 64), b0 = wave * per, b1 = b0 + per < nblk ? b0 + per : nblk;
+  for (int b = b0; b < b1; ++b) {
     if (lane < DH) f += p[b * (DH + 1) + lane];
+    if (DH == 64 ? lane == 0 : lane == DH) f2 += p[b * (DH + 1) + DH];
   }
-  if (lane < DH) IO<TIO>::st(o.base(bh) + lane, f / gs);
-  if (lane == 0) g.base(bh)[0] = gs;
+  if (lane < DH) red[wave][lane] = f;
+  if (DH == 64 ? lane == 0 : lane == DH) red[wave][DH] = f2;
+  FM_SYNC();
+  if (tid <= DH) {
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < FM_THREADS / 64; ++w) sum += red[w][tid];
+    red[0][tid] = sum;
+  }
+  FM_SYNC();
+  const float gs = red[0][DH];
+  if (tid < DH) IO<TIO>::st(o.base(bh) + tid, red[0][tid] / gs);
+  if (tid == 0) g.base(bh)[0] = gs;
 }
 
 template <typename TIO, int DH>
@@ -139,7 +176,7 @@ int fm_decode_run(const FastmaxDesc* d, const void* q, const void* k, const void
   FM_KERNEL_LAUNCH((k_decode_absorb<TIO, DH>), fm_dim3(nblk, d->bh), fm_dim3(FM_THREADS), 0, stream, kr, vr, qr, n_new, quad ? 1 : 0,
                    d->inv_tau, d->a0, d->a1, quad ? d->a2 : 0.0f, state, q ? scratch : nullptr);
   if (q)
-    FM_KERNEL_LAUNCH((k_decode_finish<TIO, DH>), fm_dim3(d->bh), fm_dim3(64), 0, stream, scratch, nblk,
+    FM_KERNEL_LAUNCH((k_decode_finish<TIO, DH>), fm_dim3(d->bh), fm_dim3(FM_THREADS), 0, stream, scratch, nblk,
                      fm_ref<TIO>(static_cast<TIO*>(o), d->so), fm_ref<float>(g, d->sg));
   return fm_after_launch() ? FASTMAX_ERR_LAUNCH : FASTMAX_OK;
 }
