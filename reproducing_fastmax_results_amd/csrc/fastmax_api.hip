@@ -344,7 +344,7 @@ template <typename E, int DH, int QT> size_t tok_lds_bytes(int kind) {
   const size_t zs = size_t(C::NZ) * DH * C::PS * sizeof(E);
   if (zs > region) region = zs;
   size_t body = size_t(C::QW) * C::PQ * sizeof(E) + region;
-  const size_t outst = size_t(C::QW) * (DH + 1) * 4;
+  const size_t outst = size_t(C::QW) * fm_store_pitch(DH) * 4;
   const size_t stage = kind == 0 ? size_t(2) * C::PV_STAGE * sizeof(E)
                                  : size_t(C::DS_NBUF) * (kind == 2 || kind == 4 ? C::DV_STAGE : C::DS_STAGE) * sizeof(E);
   if (kind == 4) body += size_t(C::QW) * (DH + 1) * 4;      // dK of the fused state readout, behind the slabs

@@ -379,15 +379,19 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 3) k_o1_fwd(O1FwdArgs<TIO> A) {
       for (int ct = 0; ct < NT; ++ct) acc[ct] = M::mma(M::load_tr(Vs, PQ, 32 * jt + 16 * ss, 32 * ct, lane), pb[ss], acc[ct]);
   }
   FM_SYNC();                                             // the tiles are spent: the output staging lies over them
-  float* Os = reinterpret_cast<float*>(smem);           // [QW][DH + 1]
+  float* Os = reinterpret_cast<float*>(smem);           // [QW][fm_store_pitch]
   float gt = gsum + fm_shfl_xor(gsum, 32) + A.a0 * float(t0);
   const float ginv = 1.0f / gt;
+  constexpr int OP = fm_store_pitch(DH);
 #pragma unroll
   for (int ct = 0; ct < NT; ++ct)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int c = 32 * ct + fm_acc_row(e, lh);
-      Os[own * (DH + 1) + c] = (acc[ct][e] + vecs[DH + c]) * ginv;
+    for (int g = 0; g < 4; ++g) {
+      const int c = 32 * ct + fm_acc_row(4 * g, lh);
+      fm_f32x4 w;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w[i] = (acc[ct][4 * g + i] + vecs[DH + c + i]) * ginv;
+      *reinterpret_cast<fm_f32x4*>(Os + own * OP + c) = w;
     }
   if (lh == 0 && t0 + own < A.n) A.g.base(bh)[int64_t(t0 + own) * A.g.s_n] = gt;
   FM_SYNC();
@@ -395,9 +399,9 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 3) k_o1_fwd(O1FwdArgs<TIO> A) {
   for (int c = tid; c < QW * (DH / 8); c += FM_THREADS) {
     const int row = c / (DH / 8), col = (c % (DH / 8)) * 8;
     if (t0 + row < A.n) {
-      float v[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) v[i] = Os[row * (DH + 1) + col + i];
+      const fm_f32x4 lo = *reinterpret_cast<const fm_f32x4*>(Os + row * OP + col);
+      const fm_f32x4 hi = *reinterpret_cast<const fm_f32x4*>(Os + row * OP + col + 4);
+      const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       IO<TIO>::st8(ob + int64_t(t0 + row) * A.o.s_n + col, A.o.vec != 0, v);
     }
   }
@@ -605,7 +609,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
   const float ginv = 1.0f / gsc;
   const int nblk = (A.n + QW - 1) / QW;
   const int xrow[1] = {own};
-  float* Os = reinterpret_cast<float*>(Vs);              // over V and GH: [QW][DH + 1] floats
+  float* Os = reinterpret_cast<float*>(Vs);              // over V and GH: [QW][fm_store_pitch] floats
   FM_SYNC();                                             // GH, V and c are spent
   {
     const float fac = A.bq ? fm_norm_factor(A.q_fold, bh, lane) : 1.0f;
@@ -630,6 +634,6 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
 template <int DH> inline size_t fm_o1_bwd_lds() {
   const size_t tile = size_t(FM_O1_SEG) * (DH + Mma<fm_half>::PAD) * 2;
   const size_t tiles = 3 * tile + size_t(FM_O1_SEG) * 2 + size_t(3) * DH * 4 + size_t(DH) * (DH + Mma<fm_half>::PAD) * 2;
-  const size_t outst = tile + size_t(FM_O1_SEG) * (DH + 1) * 4;      // Q' / K' tile kept, staging over V and GH
+  const size_t outst = tile + size_t(FM_O1_SEG) * fm_store_pitch(DH) * 4;      // Q' / K' tile kept, staging over V and GH
   return tiles > outst ? tiles : outst;
 }

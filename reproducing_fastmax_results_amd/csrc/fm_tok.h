@@ -95,20 +95,26 @@ FM_DEVICE fm_f32x16 fm_zy(const E* Zs, const typename Mma<E>::frag* tf, int mt, 
 // brows (optional): compute-type rows of the same tokens (row t at brows + (t - brow0) * bpitch: a copy in
 // memory, or a tile still in LDS); the workgroup's sum over its stored values times those rows, times bscale,
 // goes to *bout (one workgroup-uniform address).
+// pitch (floats) of the fp32 staging of fm_store_tokens: rows stay 16-byte aligned
+constexpr int fm_store_pitch(int dh) { return dh + 4; }
 template <typename TIO, typename E, int DH, int QT>
 FM_DEVICE void fm_store_tokens(fm_f32x16 (*acc)[DH / 32], const int* xrow, const float* addvec, float scale, float* Os,
                                TRef<TIO> out, int bh, int row0, int nrows, int tid, const E* brows = nullptr,
                                float bscale = 0.f, float* bout = nullptr, int bpitch = DH, int brow0 = 0) {
   typedef TokCfg<E, DH, QT> C;
+  constexpr int OP = fm_store_pitch(DH);                 // rows of the staging 16-byte aligned: four entries per LDS write
   const int lane = tid & 63, lh = lane >> 5;
 #pragma unroll
   for (int j = 0; j < QT; ++j)
 #pragma unroll
     for (int ct = 0; ct < C::NT; ++ct)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int c = 32 * ct + fm_acc_row(e, lh);
-        Os[xrow[j] * (DH + 1) + c] = scale * (acc[j][ct][e] + (addvec ? addvec[c] : 0.f));
+      for (int g = 0; g < 4; ++g) {
+        const int c = 32 * ct + fm_acc_row(4 * g, lh);
+        fm_f32x4 w;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = scale * (acc[j][ct][4 * g + i] + (addvec ? addvec[c + i] : 0.f));
+        *reinterpret_cast<fm_f32x4*>(Os + xrow[j] * OP + c) = w;
       }
   FM_SYNC();
   TIO* ob = out.base(bh);
@@ -116,9 +122,9 @@ FM_DEVICE void fm_store_tokens(fm_f32x16 (*acc)[DH / 32], const int* xrow, const
   for (int c = tid; c < C::QW * (DH / 8); c += FM_THREADS) {
     const int row = c / (DH / 8), col = (c % (DH / 8)) * 8;
     if (row0 + row < nrows) {
-      float v[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) v[i] = Os[row * (DH + 1) + col + i];
+      const fm_f32x4 lo = *reinterpret_cast<const fm_f32x4*>(Os + row * OP + col);
+      const fm_f32x4 hi = *reinterpret_cast<const fm_f32x4*>(Os + row * OP + col + 4);
+      const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       if (brows) {
         const E* br = brows + int64_t(row0 + row - brow0) * bpitch + col;
 #pragma unroll
@@ -435,7 +441,8 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
   }
 
   // ---- epilogue, staged through LDS for coalesced stores ----
-  float* Os = reinterpret_cast<float*>(Own);           // [QW][DH + 1]
+  float* Os = reinterpret_cast<float*>(Own);           // [QW][fm_store_pitch]
+  constexpr int OP = fm_store_pitch(DH);
   if (OWN == FM_OWN_Q) {
     // o = (F + vb) / g
     const float cnt = causal ? float(G.sbeg) : float(A.n_str);   // keys covered by the state
@@ -448,10 +455,12 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
 #pragma unroll
       for (int ct = 0; ct < NT; ++ct)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int c = 32 * ct + fm_acc_row(e, lh);
-          const float f = acc[j][ct][e] + (G.use_state ? vecs[DH + c] : 0.f);
-          Os[xrow[j] * (DH + 1) + c] = f * ginv;
+        for (int g4 = 0; g4 < 4; ++g4) {
+          const int c = 32 * ct + fm_acc_row(4 * g4, lh);
+          fm_f32x4 w;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) w[i] = (acc[j][ct][4 * g4 + i] + (G.use_state ? vecs[DH + c + i] : 0.f)) * ginv;
+          *reinterpret_cast<fm_f32x4*>(Os + xrow[j] * OP + c) = w;
         }
       const int qi = t0 + xrow[j];
       if (lh == 0 && qi < A.n_own) A.g.base(bh)[int64_t(qi) * A.g.s_n] = gt;
@@ -461,9 +470,9 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
     for (int c = tid; c < QW * (DH / 8); c += FM_THREADS) {
       const int row = c / (DH / 8), col = (c % (DH / 8)) * 8;
       if (t0 + row < A.n_own) {
-        float v[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = Os[row * (DH + 1) + col + i];
+        const fm_f32x4 lo = *reinterpret_cast<const fm_f32x4*>(Os + row * OP + col);
+        const fm_f32x4 hi = *reinterpret_cast<const fm_f32x4*>(Os + row * OP + col + 4);
+        const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         IO<TIO>::st8(ob + int64_t(t0 + row) * A.out.s_n + col, A.out.vec != 0, v);
       }
     }
