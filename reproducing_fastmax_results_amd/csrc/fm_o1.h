@@ -24,6 +24,7 @@
 #include "fm_tok.h"
 
 static constexpr int FM_O1_SEG = 128;
+static constexpr int FM_O1_DQ_PITCH = 40;   // elements per row of k_o1_bwd's dq staging (32 features, rows 16-byte aligned)
 
 // One 128-token segment of a bf16 caller tensor as raw 16-byte chunks: with CPR = DH / 8 chunks per row,
 // thread t holds chunk t % CPR of the rows t / CPR + (256 / CPR) i.  Rows past the end are zeros.
@@ -416,7 +417,8 @@ template <int DH> inline size_t fm_o1_fwd_lds() {
 // ------------------------------------------------------------------------------
 // k_o1_bwd: dq, dk and dv of one segment.  grid (nseg, bh); wavefront w owns the 32 tokens of tile w for all
 // three.  First the tiles K', V, GH are in LDS (the raw q rows wait in registers): the prefix product and the
-// dense tiles of dq; then Q' takes the place of K' for the dense tiles of dk and dv and the suffix products.
+// dense tiles of dq, which is stored at once (its stores travel during the second phase); then Q' takes the place
+// of K' for the dense tiles of dk and dv and the suffix products.
 //   bigq (prefix, slot s: segments < s): slab [c][f] = a1 sum v_c k'_f, the forward's own state; smallq: va = a1 sum k'
 //   bigk (suffix, slot s: segments > s): slab [f][c] = a1 sum q'_f gh_c;  smallk: va = a1 sum c q', vb = a0 sum gh
 // each in two parts, the segments inside the run (big*, small*) and the whole runs (run*, see k_o1_sums), added on load.
@@ -558,6 +560,39 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
 #pragma unroll
       for (int mt = 0; mt < NT; ++mt) dq[mt] = M::mma(M::load_tr(Ks, PQ, 32 * jt + 16 * ss, 32 * mt, lane), db[ss], dq[mt]);
   }
+  // dq leaves now, so that its stores travel while dk and dv are computed: every wavefront through an LDS region of
+  // its own (its 32 tokens, 32 features at a time, already in the output type), no barrier.  (With the Jacobian of a
+  // folded normalisation, or rows that are not 16-byte aligned, dq goes out with the others at the end.)
+  const float ginv = 1.0f / gsc;
+  bool dq_stored = false;
+  if constexpr (sizeof(TIO) == 2) {
+    if (!A.bq && A.dq.vec != 0) {
+      constexpr int DP = FM_O1_DQ_PITCH;
+      TIO* st = reinterpret_cast<TIO*>(Sl + DH * PS) + wave * 32 * DP;
+      const float f = A.sc * ginv;
+      TIO* ob = A.dq.base(bh);
+#pragma unroll
+      for (int mt = 0; mt < NT; ++mt) {
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          fm_u32x2 w;
+          w[0] = uint32_t(fm_f32_to_bf16(f * dq[mt][4 * g4])) | (uint32_t(fm_f32_to_bf16(f * dq[mt][4 * g4 + 1])) << 16);
+          w[1] = uint32_t(fm_f32_to_bf16(f * dq[mt][4 * g4 + 2])) | (uint32_t(fm_f32_to_bf16(f * dq[mt][4 * g4 + 3])) << 16);
+          *reinterpret_cast<fm_u32x2*>(st + lr * DP + fm_acc_row(4 * g4, lh)) = w;
+        }
+        FM_WAVE_SYNC();
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const int c = lane + 64 * i, row = c >> 2, col = (c & 3) * 8;
+          const int tok = t0 + wave * 32 + row;
+          if (tok < A.n)
+            *reinterpret_cast<fm_u32x4*>(ob + int64_t(tok) * A.dq.s_n + 32 * mt + col) = *reinterpret_cast<const fm_u32x4*>(st + row * DP + col);
+        }
+        FM_WAVE_SYNC();
+      }
+      dq_stored = true;
+    }
+  }
   FM_SYNC();                                             // K' and the prefix slab are spent
   rq.store(Qs, PQ, tid, qsc);
   slab_store(rs, rs2);
@@ -606,12 +641,11 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
   // ---- stores, through LDS.  With the Jacobian of a folded normalisation (bq / bk): the stored gradient carries
   // lim / max-norm and the workgroup's part of B = sum dy . y is left for k_norm_fix; the rows y * sc are the tiles
   // still in LDS (Q', and K' which is written back first) ----
-  const float ginv = 1.0f / gsc;
   const int nblk = (A.n + QW - 1) / QW;
   const int xrow[1] = {own};
   float* Os = reinterpret_cast<float*>(Vs);              // over V and GH: [QW][fm_store_pitch] floats
   FM_SYNC();                                             // GH, V and c are spent
-  {
+  if (!dq_stored) {
     const float fac = A.bq ? fm_norm_factor(A.q_fold, bh, lane) : 1.0f;
     fm_store_tokens<TIO, E, DH, 1>(&dq, xrow, nullptr, A.sc * ginv * fac, Os, A.dq, bh, t0, A.n, tid,
                                    A.bq ? Qs : nullptr, fac > 0.f ? 1.0f / (fac * A.sc) : 0.f,
@@ -633,7 +667,8 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
 }
 template <int DH> inline size_t fm_o1_bwd_lds() {
   const size_t tile = size_t(FM_O1_SEG) * (DH + Mma<fm_half>::PAD) * 2;
-  const size_t tiles = 3 * tile + size_t(FM_O1_SEG) * 2 + size_t(3) * DH * 4 + size_t(DH) * (DH + Mma<fm_half>::PAD) * 2;
+  const size_t tiles = 3 * tile + size_t(FM_O1_SEG) * 2 + size_t(3) * DH * 4 + size_t(DH) * (DH + Mma<fm_half>::PAD) * 2 +
+                       size_t(FM_THREADS / 64) * 32 * FM_O1_DQ_PITCH * 2;            // and the wavefronts' dq staging
   const size_t outst = tile + size_t(FM_O1_SEG) * fm_store_pitch(DH) * 4;      // Q' / K' tile kept, staging over V and GH
   return tiles > outst ? tiles : outst;
 }

@@ -45,6 +45,7 @@ typedef hostsim::Dim3 fm_dim3;
 #define FM_GDIM_Y (int(hostsim::g_t.gdim.y))
 #define FM_GDIM_Z (int(hostsim::g_t.gdim.z))
 #define FM_SYNC() hostsim::syncthreads()
+#define FM_WAVE_SYNC() hostsim::syncthreads()
 #define FM_DYN_SMEM(name) unsigned char* name = hostsim::g_t.blk->dyn_smem
 #define FM_KERNEL_LAUNCH(kern, grid, block, smem, stream, ...) \
   hostsim::launch((grid), (block), (smem), [=]() { kern(__VA_ARGS__); })
@@ -123,6 +124,9 @@ typedef dim3 fm_dim3;
 #define FM_GDIM_Y (int(gridDim.y))
 #define FM_GDIM_Z (int(gridDim.z))
 #define FM_SYNC() __syncthreads()
+// Between LDS writes and reads of the same wavefront (lanes exchange data through a region no other wavefront touches):
+// the LDS serves a wavefront's operations in order, so only the compiler has to keep them in order.
+#define FM_WAVE_SYNC() do { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront"); } while (0)
 #define FM_DYN_SMEM(name) extern __shared__ __align__(16) unsigned char name[]
 // A launch the runtime refuses leaves its error as the calling thread's last error.  Only an error that
 // appears across the launch is this library's: it is taken (cleared) and remembered until
