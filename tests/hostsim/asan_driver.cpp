@@ -47,10 +47,42 @@ static int run_pointwise(int bh, int n, int d, int dtype) {
   printf("pointwise bh=%d n=%d d=%d dtype=%d -> status %d\n", bh, n, d, dtype, st);
   return st;
 }
+// the decoding state: a prompt absorbed, then single-token steps (buffers of exactly the sizes the library names)
+static int run_decode(int bh, int d, int p, int prompt, int steps, int dtype) {
+  FastmaxDesc D; memset(&D, 0, sizeof D);
+  D.bh = bh; D.nq = 1; D.nk = prompt; D.d = d; D.dtype = dtype; D.mask = 1; D.p = p; D.a0 = 1; D.a1 = 1; D.a2 = .5f;
+  D.inv_tau = 1.f / (2.f * std::sqrt(float(d)));
+  FastmaxStrides s = {int64_t(prompt) * d, d, 0, 0}, s1 = {int64_t(d), d, 0, 0};
+  D.sq = s1; D.sk = D.sv = s; D.so = s1; D.sg.bh = 1; D.sg.n = 1;
+  const size_t esz = dtype == FASTMAX_BF16 ? 2 : 4, ne = size_t(bh) * prompt * d;
+  std::vector<char> k(ne * esz), v(ne * esz), q1(size_t(bh) * d * esz), k1(q1.size()), v1(q1.size()), o1(q1.size());
+  auto fill = [&](std::vector<char>& b) {
+    for (size_t i = 0; i < b.size() / esz; ++i) {
+      const float x = frand();
+      if (esz == 2) reinterpret_cast<uint16_t*>(b.data())[i] = bf16(x); else reinterpret_cast<float*>(b.data())[i] = x;
+    }
+  };
+  fill(k); fill(v); fill(q1); fill(k1); fill(v1);
+  const size_t sb = fastmax_decode_state_bytes(&D), cb = fastmax_decode_scratch_bytes(&D);
+  if (!sb || !cb) return 99;
+  float* state = static_cast<float*>(aligned_alloc(256, (sb + 255) / 256 * 256));
+  memset(state, 0, sb);
+  float* scratch = static_cast<float*>(aligned_alloc(256, (cb + 255) / 256 * 256));
+  std::vector<float> g(bh);
+  int st = fastmax_decode_absorb(&D, k.data(), v.data(), state, nullptr);
+  D.sk = D.sv = s1;
+  for (int i = 0; i < steps && !st; ++i)
+    st = fastmax_decode_step(&D, q1.data(), k1.data(), v1.data(), state, o1.data(), g.data(), scratch, nullptr);
+  free(state); free(scratch);
+  printf("decode bh=%d d=%d p=%d prompt=%d steps=%d dtype=%d -> status %d, g[0] %.3f\n", bh, d, p, prompt, steps, dtype, st, g[0]);
+  return st;
+}
 int main() {
   int bad = 0;
   bad |= run_pointwise(3, 333, 64, FASTMAX_BF16);
   bad |= run_pointwise(2, 70, 32, FASTMAX_F32);
+  bad |= run_decode(2, 64, 2, 37, 2, FASTMAX_BF16);
+  bad |= run_decode(3, 32, 1, 5, 2, FASTMAX_F32);
   bad |= run(1, 600, 32, 2, 256, FASTMAX_BF16, 1);    // order-2 walk (a CU to itself: two buffers), both walks
   bad |= run(1, 600, 32, 2, 256, FASTMAX_BF16, 0);
   bad |= run(1, 520, 64, 2, 256, FASTMAX_BF16, 1);
