@@ -24,7 +24,7 @@
 #include "fm_tok.h"
 
 static constexpr int FM_O1_SEG = 128;
-static constexpr int FM_O1_DQ_PITCH = 40;   // elements per row of k_o1_bwd's dq staging (32 features, rows 16-byte aligned)
+static constexpr int FM_O1_DQ_PITCH = 40;   // elements per row of k_o1_bwd's per-wavefront output staging (32 features, rows 16-byte aligned)
 
 // One 128-token segment of a bf16 caller tensor as raw 16-byte chunks: with CPR = DH / 8 chunks per row,
 // thread t holds chunk t % CPR of the rows t / CPR + (256 / CPR) i.  Rows past the end are zeros.
@@ -560,24 +560,24 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
 #pragma unroll
       for (int mt = 0; mt < NT; ++mt) dq[mt] = M::mma(M::load_tr(Ks, PQ, 32 * jt + 16 * ss, 32 * mt, lane), db[ss], dq[mt]);
   }
-  // dq leaves now, so that its stores travel while dk and dv are computed: every wavefront through an LDS region of
-  // its own (its 32 tokens, 32 features at a time, already in the output type), no barrier.  (With the Jacobian of a
-  // folded normalisation, or rows that are not 16-byte aligned, dq goes out with the others at the end.)
+  // A gradient leaves through an LDS region of the wavefront's own (its 32 tokens, 32 features at a time, already in
+  // the output type): no barrier, so dq goes out right after its phase (its stores travel while dk and dv are
+  // computed) and a wavefront that is done with dk and dv (the later its tokens, the fewer dense tiles) stores them
+  // without waiting for the others.  (With the Jacobian of a folded normalisation, or rows that are not 16-byte
+  // aligned, a gradient goes through the workgroup's fp32 staging at the end.)
   const float ginv = 1.0f / gsc;
-  bool dq_stored = false;
-  if constexpr (sizeof(TIO) == 2) {
-    if (!A.bq && A.dq.vec != 0) {
+  auto store_own = [&](const fm_f32x16* acc, float f, const TRef<TIO>& out) FM_ALWAYS_INLINE {
+    if constexpr (sizeof(TIO) == 2) {
       constexpr int DP = FM_O1_DQ_PITCH;
       TIO* st = reinterpret_cast<TIO*>(Sl + DH * PS) + wave * 32 * DP;
-      const float f = A.sc * ginv;
-      TIO* ob = A.dq.base(bh);
+      TIO* ob = out.base(bh);
 #pragma unroll
       for (int mt = 0; mt < NT; ++mt) {
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4) {
           fm_u32x2 w;
-          w[0] = uint32_t(fm_f32_to_bf16(f * dq[mt][4 * g4])) | (uint32_t(fm_f32_to_bf16(f * dq[mt][4 * g4 + 1])) << 16);
-          w[1] = uint32_t(fm_f32_to_bf16(f * dq[mt][4 * g4 + 2])) | (uint32_t(fm_f32_to_bf16(f * dq[mt][4 * g4 + 3])) << 16);
+          w[0] = uint32_t(fm_f32_to_bf16(f * acc[mt][4 * g4])) | (uint32_t(fm_f32_to_bf16(f * acc[mt][4 * g4 + 1])) << 16);
+          w[1] = uint32_t(fm_f32_to_bf16(f * acc[mt][4 * g4 + 2])) | (uint32_t(fm_f32_to_bf16(f * acc[mt][4 * g4 + 3])) << 16);
           *reinterpret_cast<fm_u32x2*>(st + lr * DP + fm_acc_row(4 * g4, lh)) = w;
         }
         FM_WAVE_SYNC();
@@ -586,13 +586,16 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
           const int c = lane + 64 * i, row = c >> 2, col = (c & 3) * 8;
           const int tok = t0 + wave * 32 + row;
           if (tok < A.n)
-            *reinterpret_cast<fm_u32x4*>(ob + int64_t(tok) * A.dq.s_n + 32 * mt + col) = *reinterpret_cast<const fm_u32x4*>(st + row * DP + col);
+            *reinterpret_cast<fm_u32x4*>(ob + int64_t(tok) * out.s_n + 32 * mt + col) = *reinterpret_cast<const fm_u32x4*>(st + row * DP + col);
         }
         FM_WAVE_SYNC();
       }
-      dq_stored = true;
     }
-  }
+  };
+  const bool dq_own = sizeof(TIO) == 2 && !A.bq && A.dq.vec != 0;
+  const bool dk_own = sizeof(TIO) == 2 && !A.bk && A.dk.vec != 0;
+  const bool dv_own = sizeof(TIO) == 2 && A.dv.vec != 0;
+  if (dq_own) store_own(dq, A.sc * ginv, A.dq);
   FM_SYNC();                                             // K' and the prefix slab are spent
   rq.store(Qs, PQ, tid, qsc);
   slab_store(rs, rs2);
@@ -641,11 +644,14 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
   // ---- stores, through LDS.  With the Jacobian of a folded normalisation (bq / bk): the stored gradient carries
   // lim / max-norm and the workgroup's part of B = sum dy . y is left for k_norm_fix; the rows y * sc are the tiles
   // still in LDS (Q', and K' which is written back first) ----
+  if (dk_own) store_own(dk, A.sc * ginv, A.dk);
+  if (dv_own) store_own(dv, ginv, A.dv);
+  if (dq_own && dk_own && dv_own) return;
   const int nblk = (A.n + QW - 1) / QW;
   const int xrow[1] = {own};
   float* Os = reinterpret_cast<float*>(Vs);              // over V and GH: [QW][fm_store_pitch] floats
   FM_SYNC();                                             // GH, V and c are spent
-  if (!dq_stored) {
+  if (!dq_own) {
     const float fac = A.bq ? fm_norm_factor(A.q_fold, bh, lane) : 1.0f;
     fm_store_tokens<TIO, E, DH, 1>(&dq, xrow, nullptr, A.sc * ginv * fac, Os, A.dq, bh, t0, A.n, tid,
                                    A.bq ? Qs : nullptr, fac > 0.f ? 1.0f / (fac * A.sc) : 0.f,
@@ -657,18 +663,18 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
     for (int ks = 0; ks < NKS; ++ks) *reinterpret_cast<frag*>(Ks + own * PQ + ks * M::KSTEP + lh * M::KPL) = kf[ks];
     FM_SYNC();
   }
-  {
+  if (!dk_own) {
     const float fac = A.bk ? fm_norm_factor(A.k_fold, bh, lane) : 1.0f;
     fm_store_tokens<TIO, E, DH, 1>(&dk, xrow, nullptr, A.sc * ginv * fac, Os, A.dk, bh, t0, A.n, tid,
                                    A.bk ? Ks : nullptr, fac > 0.f ? 1.0f / (fac * A.sc) : 0.f,
                                    A.bk ? A.bk + int64_t(bh) * nblk + seg : nullptr, PQ, t0);
   }
-  fm_store_tokens<TIO, E, DH, 1>(&dv, xrow, nullptr, ginv, Os, A.dv, bh, t0, A.n, tid);
+  if (!dv_own) fm_store_tokens<TIO, E, DH, 1>(&dv, xrow, nullptr, ginv, Os, A.dv, bh, t0, A.n, tid);
 }
 template <int DH> inline size_t fm_o1_bwd_lds() {
   const size_t tile = size_t(FM_O1_SEG) * (DH + Mma<fm_half>::PAD) * 2;
   const size_t tiles = 3 * tile + size_t(FM_O1_SEG) * 2 + size_t(3) * DH * 4 + size_t(DH) * (DH + Mma<fm_half>::PAD) * 2 +
-                       size_t(FM_THREADS / 64) * 32 * FM_O1_DQ_PITCH * 2;            // and the wavefronts' dq staging
+                       size_t(FM_THREADS / 64) * 32 * FM_O1_DQ_PITCH * 2;            // and the wavefronts' own output staging
   const size_t outst = tile + size_t(FM_O1_SEG) * fm_store_pitch(DH) * 4;      // Q' / K' tile kept, staging over V and GH
   return tiles > outst ? tiles : outst;
 }
