@@ -219,7 +219,7 @@ def main() -> int:
                            ("c3_order1_bf16", dict(LONG_WORKLOAD, p=1), "bf16"),
                            ("c3_order2_bf16", dict(LONG_WORKLOAD, p=2), "bf16")):
             plain = argparse.Namespace(**dict(vars(args), chunk=0, graph=False, independent_backward=False))
-            r = operator_line(lib, dev, w, dt, plain, steps=10, warmup=3, full=False)
+            r = operator_line(lib, dev, w, dt, plain, steps=30, warmup=10, full=False)
             extra[key] = {"workload": r["config"]["workload"], "dtype": dt, "ms_per_step": r["ms_per_step"],
                           "step_ms": r["step_ms"], "tokens_per_s": r["value"], "forward_only_ms": r["forward_only"]["ms"],
                           "roofline": r["roofline"], "hbm_bound_helpers": r["hbm_bound_helpers"]}
