@@ -24,8 +24,8 @@
 #include "fm_kernels.h"
 
 static constexpr int FM_DEC_ROWS = 64;      // moment rows per workgroup
-inline int64_t fm_decode_rows(int d, bool quad) { return 1 + int64_t(d) + (quad ? int64_t(d) * d : 0); }
-inline int fm_decode_blocks(int d, bool quad) { return int((fm_decode_rows(d, quad) + FM_DEC_ROWS - 1) / FM_DEC_ROWS); }
+constexpr int64_t fm_decode_rows(int d, bool quad) { return 1 + int64_t(d) + (quad ? int64_t(d) * d : 0); }
+constexpr int fm_decode_blocks(int d, bool quad) { return int((fm_decode_rows(d, quad) + FM_DEC_ROWS - 1) / FM_DEC_ROWS); }
 // floats of one batch*head's state: num [R][D] then den [R], R rounded up to whole blocks
 inline int64_t fm_decode_state_floats(int d, bool quad) {
   return int64_t(fm_decode_blocks(d, quad)) * FM_DEC_ROWS * (d + 1);
@@ -147,10 +147,19 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_decode_finish(const float* FM_REST
   const float* p = part + int64_t(bh) * nblk * (DH + 1);
   float f = 0.f, f2 = 0.f;
   const int per = (nblk + FM_THREADS / 64 - 1) / (FM_THREADS / 64), b0 = wave * per, b1 = b0 + per < nblk ? b0 + per : nblk;
-  for (int b = b0; b < b1; ++b) {
-    if (lane < DH) f += p[b * (DH + 1) + lane];
-    if (DH == 64 ? lane == 0 : lane == DH) f2 += p[b * (DH + 1) + DH];
+  // all loads of the wavefront's blocks are issued before the first sum (a loop over a run-time count waits for
+  // every load in turn: 17 memory latencies for the 66 blocks of D = 64, order 2)
+  constexpr int PER_MAX = (fm_decode_blocks(DH, true) + FM_THREADS / 64 - 1) / (FM_THREADS / 64);
+  const bool gl = DH == 64 ? lane == 0 : lane == DH;     // the lane that also adds the g parts
+  float x[PER_MAX], x2[PER_MAX];
+#pragma unroll
+  for (int i = 0; i < PER_MAX; ++i) {
+    const int b = b0 + i;
+    x[i] = (b < b1 && lane < DH) ? p[b * (DH + 1) + lane] : 0.f;
+    x2[i] = (b < b1 && gl) ? p[b * (DH + 1) + DH] : 0.f;
   }
+#pragma unroll
+  for (int i = 0; i < PER_MAX; ++i) { f += x[i]; f2 += x2[i]; }
   if (lane < DH) red[wave][lane] = f;
   if (DH == 64 ? lane == 0 : lane == DH) red[wave][DH] = f2;
   FM_SYNC();
