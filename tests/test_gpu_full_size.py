@@ -67,15 +67,36 @@ def _check_sparse_rows(lib, bh, n, d, dtype, p, seed, scale, chunk=0, count=48, 
     off[rows] = False
     assert float(dq[:, off].float().abs().max()) == 0.0, "dq of a row without upstream gradient"
     got = (o.cpu()[:, rows], g.cpu()[:, rows], dq[:, rows], dk.cpu(), dv.cpu())
-    errs = {name: rel_err(x, r) for name, x, r in zip(("o", "g", "dq", "dk", "dv"), got, ref)}
+    names = ("o", "g", "dq", "dk", "dv")
+    errs = {name: rel_err(x, r) for name, x, r in zip(names, got, ref)}
     for name, e in errs.items():
         assert e < TOL[dtype], f"{name} rel-L2 {e:.3e} (all: {errs})"
     # per slice as well: one bad (b, h) must not hide among the others
     for i in range(bh):
-        for name, x, r in zip(("o", "dk", "dv"), (got[0], got[3], got[4]), (ref[0], ref[3], ref[4])):
+        for name, x, r in zip(names, got, ref):
             e = rel_err(x[i], r[i])
             assert e < TOL[dtype], f"slice {i}: {name} rel-L2 {e:.3e}"
+    # dk and dv per stretch of ``seg`` keys and slice: one wrong suffix state must not hide in a sum over
+    # the whole sequence.  Keys behind the last row with upstream gradient have dk = dv = 0 exactly, on both sides.
+    worst = {}
+    for name, x, r in (("dk", got[3], ref[3]), ("dv", got[4], ref[4])):
+        x = _by_segment(x.double(), seg); r = _by_segment(r.double(), seg)
+        num = (x - r).flatten(2).norm(dim=2); den = r.flatten(2).norm(dim=2)
+        assert bool((num[den == 0] == 0).all()), f"{name}: non-zero where the reference is exactly zero"
+        e = (num / den.clamp_min(1e-300))[den > 0]
+        worst[name] = float(e.max())
+        assert worst[name] < TOL[dtype], f"{name}: worst rel-L2 over {seg}-key stretches {worst[name]:.3e}"
+    print(f"  errs {errs} worst per stretch {worst}", flush=True)
     return errs
+
+
+def _by_segment(x, seg):
+    """(bh, n, d) -> (bh, ceil(n / seg), seg, d), zero padded"""
+    bh, n, d = x.shape
+    pad = (-n) % seg
+    if pad:
+        x = torch.cat([x, x.new_zeros(bh, pad, d)], dim=1)
+    return x.view(bh, -1, seg, d)
 
 
 def _check_running_mean(lib, bh, n, d, dtype, p, seed, chunk=0):
@@ -135,6 +156,14 @@ def test_order1_runs_of_segments(lib, bh, n):
     enter o, dq, dk and dv."""
     print(f"case order-1 runs bh={bh} n={n}", flush=True)
     _check_sparse_rows(lib, bh, n, 64, torch.bfloat16, 1, seed=90 + bh, scale=0.7, seg=128)
+
+
+def test_order1_runs_of_segments_dense_gradient(lib):
+    """The same path with an upstream gradient on every row (runs of three segments), every result against the
+    fp64 closed form."""
+    from tests.parity import check_forward_backward
+    print("case order-1 runs, dense dO", flush=True)
+    check_forward_backward(lib, 40, 5000, 64, torch.bfloat16, DEV, mask=True, p=1, seed=77, scale=0.7, saved=True)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

@@ -271,6 +271,9 @@ def test_upstream_gradient_of_any_size(lib, go_scale):
     for p, chunk in ((2, 0), (2, 256), (1, 0), (1, 256)):
         check_forward_backward(lib, 4, 1024, 64, torch.bfloat16, DEV, mask=True, p=p, chunk=chunk, seed=61,
                                go_scale=go_scale, saved=True)
+    # order 1 beyond 1024 tokens runs on 128-token segments summed in runs, with a scale of its own
+    for n in (1100, 4096):
+        check_forward_backward(lib, 4, n, 64, torch.bfloat16, DEV, mask=True, p=1, seed=64, go_scale=go_scale, saved=True)
     check_forward_backward(lib, 2, 300, 32, torch.bfloat16, DEV, mask=False, p=2, nk=700, seed=62, go_scale=go_scale)
     check_forward_backward(lib, 2, 513, 64, torch.bfloat16, DEV, mask=True, p=2, nk=2100, seed=63, go_scale=go_scale)
 
