@@ -10,7 +10,8 @@ HBM, called through the C ABI (libfastmax_hip.so).  Prints ONE JSON line.
 
 Besides the contract fields the line carries
   roofline:     the dominant kernel, measured live with HIP events on the launch
-                stream (fastmax_profile_begin/end), priced with the ALGORITHMIC
+                stream (the same steps run through libfastmax_hip_bench.so, the product's
+                sources built with per-kernel event brackets), priced with the ALGORITHMIC
                 flop count 2*(D + D^2)*(Dv + 1) per (b, h, token) and unit of
                 work (state build, readout, dQ, dK, dV each count one unit);
   cpu_baseline: the oracle's port of the reference's einops algorithm timed on
@@ -200,7 +201,7 @@ def main() -> int:
         return 2
 
     import torch
-    from reproducing_fastmax_results_amd._capi import get_lib
+    from reproducing_fastmax_results_amd._capi import get_bench_lib, get_lib
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -361,12 +362,20 @@ def operator_line(lib, dev, W, dtype, args, steps, warmup, full):
     torch.cuda.synchronize()
     fwd_ms = 1e3 * (time.perf_counter() - t0) / steps
 
-    # per-kernel durations, HIP events on the launch stream
+    # per-kernel durations, HIP events on the launch stream: the same step through the bench build of the library
+    # (same kernels, every launch bracketed by events; the product library carries no such hooks)
+    from reproducing_fastmax_results_amd._capi import get_bench_lib
+    blib = get_bench_lib()
+    prod, lib = lib, blib
     nprof = max(3, min(10, steps))
-    lib.profile_begin()
+    for _ in range(max(3, warmup)):          # the bench build is a code object of its own: warm it like the product
+        step()
+    torch.cuda.synchronize()
+    blib.profile_begin()
     for _ in range(nprof):
         step()
-    recs = lib.profile_end()
+    recs = blib.profile_end()
+    lib = prod
     per_kernel = {}
     for name, ms in recs:
         tot, cnt = per_kernel.get(name, (0.0, 0))
@@ -437,17 +446,17 @@ def operator_line(lib, dev, W, dtype, args, steps, warmup, full):
     helpers = {}
     for name, fn, nbytes in (
             # the statistics pass of the folded max-norm normalisation: q and k read once (the kernels scale as they load)
-            ("normalize", lambda: lib.maxnorm_stats(q, k), 2 * tensor),) + (() if not full else (
+            ("normalize", lambda: blib.maxnorm_stats(q, k), 2 * tensor),) + (() if not full else (
             # the stand-alone passes (token-mean centring and other callers): forward one statistics read, one apply
             # read, one write; backward: x and dy twice, dx once
-            ("normalize_pass", lambda: lib.normalize(q, centre=0, max_norm=True, scale=1.0), 3 * tensor),
-            ("normalize_backward", lambda: lib.normalize_backward(q, go, centre=0, max_norm=True, scale=1.0), 5 * tensor))):
+            ("normalize_pass", lambda: blib.normalize(q, centre=0, max_norm=True, scale=1.0), 3 * tensor),
+            ("normalize_backward", lambda: blib.normalize_backward(q, go, centre=0, max_norm=True, scale=1.0), 5 * tensor))):
         fn()
         torch.cuda.synchronize()
-        lib.profile_begin()
+        blib.profile_begin()
         for _ in range(5):
             fn()
-        ms = sum(t for nme, t in lib.profile_end() if nme == "normalize") / 5
+        ms = sum(t for nme, t in blib.profile_end() if nme == "normalize") / 5
         helpers[name] = {"ms": ms, "bytes": nbytes, "achieved_GBps": nbytes / (ms * 1e-3) / 1e9,
                          "frac_of_8TBps": nbytes / (ms * 1e-3) / 8e12}
     if "transpose" in roofline["kernels_ms_per_step"]:
@@ -493,11 +502,11 @@ def operator_line(lib, dev, W, dtype, args, steps, warmup, full):
         dst.copy_(src)
     e1.record()
     e1.synchronize()
-    out["measured_on_this_box"] = {"mfma_f16_loop_TFLOPs": lib.mfma_rate(dev),
+    out["measured_on_this_box"] = {"mfma_f16_loop_TFLOPs": blib.mfma_rate(dev),
                                    # the same products fed from LDS with the dense kernels' instruction mix: what a
                                    # kernel of this structure can reach (one / two own tiles per wavefront)
-                                   "mfma_f16_lds_fed_mix_TFLOPs": lib.mix_rate(dev, 1),
-                                   "mfma_f16_lds_fed_mix_two_tiles_TFLOPs": lib.mix_rate(dev, 2),
+                                   "mfma_f16_lds_fed_mix_TFLOPs": blib.mix_rate(dev, 1),
+                                   "mfma_f16_lds_fed_mix_two_tiles_TFLOPs": blib.mix_rate(dev, 2),
                                    "hbm_copy_GBps": 5 * 2 * float(1 << 30) / (e0.elapsed_time(e1) * 1e-3) / 1e9,
                                    "published": {"mfma_bf16_TFLOPs": PEAK_TFLOPS["bf16"], "mfma_f32_TFLOPs": PEAK_TFLOPS["f32"],
                                                  "hbm_GBps": PEAK_HBM_GBS}}

@@ -248,35 +248,10 @@ const char* fastmax_status_string(int status);
 /* Library version: major * 10000 + minor * 100 + patch. */
 int fastmax_version(void);
 
-/* Per-kernel timing for benchmarks (no counterpart in the reference).  Between begin and end the
- * library brackets every kernel it launches with HIP events on the launch stream; end waits for
- * them and returns how many launches were recorded, filling up to `capacity` entries with the
- * kernel id (0 transpose, 1 backward prep, 2 state build, 3 forward, 4 dQ, 5 dK, 6 normalise, 7 dV,
- * 8 dK and dV in one pass)
- * and its duration.  Process-global and not re-entrant: do not use from concurrent threads. */
-int fastmax_profile_begin(void);
-int fastmax_profile_end(int* kernel_ids, float* milliseconds, int capacity);
-
 /* Self-check of the matrix-core lane layout the kernels assume: runs one 32x32 MFMA tile per
  * element type on known operands and writes, for each of the 64 lanes and 16 accumulator
  * registers, the value found (out_f16 and out_f32: 1024 floats each, device memory). */
 int fastmax_probe_mfma(float* out_f16, float* out_f32, void* hip_stream);
-
-/* Yardstick for benchmarks (no counterpart in the reference): `workgroups` workgroups of four
- * wavefronts each issue `iters` rounds of eight independent 32x32x16 _Float16 matrix products on
- * register operands, i.e. workgroups * 4 * iters * 8 * 32768 flop with no memory traffic; timed by
- * the caller with events on `hip_stream`, it gives the matrix rate this device sustains.
- * out: workgroups * 256 floats (device memory, checksums).  workgroups <= 65536, iters <= 2^20. */
-int fastmax_probe_mfma_rate(int workgroups, int iters, float* out, void* hip_stream);
-
-/* Second yardstick (no counterpart in the reference): the same, with the operands coming out of LDS the way the
- * dense kernels' do.  Per round and own tile a wavefront issues the 16 products of one 32x32 tile pair of the
- * dK + dV pass, fed by 8 sixteen-byte LDS reads and 16 transposing eight-byte reads per round (shared by the
- * wavefront's own_tiles = 1 or 2 tiles) and accompanied by 64 packed-half vector instructions per own tile;
- * workgroups * 4 * iters * 16 * own_tiles * 32768 flop.  Timed by the caller, it gives the matrix rate this
- * instruction mix can reach on the device, which is what the dense kernels' own rate is to be held against.
- * out: workgroups * 256 floats.  own_tiles = 1 is built for two workgroups per CU, 2 for one. */
-int fastmax_probe_mix_rate(int workgroups, int iters, int own_tiles, float* out, void* hip_stream);
 
 /* Self-check of the transposing LDS read (ds_read_b64_tr_b16) the _Float16 kernels use for transposed
  * fragments: one wavefront reads a 16 x 64 tile holding 64 * row + col; lane l addresses the four

@@ -16,6 +16,9 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_NAME = "libfastmax_hip.so"
+# The same sources built with -DFM_BENCH_AIDS: per-kernel event timing and two matrix-rate yardsticks on top
+# of the product's entry points.  Only bench.py and the tests of those aids load it.
+BENCH_LIB_NAME = "libfastmax_hip_bench.so"
 
 F32, BF16 = 0, 1
 FLAG_FORCE_MOMENTS, FLAG_FORCE_DENSE, FLAG_SAVE_FOR_BACKWARD, FLAG_F32_COMPUTE = 1, 2, 4, 8
@@ -59,11 +62,11 @@ EXPORTS = (
     "fastmax_workspace_bytes", "fastmax_forward", "fastmax_backward", "fastmax_backward_saved", "fastmax_normalize",
     "fastmax_normalize_stats_bytes", "fastmax_normalize_backward", "fastmax_normalize_backward_stats_bytes",
     "fastmax_status_string", "fastmax_version", "fastmax_probe_mfma", "fastmax_probe_lds_transpose",
-    "fastmax_probe_mfma_rate", "fastmax_probe_mix_rate", "fastmax_key_rpe", "fastmax_output_noise",
-    "fastmax_profile_begin", "fastmax_profile_end", "fastmax_forward_static",
+    "fastmax_key_rpe", "fastmax_output_noise", "fastmax_forward_static",
     "fastmax_maxnorm_stats", "fastmax_maxnorm_stats_bytes",
     "fastmax_decode_state_bytes", "fastmax_decode_scratch_bytes", "fastmax_decode_absorb", "fastmax_decode_step",
 )
+BENCH_EXPORTS = ("fastmax_profile_begin", "fastmax_profile_end", "fastmax_probe_mfma_rate", "fastmax_probe_mix_rate")
 STATIC_SCRATCH_BYTES = 64 << 20     # FASTMAX_STATIC_SCRATCH_BYTES
 
 
@@ -114,8 +117,9 @@ def _gstrides(g: torch.Tensor) -> Strides:
 class FastmaxLib:
     """One loaded copy of the shared library."""
 
-    def __init__(self, path: Optional[str] = None):
-        path = path or os.path.join(_HERE, LIB_NAME)
+    def __init__(self, path: Optional[str] = None, bench: bool = False):
+        path = path or os.path.join(_HERE, BENCH_LIB_NAME if bench else LIB_NAME)
+        self.bench = bench
         if not os.path.exists(path):
             raise ImportError(
                 f"{path} not found: build it with `python __graft_entry__.py` "
@@ -161,17 +165,18 @@ class FastmaxLib:
         L.fastmax_probe_mfma.restype = C.c_int
         L.fastmax_probe_lds_transpose.argtypes = [C.c_void_p, C.c_void_p]
         L.fastmax_probe_lds_transpose.restype = C.c_int
-        L.fastmax_probe_mfma_rate.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p]
-        L.fastmax_probe_mfma_rate.restype = C.c_int
-        L.fastmax_probe_mix_rate.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
-        L.fastmax_probe_mix_rate.restype = C.c_int
         L.fastmax_key_rpe.argtypes = [C.POINTER(NormDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p]
         L.fastmax_key_rpe.restype = C.c_int
         L.fastmax_output_noise.argtypes = [C.POINTER(NormDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p]
         L.fastmax_output_noise.restype = C.c_int
-        L.fastmax_profile_begin.restype = C.c_int
-        L.fastmax_profile_end.argtypes = [C.POINTER(C.c_int), C.POINTER(C.c_float), C.c_int]
-        L.fastmax_profile_end.restype = C.c_int
+        if bench:
+            L.fastmax_probe_mfma_rate.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+            L.fastmax_probe_mfma_rate.restype = C.c_int
+            L.fastmax_probe_mix_rate.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+            L.fastmax_probe_mix_rate.restype = C.c_int
+            L.fastmax_profile_begin.restype = C.c_int
+            L.fastmax_profile_end.argtypes = [C.POINTER(C.c_int), C.POINTER(C.c_float), C.c_int]
+            L.fastmax_profile_end.restype = C.c_int
 
     # -- helpers ---------------------------------------------------------------
     def status_string(self, st: int) -> str:
@@ -414,6 +419,7 @@ class FastmaxLib:
 
     KERNEL_NAMES = ("transpose", "prep_bwd", "build", "fwd", "dq", "dk", "normalize", "dv", "dkv")
 
+    # -- bench aids (only in the library built with -DFM_BENCH_AIDS) --------------------
     def profile_begin(self) -> None:
         self.lib.fastmax_profile_begin()
 
@@ -476,3 +482,15 @@ def get_lib() -> FastmaxLib:
         if _default is None:
             _default = FastmaxLib()
         return _default
+
+
+_bench: Optional[FastmaxLib] = None
+
+
+def get_bench_lib() -> FastmaxLib:
+    """The bench build of the same sources (per-kernel event timing, matrix-rate yardsticks)."""
+    global _bench
+    with _lock:
+        if _bench is None:
+            _bench = FastmaxLib(bench=True)
+        return _bench

@@ -8,6 +8,9 @@
 #include "fm_decode.h"
 #include "fm_o1.h"
 #include "fm_pointwise.h"
+#if defined(FM_BENCH_AIDS)
+#include "fm_bench_aids.h"
+#endif
 #include <atomic>
 #include <cmath>
 #include <mutex>
@@ -66,9 +69,10 @@ inline void fm_allow_lds(const void* fn, size_t bytes) {
 }
 #endif
 
-// ---- optional per-kernel timing (used by the benchmark; not re-entrant) --------
+// ---- per-kernel timing: compiled only into the bench build of this file (-DFM_BENCH_AIDS); in the product
+// library a ProfScope is an empty object and no launch touches any process-wide state ---------------------
 enum { FM_K_TRANSPOSE = 0, FM_K_PREP_BWD = 1, FM_K_BUILD = 2, FM_K_FWD = 3, FM_K_DQ = 4, FM_K_DK = 5, FM_K_NORM = 6, FM_K_DV = 7, FM_K_DKV = 8 };
-#if defined(FM_HOSTSIM)
+#if defined(FM_HOSTSIM) || !defined(FM_BENCH_AIDS)
 struct ProfScope { ProfScope(int, fm_stream_t) {} };
 #else
 struct ProfRec { int id; hipEvent_t a, b; };
@@ -865,18 +869,28 @@ int fastmax_normalize_backward(const FastmaxNormDesc* desc, const void* x, const
   return fm_normalize_bwd_dispatch(desc, x, dy, dx, stats, static_cast<fm_stream_t>(hip_stream));
 }
 
+int fastmax_probe_mfma(float* out_f16, float* out_f32, void* hip_stream) {
+  if (!out_f16 || !out_f32) return FASTMAX_ERR_NULL;
+  FM_KERNEL_LAUNCH(k_probe_mfma, fm_dim3(1), fm_dim3(64), 0, static_cast<fm_stream_t>(hip_stream), out_f16, out_f32);
+  return fm_launch_status();
+}
+
+int fastmax_probe_lds_transpose(float* out, void* hip_stream) {
+  if (!out) return FASTMAX_ERR_NULL;
+  FM_KERNEL_LAUNCH(k_probe_lds_tr, fm_dim3(1), fm_dim3(64), 0, static_cast<fm_stream_t>(hip_stream), out);
+  return fm_launch_status();
+}
+
+#if defined(FM_BENCH_AIDS) && !defined(FM_HOSTSIM)
 int fastmax_profile_begin(void) {
-#if !defined(FM_HOSTSIM)
   for (auto& r : g_prof) { hipEventDestroy(r.a); hipEventDestroy(r.b); }
   g_prof.clear();
   g_prof_on = true;
-#endif
   return FASTMAX_OK;
 }
 
 int fastmax_profile_end(int* kernel_ids, float* milliseconds, int capacity) {
   int n = 0;
-#if !defined(FM_HOSTSIM)
   g_prof_on = false;
   for (auto& r : g_prof) {
     hipEventSynchronize(r.b);
@@ -887,16 +901,7 @@ int fastmax_profile_end(int* kernel_ids, float* milliseconds, int capacity) {
     hipEventDestroy(r.a); hipEventDestroy(r.b);
   }
   g_prof.clear();
-#else
-  (void)kernel_ids; (void)milliseconds; (void)capacity;
-#endif
   return n;
-}
-
-int fastmax_probe_mfma(float* out_f16, float* out_f32, void* hip_stream) {
-  if (!out_f16 || !out_f32) return FASTMAX_ERR_NULL;
-  FM_KERNEL_LAUNCH(k_probe_mfma, fm_dim3(1), fm_dim3(64), 0, static_cast<fm_stream_t>(hip_stream), out_f16, out_f32);
-  return fm_launch_status();
 }
 
 int fastmax_probe_mfma_rate(int workgroups, int iters, float* out, void* hip_stream) {
@@ -917,10 +922,6 @@ int fastmax_probe_mix_rate(int workgroups, int iters, int own_tiles, float* out,
   return fm_launch_status();
 }
 
-int fastmax_probe_lds_transpose(float* out, void* hip_stream) {
-  if (!out) return FASTMAX_ERR_NULL;
-  FM_KERNEL_LAUNCH(k_probe_lds_tr, fm_dim3(1), fm_dim3(64), 0, static_cast<fm_stream_t>(hip_stream), out);
-  return fm_launch_status();
-}
+#endif  // FM_BENCH_AIDS
 
 }  // extern "C"

@@ -32,6 +32,22 @@ def test_exports_match_header(lib):
         assert getattr(lib.lib, n) is not None
 
 
+def test_bench_build_exports_the_aids_on_top(lib):
+    """libfastmax_hip_bench.so: everything the product exports plus the bench aids; the product has none of them."""
+    path = os.path.join(ROOT, "reproducing_fastmax_results_amd", _capi.BENCH_LIB_NAME)
+    if not os.path.exists(path):
+        pytest.skip("bench build of the library not built")
+    bench = _capi.FastmaxLib(path, bench=True)
+    for n in _capi.EXPORTS + _capi.BENCH_EXPORTS:
+        assert getattr(bench.lib, n) is not None
+    for n in _capi.BENCH_EXPORTS:
+        assert not hasattr(lib.lib, n)
+    one = C.c_void_p(256)
+    assert bench.lib.fastmax_probe_mfma_rate(1, 1, None, None) == 1
+    assert bench.lib.fastmax_probe_mfma_rate(0, 1, one, None) == 2
+    assert bench.lib.fastmax_probe_mfma_rate(1, (1 << 20) + 1, one, None) == 2
+
+
 def test_missing_library_fails_loudly(tmp_path):
     with pytest.raises(ImportError, match="no CPU fallback"):
         _capi.FastmaxLib(str(tmp_path / "libfastmax_hip.so"))
@@ -113,9 +129,6 @@ def test_forward_backward_reject_bad_arguments_before_launching(lib):
     assert lib.lib.fastmax_normalize(C.byref(nd), one, one, None, None) == 4   # max_norm needs stats scratch
     assert lib.lib.fastmax_probe_mfma(None, None, None) == 1
     assert lib.lib.fastmax_probe_lds_transpose(None, None) == 1
-    assert lib.lib.fastmax_probe_mfma_rate(1, 1, None, None) == 1
-    assert lib.lib.fastmax_probe_mfma_rate(0, 1, one, None) == 2
-    assert lib.lib.fastmax_probe_mfma_rate(1, (1 << 20) + 1, one, None) == 2
     assert lib.lib.fastmax_version() >= 200
 
 

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from tests.parity import (check_batch_head_strides, check_decode, check_forward, check_forward_backward,
-                          check_norm_fold)
+                          check_norm_fold, make_inputs)
 from reproducing_fastmax_results_amd._capi import FLAG_FORCE_DENSE, FLAG_FORCE_MOMENTS
 
 pytestmark = pytest.mark.gpu
@@ -15,6 +15,13 @@ pytestmark = pytest.mark.gpu
 def lib():
     from reproducing_fastmax_results_amd._capi import get_lib
     return get_lib()
+
+
+@pytest.fixture(scope="module")
+def bench_lib():
+    """The bench build of the library (the product's sources with -DFM_BENCH_AIDS)."""
+    from reproducing_fastmax_results_amd._capi import get_bench_lib
+    return get_bench_lib()
 
 
 DEV = "cuda:0"
@@ -33,9 +40,10 @@ def test_mfma_lane_layout(lib):
     assert torch.equal(a32.cpu(), want)
 
 
-def test_matrix_rate_probe_runs(lib):
+def test_matrix_rate_probe_runs(bench_lib):
     """The bench's yardstick: a register-only loop of matrix products; here only that it runs, writes
     every checksum and reports a rate (16 workgroups, 64 rounds)."""
+    lib = bench_lib
     import ctypes as C
     out = torch.full((16 * 256,), float("nan"), device=DEV)
     stream = torch.cuda.current_stream().cuda_stream
@@ -45,9 +53,10 @@ def test_matrix_rate_probe_runs(lib):
     assert lib.mfma_rate(DEV, workgroups=256, iters=200) > 0.0
 
 
-def test_lds_fed_mix_probe_runs(lib):
+def test_lds_fed_mix_probe_runs(bench_lib):
     """The second yardstick (matrix products fed from LDS with the dense kernels' instruction mix): runs for one and
     two own tiles, writes every checksum, rejects anything else."""
+    lib = bench_lib
     import ctypes as C
     stream = torch.cuda.current_stream().cuda_stream
     for tiles in (1, 2):
@@ -60,6 +69,19 @@ def test_lds_fed_mix_probe_runs(lib):
     assert lib.lib.fastmax_probe_mix_rate(0, 16, 1, C.c_void_p(out.data_ptr()), C.c_void_p(stream)) != 0
     assert lib.lib.fastmax_probe_mix_rate(8, 16, 1, None, C.c_void_p(stream)) != 0
     assert lib.mix_rate(DEV, 1, iters=100) > 0.0
+
+
+def test_bench_build_matches_the_product_and_times_its_kernels(lib, bench_lib):
+    """The bench build runs the same kernels (bit-identical results) and its per-kernel events name them."""
+    q, k, v, go = make_inputs(3, 700, 700, 64, torch.bfloat16, DEV, seed=5)
+    kw = dict(mask=True, inv_tau=0.05, p=2)
+    o0, g0 = lib.forward(q, k, v, **kw)
+    bench_lib.profile_begin()
+    o1, g1 = bench_lib.forward(q, k, v, **kw)
+    recs = bench_lib.profile_end()
+    assert torch.equal(o0, o1) and torch.equal(g0, g1)
+    assert {"transpose", "fwd"} <= {name for name, _ in recs} and all(ms > 0.0 for _, ms in recs)
+    assert not hasattr(lib.lib, "fastmax_profile_begin")      # the product library carries no bench aid
 
 
 def test_lds_transpose_read_layout(lib):

@@ -19,23 +19,29 @@ def lib():
     return _capi.get_lib()
 
 
-def _pair(lib, bh, n, d, dtype, seed, **kw):
+def _pair(lib, bh, n, d, dtype, seed, first=False, **kw):
     gen = torch.Generator().manual_seed(seed)
     q, k, v = (torch.randn(bh, n, d, generator=gen).to(dtype).to(DEV) for _ in range(3))
     o1, g1 = lib.forward(q, k, v, **kw)
     o2 = torch.full_like(o1, float("nan"))
     g2 = torch.full_like(g1, float("nan"))
-    before = torch.cuda.memory_stats()["allocation.all.allocated"]
-    lib.forward_static(q, k, v, o2, g2, **kw)
-    assert torch.cuda.memory_stats()["allocation.all.allocated"] == before     # torch's allocator saw nothing
     torch.cuda.synchronize()
+    before = torch.cuda.memory_stats()["allocation.all.allocated"]
+    free_before = torch.cuda.mem_get_info()[0]               # the driver's own count of free device memory
+    lib.forward_static(q, k, v, o2, g2, **kw)
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_stats()["allocation.all.allocated"] == before     # torch's allocator saw nothing
+    if not first:
+        # nor did the device: a hipMalloc inside the library would lower the driver's free count (the very first
+        # call on a device looks the static array's address up, which is allowed to load the code object)
+        assert torch.cuda.mem_get_info()[0] == free_before
     assert torch.equal(o1, o2) and torch.equal(g1, g2), f"bh={bh} n={n} d={d} {dtype}"
 
 
 def test_static_scratch_forward_matches_forward(lib):
     print("case no-alloc forward", flush=True)
     kw = dict(mask=True, inv_tau=1.0 / (8.0 * math.sqrt(64)), p=2)
-    _pair(lib, 8, 2048, 64, torch.bfloat16, 1, **kw)          # first call on this device: looks the buffer up
+    _pair(lib, 8, 2048, 64, torch.bfloat16, 1, first=True, **kw)          # first call on this device: looks the buffer up
     _pair(lib, 3, 333, 64, torch.bfloat16, 2, **kw)           # smaller, straight after, on the used buffer
     _pair(lib, 2, 1100, 64, torch.float32, 3, chunk=256, **kw)                 # through moment states
     _pair(lib, 2, 300, 32, torch.bfloat16, 4, mask=False, inv_tau=0.1, p=1)
