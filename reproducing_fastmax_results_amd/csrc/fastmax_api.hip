@@ -107,7 +107,8 @@ struct Plan {
   float a0, a1, a2;     // polynomial on the score s = (q.k) / tau
   float sc;             // sqrt(1/tau), folded into q and k when they are converted
   // workspace offsets (bytes)
-  size_t kt, vt, kr, vr, big, big2, small, run, runh, fwd_bytes;   // run, runh: see k_o1_sums
+  size_t kt, vt, kr, vr, big, big2, small, run, runh, ores, fwd_bytes;
+  bool keep_resid;      // the forward leaves o - bf16(o) for the backward (see TokArgs::out_resid)   // run, runh: see k_o1_sums
   bool save;
   size_t b_kr, b_vr, b_qr, b_kt, b_vt, b_qt, b_qct, b_gh, b_ght, b_cv, b_bigq, b_smallq, b_bigk, b_smallk, b_bigv, b_gpart, b_bq, b_bk, b_runq, b_runqh, b_runk, b_runkh, bwd_bytes;
 };
@@ -223,6 +224,8 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   const size_t runarr = size_t(d->bh) * nruns * (d->d == 64 ? O1Run<64>::RS : O1Run<32>::RS) * 4;
   const size_t runharr = size_t(d->bh) * nruns * d->d * d->d * 2;
   p.run = take(runarr); p.runh = take(runharr);
+  p.keep_resid = p.save && d->dtype == FASTMAX_BF16 && !p.o1;
+  p.ores = take(p.keep_resid ? size_t(d->bh) * p.npad_q * d->d * 2 : 0);
   p.fwd_bytes = off ? off : 256;
   off = 0;
   p.b_kt = take(tkt); p.b_vt = take(tkt); p.b_qt = take(tqt); p.b_qct = take(tqt);
@@ -376,6 +379,7 @@ template <typename TIO, typename E> void tok_common(TokArgs<TIO, E>& a, const Fa
   a.quad = p.quad; a.a0 = p.a0; a.a1 = p.a1; a.a2 = p.a2; a.sc = p.sc; a.out_scale = 1.0f; a.zscale = 1.0f;
   a.own_o = TRef<const TIO>{nullptr, 0, 0, 0, 0, 0}; a.own_do = a.own_o;
   a.w_gh = nullptr; a.w_qr = nullptr; a.w_cv = nullptr; a.gpart = nullptr; a.gnblk = 0;
+  a.out_resid = nullptr; a.own_ores = nullptr;
 }
 
 template <typename TIO, typename E, int DH, int QT, int OWN, int QF = 0>
@@ -496,6 +500,7 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   a.out = mref<TIO>(o, d->so);
   a.g = mref<float>(g, d->sg);
   a.n_own = d->nq; a.n_str = d->nk;
+  if (p.keep_resid) a.out_resid = reinterpret_cast<fm_half*>(ws + p.ores);
   // order-2 states: two tiles per wavefront halve the state bytes a token reads (forward 1.38 -> 0.94 ms
   // at B*H = 16, N = 65536 on MI355X); without states one tile per wavefront and more workgroups per CU win
   if (sizeof(E) == 2 && p.use_state && p.quad)

@@ -344,7 +344,7 @@ FM_DEVICE float fm_grad_scale(const float* part, int nblk, int lane) {
 //   qt  [bh][DH][npad]  (q' transposed)                 qct [bh][DH][npad]  (c_i q'_i; skipped when null:
 //                                                        only the state walk reads it)
 //   qr  [bh][npad][DH]  (q' row-major)
-//   cv  [bh][npad]      (c, compute type)
+//   cv  [bh][npad]      (c, fp32)
 // gscale is the power of two of fm_grad_scale (see k_grad_scale): it keeps gh inside the _Float16
 // range; every gradient is linear in (gh, c) and is divided by gscale again when it is stored.
 // Tokens >= n are written as zeros.  grid (npad/64, bh).
@@ -354,8 +354,9 @@ FM_DEVICE float fm_grad_scale(const float* part, int nblk, int lane) {
 template <typename TIO, typename E, int DH>
 FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS)
 k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, TRef<const float> g, int n, int npad, E* FM_RESTRICT gh, E* FM_RESTRICT ght,
-           E* FM_RESTRICT qt, E* FM_RESTRICT qct, E* FM_RESTRICT qr, E* FM_RESTRICT cv, float qscale0,
-           const float* FM_RESTRICT gpart, int gnblk, NormFold qfold) {
+           E* FM_RESTRICT qt, E* FM_RESTRICT qct, E* FM_RESTRICT qr, float* FM_RESTRICT cv, float qscale0,
+           const float* FM_RESTRICT gpart, int gnblk, NormFold qfold, const fm_half* FM_RESTRICT ores) {
+  // ores: what bf16 rounding took away from o ([bh][npad][DH] halves, written by a forward that kept its workspace), or null
   constexpr int PT = 64 + Mma<E>::PAD;
   constexpr int VEC = Mma<E>::VEC;
   constexpr int EPT = DH / 4;                      // elements per thread (4 threads per token)
@@ -370,19 +371,24 @@ k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, TRef<const
   float vg[EPT], vq[EPT];
   float csum = 0.f;
   if (row < n) {
-    const float ginv = gscale / g.base(bh)[int64_t(row) * g.s_n];
+    // every load of the thread is issued before the first result is used
+    float a[EPT], b[EPT], c[EPT];
+    fm_half8 r[EPT / 8];
+    const float gi = g.base(bh)[int64_t(row) * g.s_n];
 #pragma unroll
     for (int j = 0; j < EPT; j += 8) {
-      float a[8], b[8], c[8];
-      IO<TIO>::ld8(d_o.base(bh) + int64_t(row) * d_o.s_n + d0 + j, d_o.vec != 0, a);
-      IO<TIO>::ld8(o.base(bh) + int64_t(row) * o.s_n + d0 + j, o.vec != 0, b);
-      IO<TIO>::ld8(q.base(bh) + int64_t(row) * q.s_n + d0 + j, q.vec != 0, c);
+      IO<TIO>::ld8(d_o.base(bh) + int64_t(row) * d_o.s_n + d0 + j, d_o.vec != 0, &a[j]);
+      IO<TIO>::ld8(o.base(bh) + int64_t(row) * o.s_n + d0 + j, o.vec != 0, &b[j]);
+      IO<TIO>::ld8(q.base(bh) + int64_t(row) * q.s_n + d0 + j, q.vec != 0, &c[j]);
+      r[j / 8] = ores ? *reinterpret_cast<const fm_half8*>(ores + (int64_t(bh) * npad + row) * DH + d0 + j)
+                      : Mma<fm_half>::splat(fm_half(0.f));
+    }
+    const float ginv = gscale / gi;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        vg[j + i] = a[i] * ginv;
-        csum += vg[j + i] * b[i];
-        vq[j + i] = c[i] * qscale;
-      }
+    for (int j = 0; j < EPT; ++j) {
+      vg[j] = a[j] * ginv;
+      csum += vg[j] * (b[j] + float(r[j / 8][j % 8]));
+      vq[j] = c[j] * qscale;
     }
   } else {
 #pragma unroll
@@ -390,7 +396,7 @@ k_prep_bwd(TRef<const TIO> q, TRef<const TIO> o, TRef<const TIO> d_o, TRef<const
   }
   csum += fm_shfl_xor(csum, 1);
   csum += fm_shfl_xor(csum, 2);
-  if (part == 0) cv[int64_t(bh) * npad + t0 + Mma<E>::tperm(tok)] = CE<E>::from(csum);
+  if (part == 0) cv[int64_t(bh) * npad + t0 + Mma<E>::tperm(tok)] = csum;
   E* ghrow = gh + (int64_t(bh) * npad + row) * DH + d0;
   E* qrrow = qr + (int64_t(bh) * npad + row) * DH + d0;
 #pragma unroll
@@ -460,7 +466,7 @@ template <typename E> struct BuildArgs {
                                            // k_state_scan turns the per-segment sums into prefix / suffix states
   // Order-1 sums from row-major operands (k_build1_rows; null: the transposed operands above are read):
   const E* pr; const E* rr;                // [bh][npad][DH] rows of the p and r operands
-  const E* cw;                             // [bh][npad] per-token weights (stored in `tperm` order): the third
+  const float* cw;                         // [bh][npad] per-token weights, fp32 (stored in `tperm` order): the third
                                            // operand is then cw_t * p_t, and zt is not read; or null
 };
 
@@ -1135,7 +1141,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_build1_rows(BuildArgs<E> A) {
   const bool has_w = A.cw != nullptr;
   const E* gp = A.pr + int64_t(bh) * A.npad * DH;
   const E* gr = A.rr + int64_t(bh) * A.npad * DH;
-  const E* gc = has_w ? A.cw + int64_t(bh) * A.npad : nullptr;
+  const float* gc = has_w ? A.cw + int64_t(bh) * A.npad : nullptr;
   // the tiles of this wavefront: A operand (tile, feature offset), B operand (tile or null = weights / ones)
   const E* ta[NS]; const E* tbt[NS];
   int fa_off[NS], fb_off[NS], tl[NS];
@@ -1160,7 +1166,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_build1_rows(BuildArgs<E> A) {
   for (int s = 0; s < NS; ++s) acc[s] = fm_zero16();
   const frag ones = M::splat(E(1.0f));
   TileRegs<E, TT, DH> rp, rr;
-  E creg = E(0.f);
+  float creg = 0.f;
   auto fetch = [&](int t0) {                            // global memory -> registers
     rp.load(gp + int64_t(t0) * DH, DH, tid);
     rr.load(gr + int64_t(t0) * DH, DH, tid);
@@ -1171,7 +1177,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS(FM_THREADS) k_build1_rows(BuildArgs<E> A) {
     if (t0 != tb) FM_SYNC();                            // the previous tile has been read
     rp.store(Lp, PQ, tid);
     rr.store(Lr, PQ, tid);
-    if (has_w && tid < TT) Lc[tid] = creg;
+    if (has_w && tid < TT) Lc[tid] = CE<E>::from(creg);
     if (t0 + TT < te) fetch(t0 + TT);
     FM_SYNC();
 #pragma unroll

@@ -187,8 +187,6 @@ template <> struct TileMath<float> {
   typedef float frag;
   struct Coef { float a0, a1, a2, ta2; };
   static FM_DEVICE Coef coef(float a0, float a1, float a2) { Coef c = {a0, a1, a2, 2.0f * a2}; return c; }
-  typedef float CSplat;
-  static FM_DEVICE float splat_c(float c) { return c; }
   static FM_DEVICE float fwd(const fm_f32x16& s, const Coef& k, bool edge, int lo, int hi, int lh, frag* pb) {
     float g = 0.f;
 #pragma unroll
@@ -201,31 +199,31 @@ template <> struct TileMath<float> {
     }
     return g;
   }
-  static FM_DEVICE void dsc(const fm_f32x16& s, const fm_f32x16& dp, float c, const Coef& k, bool edge, int lo, int hi,
+  static FM_DEVICE void dsc(const fm_f32x16& s, const fm_f32x16& dp, float negc, const Coef& k, bool edge, int lo, int hi,
                             int lh, frag* db) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      float ds = (k.a1 + k.ta2 * s[e]) * (dp[e] - c);
+      float ds = (k.a1 + k.ta2 * s[e]) * (dp[e] + negc);
       if (edge) { const int r = fm_acc_row(e, lh); if (r < lo || r > hi) ds = 0.f; }
       db[e] = ds;
     }
   }
-  static FM_DEVICE void dsr(const fm_f32x16& s, const fm_f32x16& dp, const frag* crow, const Coef& k, bool edge, int lo,
+  static FM_DEVICE void dsr(const fm_f32x16& s, const fm_f32x16& dp, const float* negc, const Coef& k, bool edge, int lo,
                             int hi, int lh, frag* db) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      float ds = (k.a1 + k.ta2 * s[e]) * (dp[e] - crow[e]);
+      float ds = (k.a1 + k.ta2 * s[e]) * (dp[e] + negc[e]);
       if (edge) { const int r = fm_acc_row(e, lh); if (r < lo || r > hi) ds = 0.f; }
       db[e] = ds;
     }
   }
-  static FM_DEVICE void both(const fm_f32x16& s, const fm_f32x16& dp, const frag* crow, const Coef& k, bool edge, int lo,
+  static FM_DEVICE void both(const fm_f32x16& s, const fm_f32x16& dp, const float* negc, const Coef& k, bool edge, int lo,
                              int hi, int lh, frag* pb, frag* db) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const float x = s[e];
       float pv = k.a0 + x * (k.a1 + k.a2 * x);
-      float ds = (k.a1 + k.ta2 * x) * (dp[e] - crow[e]);
+      float ds = (k.a1 + k.ta2 * x) * (dp[e] + negc[e]);
       if (edge) { const int r = fm_acc_row(e, lh); if (r < lo || r > hi) { pv = 0.f; ds = 0.f; } }
       pb[e] = pv;
       db[e] = ds;
@@ -253,8 +251,6 @@ template <> struct TileMath<fm_half> {
     c.a0 = pair(a0); c.a1 = pair(a1); c.a2 = pair(a2); c.ta2 = pair(2.0f * a2);
     return c;
   }
-  typedef fm_half2 CSplat;
-  static FM_DEVICE fm_half2 splat_c(float c) { return pair(c); }
   static FM_DEVICE fm_half2 cvt2(float a, float b) {
     fm_f32x2 v = {a, b};
     return __builtin_convertvector(v, fm_half2);
@@ -292,19 +288,25 @@ template <> struct TileMath<fm_half> {
       for (int i = 0; i < 4; ++i) g = fm_dot2(get2(pb[ss], i), one, g);
     return g;
   }
-  static FM_DEVICE void dsc(const fm_f32x16& s, const fm_f32x16& dp, fm_half2 c, const Coef& k, bool edge, int lo, int hi,
+  // Own = queries (dsc): c of the lane's query is subtracted as a half from the rounded gh.v (its rounding moves the
+  // query's own gradient by a few parts in a thousand at worst).  Own = keys (dsr, both): c is taken off gh.v in
+  // fp32, before the difference is rounded: the two are of one size, and an error in c has one sign along a query's
+  // whole row of keys, so over the keys it adds up in sum_j dk_j (what a projection's weight gradient sees) instead
+  // of averaging out.
+  static FM_DEVICE void dsc(const fm_f32x16& s, const fm_f32x16& dp, float negc, const Coef& k, bool edge, int lo, int hi,
                             int lh, frag* db) {
+    const fm_half2 nc = pair(negc);
 #pragma unroll
     for (int ss = 0; ss < 2; ++ss)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int e = 8 * ss + 2 * i;
         const fm_half2 x = cvt2(s[e], s[e + 1]);
-        put2(db[ss], i, (x * k.ta2 + k.a1) * (cvt2(dp[e], dp[e + 1]) - c));
+        put2(db[ss], i, (x * k.ta2 + k.a1) * (cvt2(dp[e], dp[e + 1]) + nc));
       }
     if (edge) { FM_KEEP_BRANCH(); window_frags(db, lo, hi, lh); }
   }
-  static FM_DEVICE void dsr(const fm_f32x16& s, const fm_f32x16& dp, const frag* crow, const Coef& k, bool edge, int lo,
+  static FM_DEVICE void dsr(const fm_f32x16& s, const fm_f32x16& dp, const float* negc, const Coef& k, bool edge, int lo,
                             int hi, int lh, frag* db) {
 #pragma unroll
     for (int ss = 0; ss < 2; ++ss)
@@ -312,11 +314,11 @@ template <> struct TileMath<fm_half> {
       for (int i = 0; i < 4; ++i) {
         const int e = 8 * ss + 2 * i;
         const fm_half2 x = cvt2(s[e], s[e + 1]);
-        put2(db[ss], i, (x * k.ta2 + k.a1) * (cvt2(dp[e], dp[e + 1]) - get2(crow[ss], i)));
+        put2(db[ss], i, (x * k.ta2 + k.a1) * cvt2(dp[e] + negc[e], dp[e + 1] + negc[e + 1]));
       }
     if (edge) { FM_KEEP_BRANCH(); window_frags(db, lo, hi, lh); }
   }
-  static FM_DEVICE void both(const fm_f32x16& s, const fm_f32x16& dp, const frag* crow, const Coef& k, bool edge, int lo,
+  static FM_DEVICE void both(const fm_f32x16& s, const fm_f32x16& dp, const float* negc, const Coef& k, bool edge, int lo,
                              int hi, int lh, frag* pb, frag* db) {
 #pragma unroll
     for (int ss = 0; ss < 2; ++ss)
@@ -325,7 +327,7 @@ template <> struct TileMath<fm_half> {
         const int e = 8 * ss + 2 * i;
         const fm_half2 x = cvt2(s[e], s[e + 1]);
         put2(pb[ss], i, (x * k.a2 + k.a1) * x + k.a0);
-        put2(db[ss], i, (x * k.ta2 + k.a1) * (cvt2(dp[e], dp[e + 1]) - get2(crow[ss], i)));
+        put2(db[ss], i, (x * k.ta2 + k.a1) * cvt2(dp[e] + negc[e], dp[e + 1] + negc[e + 1]));
       }
     if (edge) { FM_KEEP_BRANCH(); window_frags(pb, lo, hi, lh); window_frags(db, lo, hi, lh); }
   }

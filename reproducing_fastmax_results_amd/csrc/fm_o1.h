@@ -75,10 +75,11 @@ template <int DH> struct O1Raw {
 
 // gh = gscale * dO / g and c = gh . o of the segment's rows, from raw dO and o chunks and the denominators gi of
 // the thread's rows (1 past the end): gh rows go to the LDS
-// tile Gs, c (compute type, 16-token groups in `tperm` order) to cs.  Every lane takes part in the shuffles.
+// tile Gs, c to cs (compute type, 16-token groups in `tperm` order: the weights of a matrix product) or to cf
+// (fp32, natural order: what the score gradient subtracts), whichever is given.  Every lane takes part in the shuffles.
 template <int DH>
 FM_DEVICE void fm_o1_gh_rows(const O1Raw<DH>& rdo, const O1Raw<DH>& ro, const float* gi, float gscale, fm_half* Gs,
-                             int pitch, fm_half* cs, int tid) {
+                             int pitch, fm_half* cs, float* cf, int tid) {
   typedef O1Raw<DH> R;
 #pragma unroll
   for (int i = 0; i < R::N; ++i) {
@@ -93,7 +94,10 @@ FM_DEVICE void fm_o1_gh_rows(const O1Raw<DH>& rdo, const O1Raw<DH>& ro, const fl
 #pragma unroll
     for (int m = 1; m < R::CPR; m <<= 1) csum += fm_shfl_xor(csum, m);
     CE<fm_half>::st8(Gs + row * pitch + R::col_of(tid), a);
-    if (tid % R::CPR == 0) cs[Mma<fm_half>::tperm(row)] = CE<fm_half>::from(csum);
+    if (tid % R::CPR == 0) {
+      if (cs) cs[Mma<fm_half>::tperm(row)] = CE<fm_half>::from(csum);
+      if (cf) cf[row] = csum;
+    }
   }
 }
 
@@ -182,7 +186,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_sums(O1SumArgs<TIO> A) {
     FM_SYNC();                                                         // the products of the segment before are done with the tiles
     if (QG) {
       r0.store(Lp, PQ, tid, s0);                                       // p = q'
-      fm_o1_gh_rows<DH>(r1, ro, gi, gscale, Lr, PQ, Lc, tid);          // r = gh, weights c
+      fm_o1_gh_rows<DH>(r1, ro, gi, gscale, Lr, PQ, Lc, nullptr, tid); // r = gh, weights c
     } else {
       r1.store(Lp, PQ, tid, 1.0f);                                     // p = v
       r0.store(Lr, PQ, tid, s0);                                       // r = k'
@@ -453,8 +457,8 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
   E* Ks = reinterpret_cast<E*>(smem);                   // [QW][PQ] each; Q' later lies over K'
   E* Vs = Ks + QW * PQ;
   E* Gs = Vs + QW * PQ;
-  E* cs = Gs + QW * PQ;                                  // [QW] c in `tperm` order
-  float* vecs = reinterpret_cast<float*>(cs + QW);       // va of the prefix sums | va, vb of the suffix sums: 3 * DH
+  float* cs = reinterpret_cast<float*>(Gs + QW * PQ);    // [QW] c, fp32
+  float* vecs = cs + QW;                                 // va of the prefix sums | va, vb of the suffix sums: 3 * DH
   E* Sl = reinterpret_cast<E*>(vecs + 3 * DH);           // one state slab [DH][PS], rows in `tperm` order
   E* Qs = Ks;
   constexpr int PS = C::PS;
@@ -515,7 +519,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
     slab_store(rs, rs2);
     rk.store(Ks, PQ, tid, ksc);
     rv.store(Vs, PQ, tid, 1.0f);
-    fm_o1_gh_rows<DH>(rdo, ro, gi, gsc, Gs, PQ, cs, tid);
+    fm_o1_gh_rows<DH>(rdo, ro, gi, gsc, Gs, PQ, nullptr, cs, tid);
   }
   FM_SYNC();
 
@@ -526,8 +530,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
     const int off = own * PQ + ks * M::KSTEP + lh * M::KPL;
     gf[ks] = M::load(Gs + off); kf[ks] = M::load(Ks + off); vf[ks] = M::load(Vs + off);
   }
-  const float ci = float(cs[wave * 32 + M::tperm(lr)]);
-  const typename TM::CSplat csp = TM::splat_c(ci);
+  const float ci = cs[wave * 32 + lr];
   const typename TM::Coef coef = TM::coef(A.a0, A.a1, 0.0f);
   fm_f32x16 dq[NT], dk[NT], dv[NT];
 #pragma unroll
@@ -554,7 +557,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) dp = M::mma(M::load(vrow + ks * M::KSTEP), gf[ks], dp);
     frag db[M::ACC_KSTEPS];
-    TM::dsc(zero, dp, csp, coef, jt == wave, 0, lr, lh, db);         // diagonal tile: key row <= the lane's query
+    TM::dsc(zero, dp, -ci, coef, jt == wave, 0, lr, lh, db);         // diagonal tile: key row <= the lane's query
 #pragma unroll
     for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
 #pragma unroll
@@ -610,10 +613,14 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
       s = M::mma(M::load(qrow + ks * M::KSTEP), kf[ks], s);
       dp = M::mma(M::load(grow + ks * M::KSTEP), vf[ks], dp);
     }
-    frag crow[M::ACC_KSTEPS], pb[M::ACC_KSTEPS], db[M::ACC_KSTEPS];
+    frag pb[M::ACC_KSTEPS], db[M::ACC_KSTEPS];
+    float negc[16];                                      // -c of the tile's queries, the lane's 16 accumulator rows
 #pragma unroll
-    for (int ss = 0; ss < M::ACC_KSTEPS; ++ss) crow[ss] = M::load_perm(cs + 32 * it, ss, lh);
-    TM::both(s, dp, crow, coef, it == wave, lr, 31, lh, pb, db);     // diagonal tile: query row >= the lane's key
+    for (int gq = 0; gq < 4; ++gq) {
+      const fm_f32x4 t = *reinterpret_cast<const fm_f32x4*>(cs + 32 * it + 4 * lh + 8 * gq);
+      negc[4 * gq] = -t[0]; negc[4 * gq + 1] = -t[1]; negc[4 * gq + 2] = -t[2]; negc[4 * gq + 3] = -t[3];
+    }
+    TM::both(s, dp, negc, coef, it == wave, lr, 31, lh, pb, db);     // diagonal tile: query row >= the lane's key
 #pragma unroll
     for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
 #pragma unroll
@@ -673,7 +680,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, 2) k_o1_bwd(O1BwdArgs<TIO> A) {
 }
 template <int DH> inline size_t fm_o1_bwd_lds() {
   const size_t tile = size_t(FM_O1_SEG) * (DH + Mma<fm_half>::PAD) * 2;
-  const size_t tiles = 3 * tile + size_t(FM_O1_SEG) * 2 + size_t(3) * DH * 4 + size_t(DH) * (DH + Mma<fm_half>::PAD) * 2 +
+  const size_t tiles = 3 * tile + size_t(FM_O1_SEG) * 4 + size_t(3) * DH * 4 + size_t(DH) * (DH + Mma<fm_half>::PAD) * 2 +
                        size_t(FM_THREADS / 64) * 32 * FM_O1_DQ_PITCH * 2;            // and the wavefronts' own output staging
   const size_t outst = tile + size_t(FM_O1_SEG) * fm_store_pitch(DH) * 4;      // Q' / K' tile kept, staging over V and GH
   return tiles > outst ? tiles : outst;

@@ -28,7 +28,7 @@ template <typename TIO, typename E> struct TokArgs {
   TRef<const TIO> own_io;   // k_pv, own = queries: q in the caller's tensor (multiplied by sc on load)
   const E* own_r;           // otherwise: own tokens, row-major compute-type copy [bh][npad_own][DH]
   const E* own2_r;          // k_ds: second own operand rows (gh for own = queries, v for own = keys)
-  const E* cv;              // k_ds: c per query [bh][npad_q] in tile order
+  const float* cv;          // k_ds: c per query [bh][npad_q], fp32, tokens of every group of 16 in `tperm` order
   const E* xr;              // stream rows that form the scores      [bh][npad_str][DH]
   const E* yr;              // k_ds: stream rows that form gh.v      [bh][npad_str][DH]
   const E* zt;              // stream tokens, transposed             [bh][DH][npad_str]
@@ -49,7 +49,7 @@ template <typename TIO, typename E> struct TokArgs {
   // its own queries itself, from the caller's tensors, and leaves them in w_gh, w_qr (row-major
   // [bh][npad_own][DH]) and w_cv ([bh][npad_own], tile order) for the key-side pass that follows
   TRef<const TIO> own_o, own_do;
-  E* w_gh; E* w_qr; E* w_cv;
+  E* w_gh; E* w_qr; float* w_cv;
   // partial maxima of |dO| / |g| ([bh][gnblk], see k_grad_scale) or null: the kernels that form gh multiply it by
   // fm_grad_scale of them, the kernels that store a gradient divide by it
   const float* gpart; int gnblk;
@@ -60,7 +60,23 @@ template <typename TIO, typename E> struct TokArgs {
   // the copy `brows` = sc * y) in bpart [bh][blocks]; k_norm_fix applies the rank-one term to one row later.
   NormFold own_fold, out_fold;
   const E* brows; float* bpart;
+  // What bf16 rounding takes away from o, [bh][npad_own][DH] halves: o = (the caller's bf16 o) + this.  The forward
+  // writes it next to o when its workspace is kept for the backward (out_resid), the backward's preparation adds it
+  // back (own_ores) before it forms c = gh . o: c is subtracted from numbers of its own size, gh . v, so the 8 bits
+  // of a bf16 o would leave dS with a few bits, and with an error of one sign along a whole row of keys.
+  fm_half* out_resid; const fm_half* own_ores;
 };
+
+// eight values as they will read back from the caller's tensor: themselves (fp32) or rounded to bf16
+template <typename TIO> FM_DEVICE float fm_as_stored(float v);
+template <> FM_DEVICE float fm_as_stored<float>(float v) { return v; }
+template <> FM_DEVICE float fm_as_stored<fm_bf16>(float v) { return fm_bf16_to_f32(fm_f32_to_bf16(v)); }
+FM_DEVICE void fm_store_resid8(fm_half* p, const float v[8], const float stored[8]) {
+  fm_half8 r;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) r[i] = fm_half(v[i] - stored[i]);
+  *reinterpret_cast<fm_half8*>(p) = r;
+}
 
 // Z (fp32, [DH][DH]) -> LDS in the compute type (hi/lo split for _Float16), va/vb -> vecs.
 template <typename E, int DH, int QT>
@@ -474,6 +490,12 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (TokCfg<E, DH, QT>::OCC_PV)) k_pv(T
         const fm_f32x4 hi = *reinterpret_cast<const fm_f32x4*>(Os + row * OP + col + 4);
         const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         IO<TIO>::st8(ob + int64_t(t0 + row) * A.out.s_n + col, A.out.vec != 0, v);
+        if (A.out_resid) {
+          float sv[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) sv[i] = fm_as_stored<TIO>(v[i]);
+          fm_store_resid8(A.out_resid + (int64_t(bh) * A.npad_own + t0 + row) * DH + col, v, sv);
+        }
       }
     }
   } else {
@@ -588,11 +610,13 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
     // (fastmax_cuda_backward.cu:494-501) and the "grad * o" row sums of fastattention_einops.py:405-407.
     constexpr int EPT = DH / 4;
     static_assert(!PREP || (OWN == FM_OWN_Q && QT == 1), "the fused preparation is for one query tile per wavefront");
+    // PREP = 2: A.own_ores is given (the forward kept what bf16 rounding took from o)
     float* cl = reinterpret_cast<float*>(R + QW * PQ);   // c per own query, behind the gh rows
     const int part = tid & 3, d0 = part * EPT;
     constexpr int NH = QW / 64;
     const float qsc = A.sc * fm_norm_factor(A.own_fold, bh, lane);
     float ra[NH][EPT], rb[NH][EPT], rc[NH][EPT], gi[NH];
+    fm_half8 rr[NH][EPT / 8];
     // every load of the block is issued before the first result is used
 #pragma unroll
     for (int h = 0; h < NH; ++h) {
@@ -604,11 +628,14 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
           IO<TIO>::ld8(A.own_do.base(bh) + int64_t(row) * A.own_do.s_n + d0 + j, A.own_do.vec != 0, &ra[h][j]);
           IO<TIO>::ld8(A.own_o.base(bh) + int64_t(row) * A.own_o.s_n + d0 + j, A.own_o.vec != 0, &rb[h][j]);
           IO<TIO>::ld8(A.own_io.base(bh) + int64_t(row) * A.own_io.s_n + d0 + j, A.own_io.vec != 0, &rc[h][j]);
+          if (PREP == 2) rr[h][j / 8] = *reinterpret_cast<const fm_half8*>(A.own_ores + (int64_t(bh) * A.npad_own + row) * DH + d0 + j);
         }
       } else {
         gi[h] = 1.0f;
 #pragma unroll
         for (int j = 0; j < EPT; ++j) { ra[h][j] = 0.f; rb[h][j] = 0.f; rc[h][j] = 0.f; }
+#pragma unroll
+        for (int j = 0; j < EPT / 8; ++j) rr[h][j] = Mma<fm_half>::splat(fm_half(0.f));
       }
     }
 #pragma unroll
@@ -620,15 +647,14 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
 #pragma unroll
       for (int j = 0; j < EPT; ++j) {
         vg[j] = ra[h][j] * ginv;
-        csum += vg[j] * rb[h][j];
+        csum += vg[j] * (PREP == 2 ? rb[h][j] + float(rr[h][j / 8][j % 8]) : rb[h][j]);   // PREP = 2: o = bf16 o + what its rounding took
         vq[j] = rc[h][j] * qsc;
       }
       csum += fm_shfl_xor(csum, 1);
       csum += fm_shfl_xor(csum, 2);
-      const E ch = CE<E>::from(csum);
       if (part == 0) {
-        A.w_cv[int64_t(bh) * A.npad_own + t0 + 64 * h + M::tperm(tid >> 2)] = ch;
-        cl[tok] = float(ch);
+        A.w_cv[int64_t(bh) * A.npad_own + t0 + 64 * h + M::tperm(tid >> 2)] = csum;
+        cl[tok] = csum;
       }
       E* ghrow = A.w_gh + (int64_t(bh) * A.npad_own + row) * DH + d0;
       E* qrrow = A.w_qr + (int64_t(bh) * A.npad_own + row) * DH + d0;
@@ -651,15 +677,13 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
   FM_SYNC();
 
   int tw[QT], xrow[QT];
-  float ci[QT];
-  typename TM::CSplat cs_own[QT];                      // own = queries: c of the lane's query
+  float ci[QT];                                        // own = queries: c of the lane's query
 #pragma unroll
   for (int j = 0; j < QT; ++j) {
     tw[j] = (j == 0) ? wave : (4 * QT - 1 - wave);
     xrow[j] = tw[j] * 32 + lr;
     ci[j] = (OWN == FM_OWN_Q) ? (PREP ? reinterpret_cast<const float*>(R + QW * PQ)[xrow[j]]
-                                      : float(A.cv[int64_t(bh) * A.npad_own + t0 + M::tperm(xrow[j])])) : 1.0f;
-    cs_own[j] = TM::splat_c(ci[j]);
+                                      : A.cv[int64_t(bh) * A.npad_own + t0 + M::tperm(xrow[j])]) : 1.0f;
   }
   frag of[QT][NKS], of2[QT][NKS];
 #pragma unroll
@@ -754,7 +778,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
     const E* xb = A.xr + int64_t(bh) * A.npad_str * DH;
     const E* yb = A.yr + int64_t(bh) * A.npad_str * DH;
     const E* zb = A.zt + int64_t(bh) * DH * A.npad_str;
-    const E* cvb = A.cv + int64_t(bh) * A.npad_str;    // own = keys: c of the streamed queries
+    const float* cvb = A.cv + int64_t(bh) * A.npad_str;   // own = keys: c of the streamed queries
     const E* z2b = DV ? A.zt2 + int64_t(bh) * DH * A.npad_str : nullptr;
     // stage order: see k_pv
     const int nst = (G.send - G.sbeg + KT - 1) / KT;
@@ -762,25 +786,23 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
     const int s_step = OWN == FM_OWN_Q ? KT : -KT;
     TileRegs<E, KT, DH> rx, ry;
     TileRegs<E, DH, KT> rz, rz2;
-    E creg = E(0.f);
+    float creg = 0.f;
     auto more = [&](int sx) { return OWN == FM_OWN_Q ? (sx < G.send) : (sx >= G.sbeg); };
     auto fetch = [&](int sx) {                          // global memory -> registers
       rx.load(xb + int64_t(sx) * DH, DH, tid);
       ry.load(yb + int64_t(sx) * DH, DH, tid);
       if (!TR) rz.load(zb + sx, A.npad_str, tid);
       if (DV && !TR) rz2.load(z2b + sx, A.npad_str, tid);
-      // QF: c is staged as -c in fp32, tokens in their natural order (the copy holds them in `tperm` order).
+      // c is staged as -c in fp32, tokens in their natural order (the copy holds them in `tperm` order).
       // Every thread takes part (the threads past KT repeat the first ones): no branch in the stage loop.
-      if (OWN == FM_OWN_K) creg = cvb[sx + (QF ? M::tperm(tid % KT) : tid % KT)];
+      if (OWN == FM_OWN_K) creg = cvb[sx + M::tperm(tid % KT)];
     };
     auto put = [&](int b) {                             // registers -> stage buffer b
       E* Xn = Own + b * STAGE; E* Yn = Xn + KT * PQ; E* Zn = Yn + KT * PQ; E* cn = Zn + (TR ? 0 : DH * PV);
       rx.store(Xn, PQ, tid); ry.store(Yn, PQ, tid);
       if (!TR) rz.store(Zn, PV, tid);
-      if (DV && !TR) rz2.store(cn + KT, PV, tid);
-      if (OWN == FM_OWN_K) {
-        if (QF) reinterpret_cast<float*>(cn)[tid % KT] = -float(creg); else cn[tid % KT] = creg;
-      }
+      if (DV && !TR) rz2.store(cn + (sizeof(E) == 2 ? 2 : 1) * KT, PV, tid);
+      if (OWN == FM_OWN_K) reinterpret_cast<float*>(cn)[tid % KT] = -creg;
     };
     // Two buffers: the tiles of stage i+1 travel global memory -> registers during stage i-1 and
     // registers -> LDS in the middle of stage i (see k_pv).  One buffer (fp32): both at the top.
@@ -792,7 +814,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
     int buf = 0;
     for (int s0 = s_first; more(s0); s0 += s_step) {
       E* Xs = Own + buf * STAGE; E* Ys = Xs + KT * PQ; E* Zt = Ys + KT * PQ; E* cs = Zt + (TR ? 0 : DH * PV);
-      E* Zt2 = cs + KT;
+      E* Zt2 = cs + (sizeof(E) == 2 ? 2 : 1) * KT;        // behind the KT floats of -c
       if (NBUF == 1) put(0);
       FM_SYNC();
       if (NBUF == 1 && more(s0 + s_step)) fetch(s0 + s_step);
@@ -835,10 +857,18 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
             for (int j = 0; j < QT; ++j) s[j] = M::mma(xf, of[j][ks], s[j]);
           }
         }
-        frag zf[NT][M::ACC_KSTEPS], crow[M::ACC_KSTEPS];
+        frag zf[NT][M::ACC_KSTEPS];
+        float negc[16];                                  // own = keys, not seeded: -c of the tile's queries, the lane's 16 accumulator rows
+        if (OWN == FM_OWN_K && !QF) {
+          const float* cf = reinterpret_cast<const float*>(cs) + 32 * st + 4 * lh;
+#pragma unroll
+          for (int gq = 0; gq < 4; ++gq) {
+            const fm_f32x4 t = *reinterpret_cast<const fm_f32x4*>(cf + 8 * gq);
+            negc[4 * gq] = t[0]; negc[4 * gq + 1] = t[1]; negc[4 * gq + 2] = t[2]; negc[4 * gq + 3] = t[3];
+          }
+        }
 #pragma unroll
         for (int ss = 0; ss < M::ACC_KSTEPS; ++ss) {
-          if (OWN == FM_OWN_K && !QF) crow[ss] = M::load_perm(cs + 32 * st, ss, lh);
 #pragma unroll
           for (int mt = 0; mt < NT; ++mt)
             zf[mt][ss] = TR ? M::load_tr(Xs, PQ, 32 * st + 16 * ss, 32 * mt, lane)
@@ -882,9 +912,9 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
           if constexpr (QF != 0) {
             if (DV) TM::bothq(s[j], dp, TM::pair(4.0f * A.a0 * A.a2 - A.a1 * A.a1), edge, wlo, whi, lh, pb, db);
             else TM::dsq(s[j], dp, edge, wlo, whi, lh, db);
-          } else if (DV) TM::both(s[j], dp, crow, coef, edge, wlo, whi, lh, pb, db);
-          else if (OWN == FM_OWN_Q) TM::dsc(s[j], dp, cs_own[j], coef, edge, wlo, whi, lh, db);
-          else TM::dsr(s[j], dp, crow, coef, edge, wlo, whi, lh, db);
+          } else if (DV) TM::both(s[j], dp, negc, coef, edge, wlo, whi, lh, pb, db);
+          else if (OWN == FM_OWN_Q) TM::dsc(s[j], dp, -ci[j], coef, edge, wlo, whi, lh, db);
+          else TM::dsr(s[j], dp, negc, coef, edge, wlo, whi, lh, db);
 #pragma unroll
           for (int ss = 0; ss < M::ACC_KSTEPS; ++ss)
 #pragma unroll

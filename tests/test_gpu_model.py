@@ -69,7 +69,7 @@ def test_gpt_step_matches_oracle_bf16():
     def lm_loss(logits, tgt):
         return torch.nn.functional.cross_entropy(logits.float().view(-1, logits.shape[-1]), tgt.view(-1))
 
-    loss, worst = compare(hip, ref, tokens, target, lm_loss, 2e-2, 6e-2)
+    loss, worst = compare(hip, ref, tokens, target, lm_loss, 2e-2, 2e-2)
     print(f"gpt bf16: loss {loss:.4f}, worst parameter-gradient rel-L2 {worst:.2e}", flush=True)
 
 
@@ -138,13 +138,13 @@ def _lm_loss(logits, tgt):
 def _gpt_full_depth(dtype):
     from reproducing_fastmax_results_amd.transformer.model import gpt_for_c5
     torch.manual_seed(14)
-    hip = gpt_for_c5(vocab_size=512, out_dim=512).to(DEV).to(dtype)
+    hip = gpt_for_c5().to(DEV).to(dtype)                   # the real vocabulary: 50 257 logits per token
     assert len(hip.blocks) == 6
     ref = copy.deepcopy(hip)
     for blk in ref.blocks:
         blk.attention_subblock.attention_fn = oracle_attention
-    tokens = torch.randint(0, 512, (16, 1024), generator=torch.Generator().manual_seed(15)).to(DEV)
-    target = torch.randint(0, 512, (16, 1024), generator=torch.Generator().manual_seed(16)).to(DEV)
+    tokens = torch.randint(0, 50257, (16, 1024), generator=torch.Generator().manual_seed(15)).to(DEV)
+    target = torch.randint(0, 50257, (16, 1024), generator=torch.Generator().manual_seed(16)).to(DEV)
     return hip, ref, tokens, target
 
 
@@ -159,26 +159,38 @@ def test_gpt_step_full_depth_fp32():
 
 
 def test_gpt_step_full_depth_bf16():
-    """The same model in bf16.  Six bf16 blocks amplify a one-rounding-step difference in an attention output,
-    so the gradients of the HIP model are judged against what an operator with a relative error of 3e-3 (well
-    inside the operator's 2e-2 bar, about what the kernels measure) does to the same model: every parameter
-    gradient of the HIP model must be at most twice as far from the oracle model's as that yardstick's."""
+    """The same model in bf16.  Six bf16 blocks amplify a one-rounding-step difference in an attention output, and
+    how much differs from one perturbation to the next (the key projection of block 1 moves between 1.5e-2 and
+    5e-2 for operators that are 1e-3 from the truth).  So the yardstick is a family: the oracle with seeded relative
+    Gaussian noise of 2e-3 on its result (about what rounding a result to bf16 does, a tenth of the operator's
+    2e-2 bar), four seeds; every parameter gradient of the HIP model must be at most twice as far from the oracle
+    model's as the worst of the four."""
     hip, ref, tokens, target = _gpt_full_depth(torch.bfloat16)
-    noisy = copy.deepcopy(ref)
-    for i, blk in enumerate(noisy.blocks):
-        blk.attention_subblock.attention_fn = noisy_oracle_attention(3e-3, 100 + i)
-    lh, lr, ln = (_lm_loss(m(tokens), target) for m in (hip, ref, noisy))
-    assert abs(lh.item() - lr.item()) <= 2e-2 * max(1.0, abs(lr.item()))
-    gh, gr, gn = grads_of(hip, lh), grads_of(ref, lr), grads_of(noisy, ln)
+    lh, lr = (_lm_loss(m(tokens), target) for m in (hip, ref))
+    assert abs(lh.item() - lr.item()) <= 2e-3 * max(1.0, abs(lr.item()))
+    gh, gr = grads_of(hip, lh), grads_of(ref, lr)
+    yard = {name: 0.0 for name in gr}
+    flips_yard = 0.0
+    for seed in range(4):
+        noisy = copy.deepcopy(ref)
+        for i, blk in enumerate(noisy.blocks):
+            blk.attention_subblock.attention_fn = noisy_oracle_attention(2e-3, 1000 * seed + i)
+        gn = grads_of(noisy, _lm_loss(noisy(tokens), target))
+        for name in gr:
+            yard[name] = max(yard[name], float((gn[name] - gr[name]).norm()) / max(float(gr[name].norm()), 1e-30))
+        if seed == 0:
+            flips_yard = adamw_step_compare(noisy, copy.deepcopy(ref), tokens, target, _lm_loss, 1e-3, 1.0)
+        del noisy
     worst_h = worst_n = 0.0
     for name in gr:
-        den = max(float(gr[name].norm()), 1e-6)
-        eh, en = float((gh[name] - gr[name]).norm()) / den, float((gn[name] - gr[name]).norm()) / den
-        worst_h, worst_n = max(worst_h, eh), max(worst_n, en)
-        assert eh <= 2.0 * max(en, 2e-2), f"{name}: HIP {eh:.3e}, yardstick {en:.3e}"
-    share = adamw_step_compare(hip, ref, tokens, target, _lm_loss, 1e-3, 0.25)
+        eh = float((gh[name] - gr[name]).norm()) / max(float(gr[name].norm()), 1e-30)
+        worst_h, worst_n = max(worst_h, eh), max(worst_n, yard[name])
+        assert eh <= 2.0 * max(yard[name], 1e-3), f"{name}: HIP {eh:.3e}, yardstick {yard[name]:.3e}"
+    # one AdamW step: elements whose update differs in sign are those whose gradient lies within the operator's error
+    # of zero; the HIP model may have at most twice as many as the yardstick model, and never more than 5 %
+    share = adamw_step_compare(hip, ref, tokens, target, _lm_loss, 1e-3, min(0.05, 2.0 * flips_yard + 1e-3))
     print(f"gpt bf16 full depth: loss {lh.item():.4f}, worst gradient rel-L2 {worst_h:.2e} (yardstick {worst_n:.2e}), "
-          f"AdamW sign flips {share:.2e}", flush=True)
+          f"AdamW sign flips {share:.2e} (yardstick {flips_yard:.2e})", flush=True)
 
 
 def test_attention_layout_needs_no_copies():

@@ -300,6 +300,41 @@ def test_upstream_gradient_of_any_size(lib, go_scale):
     check_forward_backward(lib, 2, 513, 64, torch.bfloat16, DEV, mask=True, p=2, nk=2100, seed=63, go_scale=go_scale)
 
 
+@pytest.mark.parametrize("chunk", [0, 512])
+def test_values_with_a_common_component(lib, chunk):
+    """Tokens of a trained layer share a large common component (here: token-mean 0.7 of an rms of 1).  Then o_i is
+    close to every v_j, gh.v_j and c_i = gh.o_i are of one size, and dS = f'(s)(gh.v - c) is their small difference:
+    an error in c has one sign along a whole row of keys and adds up in sum_j dk_j, which is what the weight
+    gradient of the key projection sees.  The backward on a kept forward workspace reads what bf16 rounding took
+    from o there and keeps c in fp32: dq, dk, dv within the bar, and the sums over tokens (rel-L2 per slice of the
+    (bh, d) sums) within three times what rounding the exact gradients to bf16 does to those sums, where the backward
+    that only has the caller's bf16 o is several times further off."""
+    import math
+    from tests.parity import TOL, oracle_all, rel_err
+    print(f"case common component chunk={chunk}", flush=True)
+    bh, n, d = 4, 2048, 64
+    gen = torch.Generator().manual_seed(44)
+    q, k, v = ((0.7 * torch.randn(bh, n, d, generator=gen) + 0.7 * torch.randn(bh, 1, d, generator=gen)).bfloat16().to(DEV)
+               for _ in range(3))
+    go = torch.randn(bh, n, d, generator=gen).bfloat16().to(DEV)
+    tau = 8.0 * math.sqrt(d)
+    kw = dict(mask=True, inv_tau=1.0 / tau, p=2, chunk=chunk)
+    o, g, ws = lib.forward(q, k, v, save=True, **kw)
+    saved = lib.backward(q, k, v, o, g, go, saved=ws, **kw)
+    plain = lib.backward(q, k, v, o, g, go, **kw)
+    ref = oracle_all(q, k, v, go, mask=True, tau=tau, p=2)
+    tol = TOL[torch.bfloat16]
+    for name, x, r in zip(("dq", "dk", "dv"), saved, ref[2:]):
+        assert rel_err(x, r) < tol, f"{name} rel-L2 {rel_err(x, r):.3e}"
+    sums = {name: rel_err(x.double().sum(1), r.sum(1)) for name, x, r in zip(("dq", "dk", "dv"), saved, ref[2:])}
+    sums_plain = {name: rel_err(x.double().sum(1), r.sum(1)) for name, x, r in zip(("dq", "dk", "dv"), plain, ref[2:])}
+    floor = {name: rel_err(r.bfloat16().double().sum(1), r.sum(1)) for name, r in zip(("dq", "dk", "dv"), ref[2:])}
+    print(f"  token sums, kept workspace {sums}, caller's o only {sums_plain}, bf16-rounded exact gradients {floor}", flush=True)
+    for name in sums:
+        assert sums[name] < 4.0 * floor[name] + 1e-3, (name, sums, floor)
+    assert sums["dk"] < 0.5 * sums_plain["dk"], (sums, sums_plain)
+
+
 def test_bf16_range_is_loud_not_wrong(lib):
     """bf16 tensors are computed in _Float16.  Inside the documented range (|s| <= 250) the results meet
     the bf16 bar; beyond it a result is either still within the bar or not finite, never a finite wrong
