@@ -8,6 +8,7 @@
 #include "fm_decode.h"
 #include "fm_o1.h"
 #include "fm_pointwise.h"
+#include "fm_walk_sym.h"
 #if defined(FM_BENCH_AIDS)
 #include "fm_bench_aids.h"
 #endif
@@ -108,7 +109,8 @@ struct Plan {
   float sc;             // sqrt(1/tau), folded into q and k when they are converted
   // workspace offsets (bytes)
   size_t kt, vt, kr, vr, big, big2, small, run, runh, ores, fwd_bytes;
-  bool keep_resid;      // the forward leaves o - bf16(o) for the backward (see TokArgs::out_resid)   // run, runh: see k_o1_sums
+  bool keep_resid;      // the forward leaves o - bf16(o) for the backward (see TokArgs::out_resid)
+  bool sym;             // order-2 states are built by the walk per value column (k_walk_sym): one layout, no transposed copy   // run, runh: see k_o1_sums
   bool save;
   size_t b_kr, b_vr, b_qr, b_kt, b_vt, b_qt, b_qct, b_gh, b_ght, b_cv, b_bigq, b_smallq, b_bigk, b_smallk, b_bigv, b_gpart, b_bq, b_bk, b_runq, b_runqh, b_runk, b_runkh, bwd_bytes;
 };
@@ -199,6 +201,12 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
     p.qf = p.half && p.quad && !p.use_state && std::fabs(p.a2) >= 0.0625f && std::fabs(p.a2) <= 4.0f &&
            std::fabs(kc) <= 1024.0f && std::fabs(p.a1) <= 64.0f;
   }
+  {
+    // _Float16, D = 64, and enough batch*heads that one walk per (four values, batch*head) fills the chip; smaller
+    // problems sum their segments apart (k_build with seg_parallel)
+    const int nsteps = d->mask ? p.nseg - 1 : 1;
+    p.sym = p.half && d->d == 64 && p.quad && p.use_state && !(nsteps > 1 && d->bh * 16 < 256);
+  }
   const size_t slots = size_t(d->bh) * p.nslots;
   const size_t bigarr = d->d == 64 ? big_array_bytes<64>(p.esz, p.quad, slots) : big_array_bytes<32>(p.esz, p.quad, slots);
   // fp32 part of a slot: Z and the two vector sums; the order-1 path of fm_o1.h keeps the two vectors only
@@ -217,7 +225,7 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   p.small = take(size_t(d->bh) * p.nslots * smallsz);
   p.save = (d->flags & FASTMAX_FLAG_SAVE_FOR_BACKWARD) != 0;
   p.vr = take(p.save || p.half ? tk : 0);      // _Float16: the forward stages v rows (transposing LDS reads)
-  p.big2 = take(p.save && !p.o1 ? bigarr : 0);
+  p.big2 = take(p.save && !p.o1 && !p.sym ? bigarr : 0);
   // the order-1 path sums runs of segments: per batch*head and run one fp32 total and its compute-type slab
   p.o1_run = fm_o1_run_len(p.nseg, d->bh);
   const size_t nruns = p.o1 ? size_t(fm_o1_runs(p.nseg, p.o1_run)) : 0;
@@ -342,6 +350,18 @@ int launch_build(const BuildArgs<E>& args, int bh, fm_stream_t stream) {
   return fm_launch_status();
 }
 
+// The order-2 walk held per value column (k_walk_sym), where the plan says so.
+template <typename E, int DH> bool walk_sym_applies(const Plan& p, int, bool) { return sizeof(E) == 2 && DH == 64 && p.sym; }
+inline int launch_walk_sym(const WalkSymArgs& a, int bh, fm_stream_t stream) {
+  const int nsteps = a.mode == FM_WALK_TOTAL ? 1 : a.nseg - 1;
+  if (nsteps <= 0) return FASTMAX_OK;
+  ProfScope prof(FM_K_BUILD, stream);
+  const size_t lds = WalkSymCfg<64>::lds_bytes();
+  fm_allow_lds(reinterpret_cast<const void*>(&k_walk_sym<64>), lds);
+  FM_KERNEL_LAUNCH((k_walk_sym<64>), fm_dim3(16, bh), fm_dim3(WalkSymCfg<64>::THREADS), lds, stream, a);
+  return fm_launch_status();
+}
+
 // Dynamic LDS of a token kernel (kind 0: k_pv, 1: k_ds, 2: k_ds with dV, 3: k_ds with the fused
 // preparation, 4: k_ds with dV and states): va, vb | own rows | region, where the dense stages and the output staging lie over
 // the own rows and the region.
@@ -379,7 +399,7 @@ template <typename TIO, typename E> void tok_common(TokArgs<TIO, E>& a, const Fa
   a.quad = p.quad; a.a0 = p.a0; a.a1 = p.a1; a.a2 = p.a2; a.sc = p.sc; a.out_scale = 1.0f; a.zscale = 1.0f;
   a.own_o = TRef<const TIO>{nullptr, 0, 0, 0, 0, 0}; a.own_do = a.own_o;
   a.w_gh = nullptr; a.w_qr = nullptr; a.w_cv = nullptr; a.gpart = nullptr; a.gnblk = 0;
-  a.out_resid = nullptr; a.own_ores = nullptr;
+  a.out_resid = nullptr; a.own_ores = nullptr; a.state_tr = 0; a.state_xscale = 1.0f;
 }
 
 template <typename TIO, typename E, int DH, int QT, int OWN, int QF = 0>
@@ -488,7 +508,19 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
     b.big2 = p.save ? reinterpret_cast<E*>(ws + p.big2) : nullptr;
     b.vb_from_r = 0; b.coef2b = 2.0f * p.a2; b.coef1b = p.a1;
     b.coef2 = p.a2; b.coef1 = p.a1; b.coefz = p.a2; b.coefva = p.a1; b.coefvb = p.a0;
-    st = launch_build<E, DH>(b, d->bh, stream);
+    bool walked = false;
+    if constexpr (sizeof(E) == 2) {
+      if (walk_sym_applies<E, DH>(p, d->bh, d->mask != 0)) {
+        // values = v, keys = k': one layout serves the forward, and the backward's dQ reads the same slabs transposed
+        WalkSymArgs w;
+        w.kt = kt; w.xt = vt; w.cw = nullptr; w.npad = p.npad_k; w.nseg = p.nseg; w.L = p.L; w.mode = b.mode; w.nslots = p.nslots;
+        w.o2 = big; w.o1_vk = big; w.o1_kv = nullptr; w.small = small;
+        w.coef2 = p.a2; w.coef1 = p.a1; w.coefz = p.a2; w.coefva = p.a1; w.coefvb = p.a0;
+        st = launch_walk_sym(w, d->bh, stream);
+        walked = true;
+      }
+    }
+    if (!walked) st = launch_build<E, DH>(b, d->bh, stream);
     if (st) return st;
   }
   TokArgs<TIO, E> a;

@@ -1319,15 +1319,30 @@ struct TokCfg {
 // slab: two buffers of SA*DH*PS elements.  All 256 threads must call this.
 // The A fragments of step i+1 are fetched from LDS before the products of step i are
 // issued, so a single wavefront per SIMD keeps the matrix pipe fed.
-template <typename E, int DH, int QT, int NACC>
+// TRA: the slabs lie transposed in memory, T[a][b][c] (rows b, columns c): the A fragments are read out of the
+// staged slab with transposing LDS reads, and yb must then hold y in the k order those reads deliver (16 s +
+// 4 lh + {0..3}, 16 s + 8 + 4 lh + {0..3}: Mma::load_nat_perm).  This is how dQ reads the forward's own
+// (k, v, k) state, whose slab a is [v][k]: U[a][v][k] = sum k_a v k is symmetric in its two key indices, so it is
+// the transposed slab of the (k, k, v) state dQ contracts.  xscale: factor on x (the order-2 part only).
+template <typename E, int DH, int QT, int NACC, bool TRA = false>
 FM_DEVICE void fm_readout(const E* FM_RESTRICT state, bool quad, const E* xs, const int* xrow,
                           const typename Mma<E>::frag (*yb)[TokCfg<E, DH, QT>::NKS],
-                          E* slab, fm_f32x16 (*acc)[NACC], int tid) {
+                          E* slab, fm_f32x16 (*acc)[NACC], int tid, float xscale = 1.0f) {
   typedef TokCfg<E, DH, QT> C;
   typedef Mma<E> M;
   typedef typename M::frag frag;
   const int lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   const int a_begin = quad ? 0 : DH;
+  const E xs_f = CE<E>::from(xscale);
+  // TRA: the lane's row (4 lh + s4 inside a k-step) and its columns inside the swizzled rows, per row tile; which half
+  // of a row the columns lie in depends on bit 1 of the row, i.e. of s4 alone
+  int tr_base[C::NT];
+  {
+    const int s4 = (lane & 15) >> 2, q = lane & 3, half16 = (lane >> 4) & 1;
+#pragma unroll
+    for (int ct = 0; ct < C::NT; ++ct)
+      tr_base[ct] = (4 * lh + s4) * DH + ((32 * ct + 16 * half16 + 4 * q) ^ (((s4 >> 1) & 1) * (DH / 2)));
+  }
   TileRegs<E, C::SA * DH, DH> regs;
   // `state` points at the first slab to read (T[0] with order-2 states, else the order-1 slab)
   regs.load(state, DH, tid);                                  // rows [a][c] are contiguous
@@ -1335,18 +1350,43 @@ FM_DEVICE void fm_readout(const E* FM_RESTRICT state, bool quad, const E* xs, co
   const int lane_off = lr * C::PS + lh * M::KPL;
   for (int as = a_begin; as <= DH; as += C::SA) {
     E* sb = slab + buf * C::SLAB;
-    regs.store(sb, C::PS, tid);
+    if constexpr (TRA) {
+      // Rows without padding, the 16-byte chunks of rows 2, 3 (mod 4) exchanged between the two halves of the row: the
+      // four rows a transposing read touches per half-wavefront then lie in four different quarters of the banks
+      // (with the padded pitch rows r and r + 2 share banks and every such read takes twice as long).
+      typedef TileRegs<E, C::SA * DH, DH> TR_;
+#pragma unroll
+      for (int i = 0; i < TR_::N; ++i) {
+        const int c = tid + FM_THREADS * i;
+        if (TR_::TOTAL % FM_THREADS == 0 || c < TR_::TOTAL) {
+          const int row = c / TR_::CPR, ch = c % TR_::CPR;
+          *reinterpret_cast<fm_u32x4*>(sb + row * DH + ((ch ^ (((row >> 1) & 1) * (TR_::CPR / 2))) * TR_::VEC)) = regs.r[i];
+        }
+      }
+    } else {
+      regs.store(sb, C::PS, tid);
+    }
     FM_SYNC();
     if (as + C::SA <= DH) regs.load(state + int64_t(as + C::SA - a_begin) * DH * DH, DH, tid);
     const int na = (as + C::SA <= DH) ? C::SA : (DH + 1 - as);
     const E* sl = sb + lane_off;
+    // fragment (value al of the slab, row tile ct, k-step ks)
+    auto afrag = [&](int al, int ct, int ks) FM_ALWAYS_INLINE {
+      if constexpr (TRA) {
+        // Mma::load_tr on the swizzled rows; the lane's part of the address was formed once (tr_base)
+        const E* p = sb + tr_base[ct] + (al * DH + ks * M::KSTEP) * DH;
+        const fm_half4 lo = fm_lds_tr4(p), hi = fm_lds_tr4(p + 8 * DH);
+        frag r = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        return r;
+      } else return M::load(sl + (al * DH + 32 * ct) * C::PS + ks * M::KSTEP);
+    };
     frag fa[C::NT];
 #pragma unroll
-    for (int ct = 0; ct < C::NT; ++ct) fa[ct] = M::load(sl + (32 * ct) * C::PS);
+    for (int ct = 0; ct < C::NT; ++ct) fa[ct] = afrag(0, ct, 0);
     // the own tokens' x_a: the value for the next a is read from LDS while this one's products run
     E xv[QT];
 #pragma unroll
-    for (int j = 0; j < QT; ++j) xv[j] = (as < DH) ? xs[xrow[j] * C::PQ + as] : E(1.0f);
+    for (int j = 0; j < QT; ++j) xv[j] = (as < DH) ? xs[xrow[j] * C::PQ + as] * xs_f : E(1.0f);
     for (int al = 0; al < na; ++al) {
       const int a = as + al;
       frag xr[QT];
@@ -1354,7 +1394,7 @@ FM_DEVICE void fm_readout(const E* FM_RESTRICT state, bool quad, const E* xs, co
       for (int j = 0; j < QT; ++j) xr[j] = M::splat(xv[j]);
       const int an = (al + 1 < na) ? a + 1 : a;        // re-reads a valid element at the end of a slab
 #pragma unroll
-      for (int j = 0; j < QT; ++j) xv[j] = (an < DH) ? xs[xrow[j] * C::PQ + an] : E(1.0f);
+      for (int j = 0; j < QT; ++j) xv[j] = (an < DH) ? xs[xrow[j] * C::PQ + an] * xs_f : E(1.0f);
 #pragma unroll
       for (int ks = 0; ks < C::NKS; ++ks) {
         // prefetch the fragments of the next (a, k-step); the last one of a slab re-reads a valid row
@@ -1362,7 +1402,7 @@ FM_DEVICE void fm_readout(const E* FM_RESTRICT state, bool quad, const E* xs, co
         const int nal = (ks + 1 < C::NKS) ? al : (al + 1 < na ? al + 1 : al);
         frag fn[C::NT];
 #pragma unroll
-        for (int ct = 0; ct < C::NT; ++ct) fn[ct] = M::load(sl + (nal * DH + 32 * ct) * C::PS + nks * M::KSTEP);
+        for (int ct = 0; ct < C::NT; ++ct) fn[ct] = afrag(nal, ct, nks);
 #pragma unroll
         for (int j = 0; j < QT; ++j) {
           const frag fb = yb[j][ks] * xr[j];

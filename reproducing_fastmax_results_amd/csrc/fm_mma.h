@@ -41,6 +41,14 @@ template <> struct Mma<fm_half> {
     for (int i = 0; i < 8; ++i) r[i] = fm_half(c[8 * s + i]);
     return r;
   }
+  // The B fragment of k-step s of a row stored in natural order, in the k order a transposing read delivers its A
+  // fragment (load_tr): elements 16 s + 4 lh + {0..3} and 16 s + 8 + 4 lh + {0..3}.
+  static FM_DEVICE frag load_nat_perm(const fm_half* row, int s, int lh) {
+    const fm_half4 lo = *reinterpret_cast<const fm_half4*>(row + 16 * s + 4 * lh);
+    const fm_half4 hi = *reinterpret_cast<const fm_half4*>(row + 16 * s + 8 + 4 * lh);
+    frag r = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return r;
+  }
   // The fragment load_perm would read from a transposed tile, taken from the ROW-MAJOR tile
   // instead (tokens x features, `pitch` elements per token) with two transposing reads: lane
   // (lr, lh) gets feature col0 + lr of the tokens tok0 + 4 lh + {0..3} and tok0 + 8 + 4 lh + {0..3},
@@ -71,6 +79,7 @@ template <> struct Mma<float> {
   static constexpr bool HAS_TR = false;
   static FM_DEVICE frag load_tr(const float*, int, int, int, int) { return 0.f; }   // never called
   static FM_DEVICE frag from_acc(const fm_f32x16& c, int s) { return c[s]; }
+  static FM_DEVICE frag load_nat_perm(const float*, int, int) { return 0.f; }   // never called
 };
 
 // Row index (0..31) of accumulator register e for a lane in half lh.

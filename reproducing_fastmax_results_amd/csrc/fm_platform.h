@@ -35,6 +35,7 @@ typedef uint16_t fm_bf16;  // raw storage of a bfloat16
 #define FM_SCHED_FENCE()
 #define FM_SCHED_MFMA_DS(n)
 #define FM_KEEP_BRANCH()
+#define FM_WAIT_GLOBAL_LOADS()
 typedef void* fm_stream_t;
 typedef hostsim::Dim3 fm_dim3;
 #define FM_TID_X (int(hostsim::g_t.tid.x))
@@ -114,6 +115,10 @@ static __device__ __forceinline__ int fm_opaque_zero() { int z = 0; asm volatile
 // Inside a rarely taken wavefront-uniform branch: keeps it a branch (the optimiser would
 // otherwise run its body on every pass and select the result).
 #define FM_KEEP_BRANCH() asm volatile("")
+// Waits for every global load of the wavefront that is still in flight (s_waitcnt vmcnt(0), the other counters left
+// alone).  Ahead of a software-pipelined loop it tells the compiler that nothing is pending on entry, so the loop
+// head does not inherit a full wait from the prologue's loads on every iteration.
+#define FM_WAIT_GLOBAL_LOADS() __builtin_amdgcn_s_waitcnt(0x0F70)
 typedef hipStream_t fm_stream_t;
 typedef dim3 fm_dim3;
 #define FM_TID_X (int(threadIdx.x))

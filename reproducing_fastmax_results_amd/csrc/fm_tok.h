@@ -65,6 +65,9 @@ template <typename TIO, typename E> struct TokArgs {
   // back (own_ores) before it forms c = gh . o: c is subtracted from numbers of its own size, gh . v, so the 8 bits
   // of a bf16 o would leave dS with a few bits, and with an error of one sign along a whole row of keys.
   fm_half* out_resid; const fm_half* own_ores;
+  // k_ds, own = queries, _Float16: the prefix state is the forward's own layout (slab a = [v][k], see fm_readout's
+  // TRA) and its order-2 part is to be counted state_xscale times
+  int state_tr; float state_xscale;
 };
 
 // eight values as they will read back from the caller's tensor: themselves (fp32) or rounded to bf16
@@ -767,7 +770,22 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS
         FM_SYNC();                                     // the slabs and dks are overwritten by the dense stages
       }
     } else {
-      fm_readout<E, DH, QT, NT>(state, A.quad != 0, Own, xrow, of2, R, acc, tid);
+      bool done = false;
+      if constexpr (OWN == FM_OWN_Q && M::HAS_TR) {
+        if (A.state_tr) {
+          // gh of the own queries in the k order of the transposing reads
+          frag ofp[QT][NKS];
+#pragma unroll
+          for (int j = 0; j < QT; ++j) {
+            const E* o2 = PREP ? R + xrow[j] * PQ : A.own2_r + (int64_t(bh) * A.npad_own + t0 + xrow[j]) * DH;
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) ofp[j][ks] = M::load_nat_perm(o2, ks, lh);
+          }
+          fm_readout<E, DH, QT, NT, true>(state, A.quad != 0, Own, xrow, ofp, R, acc, tid, A.state_xscale);
+          done = true;
+        }
+      }
+      if (!done) fm_readout<E, DH, QT, NT>(state, A.quad != 0, Own, xrow, of2, R, acc, tid);
     }
   } else {
     FM_SYNC();                                         // own rows are overwritten by the dense stages

@@ -137,6 +137,15 @@ def test_normalize_backward(sim):
     assert O.rel_l2(sim.normalize_backward(x, dy, centre=2, max_norm=True, scale=1.5), xd.grad) < 1e-5
 
 
+def test_order2_walk_per_value_column(sim):
+    """k_walk_sym (D = 64, _Float16): prefix walk for the forward, suffix walk with the weights c for the backward,
+    dQ reading the forward's state transposed; with and without the forward's kept workspace, and the one global
+    state of unmasked attention."""
+    check_forward_backward(sim, 1, 300, 64, torch.bfloat16, "cpu", mask=True, p=2, chunk=256, seed=21)
+    check_forward_backward(sim, 1, 512, 64, torch.bfloat16, "cpu", mask=True, p=2, chunk=256, seed=22, saved=True)
+    check_forward_backward(sim, 1, 130, 64, torch.bfloat16, "cpu", mask=False, p=2, nk=300, seed=23, flags=_capi.FLAG_FORCE_MOMENTS)
+
+
 def test_causal_with_more_keys_than_queries(sim):
     # query i sees keys 0 .. nk - nq + i (fastmax_cuda_forward.cu:161-172): head + square tail, merged
     check_forward_backward(sim, 1, 40, 32, torch.float32, "cpu", mask=True, p=2, nk=75, seed=13)
