@@ -160,17 +160,20 @@ int fastmax_backward_saved(const FastmaxDesc* desc, const void* q, const void* k
 /* Incremental decoding on a persistent moment state (the running sums of fastmax_cuda_forward.cu:160-276
  * kept between calls; the reference's generation loop, transformer/eval.py:8-32, re-runs the whole context
  * for every new token).  The state of a batch*head is the fp32 sums over all keys so far of [1, k', k' x k']
- * times [v, 1] with k' = k * inv_tau: fastmax_decode_state_bytes(desc) bytes for desc->bh of them (1.10 MB
- * per batch*head at d = 64, order 2; 33 KB at order 1), whatever the number of keys.  A zero-filled buffer
+ * times [v, 1] with k' = k * inv_tau, the symmetric order-2 part kept once per pair of features:
+ * fastmax_decode_state_bytes(desc) bytes for desc->bh of them (0.70 MB per batch*head at d = 64, order 2;
+ * 41 KB at order 1), whatever the number of keys.  The layout is the library's own (a state is only ever
+ * passed back to these two calls).  A zero-filled buffer
  * is the empty state.  desc: bh, d, dtype, p, a0..a2, inv_tau and the strides named below are used; mask,
  * chunk, flags and norm are ignored (decoding is causal by construction and needs unnormalised q, k: the
  * max-norm depends on every token).
  *   fastmax_decode_absorb: adds desc->nk tokens (k, v: strides sk, sv) to the state, e.g. a prompt whose
  *     own outputs come from fastmax_forward.
  *   fastmax_decode_step: adds one token (k, v) and reads the state out for its query q (strides sq; the
- *     query sees its own key, as in causal attention): o (strides so, one token) and g (sg).  scratch:
- *     fastmax_decode_scratch_bytes(desc) bytes of device memory.  desc->nq and nk are ignored (one token).
- * Both enqueue on the stream and allocate nothing; a step reads and writes the state once. */
+ *     query sees its own key, as in causal attention): o (strides so, one token) and g (sg).  scratch is
+ *     not used any more (a step is one launch; the argument and fastmax_decode_scratch_bytes stay for
+ *     callers built against the earlier signature; null is accepted).  desc->nq and nk are ignored (one token).
+ * Both enqueue on the stream and allocate nothing; a step is one launch that reads and writes the state once. */
 size_t fastmax_decode_state_bytes(const FastmaxDesc* desc);
 size_t fastmax_decode_scratch_bytes(const FastmaxDesc* desc);
 int fastmax_decode_absorb(const FastmaxDesc* desc, const void* k, const void* v, float* state, void* hip_stream);
