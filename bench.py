@@ -186,6 +186,8 @@ def main() -> int:
                          "the minimal ViT (fp32, 256 images of 28x28) or decoder-only LM (bf16, 16 x 1024 tokens)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the short runs of the other configurations")
+    ap.add_argument("--decode-only", action="store_true",
+                    help="only the incremental-decoding line (for profiling its kernel)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device copy, the yardstick for the HBM traffic counters")
     ap.add_argument("--workload", choices=["headline", "long"], default="headline",
@@ -210,6 +212,9 @@ def main() -> int:
     dev = torch.device("cuda:0")
     if args.model_step:
         print(json.dumps(model_step(args, dev)))
+        return 0
+    if args.decode_only:
+        print(json.dumps(decode_line(lib, dev)))
         return 0
     W = dict(WORKLOAD if args.workload == "headline" else LONG_WORKLOAD, p=args.order)
     out = operator_line(lib, dev, W, args.dtype, args, args.steps, args.warmup, full=True)
