@@ -44,10 +44,10 @@ PEAK_HBM_GBS = 8000.0
 # (N, order, dtype, --chunk, kernel).  A constant, not a live measurement: it belongs to the kernels as they
 # were when the named summary was made.
 TRAFFIC = {
-    (4096, 2, "bf16", 0, "dkv"): {"bytes": (44639 * 2 + 32770) * 1024, "source": "profiles/c2_bf16_hbm_traffic.md"},
-    (65536, 1, "bf16", 0, "dkv"): {"bytes": (402970 * 2 + 393240) * 1024, "source": "profiles/long_order1_bf16_hbm_traffic.md"},
-    (65536, 2, "bf16", 0, "build"): {"bytes": (160828 * 2 + 982268) * 1024, "source": "profiles/long_order2_bf16_hbm_traffic.md"},
-    (65536, 2, "bf16", 0, "dkv"): {"bytes": (564148 * 2 + 262171) * 1024, "source": "profiles/long_order2_bf16_hbm_traffic.md"},
+    (4096, 2, "bf16", 0, "dkv"): {"bytes": int((42456.4 * 2 + 32768.4) * 1024), "source": "profiles/c2_bf16_hbm_traffic.md"},
+    (65536, 1, "bf16", 0, "dkv"): {"bytes": int((402949.3 * 2 + 393223.9) * 1024), "source": "profiles/long_order1_bf16_hbm_traffic.md"},
+    (65536, 2, "bf16", 0, "build"): {"bytes": int((130104.8 * 2 + 544651.2) * 1024), "source": "profiles/long_order2_bf16_hbm_traffic.md"},
+    (65536, 2, "bf16", 0, "dkv"): {"bytes": int((546856.1 * 2 + 262149.1) * 1024), "source": "profiles/long_order2_bf16_hbm_traffic.md"},
 }
 
 WORKLOAD = dict(name="configs[1]: causal order-2 fwd+bwd", B=4, H=8, N=4096, D=64, p=2, mask=True, scale=1.0)

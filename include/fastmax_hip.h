@@ -49,8 +49,10 @@ enum {
  * multiplies but no packed bf16 arithmetic).  _Float16 has 11 significand bits (bf16: 8) but a
  * narrow exponent: values beyond 65504 become infinities and values below 6e-5 lose precision.
  * Supported: |s_ij| = |q_i . k_j| * inv_tau <= 250 for every pair (so that a2 * s^2 <= 65504 / 2 for
- * a2 = 1/2; in general |a1 s| + |a2| s^2 < 6e4), |q|, |k| * sqrt(inv_tau) <= 6e4, and v, dO of
- * ordinary magnitude (about 1e-3 .. 1e4).  The reference model's normalised q and k (|q_i|, |k_j| <=
+ * a2 = 1/2; in general |a1 s| + |a2| s^2 < 6e4), |q|, |k| * sqrt(inv_tau) <= 6e4, and values v whose
+ * entries lie between about 1e-4 and 1e2 in magnitude (the backward forms (dO / g) . v with dO / g brought to
+ * [32, 64), and the moment states sum k k v over a segment, both rounded to _Float16; at 1e3 the gradients of q
+ * and k, at 1e4 also the outputs of segmented sequences turn non-finite).  The reference model's normalised q and k (|q_i|, |k_j| <=
  * lim, transformer/model.py:97-102) satisfy this by construction.  Nothing saturates: an input
  * beyond the range turns into infinities that reach the outputs as inf / NaN rather than as finite
  * wrong numbers.  FASTMAX_FLAG_F32_COMPUTE lifts the limits at fp32 speed.  The size of dO is free (the

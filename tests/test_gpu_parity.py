@@ -335,6 +335,45 @@ def test_values_with_a_common_component(lib, chunk):
     assert sums["dk"] < 0.5 * sums_plain["dk"], (sums, sums_plain)
 
 
+@pytest.mark.parametrize("n,p,chunk", [(700, 2, 0), (2048, 2, 512), (2048, 1, 0)])
+def test_bf16_value_range(lib, n, p, chunk):
+    """The range of v that include/fastmax_hip.h states for bf16 tensors: entries of 1e-4 .. 1e2 in magnitude meet
+    the bar on every tensor (one segment, order-2 states, the order-1 path of long sequences); beyond it (1e3, 1e4) a
+    result is within the bar or not finite, never finite and wrong; FASTMAX_FLAG_F32_COMPUTE meets the bar there."""
+    import math
+    from reproducing_fastmax_results_amd._capi import FLAG_F32_COMPUTE
+    from tests.parity import TOL, oracle_all, rel_err
+    bh, d, tol = 2, 64, TOL[torch.bfloat16]
+    tau = 8.0 * math.sqrt(d)
+
+    def run(vs, flags=0):
+        gen = torch.Generator().manual_seed(3)
+        q, k = (torch.randn(bh, n, d, generator=gen).bfloat16() for _ in range(2))
+        v = (vs * torch.randn(bh, n, d, generator=gen)).bfloat16()
+        go = torch.randn(bh, n, d, generator=gen).bfloat16()
+        kw = dict(mask=True, inv_tau=1.0 / tau, p=p, chunk=chunk, flags=flags)
+        qd, kd, vd, gd = (t.to(DEV) for t in (q, k, v, go))
+        if flags:
+            o, g = lib.forward(qd, kd, vd, **kw)
+            grads = lib.backward(qd, kd, vd, o, g, gd, **kw)
+        else:
+            o, g, ws = lib.forward(qd, kd, vd, save=True, **kw)
+            grads = lib.backward(qd, kd, vd, o, g, gd, saved=ws, **kw)
+        ref = oracle_all(q, k, v, go, mask=True, tau=tau, p=p)
+        return list(zip(("o", "g", "dq", "dk", "dv"), (o, g) + tuple(grads), ref))
+
+    for vs in (1e-4, 1e-2, 1e2):
+        print(f"case bf16 value range n={n} p={p} chunk={chunk} v x {vs:g}", flush=True)
+        for name, x, r in run(vs):
+            assert bool(torch.isfinite(x).all()) and rel_err(x, r) < tol, f"{name} at v x {vs:g}: {rel_err(x, r):.3e}"
+    for vs in (1e3, 1e4):
+        print(f"case bf16 value range n={n} p={p} chunk={chunk} v x {vs:g} (beyond)", flush=True)
+        for name, x, r in run(vs):
+            assert (not bool(torch.isfinite(x).all())) or rel_err(x, r) < tol, f"{name} finite but wrong at v x {vs:g}"
+        for name, x, r in run(vs, FLAG_F32_COMPUTE):
+            assert bool(torch.isfinite(x).all()) and rel_err(x, r) < tol, f"{name} in fp32 at v x {vs:g}"
+
+
 def test_bf16_range_is_loud_not_wrong(lib):
     """bf16 tensors are computed in _Float16.  Inside the documented range (|s| <= 250) the results meet
     the bf16 bar; beyond it a result is either still within the bar or not finite, never a finite wrong
