@@ -70,6 +70,43 @@ def alg_flops_unit(bh: int, n: int, d: int, p: int) -> float:
     return 2.0 * m * (d + 1) * bh * n
 
 
+def sclk_under(run, sync, seconds: float = 0.4):
+    """Shader clock while `run` is called in a loop for `seconds`: the driver's pp_dpm_sclk file sampled every 10 ms
+    from a second thread, median of the samples of the second half (MHz), or None where the file cannot be read."""
+    import glob
+    import threading
+    files = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
+    if not files:
+        return None
+    samples, stop = [], threading.Event()
+
+    def sampler():
+        while not stop.is_set():
+            try:
+                with open(files[0]) as fh:
+                    for line in fh:
+                        if "*" in line:
+                            samples.append(float(line.split(":")[1].lower().split("mhz")[0]))
+            except (OSError, ValueError, IndexError):
+                return
+            time.sleep(0.01)
+
+    th = threading.Thread(target=sampler, daemon=True)
+    th.start()
+    t_end = time.perf_counter() + seconds
+    while time.perf_counter() < t_end:
+        for _ in range(8):
+            run()
+        sync()
+    stop.set()
+    th.join()
+    half = sorted(samples[len(samples) // 2:])
+    return half[len(half) // 2] if len(half) >= 3 else None
+
+
+NOMINAL_SCLK_MHZ = 2400.0     # the engine clock the published matrix peaks are quoted at
+
+
 def cpu_model_name() -> str:
     try:
         with open("/proc/cpuinfo") as fh:
@@ -509,6 +546,7 @@ def operator_line(lib, dev, W, dtype, args, steps, warmup, full):
     ms_per_step = 1e3 * elapsed / steps
     tokens = B * N
     value = tokens * steps / elapsed
+    sclk = sclk_under(run, torch.cuda.synchronize)
 
     # forward alone (the inference call: no workspace kept for a backward)
     for _ in range(3):
@@ -577,6 +615,15 @@ def operator_line(lib, dev, W, dtype, args, steps, warmup, full):
         roofline["executed_mfma"] = {"flop_per_step": executed,
                                      "achieved": executed / (ms_per_step * 1e-3) / 1e12,
                                      "frac": executed / (ms_per_step * 1e-3) / 1e12 / peak}
+    if sclk:
+        # the published peak is quoted at the nominal engine clock; under these kernels the device holds a lower one
+        # (power management), and the matrix rate it can deliver scales with it
+        roofline["clock"] = {"sclk_MHz_under_this_step": sclk, "nominal_MHz": NOMINAL_SCLK_MHZ,
+                             "what": "median of the driver's current shader clock, sampled every 10 ms while the step "
+                                     "runs in a loop for 0.4 s"}
+        if roofline["bound"] == "mfma":
+            roofline["clock"]["peak_at_that_clock"] = peak * sclk / NOMINAL_SCLK_MHZ
+            roofline["clock"]["frac_at_that_clock"] = roofline["frac"] * NOMINAL_SCLK_MHZ / sclk
     tkey = (W["N"], p, dtype, args.chunk, dominant)
     if tkey in TRAFFIC:
         roofline["traffic"] = TRAFFIC[tkey]["bytes"]
