@@ -351,9 +351,24 @@ def decode_line(lib, dev, bh=16, d=64, prompt=4096, steps=200):
     q, k, v = ((torch.randn(bh, prompt + steps, d, generator=gen)).to(torch.bfloat16).to(dev) for _ in range(3))
     kw = dict(inv_tau=1.0 / (8.0 * math.sqrt(d)), p=2)
     state = lib.decode_state(k, **kw)
-    lib.decode_absorb(k[:, :prompt], v[:, :prompt], state, **kw)
-    # the C entry point itself, on buffers made once (the Python front allocates o, g and the scratch per call)
+    # the prompt's keys and values summed into the state (one launch; bf16 at D = 64: matrix instructions), timed as
+    # five calls in a row between two events, then once more into the cleared state the steps below continue from
     import ctypes as C
+    kp, vp = k[:, :prompt], v[:, :prompt]
+    pdesc = lib.make_desc(kp, kp, vp, mask=True, a0=1.0, a1=1.0, a2=0.5, **kw)
+    s0 = torch.cuda.current_stream().cuda_stream
+    ea, eb = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    lib.check(lib.lib.fastmax_decode_absorb(C.byref(pdesc), kp.data_ptr(), vp.data_ptr(), state.data_ptr(), s0), "fastmax_decode_absorb")
+    torch.cuda.synchronize()
+    ea.record()
+    for _ in range(5):
+        lib.lib.fastmax_decode_absorb(C.byref(pdesc), kp.data_ptr(), vp.data_ptr(), state.data_ptr(), s0)
+    eb.record()
+    eb.synchronize()
+    absorb_ms = ea.elapsed_time(eb) / 5
+    state.zero_()
+    lib.decode_absorb(kp, vp, state, **kw)
+    # the C entry point itself, on buffers made once (the Python front allocates o, g and the scratch per call)
     from reproducing_fastmax_results_amd._capi import _strides, _gstrides
     q1, k1, v1 = q[:, :1], k[:, :1], v[:, :1]
     desc = lib.make_desc(q1, k1, v1, mask=True, a0=1.0, a1=1.0, a2=0.5, **kw)
@@ -407,6 +422,7 @@ def decode_line(lib, dev, bh=16, d=64, prompt=4096, steps=200):
     state_bytes = state.numel() * 4
     return {"workload": f"one token per call on the moment state, B*H={bh}, D={d}, after a {prompt}-token prompt",
             "us_per_token": us, "tokens_per_s": 1e6 / us, "us_per_token_eager_python_calls": us_eager, "state_bytes": state_bytes,
+            "prompt_absorb_ms": absorb_ms, "prompt_tokens_per_s": bh * prompt / (absorb_ms * 1e-3),
             "roofline": {"bound": "hbm", "achieved": 2 * state_bytes / (us * 1e-6) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": 2 * state_bytes / (us * 1e-6) / 1e9 / PEAK_HBM_GBS,
                          "what": "state read and written once per step, one launch per token; timed as replays of a HIP "

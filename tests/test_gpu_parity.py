@@ -273,6 +273,7 @@ def test_incremental_decoding_on_the_moment_state(lib, dtype, p, d):
     check_decode(lib, 6, 700, 640, d, dtype, DEV, p=p, seed=90)
     check_decode(lib, 4, 48, 0, d, dtype, DEV, p=p, seed=91, tau_mult=1.0)
     check_decode(lib, 4, 300, 290, d, dtype, DEV, p=p, seed=92, four_d=True)
+
     # one step against the library's own route over cached keys (causal, one query, all keys)
     import math
     from tests.parity import make_inputs, rel_err, TOL
@@ -283,6 +284,34 @@ def test_incremental_decoding_on_the_moment_state(lib, dtype, p, d):
     o, g = lib.decode_step(q[:, 512:], k[:, 512:], v[:, 512:], state, **kw)
     o2, g2 = lib.forward(q[:, 512:].contiguous(), k, v, mask=True, **kw)
     assert rel_err(o, o2) < TOL[dtype] and rel_err(g, g2) < TOL[dtype]
+
+
+def test_prompt_absorbed_with_matrix_instructions(lib):
+    """bf16 tensors, D = 64, order 2: prompts of 64 tokens and more are summed by k_decode_absorb_mma.  Decoding after
+    a long prompt against the causal closed form; the state against the one k_decode builds from the same tokens in
+    pieces below the threshold (operands rounded to _Float16: 5e-3 per entry, 1e-4 over the state); absorbing in two
+    calls (into a state that is not empty, strided (b, h, n, d) views) against one call."""
+    import math
+    from tests.parity import check_decode, make_inputs
+    print("case absorb mma: decode after a 4000-token prompt", flush=True)
+    check_decode(lib, 2, 4008, 4000, 64, torch.bfloat16, DEV, p=2, seed=95)
+    check_decode(lib, 4, 203, 199, 64, torch.bfloat16, DEV, p=2, seed=96, four_d=True)
+    bh, n, d = 16, 2500, 64
+    q, k, v, _ = make_inputs(bh, n, n, d, torch.bfloat16, DEV, 7)
+    kw = dict(inv_tau=1.0 / (8.0 * math.sqrt(d)), p=2, a0=1.0, a1=1.0, a2=0.5)
+    one, two, small = (lib.decode_state(k, **kw) for _ in range(3))
+    print("case absorb mma: one call, two calls, pieces of 48", flush=True)
+    lib.decode_absorb(k, v, one, **kw)
+    lib.decode_absorb(k[:, :1000], v[:, :1000], two, **kw)
+    lib.decode_absorb(k[:, 1000:], v[:, 1000:], two, **kw)
+    for t0 in range(0, n, 48):
+        lib.decode_absorb(k[:, t0:t0 + 48], v[:, t0:t0 + 48], small, **kw)
+    torch.cuda.synchronize()
+    assert float((one - two).norm() / one.norm()) < 1e-6
+    assert float((one - small).norm() / small.norm()) < 1e-4
+    live = small.abs() > 1e-3 * small.abs().max()
+    assert float(((one - small).abs() / small.abs().clamp_min(1e-30))[live].max()) < 5e-3
+
 
 
 @pytest.mark.parametrize("go_scale", [1e-7, 1e-4, 3e4])

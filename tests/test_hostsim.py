@@ -246,6 +246,23 @@ def test_incremental_decoding_on_the_moment_state(sim):
     check_decode(sim, 2, 30, 20, 32, torch.float32, "cpu", p=1, seed=32, four_d=True)
 
 
+def test_prompt_absorbed_with_matrix_instructions(sim):
+    # bf16, D = 64, order 2, 64 tokens or more: k_decode_absorb_mma (two tiles here, the second ragged), then steps
+    check_decode(sim, 1, 134, 130, 64, torch.bfloat16, "cpu", p=2, seed=33)
+    # the same sums as token by token (k_decode), also added to a state that is not empty
+    import math
+    q, k, v, _ = make_inputs(1, 100, 100, 64, torch.bfloat16, "cpu", 5)
+    kw = dict(inv_tau=1.0 / (8 * math.sqrt(64)), p=2, a0=1.0, a1=1.0, a2=0.5)
+    s1, s2 = sim.decode_state(k, **kw), sim.decode_state(k, **kw)
+    sim.decode_absorb(k[:, :30], v[:, :30], s1, **kw)          # k_decode
+    sim.decode_absorb(k[:, 30:], v[:, 30:], s1, **kw)          # 70 tokens: matrix instructions, into a state that is not empty
+    sim.decode_absorb(k[:, :50], v[:, :50], s2, **kw)
+    sim.decode_absorb(k[:, 50:], v[:, 50:], s2, **kw)
+    assert float((s1 - s2).norm() / s2.norm()) < 1e-5
+    live = s2.abs() > 1e-3 * s2.abs().max()
+    assert float(((s1 - s2).abs() / s2.abs().clamp_min(1e-30))[live].max()) < 5e-3      # operands rounded to _Float16
+
+
 def test_order1_segment_backward_in_one_pass(sim):
     # beyond 1024 tokens order 1 on _Float16 runs in 128-token segments and k_o1_bwd makes dq, dk, dv of a segment
     # in one workgroup (9 segments here, the last one ragged); also with the folded normalisation's Jacobian
