@@ -29,7 +29,7 @@
 #include "fm_kernels.h"
 
 static constexpr int FM_DEC_ROWS = 64;      // the moment rows of a state are padded to a multiple of this
-static constexpr int FM_DEC_THREADS = 512;  // eight wavefronts per workgroup: five rows per thread at D = 64, order 2 (256: 9.3 us per token, 1024: 7.9)
+static constexpr int FM_DEC_THREADS = 512;  // eight wavefronts per workgroup: five rows per thread at D = 64, order 2 (per token: 256 threads 9.3 us, 384 7.7, 512 and 768 7.4, 1024 7.7)
 constexpr int64_t fm_decode_rows(int d, bool quad) { return 1 + int64_t(d) + (quad ? int64_t(d) * (d + 1) / 2 : 0); }
 constexpr int fm_decode_blocks(int d, bool quad) { return int((fm_decode_rows(d, quad) + FM_DEC_ROWS - 1) / FM_DEC_ROWS); }
 // floats of one batch*head's state: per group of four value columns num [Rp][4] then den [Rp], Rp = R rounded up to whole blocks
@@ -89,6 +89,7 @@ k_decode(TRef<const TIO> k, TRef<const TIO> v, TRef<const TIO> q, int n_new, int
       fm_decode_row<DH>(r, quad != 0, rm[i], rl[i], rlive[i], rmult[i]);
     }
   }
+  if (has_q && tid <= DH) qs[tid] = qreg;             // read after the barriers of the token loop
   for (int t0 = 0; t0 < n_new; t0 += TB) {
     FM_SYNC();
     for (int i = tid; i < TB * (DH + 1); i += FM_DEC_THREADS) {
@@ -124,9 +125,8 @@ k_decode(TRef<const TIO> k, TRef<const TIO> v, TRef<const TIO> q, int n_new, int
   }
   if (!has_q) return;
   // readout of the new token's query: the thread's rows, then the wavefront (a butterfly: every lane ends with the
-  // same sum), then the four wavefronts in order
-  if (tid <= DH) qs[tid] = qreg;
-  FM_SYNC();
+  // same sum), then the wavefronts in order
+  if (n_new <= 0) FM_SYNC();                           // (no token: qs has not met a barrier yet)
   float f[5] = {0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int i = 0; i < NI; ++i) {
@@ -147,16 +147,14 @@ k_decode(TRef<const TIO> k, TRef<const TIO> v, TRef<const TIO> q, int n_new, int
     for (int j = 0; j < 5; ++j) red[tid >> 6][j] = f[j];
   }
   FM_SYNC();
-  if (tid < 5) {
-    float sum = 0.f;
+  if (tid < 4) {
+    // each of the four output threads adds its column and the denominator itself (one barrier less than a shared sum)
+    float sum = 0.f, gs = 0.f;
 #pragma unroll
-    for (int w = 0; w < FM_DEC_THREADS / 64; ++w) sum += red[w][tid];
-    red[0][tid] = sum;
+    for (int w = 0; w < FM_DEC_THREADS / 64; ++w) { sum += red[w][tid]; gs += red[w][4]; }
+    IO<TIO>::st(o.base(bh) + c4 + tid, sum / gs);
+    if (tid == 0 && cb == 0) g.base(bh)[0] = gs;
   }
-  FM_SYNC();
-  const float gs = red[0][4];
-  if (tid < 4) IO<TIO>::st(o.base(bh) + c4 + tid, red[0][tid] / gs);
-  if (tid == 0 && cb == 0) g.base(bh)[0] = gs;
 }
 
 // ------------------------------------------------------------------------------
