@@ -172,7 +172,7 @@ int fastmax_backward_saved(const FastmaxDesc* desc, const void* q, const void* k
  *   fastmax_decode_absorb: adds desc->nk tokens (k, v: strides sk, sv) to the state, e.g. a prompt whose
  *     own outputs come from fastmax_forward.  One launch.  bf16 tensors at d = 64, order 2, 64 tokens or more:
  *     summed with matrix instructions on _Float16 operands (k', and the products v k'), fp32 sums (4 096 tokens
- *     at 16 batch*heads: 0.13 ms); otherwise token after token in fp32.
+ *     at 16 batch*heads: 0.10 ms); otherwise token after token in fp32.
  *   fastmax_decode_step: adds one token (k, v) and reads the state out for its query q (strides sq; the
  *     query sees its own key, as in causal attention): o (strides so, one token) and g (sg).  scratch is
  *     not used any more (a step is one launch; the argument and fastmax_decode_scratch_bytes stay for

@@ -83,6 +83,9 @@ int main() {
   bad |= run_pointwise(2, 70, 32, FASTMAX_F32);
   bad |= run_decode(2, 64, 2, 37, 2, FASTMAX_BF16);
   bad |= run_decode(3, 32, 1, 5, 2, FASTMAX_F32);
+  bad |= run_decode(1, 64, 2, 150, 1, FASTMAX_BF16);  // a prompt summed with matrix instructions (two tiles, the second ragged)
+  bad |= run(1, 300, 64, 2, 256, FASTMAX_BF16, 1);    // order-2 walk held per value column (two segments), saved and rebuilt
+  bad |= run(1, 300, 64, 2, 256, FASTMAX_BF16, 0);
   bad |= run(1, 600, 32, 2, 256, FASTMAX_BF16, 1);    // order-2 walk (a CU to itself: two buffers), both walks
   bad |= run(1, 600, 32, 2, 256, FASTMAX_BF16, 0);
   bad |= run(1, 520, 64, 2, 256, FASTMAX_BF16, 1);
