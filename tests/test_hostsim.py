@@ -263,6 +263,25 @@ def test_prompt_absorbed_with_matrix_instructions(sim):
     assert float(((s1 - s2).abs() / s2.abs().clamp_min(1e-30))[live].max()) < 5e-3      # operands rounded to _Float16
 
 
+def test_bf16_value_range_on_the_cpu(sim):
+    # the range of v the header states for bf16 tensors: 1e2 within the bar, beyond it within the bar or not finite
+    import math
+    bh, n, d = 1, 70, 32
+    tau = 8.0 * math.sqrt(d)
+    for vs, inside in ((1e2, True), (1e3, False), (1e4, False)):
+        gen = torch.Generator().manual_seed(3)
+        q, k = (torch.randn(bh, n, d, generator=gen).bfloat16() for _ in range(2))
+        v = (vs * torch.randn(bh, n, d, generator=gen)).bfloat16()
+        go = torch.randn(bh, n, d, generator=gen).bfloat16()
+        kw = dict(mask=True, inv_tau=1.0 / tau, p=2)
+        o, g, ws = sim.forward(q, k, v, save=True, **kw)
+        grads = sim.backward(q, k, v, o, g, go, saved=ws, **kw)
+        ref = oracle_all(q, k, v, go, mask=True, tau=tau, p=2)
+        for x, r in zip((o, g) + tuple(grads), ref):
+            ok = rel_err(x, r) < TOL[torch.bfloat16]
+            assert ok if inside else (ok or not bool(torch.isfinite(x).all())), f"v x {vs:g}"
+
+
 def test_order1_segment_backward_in_one_pass(sim):
     # beyond 1024 tokens order 1 on _Float16 runs in 128-token segments and k_o1_bwd makes dq, dk, dv of a segment
     # in one workgroup (9 segments here, the last one ragged); also with the folded normalisation's Jacobian
