@@ -99,7 +99,10 @@ typedef struct FastmaxNormFold {
 typedef struct FastmaxDesc {
   int32_t bh;        /* batch * heads */
   int32_t nq, nk;    /* query and key/value tokens */
-  int32_t d;         /* head size, D == Dv; 32 or 64 */
+  int32_t d;         /* head size, D == Dv; 32 or 64.  Also 128 for bf16 tensors on the _Float16 kernels (no
+                        FASTMAX_FLAG_F32_COMPUTE, a0 > 0): dense tiles at any length (at that width the moment form
+                        only pays beyond about D^2 keys), no normalisation fold, no causal nk > nq, no decoding state,
+                        no FORCE_MOMENTS; anything else at 128 is FASTMAX_ERR_UNSUPPORTED */
   int32_t dtype;     /* FASTMAX_F32 or FASTMAX_BF16: element type of q,k,v,o,dO,dq,dk,dv */
   int32_t mask;
   int32_t p;         /* 1 or 2 */

@@ -36,21 +36,25 @@ __all__ = [
 CENTRE_NONE, CENTRE_FEATURE, CENTRE_TOKEN = 0, 1, 2
 
 
-_HEAD_SIZES = (32, 64)      # what the kernels are built for
+_HEAD_SIZES = (32, 64)      # what every kernel is built for
+_WIDE_HEAD = 128            # bf16 attention alone also runs at this width (dense tiles; no normalisation or decoding kernels)
 
 
-def _pad_features(x):
+def _pad_features(x, wide=False):
     """x itself, or a copy zero-padded along the feature axis to the next head size the kernels
     are built for.  Zero features change neither q.k nor any norm, padded value columns come out
     as zero output columns, and the padded columns of every gradient are zero as well, so callers
-    pad on the way in and slice on the way out."""
+    pad on the way in and slice on the way out.  ``wide``: the caller's kernels also exist at 128
+    (attention on bf16 tensors)."""
     d = x.shape[-1]
-    for size in _HEAD_SIZES:
+    sizes = _HEAD_SIZES + ((_WIDE_HEAD,) if wide and x.dtype == torch.bfloat16 else ())
+    for size in sizes:
         if d == size:
             return x
         if d < size:
             return torch.nn.functional.pad(x, (0, size - d))
-    raise RuntimeError(f"fastmax: unsupported head size {d} (the kernels cover up to {_HEAD_SIZES[-1]})")
+    raise RuntimeError(f"fastmax: unsupported head size {d} for {x.dtype} (the kernels cover up to {_HEAD_SIZES[-1]}, "
+                       f"attention on bfloat16 tensors up to {_WIDE_HEAD})")
 
 
 class FastmaxNormalize(torch.autograd.Function):
@@ -175,7 +179,7 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
     ``normalize`` the tensors are first mapped to ``lim * x / max_n ||x_n||`` (the
     semantics spelled out in ``transformer/model.py:97-102``) and, like the reference,
     the returned gradients are those with respect to the normalised q and k.  Head sizes other
-    than 32 and 64 (up to 64) run zero-padded to the next of the two.
+    than 32 and 64 (up to 64; on bfloat16 tensors up to 128) run zero-padded to the next size the kernels have.
     """
 
     @staticmethod
@@ -185,9 +189,15 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
             raise ValueError("q, k, and v should be either 3 or 4 dimensional tensors. "
                              "If 3D: (b*h,n,d), if 4D: (b,h,n,d).")
         d = q.shape[-1]
-        q, k, v = _pad_features(q), _pad_features(k), _pad_features(v)
+        q, k, v = _pad_features(q, True), _pad_features(k, True), _pad_features(v, True)
         inv_tau = 1.0 / float(temperature)
         ctx.fold = None
+        if normalize and q.shape[-1] > _HEAD_SIZES[-1]:
+            # no normalisation kernels at that width: the scaling itself (lim * x / max_n ||x_n||, transformer/model.py:97-102)
+            # as tensor operations; like the reference, the gradients returned are those of the normalised q and k
+            q = q * (float(lim) / q.float().norm(dim=-1).amax(dim=-1)[..., None, None]).to(q.dtype)
+            k = k * (float(lim) / k.float().norm(dim=-1).amax(dim=-1)[..., None, None]).to(k.dtype)
+            normalize = False
         if normalize and _fold_possible(q, k, mask):
             # normalised on load; like the reference, the backward returns the gradients with respect to the
             # normalised q and k (its extension has no backward of apply_norm)
@@ -224,7 +234,7 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
             return (gq[..., :d], gk[..., :d], gv[..., :d]) + (None,) * 11
         q, k, v, o, g, saved = ctx.saved_tensors
         if q.shape[-1] != d:
-            grad_output = _pad_features(grad_output)
+            grad_output = _pad_features(grad_output, True)
         gq, gk, gv = _ext.backward_saved(q, k, v, o, g, grad_output, saved, mask, inv_tau, a0, a1, a2, p, 0, 0)
         return (gq[..., :d], gk[..., :d], gv[..., :d]) + (None,) * 11
 

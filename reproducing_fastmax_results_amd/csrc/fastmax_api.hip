@@ -12,6 +12,8 @@
 #if defined(FM_BENCH_AIDS)
 #include "fm_bench_aids.h"
 #endif
+// the one head size beyond 64: served by the _Float16 token kernels on dense tiles (see validate)
+static constexpr int FM_WIDE_HEAD = 128;
 #include <atomic>
 #include <cmath>
 #include <mutex>
@@ -136,7 +138,14 @@ int validate(const FastmaxDesc* d) {
   // assumes token counts and the segment length stay below 2^30
   if (d->nq > (1 << 30) || d->nk > (1 << 30) || d->chunk > (1 << 30)) return FASTMAX_ERR_SHAPE;
   if (d->p != 1 && d->p != 2) return FASTMAX_ERR_UNSUPPORTED;
-  if (d->d != 32 && d->d != 64) return FASTMAX_ERR_UNSUPPORTED;
+  if (d->d != 32 && d->d != 64 && d->d != FM_WIDE_HEAD) return FASTMAX_ERR_UNSUPPORTED;
+  if (d->d == FM_WIDE_HEAD) {
+    // heads of 128: bf16 tensors on the _Float16 kernels, dense tiles only (no moment states, no normalisation fold,
+    // no causal nk > nq): at that width the moment form only pays beyond about D^2 = 16 384 keys
+    if (d->dtype != FASTMAX_BF16 || (d->flags & FASTMAX_FLAG_F32_COMPUTE) || !(d->a0 > 0.0f)) return FASTMAX_ERR_UNSUPPORTED;
+    if (d->norm.q_keys || d->norm.k_keys || (d->mask && d->nk > d->nq)) return FASTMAX_ERR_UNSUPPORTED;
+    if (d->flags & FASTMAX_FLAG_FORCE_MOMENTS) return FASTMAX_ERR_UNSUPPORTED;
+  }
   if (d->mask && d->nq > d->nk) return FASTMAX_ERR_UNSUPPORTED;   // nk > nq: see SplitPlan
   if (d->chunk < 0) return FASTMAX_ERR_SHAPE;
   if (!(d->inv_tau > 0.0f) || !(d->inv_tau < 3.0e38f)) return FASTMAX_ERR_SHAPE;   // also rejects NaN
@@ -170,7 +179,7 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
   p.a1 = d->a1;
   p.a2 = p.quad ? d->a2 : 0.0f;
   p.sc = std::sqrt(std::fabs(d->inv_tau));
-  const bool force_dense = (d->flags & FASTMAX_FLAG_FORCE_DENSE) != 0;
+  const bool force_dense = (d->flags & FASTMAX_FLAG_FORCE_DENSE) != 0 || d->d == FM_WIDE_HEAD;
   if (d->mask) {
     // Segment length.  Dense tiles cost grows with L, the moment states cost the same per token
     // whatever L is (readout) plus the walk that builds them.  Measured on MI355X (D = 64, bf16):
@@ -199,7 +208,7 @@ int make_plan(const FastmaxDesc* d, Plan& p) {
     // f = (h^2 + kc) / (4 a2) with h = 2 a2 s + a1: worth it, and safe in _Float16, when a2 and kc are of ordinary size
     const float kc = 4.0f * p.a0 * p.a2 - p.a1 * p.a1;
     p.qf = p.half && p.quad && !p.use_state && std::fabs(p.a2) >= 0.0625f && std::fabs(p.a2) <= 4.0f &&
-           std::fabs(kc) <= 1024.0f && std::fabs(p.a1) <= 64.0f;
+           std::fabs(kc) <= 1024.0f && std::fabs(p.a1) <= 64.0f && d->d <= 64;
   }
   {
     // _Float16, D = 64, and enough batch*heads that one walk per (four values, batch*head) fills the chip; smaller
@@ -370,6 +379,7 @@ template <typename E, int DH, int QT> size_t tok_lds_bytes(int kind) {
   size_t region = size_t(2) * (kind == 0 ? C::SLAB_SYM : C::SLAB) * sizeof(E);   // k_pv reads its states with fm_readout_sym
   const size_t zs = size_t(C::NZ) * DH * C::PS * sizeof(E);
   if (zs > region) region = zs;
+  if (C::WIDE) region = 0;                             // no states at that width
   size_t body = size_t(C::QW) * C::PQ * sizeof(E) + region;
   const size_t outst = size_t(C::QW) * fm_store_pitch(DH) * 4;
   const size_t stage = kind == 0 ? size_t(2) * C::PV_STAGE * sizeof(E)
@@ -482,7 +492,7 @@ int run_forward_o1(const FastmaxDesc* d, const Plan& p, const void* q, const voi
 template <typename TIO, typename E, int DH, int QT>
 int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* k, const void* v, void* o,
                 float* g, char* ws, fm_stream_t stream) {
-  if constexpr (sizeof(E) == 2) {
+  if constexpr (sizeof(E) == 2 && DH <= 64) {
     if (p.o1) return run_forward_o1<TIO, DH>(d, p, q, k, v, o, g, ws, stream);
   }
   E* kt = reinterpret_cast<E*>(ws + p.kt);
@@ -497,6 +507,7 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   int st = launch_transpose2<TIO, E, DH>(v, d->sv, vt, vr, 1.0f, no_fold, k, d->sk, kt, kr, p.sc, k_fold(d), d->bh, d->nk,
                                          p.npad_k, stream);
   if (st) return st;
+  if constexpr (DH <= 64) {
   if (p.use_state) {
     BuildArgs<E> b;
     b.seg_parallel = 0; b.skip_big = 0;
@@ -523,6 +534,7 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
     if (!walked) st = launch_build<E, DH>(b, d->bh, stream);
     if (st) return st;
   }
+  }
   TokArgs<TIO, E> a;
   tok_common(a, d, p);
   a.own_io = cref<TIO>(q, d->sq);
@@ -535,9 +547,11 @@ int run_forward(const FastmaxDesc* d, const Plan& p, const void* q, const void* 
   if (p.keep_resid) a.out_resid = reinterpret_cast<fm_half*>(ws + p.ores);
   // order-2 states: two tiles per wavefront halve the state bytes a token reads (forward 1.38 -> 0.94 ms
   // at B*H = 16, N = 65536 on MI355X); without states one tile per wavefront and more workgroups per CU win
-  if (sizeof(E) == 2 && p.use_state && p.quad)
-    return launch_pv<TIO, E, DH, (sizeof(E) == 2 ? 2 : QT), FM_OWN_Q>(a, d->bh, FM_K_FWD, stream);
-  if constexpr (sizeof(E) == 2) {
+  if constexpr (DH <= 64) {
+    if (sizeof(E) == 2 && p.use_state && p.quad)
+      return launch_pv<TIO, E, DH, (sizeof(E) == 2 ? 2 : QT), FM_OWN_Q>(a, d->bh, FM_K_FWD, stream);
+  }
+  if constexpr (sizeof(E) == 2 && DH <= 64) {
     if (p.qf) return launch_pv<TIO, E, DH, 1, FM_OWN_Q, 1>(a, d->bh, FM_K_FWD, stream);
   }
   return launch_pv<TIO, E, DH, QT, FM_OWN_Q>(a, d->bh, FM_K_FWD, stream);
@@ -664,6 +678,7 @@ static int forward_one(const FastmaxDesc* desc, const void* q, const void* k, co
   char* ws = static_cast<char*>(workspace);
   fm_stream_t stream = static_cast<fm_stream_t>(hip_stream);
   if (p.half) {
+    if (desc->d == FM_WIDE_HEAD) return run_forward<fm_bf16, fm_half, FM_WIDE_HEAD, 1>(desc, p, q, k, v, o, g, ws, stream);
     if (desc->d == 64) return run_forward<fm_bf16, fm_half, 64, 1>(desc, p, q, k, v, o, g, ws, stream);
     return run_forward<fm_bf16, fm_half, 32, 1>(desc, p, q, k, v, o, g, ws, stream);
   }
@@ -741,6 +756,7 @@ static int backward_one(const FastmaxDesc* desc, const void* q, const void* k, c
   const char* fws = static_cast<const char*>(fwd_ws);
   fm_stream_t stream = static_cast<fm_stream_t>(hip_stream);
   if (p.half) {
+    if (desc->d == FM_WIDE_HEAD) return run_backward_wide<fm_bf16, fm_half, FM_WIDE_HEAD>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);
     if (desc->d == 64) return run_backward<fm_bf16, fm_half, 64, 1>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);
     return run_backward<fm_bf16, fm_half, 32, 1>(desc, p, q, k, v, o, g, d_o, dq, dk, dv, fws, ws, stream);
   }

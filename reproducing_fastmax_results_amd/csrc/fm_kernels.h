@@ -1288,8 +1288,12 @@ struct TokCfg {
   // _Float16, QT = 2: two tiles per wavefront share every state fragment read from LDS and halve
   // the state bytes staged per token; used by k_ds when there are states to read (dQ + dK
   // 0.20 vs 0.23 ms at the same shape with 1024-token segments).
-  static constexpr int OCC_PV = sizeof(E) == 2 ? (QT == 1 ? 4 : 2) : 1;   // workgroups per CU the kernels are sized for
-  static constexpr int OCC_DS = sizeof(E) == 2 ? (QT == 1 ? 3 : 2) : 1;
+  // Heads wider than 64 (DH = 128, _Float16, dense tiles only: see FM_WIDE_HEAD in fastmax_api.hip) hold twice the
+  // accumulators and own fragments: two workgroups per CU for k_pv, one for k_ds.
+  static constexpr bool WIDE = DH > 64;
+  static constexpr int OCC_PV = WIDE ? 2 : (sizeof(E) == 2 ? (QT == 1 ? 4 : 2) : 1);   // workgroups per CU the kernels are sized for
+  static constexpr int OCC_DS = WIDE ? 1 : (sizeof(E) == 2 ? (QT == 1 ? 3 : 2) : 1);
+  static constexpr int OCC_DV = WIDE ? 1 : 2;
   static constexpr int SA = sizeof(E) == 2 ? QT : 2;                      // values of a per state slab
   static constexpr int KT_PV = sizeof(E) == 2 ? 32 : 64;   // stream tokens per stage of the dense loop, k_pv
   static constexpr int KT_DS = 64;                        //                                           k_ds

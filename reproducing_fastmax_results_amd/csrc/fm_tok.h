@@ -579,7 +579,7 @@ FM_DEVICE void fm_readout_kv(const E* FM_RESTRICT state2, const E* xs, int xrow,
 // QF = 1 (order 2 without states, _Float16): completed-square weights and seeded accumulators (see
 // TileMath<fm_half>::dsq / bothq); the host picks it when a2 is of ordinary size.
 template <typename TIO, typename E, int DH, int QT, int OWN, int DV, int PREP, int QF = 0>
-FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? 2 : TokCfg<E, DH, QT>::OCC_DS)) k_ds(TokArgs<TIO, E> A) {
+FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? TokCfg<E, DH, QT>::OCC_DV : TokCfg<E, DH, QT>::OCC_DS)) k_ds(TokArgs<TIO, E> A) {
   static_assert(!QF || (QT == 1 && sizeof(E) == 2 && (DV != 0 || OWN == FM_OWN_Q)), "completed-square weights: dQ, or dK with dV, one tile per wavefront");
   typedef TokCfg<E, DH, QT> C;
   typedef Mma<E> M;

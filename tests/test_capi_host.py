@@ -76,6 +76,18 @@ def test_workspace_sizes_and_status_codes(lib):
     st, f, b = ws(lib, base_desc())
     assert st == 0 and f >= 256 and b >= f
     assert ws(lib, base_desc(d=48))[0] == 3          # unsupported head size
+    # heads of 128: bf16 tensors on the _Float16 kernels, dense tiles only
+    st3, f3, b3 = ws(lib, base_desc(d=128))
+    assert st3 == 0 and f3 >= 2 * 4 * 256 * 128 * 2                      # the converted k and v
+    assert ws(lib, base_desc(d=128, dtype=_capi.F32))[0] == 3
+    assert ws(lib, base_desc(d=128, flags=_capi.FLAG_F32_COMPUTE))[0] == 3
+    assert ws(lib, base_desc(d=128, flags=_capi.FLAG_FORCE_MOMENTS, mask=0))[0] == 3
+    assert ws(lib, base_desc(d=128, a0=0.0))[0] == 3                     # would need the fp32 kernels
+    assert ws(lib, base_desc(d=128, nk=256))[0] == 3                     # causal with more keys than queries
+    assert ws(lib, base_desc(d=128, nk=256, mask=0))[0] == 0
+    long128 = ws(lib, base_desc(d=128, nq=16384, nk=16384))
+    assert long128[0] == 0 and long128[2] < 8 * 4 * 16384 * 128 * 2     # copies of the tensors, no states
+    assert ws(lib, base_desc(d=256))[0] == 3
     assert ws(lib, base_desc(p=3))[0] == 3           # unsupported order
     assert ws(lib, base_desc(nq=256))[0] == 3        # masked needs nq <= nk
     st2, f2, b2 = ws(lib, base_desc(nk=256))         # masked, more keys than queries: two parts and a merge

@@ -364,6 +364,36 @@ def test_other_head_sizes_run_padded(sf, d, normalize):
 
 
 
+@pytest.mark.parametrize("d", [100, 128])
+@pytest.mark.parametrize("normalize", [False, True])
+def test_wide_heads_on_bf16(sf, d, normalize):
+    """Heads of up to 128 on bfloat16 tensors through the autograd wrapper (100: zero-padded to 128), with and without
+    the normalisation (at that width the scaling is tensor operations; gradients of the normalised q, k as always)."""
+    b, h, n, t = 2, 2, 400, 6.0
+    q, k, v, go = (rnd(b, h, n, d, seed=s).bfloat16() for s in (80, 81, 82, 83))
+    qd, kd, vd = (x.to(DEV).requires_grad_(True) for x in (q, k, v))
+    o = sf.FASTMultiHeadAttention_Function.apply(qd, kd, vd, None, None, True, 0.0, normalize, t, 1.0, 1.0, 0.5, 1.5, 2)
+    assert o.shape == (b, h, n, d) and o.dtype == torch.bfloat16
+    o.backward(go.to(DEV))
+    qr, kr, vr = (x.double().requires_grad_(True) for x in (q, k, v))
+    if normalize:
+        # the wrapper scales bf16 tensors by a bf16 factor: the same rounded factor here
+        fq = (1.5 / q.float().norm(dim=-1).amax(dim=-1)[..., None, None]).bfloat16().double()
+        fk = (1.5 / k.float().norm(dim=-1).amax(dim=-1)[..., None, None]).bfloat16().double()
+        qn, kn = (qr * fq).bfloat16().double(), (kr * fk).bfloat16().double()
+        qn.requires_grad_(True); kn.requires_grad_(True)
+    else:
+        qn, kn = qr, kr
+    qn.retain_grad(); kn.retain_grad()
+    oref, _ = O.closed_form_forward(qn, kn, vr, mask=True, tau=t, p=2)
+    oref.backward(go.double())
+    assert rel_err(o, oref) < TOL[torch.bfloat16]
+    for got, want in ((qd.grad, qn.grad), (kd.grad, kn.grad), (vd.grad, vr.grad)):
+        assert got.shape == want.shape and rel_err(got, want) < TOL[torch.bfloat16]
+    with pytest.raises(RuntimeError, match="unsupported head size"):
+        sf.FASTMultiHeadAttention_Function.apply(*(rnd(1, 1, 8, 130).bfloat16().to(DEV) for _ in range(3)))
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("shape", [(2, 3, 333, 64), (5, 700, 32), (1, 1, 1, 64)])
 def test_dormant_steps_kernels(dtype, shape):

@@ -286,6 +286,26 @@ def test_incremental_decoding_on_the_moment_state(lib, dtype, p, d):
     assert rel_err(o, o2) < TOL[dtype] and rel_err(g, g2) < TOL[dtype]
 
 
+@pytest.mark.parametrize("p", [1, 2])
+@pytest.mark.parametrize("mask", [True, False])
+def test_heads_of_128(lib, p, mask):
+    """bf16 tensors at D = 128 (dense tiles only): forward and backward, saved and not, ragged lengths, unequal nq and
+    nk without a mask, a sequence long enough that D = 64 would use states, and the statuses of what it leaves out."""
+    print(f"case heads of 128 p={p} mask={mask}", flush=True)
+    check_forward_backward(lib, 3, 300, 128, torch.bfloat16, DEV, mask=mask, p=p, seed=120, saved=True)
+    check_forward_backward(lib, 2, 1000, 128, torch.bfloat16, DEV, mask=mask, p=p, seed=121, saved=False, tau_mult=1.0)
+    check_forward_backward(lib, 8, 2048, 128, torch.bfloat16, DEV, mask=mask, p=p, seed=122, saved=True)
+    if not mask:
+        check_forward_backward(lib, 2, 130, 128, torch.bfloat16, DEV, mask=False, p=p, nk=517, seed=123, saved=True)
+    else:
+        check_forward_backward(lib, 1, 8200, 128, torch.bfloat16, DEV, mask=True, p=p, seed=124, saved=True)
+        check_batch_head_strides(lib, 2, 3, 260, 128, torch.bfloat16, DEV, mask=True, p=p, seed=125)
+    from reproducing_fastmax_results_amd._capi import FastmaxError
+    q, k, v, go = (torch.randn(2, 64, 128, device=DEV) for _ in range(4))
+    with pytest.raises(FastmaxError):
+        lib.forward(q, k, v, mask=mask, inv_tau=0.1, p=p)                # fp32 tensors
+
+
 def test_prompt_absorbed_with_matrix_instructions(lib):
     """bf16 tensors, D = 64, order 2: prompts of 64 tokens and more are summed by k_decode_absorb_mma.  Decoding after
     a long prompt against the causal closed form; the state against the one k_decode builds from the same tokens in

@@ -282,6 +282,12 @@ def test_bf16_value_range_on_the_cpu(sim):
             assert ok if inside else (ok or not bool(torch.isfinite(x).all())), f"v x {vs:g}"
 
 
+def test_heads_of_128(sim):
+    # bf16 tensors, D = 128: the _Float16 token kernels on dense tiles, four accumulator tiles per feature axis
+    check_forward_backward(sim, 1, 70, 128, torch.bfloat16, "cpu", mask=True, p=2, seed=50, saved=True)
+    check_forward_backward(sim, 1, 40, 128, torch.bfloat16, "cpu", mask=False, p=1, nk=75, seed=51)
+
+
 def test_order1_segment_backward_in_one_pass(sim):
     # beyond 1024 tokens order 1 on _Float16 runs in 128-token segments and k_o1_bwd makes dq, dk, dv of a segment
     # in one workgroup (9 segments here, the last one ragged); also with the folded normalisation's Jacobian
