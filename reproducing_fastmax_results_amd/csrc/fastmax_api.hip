@@ -409,7 +409,7 @@ template <typename TIO, typename E> void tok_common(TokArgs<TIO, E>& a, const Fa
   a.quad = p.quad; a.a0 = p.a0; a.a1 = p.a1; a.a2 = p.a2; a.sc = p.sc; a.out_scale = 1.0f; a.zscale = 1.0f;
   a.own_o = TRef<const TIO>{nullptr, 0, 0, 0, 0, 0}; a.own_do = a.own_o;
   a.w_gh = nullptr; a.w_qr = nullptr; a.w_cv = nullptr; a.gpart = nullptr; a.gnblk = 0;
-  a.out_resid = nullptr; a.own_ores = nullptr; a.state_tr = 0; a.state_xscale = 1.0f;
+  a.out_resid = nullptr; a.own_ores = nullptr; a.state_xscale = 1.0f;
 }
 
 template <typename TIO, typename E, int DH, int QT, int OWN, int QF = 0>
@@ -423,13 +423,13 @@ int launch_pv(const TokArgs<TIO, E>& a, int bh, int kernel_id, fm_stream_t strea
   return fm_launch_status();
 }
 
-template <typename TIO, typename E, int DH, int QT, int OWN, int DV = 0, int PREP = 0, int QF = 0>
+template <typename TIO, typename E, int DH, int QT, int OWN, int DV = 0, int PREP = 0, int QF = 0, int STR = 0>
 int launch_ds(const TokArgs<TIO, E>& a, int bh, int kernel_id, fm_stream_t stream) {
   typedef TokCfg<E, DH, QT> C;
   const size_t lds = tok_lds_bytes<E, DH, QT>(PREP ? 3 : (DV ? (a.use_state ? 4 : 2) : 1));
-  fm_allow_lds(reinterpret_cast<const void*>(&k_ds<TIO, E, DH, QT, OWN, DV, PREP, QF>), lds);
+  fm_allow_lds(reinterpret_cast<const void*>(&k_ds<TIO, E, DH, QT, OWN, DV, PREP, QF, STR>), lds);
   ProfScope prof(kernel_id, stream);
-  FM_KERNEL_LAUNCH((k_ds<TIO, E, DH, QT, OWN, DV, PREP, QF>), fm_dim3((a.n_own + C::QW - 1) / C::QW, bh), fm_dim3(FM_THREADS), lds,
+  FM_KERNEL_LAUNCH((k_ds<TIO, E, DH, QT, OWN, DV, PREP, QF, STR>), fm_dim3((a.n_own + C::QW - 1) / C::QW, bh), fm_dim3(FM_THREADS), lds,
                    stream, a);
   return fm_launch_status();
 }

@@ -67,7 +67,7 @@ template <typename TIO, typename E> struct TokArgs {
   fm_half* out_resid; const fm_half* own_ores;
   // k_ds, own = queries, _Float16: the prefix state is the forward's own layout (slab a = [v][k], see fm_readout's
   // TRA) and its order-2 part is to be counted state_xscale times
-  int state_tr; float state_xscale;
+  float state_xscale;
 };
 
 // eight values as they will read back from the caller's tensor: themselves (fp32) or rounded to bf16
@@ -578,8 +578,12 @@ FM_DEVICE void fm_readout_kv(const E* FM_RESTRICT state2, const E* xs, int xrow,
 // ------------------------------------------------------------------------------
 // QF = 1 (order 2 without states, _Float16): completed-square weights and seeded accumulators (see
 // TileMath<fm_half>::dsq / bothq); the host picks it when a2 is of ordinary size.
-template <typename TIO, typename E, int DH, int QT, int OWN, int DV, int PREP, int QF = 0>
+// STR = 1 (own = queries, _Float16, two tiles per wavefront): the prefix state is the forward's own layout and is
+// read out transposed (see fm_readout, TRA); the fragments of the dense tiles are fetched behind that readout, so that
+// the kernel holds 64 registers fewer across it.
+template <typename TIO, typename E, int DH, int QT, int OWN, int DV, int PREP, int QF = 0, int STR = 0>
 FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? TokCfg<E, DH, QT>::OCC_DV : TokCfg<E, DH, QT>::OCC_DS)) k_ds(TokArgs<TIO, E> A) {
+  static_assert(!STR || (OWN == FM_OWN_Q && sizeof(E) == 2 && !PREP && !QF && !DV), "the transposed readout is dQ's, on _Float16");
   static_assert(!QF || (QT == 1 && sizeof(E) == 2 && (DV != 0 || OWN == FM_OWN_Q)), "completed-square weights: dQ, or dK with dV, one tile per wavefront");
   typedef TokCfg<E, DH, QT> C;
   typedef Mma<E> M;
@@ -689,16 +693,23 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? TokCfg<E, DH, QT>::OCC_DV : T
                                       : A.cv[int64_t(bh) * A.npad_own + t0 + M::tperm(xrow[j])]) : 1.0f;
   }
   frag of[QT][NKS], of2[QT][NKS];
+  auto load_of = [&]() FM_ALWAYS_INLINE {
 #pragma unroll
-  for (int j = 0; j < QT; ++j) {
-    const E* o2 = PREP ? R + xrow[j] * PQ + lh * M::KPL
-                       : A.own2_r + (int64_t(bh) * A.npad_own + t0 + xrow[j]) * DH + lh * M::KPL;
+    for (int j = 0; j < QT; ++j)
 #pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) {
-      of[j][ks] = M::load(Own + xrow[j] * PQ + ks * M::KSTEP + lh * M::KPL);
-      of2[j][ks] = M::load(o2 + ks * M::KSTEP);
+      for (int ks = 0; ks < NKS; ++ks) of[j][ks] = M::load(Own + xrow[j] * PQ + ks * M::KSTEP + lh * M::KPL);
+  };
+  auto load_of2 = [&]() FM_ALWAYS_INLINE {
+#pragma unroll
+    for (int j = 0; j < QT; ++j) {
+      const E* o2 = PREP ? R + xrow[j] * PQ + lh * M::KPL
+                         : A.own2_r + (int64_t(bh) * A.npad_own + t0 + xrow[j]) * DH + lh * M::KPL;
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) of2[j][ks] = M::load(o2 + ks * M::KSTEP);
     }
-  }
+  };
+  load_of();
+  if (!STR) load_of2();
   fm_f32x16 sseed = fm_zero16(), dpseed = fm_zero16();
   if constexpr (QF != 0) {
     // the score products deliver h = 2 a2 s + a1; the gh.v products start from -c (own = queries: the lane's own c)
@@ -770,24 +781,24 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? TokCfg<E, DH, QT>::OCC_DV : T
         FM_SYNC();                                     // the slabs and dks are overwritten by the dense stages
       }
     } else {
-      bool done = false;
-      if constexpr (OWN == FM_OWN_Q && M::HAS_TR) {
-        if (A.state_tr) {
-          // gh of the own queries in the k order of the transposing reads
-          frag ofp[QT][NKS];
+      if constexpr (STR != 0) {
+        // gh of the own queries in the k order of the transposing reads
+        frag ofp[QT][NKS];
 #pragma unroll
-          for (int j = 0; j < QT; ++j) {
-            const E* o2 = PREP ? R + xrow[j] * PQ : A.own2_r + (int64_t(bh) * A.npad_own + t0 + xrow[j]) * DH;
+        for (int j = 0; j < QT; ++j) {
+          const E* o2 = A.own2_r + (int64_t(bh) * A.npad_own + t0 + xrow[j]) * DH;
 #pragma unroll
-            for (int ks = 0; ks < NKS; ++ks) ofp[j][ks] = M::load_nat_perm(o2, ks, lh);
-          }
-          fm_readout<E, DH, QT, NT, true>(state, A.quad != 0, Own, xrow, ofp, R, acc, tid, A.state_xscale);
-          done = true;
+          for (int ks = 0; ks < NKS; ++ks) ofp[j][ks] = M::load_nat_perm(o2, ks, lh);
         }
+        fm_readout<E, DH, QT, NT, true>(state, A.quad != 0, Own, xrow, ofp, R, acc, tid, A.state_xscale);
+        load_of(); load_of2();                         // the own rows are still in LDS (fm_readout ends on a barrier)
+        FM_SYNC();                                     // ... and are overwritten by the dense stages
+      } else {
+        fm_readout<E, DH, QT, NT>(state, A.quad != 0, Own, xrow, of2, R, acc, tid);
       }
-      if (!done) fm_readout<E, DH, QT, NT>(state, A.quad != 0, Own, xrow, of2, R, acc, tid);
     }
   } else {
+    if (STR) load_of2();                               // (a workgroup of the first segment: no state, no readout)
     FM_SYNC();                                         // own rows are overwritten by the dense stages
   }
 

@@ -92,6 +92,8 @@ int main() {
   bad |= run(1, 1100, 32, 1, 0, FASTMAX_BF16, 1);     // order-1 runs of segments
   bad |= run(3, 1300, 64, 1, 0, FASTMAX_BF16, 0);
   bad |= run(2, 200, 64, 2, 0, FASTMAX_BF16, 1);      // one segment, dense kernels
+  bad |= run(1, 200, 128, 2, 0, FASTMAX_BF16, 1);     // heads of 128: four accumulator tiles per feature axis
+  bad |= run(1, 150, 128, 1, 0, FASTMAX_BF16, 0);
   bad |= run(1, 300, 32, 2, 256, FASTMAX_F32, 1);
   return bad;
 }
