@@ -708,8 +708,10 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? TokCfg<E, DH, QT>::OCC_DV : T
       for (int ks = 0; ks < NKS; ++ks) of2[j][ks] = M::load(o2 + ks * M::KSTEP);
     }
   };
+  // LATE2: the second set is fetched where it is first needed (behind or late in the state readout), not held across it
+  constexpr bool LATE2 = STR != 0 || (DV != 0 && OWN == FM_OWN_K && QT == 1 && sizeof(E) == 2 && !QF);
   load_of();
-  if (!STR) load_of2();
+  if (!LATE2) load_of2();
   fm_f32x16 sseed = fm_zero16(), dpseed = fm_zero16();
   if constexpr (QF != 0) {
     // the score products deliver h = 2 a2 s + a1; the gh.v products start from -c (own = queries: the lane's own c)
@@ -760,6 +762,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? TokCfg<E, DH, QT>::OCC_DV : T
           }
       }
       fm_readout_kv<E, DH>(state2, Own, xrow[0], of[0], vacc, R, dks, av[0], tid);
+      load_of2();
       {
         TileRegs<E, DH, DH> s1, s1b;
         s1.load(state + int64_t(DH) * DH * DH, DH, tid);
@@ -798,7 +801,7 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? TokCfg<E, DH, QT>::OCC_DV : T
       }
     }
   } else {
-    if (STR) load_of2();                               // (a workgroup of the first segment: no state, no readout)
+    if (LATE2) load_of2();                             // (a workgroup without a state: no readout)
     FM_SYNC();                                         // own rows are overwritten by the dense stages
   }
 
