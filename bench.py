@@ -44,11 +44,11 @@ PEAK_HBM_GBS = 8000.0
 # (N, order, dtype, --chunk, kernel).  A constant, not a live measurement: it belongs to the kernels as they
 # were when the named summary was made.
 TRAFFIC = {
-    (4096, 2, "bf16", 0, "dkv"): {"bytes": int((42456.4 * 2 + 32768.4) * 1024), "source": "profiles/c2_bf16_hbm_traffic.md"},
+    (4096, 2, "bf16", 0, "dkv"): {"bytes": int((42622.6 * 2 + 32768.1) * 1024), "source": "profiles/c2_bf16_hbm_traffic.md"},
     (4096, 2, "f32", 0, "dk"): {"bytes": int((324657.1 * 2 + 32768.9) * 1024), "source": "profiles/c2_fp32_kernel_trace.md"},
     (65536, 1, "bf16", 0, "dkv"): {"bytes": int((402949.3 * 2 + 393223.9) * 1024), "source": "profiles/long_order1_bf16_hbm_traffic.md"},
-    (65536, 2, "bf16", 0, "build"): {"bytes": int((130104.8 * 2 + 544651.2) * 1024), "source": "profiles/long_order2_bf16_hbm_traffic.md"},
-    (65536, 2, "bf16", 0, "dkv"): {"bytes": int((546856.1 * 2 + 262149.1) * 1024), "source": "profiles/long_order2_bf16_hbm_traffic.md"},
+    (65536, 2, "bf16", 0, "build"): {"bytes": int((130128.6 * 2 + 544747.5) * 1024), "source": "profiles/long_order2_bf16_hbm_traffic.md"},
+    (65536, 2, "bf16", 0, "dkv"): {"bytes": int((609337.0 * 2 + 262146.4) * 1024), "source": "profiles/long_order2_bf16_hbm_traffic.md"},
 }
 
 WORKLOAD = dict(name="configs[1]: causal order-2 fwd+bwd", B=4, H=8, N=4096, D=64, p=2, mask=True, scale=1.0)

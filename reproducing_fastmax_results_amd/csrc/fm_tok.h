@@ -710,8 +710,19 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS, (DV ? TokCfg<E, DH, QT>::OCC_DV : T
   };
   // LATE2: the second set is fetched where it is first needed (behind or late in the state readout), not held across it
   constexpr bool LATE2 = STR != 0 || (DV != 0 && OWN == FM_OWN_K && QT == 1 && sizeof(E) == 2 && !QF);
-  load_of();
-  if (!LATE2) load_of2();
+  if constexpr (LATE2) load_of();
+  else {
+#pragma unroll
+    for (int j = 0; j < QT; ++j) {
+      const E* o2 = PREP ? R + xrow[j] * PQ + lh * M::KPL
+                         : A.own2_r + (int64_t(bh) * A.npad_own + t0 + xrow[j]) * DH + lh * M::KPL;
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        of[j][ks] = M::load(Own + xrow[j] * PQ + ks * M::KSTEP + lh * M::KPL);
+        of2[j][ks] = M::load(o2 + ks * M::KSTEP);
+      }
+    }
+  }
   fm_f32x16 sseed = fm_zero16(), dpseed = fm_zero16();
   if constexpr (QF != 0) {
     // the score products deliver h = 2 a2 s + a1; the gh.v products start from -c (own = queries: the lane's own c)
