@@ -124,13 +124,19 @@ FM_GLOBAL void FM_LAUNCH_BOUNDS2(FM_THREADS + 64, 1) k_walk_sym(WalkSymArgs A) {
     constexpr int CH = 4 * DH * (DH / 8);                 // 16-byte chunks of a snapshot
     const int per_tile = (CH * TT / A.L + 63) / 64 * 64;  // chunks per tile: a segment's tiles cover the snapshot
     int pend_lo = CH, pend_snap = 0, pend_slot = 0, nsn = 0;
+    // chunk c = a * 32 + w * 8 + j (value of a, wavefront's column w, 16-byte piece j of the row): pend_lo is a multiple
+    // of 64, so a lane keeps its (w, j) and steps a by two from one chunk to its next -- one LDS read, one store and
+    // two additions per chunk (this wavefront shares its SIMD with a summing one: what it issues, that one waits for)
+    static_assert(4 * (DH / 8) == 32, "a lane's chunks differ in a only");
+    const int cp_w = (lane / (DH / 8)) % 4, cp_b8 = (lane % (DH / 8)) * 8, cp_a0 = lane / 32;
     auto copy = [&](int upto) {
-      const E* all = snap0 + (pend_snap & 1) * SNAP_E;
-      E* dst = A.o2 + (int64_t(bh) * A.nslots + pend_slot) * StateDims<DH>::BIG + int64_t(c0) * DH;
-      for (int c = pend_lo + lane; c < upto; c += 64) {
-        const int a = c / (4 * (DH / 8)), w = (c / (DH / 8)) % 4, b8 = (c % (DH / 8)) * 8;
-        *reinterpret_cast<fm_u32x4*>(dst + (int64_t(a) * DH + w) * DH + b8) =
-            *reinterpret_cast<const fm_u32x4*>(all + (w * DH + a) * SP + b8);
+      const int a = pend_lo / 32 + cp_a0;
+      const E* src = snap0 + (pend_snap & 1) * SNAP_E + (cp_w * DH + a) * SP + cp_b8;
+      E* dst = A.o2 + (int64_t(bh) * A.nslots + pend_slot) * StateDims<DH>::BIG + int64_t(c0) * DH +
+               (int64_t(a) * DH + cp_w) * DH + cp_b8;
+      for (int c = pend_lo; c < upto; c += 64) {
+        *reinterpret_cast<fm_u32x4*>(dst) = *reinterpret_cast<const fm_u32x4*>(src);
+        src += 2 * SP; dst += 2 * DH * DH;
       }
       pend_lo = upto;
     };
