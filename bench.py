@@ -4,7 +4,7 @@
     python bench.py --gpus 1 --steps K --warmup W
 
 One step = one forward + one backward of causal order-2 Fastmax on one batch of
-synthetic input (BASELINE.json configs[1]: B=4, H=8, N=4096, D=Dv=64, bf16,
+synthetic input (the configuration the metric is quoted on: B=4, H=8, N=4096, D=Dv=64, bf16,
 q, k, v, dO ~ N(0,1), tau = 8*sqrt(D), Taylor coefficients), inputs resident in
 HBM, called through the C ABI (libfastmax_hip.so).  Prints ONE JSON line.
 
@@ -286,7 +286,7 @@ def main() -> int:
 
 
 def c1_line(lib, dev, with_cpu):
-    """BASELINE configs[0]: order-2 forward, unmasked, fp32, B=1, H=2, N=256, D=Dv=32: the GPU call event-timed and the
+    """The small unmasked case (the one the reference can run on a CPU): order-2 forward, unmasked, fp32, B=1, H=2, N=256, D=Dv=32: the GPU call event-timed and the
     oracle's port of the reference's factorised path on the host cores, measured directly."""
     import torch
     from oracle import fastmax_oracle as O
@@ -320,7 +320,7 @@ def c1_line(lib, dev, with_cpu):
 
 
 def cpu_long_baselines():
-    """The oracle's port of the reference's factorised path on BASELINE configs[2] (B=1, H=16, N=65536, D=64), fp32,
+    """The oracle's port of the reference's factorised path on the long-context shape (B=1, H=16, N=65536, D=64), fp32,
     fwd+bwd, on a bounded sample: one head, a slice of the sequence, scaled linearly in N (the algorithm is linear in
     N) and by the 16 heads.  Order 1 would fit whole (1.07 GB per intermediate and head); order 2 would not (68.7 GB per
     intermediate and head): both are flagged as extrapolated."""

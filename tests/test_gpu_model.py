@@ -101,7 +101,7 @@ def adamw_step_compare(model_hip, model_ref, inputs, target, loss_fn, lr, max_si
 
 
 def test_vit_step_full_depth_fp32():
-    """BASELINE configs[3] at its real size: 4 blocks, 256 images, 49 patches + class token, d_model 128,
+    """The vision-transformer configuration at its real size: 4 blocks, 256 images, 49 patches + class token, d_model 128,
     4 heads of 32; loss, every parameter gradient, then one AdamW step."""
     from reproducing_fastmax_results_amd.transformer.model import vit_for_c4
     torch.manual_seed(13)
@@ -149,7 +149,7 @@ def _gpt_full_depth(dtype):
 
 
 def test_gpt_step_full_depth_fp32():
-    """BASELINE configs[4] at its real depth and context in fp32: 6 blocks, d_model 512, 8 heads of 64,
+    """The decoder-only language-model configuration at its real depth and context in fp32: 6 blocks, d_model 512, 8 heads of 64,
     16 x 1024 tokens (the vocabulary is cut to 512: embedding and head are torch's, not the operator's);
     loss, every parameter gradient, one AdamW step."""
     hip, ref, tokens, target = _gpt_full_depth(torch.float32)
