@@ -467,7 +467,9 @@ def operator_line(lib, dev, W, dtype, args, steps, warmup, full):
     import ctypes as C
     from reproducing_fastmax_results_amd._capi import _gstrides, _strides
 
-    def make_step(L):
+    def make_step(L, live_stream=False):
+        # live_stream: the stream is looked up at every call (under HIP graph capture torch's current stream is the
+        # capturing one, not the one this closure was made on)
         df = L.make_desc(q, k, v, flags=0 if indep else FLAG_SAVE_FOR_BACKWARD, **kw)
         df.so, df.sg = _strides(o), _gstrides(g)
         db = L.make_desc(q, k, v, flags=0 if indep else FLAG_SAVE_FOR_BACKWARD, **kw)
@@ -480,6 +482,9 @@ def operator_line(lib, dev, W, dtype, args, steps, warmup, full):
         fwd, bwd, bwds = L.lib.fastmax_forward, L.lib.fastmax_backward, L.lib.fastmax_backward_saved
 
         def step():
+            nonlocal stream
+            if live_stream:
+                stream = torch.cuda.current_stream().cuda_stream
             st = fwd(pf, ptr[0], ptr[1], ptr[2], ptr[3], ptr[4], ptr[9], nf, stream)
             if indep:
                 st |= bwd(pb, ptr[0], ptr[1], ptr[2], ptr[3], ptr[4], ptr[5], ptr[6], ptr[7], ptr[8], ptr[10], nb, stream)
@@ -489,7 +494,7 @@ def operator_line(lib, dev, W, dtype, args, steps, warmup, full):
                 raise RuntimeError(f"fastmax step failed with status {st}")
         return step
 
-    step = make_step(lib)
+    step = make_step(lib, live_stream=args.graph)
     from reproducing_fastmax_results_amd._capi import get_bench_lib
     blib = get_bench_lib()
     box = None
