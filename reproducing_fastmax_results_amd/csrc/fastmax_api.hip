@@ -628,7 +628,7 @@ int add_rows(const FastmaxDesc* d, const SplitPlan& sp, const void* dqa, void* d
 
 extern "C" {
 
-int fastmax_version(void) { return 200; }   // 0.2.0: FastmaxDesc gained `norm`; decode, static-scratch and statistics entry points
+int fastmax_version(void) { return 300; }   // 0.3.0: heads of 128 (bf16), the decoding state in its symmetric column-block layout (a state of 0.2.x is not readable), bench aids out of the product library
 
 const char* fastmax_status_string(int status) {
   switch (status) {
